@@ -1,0 +1,249 @@
+"""Pins the oracle's forward against brute force, library routines and the invariants of the
+maths -- chosen so that a dropped term, a wrong sign/index or a transposed operand fails."""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import hstu_oracle as O
+
+
+def _jag(rng, lens_q, nq, nk, dqk, dv, lens_k=None, dtype=torch.float32):
+    lens_k = lens_q if lens_k is None else lens_k
+    tq, tk = sum(lens_q), sum(lens_k)
+    q = torch.from_numpy(rng.normal(0, 0.5, (tq, nq, dqk))).to(dtype)
+    k = torch.from_numpy(rng.normal(0, 0.5, (tk, nk, dqk))).to(dtype)
+    v = torch.from_numpy(rng.normal(0, 0.5, (tk, nk, dv))).to(dtype)
+    oq = torch.tensor([0] + list(np.cumsum(lens_q)), dtype=torch.int64)
+    ok = torch.tensor([0] + list(np.cumsum(lens_k)), dtype=torch.int64)
+    return q, k, v, oq, ok
+
+
+@pytest.mark.parametrize("case", [
+    dict(lens_q=[3, 1, 5], nq=2, nk=2, dqk=4, dv=4),
+    dict(lens_q=[4, 0, 6], nq=4, nk=2, dqk=3, dv=5),                      # interior empty sequence, GQA, Dqk != Dv
+    dict(lens_q=[2, 4], lens_k=[5, 4], nq=2, nk=1, dqk=4, dv=2),          # delta-q
+    dict(lens_q=[6, 7], nq=1, nk=1, dqk=2, dv=2, ctx=[1, 2], tgt=[2, 3], tgs=1),
+    dict(lens_q=[8], nq=2, nk=2, dqk=2, dv=3, ctx=[2], tgt=[4], tgs=3, bias=True),
+    dict(lens_q=[5, 3], nq=2, nk=2, dqk=4, dv=4, mask_type=3, bias=True),
+    dict(lens_q=[5, 3], nq=2, nk=2, dqk=4, dv=4, mask_type=2),
+])
+def test_exact_vs_bruteforce(case):
+    rng = np.random.default_rng(7)
+    c = dict(case)
+    lens_q = c.pop("lens_q"); lens_k = c.pop("lens_k", None)
+    q, k, v, oq, ok = _jag(rng, lens_q, c["nq"], c["nk"], c["dqk"], c["dv"], lens_k)
+    mq, mk = max(max(lens_q), 1), max(max(lens_k or lens_q), 1)
+    mask_type = c.get("mask_type", 0)
+    bias = torch.from_numpy(rng.normal(0, 0.3, (len(lens_q), c["nq"], mq, mk))).float() if c.get("bias") else None
+    mask = torch.from_numpy(rng.integers(0, 2, (len(lens_q), c["nq"], mq, mk))).float() if mask_type == 3 else None
+    kw = dict(max_seq_len_q=mq + 3, mask_type=mask_type, mask=mask, attn_bias=bias, alpha=0.37, silu_scale=0.0,
+              num_context=c.get("ctx"), num_target=c.get("tgt"), target_group_size=c.get("tgs", 0))
+    ref = O.hstu_bruteforce(q, k, v, oq, ok, **kw)
+    got = O.hstu_jagged_forward(q, k, v, oq, ok, max_seq_len_k=mk, compute_dtype=torch.float64, **kw)
+    assert torch.allclose(got, ref, rtol=1e-12, atol=1e-13)
+    got32 = O.hstu_jagged_forward(q, k, v, oq, ok, max_seq_len_k=mk, **kw)
+    assert torch.allclose(got32.double(), ref, rtol=1e-5, atol=1e-6)
+
+
+def test_reduces_to_library_routines():
+    """One sequence, one head, no mask: out == (silu(alpha*(QK^T+bias))*scale) @ V by torch's own routines."""
+    rng = np.random.default_rng(1)
+    q, k, v, oq, ok = _jag(rng, [9], 1, 1, 8, 6)
+    bias = torch.from_numpy(rng.normal(0, 1, (1, 1, 9, 9))).float()
+    got = O.hstu_jagged_forward(q, k, v, oq, max_seq_len_q=9, mask_type=2, attn_bias=bias, alpha=0.5,
+                                silu_scale=0.25)
+    ref = (F.silu(0.5 * (q[:, 0] @ k[:, 0].T + bias[0, 0])) * 0.25) @ v[:, 0]
+    assert torch.allclose(got[:, 0], ref, rtol=1e-6, atol=1e-7)
+
+
+def _cfg(rng):
+    lens = [int(x) for x in rng.integers(4, 24, 5)]
+    return lens, _jag(rng, lens, 4, 2, 8, 8)
+
+
+def test_linearity_and_alpha_zero():
+    rng = np.random.default_rng(2)
+    lens, (q, k, v, oq, ok) = _cfg(rng)
+    f = lambda vv, sc=0.0, al=0.3: O.hstu_jagged_forward(q, k, vv, oq, max_seq_len_q=32, silu_scale=sc, alpha=al,
+                                                         compute_dtype=torch.float64)
+    v = v.double()
+    v2 = torch.from_numpy(rng.normal(0, 0.5, tuple(v.shape)))
+    assert torch.allclose(f(v + 2 * v2), f(v) + 2 * f(v2), rtol=1e-10, atol=1e-12)
+    assert torch.allclose(f(v, 0.5), 16 * f(v, 1 / 32), rtol=1e-10, atol=1e-12)
+    assert torch.equal(f(v, 0.0, 0.0), torch.zeros_like(f(v)))
+    # default silu_scale is 1/max_seq_len_q (the attribute, not the per-sequence length)
+    assert torch.allclose(f(v, 0.0), f(v, 1 / 32), rtol=1e-12, atol=0)
+
+
+def test_batch_permutation_and_causality():
+    rng = np.random.default_rng(3)
+    lens = [5, 9, 3]
+    q, k, v, oq, ok = _jag(rng, lens, 2, 2, 4, 4)
+    base = O.hstu_jagged_forward(q, k, v, oq, max_seq_len_q=16, alpha=0.7)
+    perm = [2, 0, 1]
+    segs = lambda x: [x[oq[i]:oq[i + 1]] for i in range(3)]
+    qp, kp, vp = (torch.cat([segs(x)[i] for i in perm]) for x in (q, k, v))
+    op = torch.tensor([0] + list(np.cumsum([lens[i] for i in perm])))
+    outp = O.hstu_jagged_forward(qp, kp, vp, op, max_seq_len_q=16, alpha=0.7)
+    assert torch.equal(torch.cat([segs(base)[i] for i in perm]), outp)
+    # row i depends only on K/V rows <= i: perturb the last 2 rows of sequence 1
+    k2, v2 = k.clone(), v.clone()
+    k2[oq[2] - 2: oq[2]] += 1.0; v2[oq[2] - 2: oq[2]] -= 1.0
+    out2 = O.hstu_jagged_forward(q, k2, v2, oq, max_seq_len_q=16, alpha=0.7)
+    assert torch.equal(out2[: oq[2] - 2], base[: oq[2] - 2]) and torch.equal(out2[oq[2]:], base[oq[2]:])
+    assert not torch.equal(out2[oq[2] - 2: oq[2]], base[oq[2] - 2: oq[2]])
+
+
+def test_dense_equals_jagged_and_explicit_tril_and_gqa():
+    rng = np.random.default_rng(4)
+    s = 11
+    q, k, v, oq, _ = _jag(rng, [s, s], 4, 2, 8, 8)
+    jag = O.hstu_jagged_forward(q, k, v, oq, max_seq_len_q=s)
+    # dense layout needs equal head counts: expand K/V heads first (also the GQA == repeat_interleave pin)
+    ke, ve = k.repeat_interleave(2, dim=1), v.repeat_interleave(2, dim=1)
+    assert torch.equal(O.hstu_jagged_forward(q, ke, ve, oq, max_seq_len_q=s), jag)
+    dense = O.hstu_dense_forward(q.reshape(2, s, 4, 8), ke.reshape(2, s, 4, 8), ve.reshape(2, s, 4, 8),
+                                 max_seq_len=s)
+    assert torch.equal(dense.reshape(2 * s, 4, 8), jag)
+    tril = torch.tril(torch.ones(s, s)).expand(2, 4, s, s)
+    assert torch.equal(O.hstu_jagged_forward(q, k, v, oq, max_seq_len_q=s, mask_type=3, mask=tril), jag)
+
+
+def test_trailing_duplicate_offset_changes_nothing():
+    rng = np.random.default_rng(5)
+    q, k, v, oq, _ = _jag(rng, [4, 6], 2, 2, 4, 4)
+    a = O.hstu_jagged_forward(q, k, v, oq, max_seq_len_q=8, num_context=[1, 1], num_target=[1, 2],
+                              target_group_size=1)
+    oq2 = torch.cat([oq, oq[-1:]])
+    b = O.hstu_jagged_forward(q, k, v, oq2, max_seq_len_q=8, num_context=[1, 1, 1], num_target=[1, 2, 2],
+                              target_group_size=1)
+    assert torch.equal(a, b)
+
+
+def test_lowp_rounding_points_bf16():
+    """"lowp" follows the golden's rounding points; it must sit within bf16 noise of "exact"."""
+    rng = np.random.default_rng(6)
+    q, k, v, oq, _ = _jag(rng, [40, 17], 2, 2, 32, 32, dtype=torch.bfloat16)
+    ex = O.hstu_jagged_forward(q, k, v, oq, max_seq_len_q=40, alpha=1 / math.sqrt(32))
+    lp = O.hstu_jagged_forward(q, k, v, oq, max_seq_len_q=40, alpha=1 / math.sqrt(32), mode="lowp")
+    assert lp.dtype == torch.bfloat16 and ex.dtype == torch.float32
+    assert torch.allclose(lp.float(), ex, rtol=2e-2, atol=2e-3)
+    assert O.double_benchmark_close(lp, lp, ex) and O.mismatch_ratio_close(lp, ex, 5e-3, 5e-3)
+
+
+# ---- paged ---------------------------------------------------------------
+def _paged_case(rng, users, ps, nq, nk, d, dtype=torch.float32):
+    hist = [int(x) for x in rng.integers(1, 3 * ps, users)]
+    new_hist = [int(x) for x in rng.integers(0, 5, users)]
+    hist = [max(h, n) for h, n in zip(hist, new_hist)]
+    tgt = [int(x) for x in rng.integers(1, 6, users)]
+    lq = [n + t for n, t in zip(new_hist, tgt)]
+    q, k, v, oq, _ = _jag(rng, lq, nq, nk, d, d, dtype=dtype)
+    npages = [(h + ps - 1) // ps for h in hist]
+    total = sum(npages) + 2
+    order = rng.permutation(total)[: sum(npages)]            # pages are not contiguous per user
+    cache = torch.zeros(total, 2, ps, nk, d, dtype=dtype)
+    hk = [torch.from_numpy(rng.normal(0, 0.5, (h, nk, d))).to(dtype) for h in hist]
+    hv = [torch.from_numpy(rng.normal(0, 0.5, (h, nk, d))).to(dtype) for h in hist]
+    page_ids, page_offsets, last = [], [0], []
+    p = 0
+    for u, h in enumerate(hist):
+        for i in range(npages[u]):
+            pid = int(order[p]); p += 1
+            n = min(ps, h - i * ps)
+            cache[pid, 0, :n] = hk[u][i * ps: i * ps + n]
+            cache[pid, 1, :n] = hv[u][i * ps: i * ps + n]
+            page_ids.append(pid)
+        page_offsets.append(p)
+        last.append(h % ps or ps)
+    t = lambda x: torch.tensor(x, dtype=torch.int32)
+    return dict(q=q, k=k, v=v, oq=oq, cache=cache, page_offsets=t(page_offsets), page_ids=t(page_ids),
+                last=t(last), tgt=tgt, hist=hist, new_hist=new_hist, hk=hk, hv=hv)
+
+
+def test_paged_equals_delta_jagged_on_depaged_kv():
+    rng = np.random.default_rng(8)
+    c = _paged_case(rng, 4, 8, 2, 2, 4)
+    mq = max(n + t for n, t in zip(c["new_hist"], c["tgt"])); mk = max(h + t for h, t in zip(c["hist"], c["tgt"]))
+    got = O.hstu_paged_forward(c["q"], c["k"], c["v"], c["cache"], c["oq"], c["page_offsets"], c["page_ids"],
+                               c["last"], c["tgt"], max_seq_len_q=mq, max_seq_len_k=mk, alpha=0.5)
+    # independent assembly: history straight from the unpaged source rows
+    oq = c["oq"].tolist()
+    kc, vc, lens = [], [], []
+    for u in range(4):
+        kc += [c["hk"][u], c["k"][oq[u] + c["new_hist"][u]: oq[u + 1]]]
+        vc += [c["hv"][u], c["v"][oq[u] + c["new_hist"][u]: oq[u + 1]]]
+        lens.append(c["hist"][u] + c["tgt"][u])
+    ok = torch.tensor([0] + list(np.cumsum(lens)))
+    # the paged golden's mask: tril(diagonal = Lk - Lq) on history columns, identity on candidates
+    masks = torch.zeros(4, 2, mq, mk)
+    for u in range(4):
+        lq_, h, t = oq[u + 1] - oq[u], c["hist"][u], c["tgt"][u]
+        m = torch.zeros(lq_, h + t)
+        m[:, :h] = torch.tril(torch.ones(lq_, h), diagonal=h + t - lq_)
+        m[lq_ - t:, h:] = torch.eye(t)
+        masks[u, :, :lq_, : h + t] = m
+    ref = O.hstu_jagged_forward(c["q"], torch.cat(kc), torch.cat(vc), c["oq"], ok, max_seq_len_q=mq,
+                                max_seq_len_k=mk, mask_type=3, mask=masks, alpha=0.5)
+    assert torch.equal(got, ref)
+
+
+def test_fp8_cache_roundtrip():
+    rng = np.random.default_rng(9)
+    cache = torch.from_numpy(rng.normal(0, 0.5, (5, 2, 16, 2, 8))).float()
+    cache[3] = 0
+    u8, sc = O.quantize_kv_cache_fp8(cache)
+    assert u8.dtype == torch.uint8 and sc.shape == (5, 2, 2) and torch.all(sc > 0)
+    dq = O.dequantize_kv_cache_fp8(u8, sc)
+    amax = cache.abs().amax(dim=(2, 4))[:, :, None, :, None]
+    assert torch.all((dq - cache).abs() <= amax * 2 ** -4 + 1e-12)      # e4m3: 3 mantissa bits
+    assert torch.equal(dq[3], torch.zeros_like(dq[3]))
+    # absmax element is reproduced (it maps to +-448 exactly)
+    assert torch.allclose(dq.abs().amax(dim=(2, 4)), cache.abs().amax(dim=(2, 4)), rtol=1e-6)
+
+
+# ---- bias closed forms ---------------------------------------------------
+def test_rel_pos_bias_closed_form():
+    n = 7
+    w = torch.arange(2 * n - 1, dtype=torch.float32)
+    b = O.rel_pos_bias(w, 5, 5, n)
+    for i in range(5):
+        for j in range(5):
+            assert b[i, j] == (n - 1) + j - i
+    b = O.rel_pos_bias(w, 2, 5, n)                     # delta-q: row i sits at position i+3
+    assert b[0, 3] == n - 1 and b[1, 4] == n - 1 and b[1, 0] == n - 1 - 4
+
+
+def test_time_bucket_ids():
+    t = torch.tensor([0, 1, 2, 3, 10, 1000, 10 ** 6, 10 ** 12, 10 ** 17], dtype=torch.int64)
+    ids = O.time_bucket_ids(t, t)
+    assert ids.dtype == torch.int64 and torch.equal(ids, ids.T)                 # |dt| is symmetric
+    assert ids[0, 0] == 0 and ids[0, 1] == 0                                     # dt = 0 and 1 -> bucket 0
+    assert ids[0, 2] == int(math.log(2) / 0.301) == 2 and ids[0, 3] == 3
+    assert ids[0, 4] == int(math.log(10) / 0.301) and ids[0, 5] == int(math.log(1000) / 0.301)
+    assert ids[0, 8] == 128 and ids.max() == 128                                 # clamp
+    # away from bucket edges the fp32 result equals the float64 closed form
+    d = torch.arange(1, 200000, dtype=torch.int64)
+    x = np.log(d.numpy().astype(np.float64)) / 0.301
+    safe = np.abs(x - np.round(x)) > 1e-4
+    got = O.time_bucket_ids(torch.zeros(1, dtype=torch.int64), d)[0].numpy()
+    assert np.array_equal(got[safe], np.floor(x[safe]).astype(np.int64))
+    tab = torch.arange(129, dtype=torch.float32) * 0.5
+    assert torch.equal(O.time_bias(tab, t, t), ids.float() * 0.5)
+
+
+def test_dense_bias_from_tables_layout():
+    oq = torch.tensor([0, 2, 5]); ok = torch.tensor([0, 4, 7])
+    n = 6
+    pos = torch.arange(2 * n - 1, dtype=torch.float32)
+    ts = torch.arange(7, dtype=torch.int64) * 100
+    tab = torch.arange(129, dtype=torch.float32) * 1000
+    d = O.dense_bias_from_tables(oq, ok, 3, 4, n, pos_table=pos, ts_table=tab, timestamps=ts)
+    assert d.shape == (2, 3, 4, 6)
+    assert torch.equal(d[0, :, 2:, :], torch.zeros(3, 2, 6)) and torch.equal(d[0, :, :, 4:], torch.zeros(3, 4, 2))
+    # sequence 0: lq=2, lk=4 -> row 0 sits at K position 2
+    assert d[0, 1, 0, 2] == (n - 1) + 0 * 1000 and d[0, 0, 0, 0] == (n - 1) - 2 + 1000 * int(math.log(200) / 0.301)
+    assert torch.equal(d[:, 0], d[:, 2])
