@@ -1,0 +1,156 @@
+/*
+ * hstu_hip.h -- C ABI of the MI355X (gfx950) HSTU fused attention forward.
+ *
+ * out = (SiLU(alpha * (Q K^T + bias)) * silu_scale * mask) V   over packed ("jagged") sequences,
+ * no softmax, no materialised score matrix.
+ *
+ * This is the boundary a host framework binds to.  It plays the role of the two-phase aclnn C entry
+ * points the reference's torch plugin resolves with dlsym and calls through EXEC_NPU_CMD
+ * (cust_op/framework/torch_plugin/torch_library/common/pytorch_npu_helper.hpp:508-558):
+ *     aclnnXGetWorkspaceSize(args..., &ws_bytes, &executor);  aclnnX(ws, ws_bytes, executor, stream);
+ * Here the argument list is a POD struct of raw device pointers and sizes; there are no torch types.
+ * Every call is asynchronous on `stream` (a hipStream_t passed as void*; NULL = the null stream),
+ * never synchronises the device and never reads a device buffer on the host.
+ * All functions return 0 on success and a negative hstu_status otherwise; the message for the
+ * calling thread is available from hstu_hip_last_error() (the role of aclGetRecentErrMsg()).
+ */
+#ifndef HSTU_HIP_H
+#define HSTU_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HSTU_HIP_ABI_VERSION 1
+
+typedef enum hstu_status {
+    HSTU_OK = 0,
+    HSTU_ERR_INVALID_ARGUMENT = -1, /* shape / attribute rejected (reference: op_host tiling checks) */
+    HSTU_ERR_UNSUPPORTED = -2,      /* valid in the reference, not built here */
+    HSTU_ERR_WORKSPACE = -3,        /* workspace pointer missing or too small */
+    HSTU_ERR_LAUNCH = -4            /* HIP runtime refused the launch */
+} hstu_status;
+
+typedef enum hstu_dtype { HSTU_F32 = 0, HSTU_F16 = 1, HSTU_BF16 = 2, HSTU_FP8_E4M3 = 3 } hstu_dtype;
+typedef enum hstu_index_type { HSTU_I32 = 0, HSTU_I64 = 1 } hstu_index_type;
+
+/* mask_type values of the reference (hstu_common.h:47-50). 1 (triu) is rejected like there. */
+enum { HSTU_MASK_TRIL = 0, HSTU_MASK_TRIU = 1, HSTU_MASK_NONE = 2, HSTU_MASK_CUSTOM = 3 };
+
+/* limits of the reference's host checks (hstu_common.h:30-45, tiling_policy.cpp:69-94) */
+#define HSTU_MAX_BATCH 2048
+#define HSTU_MAX_SEQ_LEN 20480
+#define HSTU_MAX_HEADS 16
+#define HSTU_MAX_HEAD_DIM 512
+
+/* flags */
+#define HSTU_FLAG_DETERMINISTIC 1u /* accepted; every output row has one producer, so results never depend on it */
+#define HSTU_FLAG_FORCE_GENERIC 2u /* run the plain fp32-FMA kernel even where an MFMA kernel exists (testing) */
+
+/*
+ * One argument block for the three forward ops.  Pointers are device pointers unless stated.
+ * Layouts (row-major, innermost last):
+ *   q   [total_q, heads_q, dim_qk]     k [total_k, heads_k, dim_qk]     v [total_k, heads_k, dim_v]
+ *   out [total_q, heads_q, dim_v]      same dtype as q
+ *   seq_offset_q / seq_offset_k  [batch+1] of index_type; sequence b owns rows off[b]..off[b+1]-1.
+ *     Q row i of a sequence sits at position i + (Lk - Lq) of its K timeline ("delta-q").
+ *     Both NULL = dense layout: every sequence has max_seq_len_q (= max_seq_len_k) rows.
+ *   mask, attn_bias  [batch, heads_q, max_seq_len_q, max_seq_len_k] in `dtype`, or NULL
+ *   num_context, num_target  [batch] of index_type, or NULL (= zeros)
+ * (reference: hstu_jagged.cpp:22-67, hstu_jagged_forward_kernel.h:457-459,507-510)
+ */
+typedef struct hstu_fwd_params {
+    uint32_t struct_size; /* sizeof(hstu_fwd_params) of the caller, for ABI checking */
+    uint32_t flags;
+    int32_t dtype;      /* hstu_dtype of q/k/v/out/mask/attn_bias: F32, F16 or BF16 */
+    int32_t index_type; /* hstu_index_type of every integer tensor */
+
+    const void* q;
+    const void* k;
+    const void* v;
+    void* out;
+    const void* mask;
+    const void* attn_bias;
+    const void* seq_offset_q;
+    const void* seq_offset_k;
+    const void* num_context;
+    const void* num_target;
+
+    int64_t total_q;
+    int64_t total_k;
+    int32_t batch;
+    int32_t heads_q;
+    int32_t heads_k;
+    int32_t dim_qk;
+    int32_t dim_v;
+    int32_t mask_type;
+    int32_t max_seq_len_q;
+    int32_t max_seq_len_k;
+    int32_t target_group_size;
+    float silu_scale; /* already resolved: the caller applies "0 means 1/max_seq_len_q" */
+    float alpha;
+
+    /*
+     * Paged history (hstu_paged only; reference hstu_paged_forward_kernel.h:469-532).
+     * K/V column j of user b:  j < hist_b  ->  kv_cache[page_ids[page_offsets[b] + j / page_size]][0|1][j % page_size][kv head][:]
+     *                          else        ->  input k/v row seq_offset_q[b] + (Lq_b - num_target_b) + (j - hist_b)
+     * with hist_b = Lk_b - num_target_b.
+     *   kv_cache [num_pages, 2, page_size, heads_k, dim] in cache_dtype (== dtype, or FP8_E4M3)
+     *   kv_scales [num_pages, 2, heads_k] float, dequantised value = fp8 * scale (FP8_E4M3 caches only;
+     *   this cache format has no counterpart in the reference)
+     */
+    const void* kv_cache;
+    const void* page_offsets;  /* [batch+1] */
+    const void* page_ids;      /* [page_offsets[batch]] */
+    const void* last_page_len; /* [batch]; implied by seq_offset_k, accepted for signature parity */
+    const float* kv_scales;
+    int64_t num_pages;
+    int32_t page_size;
+    int32_t cache_dtype;
+
+    /*
+     * Fused bias tables (no counterpart in the reference op, which takes the dense attn_bias that
+     * relative_attn_bias_pos/_time produce: cust_op/test/relative_attn_bias/torch/utils.py:38-51,99-129).
+     *   pos_table [2*max_seq_len_k - 1] float:  bias += pos_table[(max_seq_len_k-1) + j - (i + Lk - Lq)]
+     *   timestamps [total_k] int64 on the K timeline; ts_table [num_buckets+1] float;
+     *   ts_bounds [num_buckets+2] float, ascending, bounds[0] = 0, bounds[num_buckets+1] = +inf:
+     *     bucket(i,j) = the b with bounds[b] <= (float)|t_i - t_j| < bounds[b+1];  bias += ts_table[bucket]
+     * Added to attn_bias when both are given.
+     */
+    const float* pos_table;
+    const float* ts_table;
+    const float* ts_bounds;
+    const int64_t* timestamps;
+    int32_t num_buckets;
+    int32_t reserved0;
+} hstu_fwd_params;
+
+/* replaces aclnnHstuJaggedForwardGetWorkspaceSize / aclnnHstuJaggedForward (hstu_jagged.cpp:63-65) */
+int hstu_hip_jagged_forward_get_workspace_size(const hstu_fwd_params* p, uint64_t* workspace_bytes);
+int hstu_hip_jagged_forward(const hstu_fwd_params* p, void* workspace, uint64_t workspace_bytes, void* stream);
+
+/* replaces aclnnHstuPagedForwardGetWorkspaceSize / aclnnHstuPagedForward (hstu_paged.cpp:67-69) */
+int hstu_hip_paged_forward_get_workspace_size(const hstu_fwd_params* p, uint64_t* workspace_bytes);
+int hstu_hip_paged_forward(const hstu_fwd_params* p, void* workspace, uint64_t workspace_bytes, void* stream);
+
+/* replaces aclnnHstuDenseForwardGetWorkspaceSize / aclnnHstuDenseForward (hstu_dense.cpp:37-39);
+ * q/k/v are [batch, max_seq_len_q, heads, dim]; seq_offset_* must be NULL */
+int hstu_hip_dense_forward_get_workspace_size(const hstu_fwd_params* p, uint64_t* workspace_bytes);
+int hstu_hip_dense_forward(const hstu_fwd_params* p, void* workspace, uint64_t workspace_bytes, void* stream);
+
+/* replaces aclGetRecentErrMsg() (pytorch_npu_helper.hpp:510-543): message of the last failing call on this thread */
+const char* hstu_hip_last_error(void);
+
+/* Name of the kernel variant the given arguments select ("mfma_bf16_d128", "generic_f32", ...);
+ * written NUL-terminated into buf.  Diagnostic: lets a caller assert that the MFMA path is the one in use. */
+int hstu_hip_describe_kernel(const hstu_fwd_params* p, char* buf, size_t buf_bytes);
+
+int hstu_hip_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HSTU_HIP_H */

@@ -1,0 +1,162 @@
+// C-ABI entry points: argument validation (the role of the reference's op_host tiling checks,
+// tiling_policy.cpp:69-94, tiling_policy_jagged.cpp:63-205, tiling_policy_paged.cpp:120-222),
+// kernel selection and launch.  No device synchronisation, no host reads of device memory.
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <string>
+
+#include "hstu_internal.h"
+
+namespace hstu {
+
+static thread_local std::string g_last_error;
+
+static int fail(int code, const char* fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    g_last_error = buf;
+    return code;
+}
+
+static bool in_range(int64_t v, int64_t lo, int64_t hi) { return v >= lo && v <= hi; }
+
+static int validate(const hstu_fwd_params* p, int op, KArgs* out) {
+    if (!p) return fail(HSTU_ERR_INVALID_ARGUMENT, "params is NULL");
+    if (p->struct_size != sizeof(hstu_fwd_params))
+        return fail(HSTU_ERR_INVALID_ARGUMENT, "hstu_fwd_params size mismatch: caller %u, library %zu (ABI version %d)",
+                    p->struct_size, sizeof(hstu_fwd_params), HSTU_HIP_ABI_VERSION);
+    if (p->dtype != HSTU_F32 && p->dtype != HSTU_F16 && p->dtype != HSTU_BF16)
+        return fail(HSTU_ERR_INVALID_ARGUMENT, "dtype expect float32, float16 or bfloat16, but value is %d", p->dtype);
+    if (p->index_type != HSTU_I32 && p->index_type != HSTU_I64)
+        return fail(HSTU_ERR_INVALID_ARGUMENT, "index_type expect int32 or int64, but value is %d", p->index_type);
+    if (!p->q || !p->k || !p->v || !p->out) return fail(HSTU_ERR_INVALID_ARGUMENT, "q, k, v and out must not be NULL");
+    if (p->batch == 0 || p->batch > HSTU_MAX_BATCH || p->batch < 0)
+        return fail(HSTU_ERR_INVALID_ARGUMENT, "batchSize limit (0, %d], but get %d", HSTU_MAX_BATCH, p->batch);
+    if (!in_range(p->max_seq_len_q, 1, HSTU_MAX_SEQ_LEN))
+        return fail(HSTU_ERR_INVALID_ARGUMENT, "maxSeqLen expect in [1, %d], but value is %d", HSTU_MAX_SEQ_LEN, p->max_seq_len_q);
+    if (!in_range(p->max_seq_len_k, 1, HSTU_MAX_SEQ_LEN))
+        return fail(HSTU_ERR_INVALID_ARGUMENT, "maxSeqLenK expect in [1, %d], but value is %d", HSTU_MAX_SEQ_LEN, p->max_seq_len_k);
+    if (!in_range(p->heads_q, 1, HSTU_MAX_HEADS) || !in_range(p->heads_k, 1, HSTU_MAX_HEADS))
+        return fail(HSTU_ERR_INVALID_ARGUMENT, "head num expect in [1, %d], but get q %d, k %d", HSTU_MAX_HEADS, p->heads_q, p->heads_k);
+    if (p->heads_q % p->heads_k != 0)
+        return fail(HSTU_ERR_INVALID_ARGUMENT, "For GQA, headNumQ must be divisible by headNumK (%d, %d)", p->heads_q, p->heads_k);
+    if (!in_range(p->dim_qk, 1, HSTU_MAX_HEAD_DIM))
+        return fail(HSTU_ERR_INVALID_ARGUMENT, "Q/K dim size expect in [1, %d], but get %d", HSTU_MAX_HEAD_DIM, p->dim_qk);
+    if (!in_range(p->dim_v, 16, HSTU_MAX_HEAD_DIM) || p->dim_v % 16 != 0)
+        return fail(HSTU_ERR_INVALID_ARGUMENT, "V dim size expect a multiple of 16 in [16, %d], but get %d", HSTU_MAX_HEAD_DIM, p->dim_v);
+    if (p->mask_type < HSTU_MASK_TRIL || p->mask_type > HSTU_MASK_CUSTOM)
+        return fail(HSTU_ERR_INVALID_ARGUMENT, "maskType expect in [0, 3], but value is %d", p->mask_type);
+    if (p->mask_type == HSTU_MASK_TRIU)
+        return fail(HSTU_ERR_INVALID_ARGUMENT, "maskType current not support triu now, pls use custom mask");
+    if (p->mask_type == HSTU_MASK_CUSTOM && !p->mask)
+        return fail(HSTU_ERR_INVALID_ARGUMENT, "use custom mask must have valid mask tensor");
+    if (p->target_group_size < 0) return fail(HSTU_ERR_INVALID_ARGUMENT, "targetGroupSize must not be negative");
+    if (p->total_q < 0 || p->total_k < 0) return fail(HSTU_ERR_INVALID_ARGUMENT, "negative row count");
+    if (!std::isfinite(p->silu_scale) || !std::isfinite(p->alpha))
+        return fail(HSTU_ERR_INVALID_ARGUMENT, "silu_scale and alpha must be finite");
+
+    if (op == OP_DENSE) {
+        if (p->seq_offset_q || p->seq_offset_k)
+            return fail(HSTU_ERR_INVALID_ARGUMENT, "dense layout takes no sequence offsets");
+        if (p->heads_q != p->heads_k || p->dim_qk != p->dim_v || p->max_seq_len_q != p->max_seq_len_k)
+            return fail(HSTU_ERR_INVALID_ARGUMENT, "dense layout needs q, k and v of one shape");
+        if (p->dim_qk % 16 != 0) return fail(HSTU_ERR_INVALID_ARGUMENT, "dense layout needs dim %% 16 == 0, but get %d", p->dim_qk);
+        if (p->total_q != (int64_t)p->batch * p->max_seq_len_q || p->total_k != p->total_q)
+            return fail(HSTU_ERR_INVALID_ARGUMENT, "dense layout: total rows must equal batch * seq_len");
+        if (p->num_context || p->num_target) return fail(HSTU_ERR_INVALID_ARGUMENT, "dense layout takes no num_context/num_target");
+    } else {
+        if (!p->seq_offset_q || !p->seq_offset_k)
+            return fail(HSTU_ERR_INVALID_ARGUMENT, "seq_offset_q and seq_offset_k must not be NULL in jagged layout");
+    }
+    if (op == OP_PAGED) {
+        if (!p->kv_cache || !p->page_offsets || !p->page_ids || !p->last_page_len)
+            return fail(HSTU_ERR_INVALID_ARGUMENT, "pagedIds, pagedOffset, lastPageLen and kvCache should not be nullptr.");
+        if (p->page_size < 1) return fail(HSTU_ERR_INVALID_ARGUMENT, "PageSize must be positive, but get %d", p->page_size);
+        if (p->dim_qk != p->dim_v) return fail(HSTU_ERR_INVALID_ARGUMENT, "K, V shape mismatch");
+        if (p->total_q != p->total_k) return fail(HSTU_ERR_INVALID_ARGUMENT, "Q, K, V seqlen mismatch");
+        if (p->cache_dtype == HSTU_FP8_E4M3) {
+            if (!p->kv_scales) return fail(HSTU_ERR_INVALID_ARGUMENT, "fp8 kv_cache needs kv_scales");
+        } else if (p->cache_dtype != p->dtype) {
+            return fail(HSTU_ERR_INVALID_ARGUMENT, "kv_cache dtype must equal the q dtype or be fp8-e4m3");
+        }
+    } else if (p->kv_cache) {
+        return fail(HSTU_ERR_INVALID_ARGUMENT, "kv_cache is only taken by the paged op");
+    }
+    if (p->ts_table) {
+        if (!p->timestamps || !p->ts_bounds || p->num_buckets < 1)
+            return fail(HSTU_ERR_INVALID_ARGUMENT, "ts_table needs timestamps, ts_bounds and num_buckets >= 1");
+    }
+
+    out->p = *p;
+    out->op = op;
+    out->head_ratio = p->heads_q / p->heads_k;
+    out->out_scale = p->alpha * p->silu_scale;
+    out->exp_scale = -p->alpha * 1.4426950408889634f;
+    return HSTU_OK;
+}
+
+static int run(const hstu_fwd_params* p, int op, void* workspace, uint64_t workspace_bytes, void* stream) {
+    (void)workspace;
+    (void)workspace_bytes;
+    KArgs a;
+    int rc = validate(p, op, &a);
+    if (rc != HSTU_OK) return rc;
+    if (p->total_q == 0) return HSTU_OK;
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    const char* name = nullptr;
+    hipError_t e;
+    if (!(p->flags & HSTU_FLAG_FORCE_GENERIC) && mfma_supported(a, &name)) {
+        e = launch_mfma(a, st);
+    } else {
+        e = launch_generic(a, st);
+    }
+    if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString(e));
+    return HSTU_OK;
+}
+
+static int ws_size(const hstu_fwd_params* p, int op, uint64_t* bytes) {
+    if (!bytes) return fail(HSTU_ERR_INVALID_ARGUMENT, "workspace_bytes is NULL");
+    KArgs a;
+    int rc = validate(p, op, &a);
+    if (rc != HSTU_OK) return rc;
+    *bytes = 0;  // every output row has exactly one producing workgroup: no partials, no flags
+    return HSTU_OK;
+}
+
+}  // namespace hstu
+
+using namespace hstu;
+
+extern "C" {
+
+int hstu_hip_jagged_forward_get_workspace_size(const hstu_fwd_params* p, uint64_t* b) { return ws_size(p, OP_JAGGED, b); }
+int hstu_hip_jagged_forward(const hstu_fwd_params* p, void* ws, uint64_t n, void* s) { return run(p, OP_JAGGED, ws, n, s); }
+int hstu_hip_paged_forward_get_workspace_size(const hstu_fwd_params* p, uint64_t* b) { return ws_size(p, OP_PAGED, b); }
+int hstu_hip_paged_forward(const hstu_fwd_params* p, void* ws, uint64_t n, void* s) { return run(p, OP_PAGED, ws, n, s); }
+int hstu_hip_dense_forward_get_workspace_size(const hstu_fwd_params* p, uint64_t* b) { return ws_size(p, OP_DENSE, b); }
+int hstu_hip_dense_forward(const hstu_fwd_params* p, void* ws, uint64_t n, void* s) { return run(p, OP_DENSE, ws, n, s); }
+
+const char* hstu_hip_last_error(void) { return g_last_error.c_str(); }
+
+int hstu_hip_describe_kernel(const hstu_fwd_params* p, char* buf, size_t n) {
+    if (!buf || n == 0) return fail(HSTU_ERR_INVALID_ARGUMENT, "buf is NULL");
+    KArgs a;
+    int op = (p && p->kv_cache) ? OP_PAGED : ((p && !p->seq_offset_q) ? OP_DENSE : OP_JAGGED);
+    int rc = validate(p, op, &a);
+    if (rc != HSTU_OK) return rc;
+    const char* name = nullptr;
+    if ((p->flags & HSTU_FLAG_FORCE_GENERIC) || !mfma_supported(a, &name)) {
+        name = p->dtype == HSTU_F32 ? "generic_f32" : (p->dtype == HSTU_F16 ? "generic_f16" : "generic_bf16");
+    }
+    snprintf(buf, n, "%s", name);
+    return HSTU_OK;
+}
+
+int hstu_hip_abi_version(void) { return HSTU_HIP_ABI_VERSION; }
+
+}  // extern "C"

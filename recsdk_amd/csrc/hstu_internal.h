@@ -1,0 +1,26 @@
+// Internal declarations shared by the C-ABI translation unit and the kernel translation units.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/hstu_hip.h"
+
+namespace hstu {
+
+enum OpKind : int32_t { OP_JAGGED = 0, OP_PAGED = 1, OP_DENSE = 2 };
+
+// Kernel argument block: the caller's parameters plus what the host derives from them.
+struct KArgs {
+    hstu_fwd_params p;
+    int32_t op;          // OpKind
+    int32_t head_ratio;  // heads_q / heads_k
+    float out_scale;     // factor applied once to the fp32 accumulator (MFMA kernels)
+    float exp_scale;     // -alpha * log2(e) (MFMA kernels)
+};
+
+// launchers (defined next to their kernels); return hipError_t of the launch
+hipError_t launch_generic(const KArgs& a, hipStream_t stream);
+bool mfma_supported(const KArgs& a, const char** name);
+hipError_t launch_mfma(const KArgs& a, hipStream_t stream);
+
+}  // namespace hstu

@@ -1,0 +1,575 @@
+// torch op registration for the HSTU forward family under the reference's names and schemas:
+//   mxrec::hstu_jagged.equal / .delta   (cust_op/framework/torch_plugin/torch_library/hstu/hstu_jagged.cpp:186-231)
+//   mxrec::hstu_paged                    (hstu_paged.cpp:73-95)
+//   mxrec::hstu_dense                    (hstu_dense.cpp:155-164)
+// plus two ops the reference has no counterpart for (fused bias tables, fp8 paged cache).
+// The host logic mirrors hstu_deltaq_forward_impl_npu (hstu_jagged.cpp:22-67): same checks and
+// messages, same defaults, output allocated here; the device work is one call into the C ABI of
+// libhstu_hip.so on the current stream.  There is no CPU implementation: CPU tensors get the same
+// argument checks and then a clear error.
+#include <ATen/ATen.h>
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <torch/library.h>
+
+#include <cmath>
+#include <limits>
+#include <mutex>
+
+#include "hstu_hip.h"
+
+namespace mxrec_hstu {
+
+constexpr int64_t kMinSeqLen = 1;
+constexpr int64_t kMaxSeqLen = 20480;
+
+static void mask_check(int64_t mask_type, bool mask_defined) {
+    TORCH_CHECK(0 <= mask_type && mask_type <= 3, "maskType expect in [0, 3], but value is ", mask_type);
+    TORCH_CHECK(mask_type != 1, "maskType current not support triu now, pls use custom mask");
+    TORCH_CHECK(!(mask_type == 3 && !mask_defined), "use custom mask must have valid mask tensor");
+}
+
+static void max_seq_len_check(int64_t n) {
+    TORCH_CHECK(n >= kMinSeqLen && n <= kMaxSeqLen, "maxSeqLen expect in [1, 20480], but value is ", n);
+}
+
+static int32_t io_dtype(const at::Tensor& t, const char* what) {
+    switch (t.scalar_type()) {
+        case at::kFloat: return HSTU_F32;
+        case at::kHalf: return HSTU_F16;
+        case at::kBFloat16: return HSTU_BF16;
+        default: TORCH_CHECK(false, what, " dtype expect float32, float16 or bfloat16, but get ", t.scalar_type());
+    }
+    return -1;
+}
+
+static const void* ptr_or_null(const at::Tensor& t) { return t.defined() ? t.const_data_ptr() : nullptr; }
+
+struct Holder {  // keeps converted temporaries alive until the launch is queued
+    std::vector<at::Tensor> keep;
+    at::Tensor index(const c10::optional<at::Tensor>& t, at::ScalarType st, int64_t expect_len, const char* name) {
+        if (!t.has_value() || !t->defined()) return at::Tensor();
+        TORCH_CHECK(t->dim() == 1, name, " should have 1 dimension, but get ", t->dim());
+        if (expect_len >= 0)
+            TORCH_CHECK(t->size(0) == expect_len, "The length of ", name, " expect ", expect_len, ", but get ", t->size(0));
+        auto x = t->to(st).contiguous();
+        keep.push_back(x);
+        return x;
+    }
+    at::Tensor same(const at::Tensor& t) {
+        auto x = t.contiguous();
+        keep.push_back(x);
+        return x;
+    }
+};
+
+static void require_gpu(const at::Tensor& q, const char* op) {
+    TORCH_CHECK(q.is_cuda(), "mxrec::", op, " has no CPU implementation: move the tensors to the MI355X (device 'cuda')");
+}
+
+static void run_abi(int (*ws_fn)(const hstu_fwd_params*, uint64_t*), int (*fn)(const hstu_fwd_params*, void*, uint64_t, void*),
+                    const hstu_fwd_params& p, const at::Tensor& q, const char* op) {
+    uint64_t ws_bytes = 0;
+    int rc = ws_fn(&p, &ws_bytes);
+    TORCH_CHECK(rc == HSTU_OK, "mxrec::", op, ": ", hstu_hip_last_error());
+    require_gpu(q, op);
+    at::Tensor ws;
+    if (ws_bytes) ws = at::empty({(int64_t)ws_bytes}, q.options().dtype(at::kByte));
+    c10::hip::OptionalHIPGuardMasqueradingAsCUDA guard(q.device());
+    auto stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA();
+    rc = fn(&p, ws_bytes ? ws.data_ptr() : nullptr, ws_bytes, (void*)stream.stream());
+    TORCH_CHECK(rc == HSTU_OK, "mxrec::", op, ": ", hstu_hip_last_error());
+}
+
+// ---------------------------------------------------------------------------------------------
+// Smallest fp32 |dt| of every time bucket, from the reference formula
+//   bucket = trunc(log(clamp(|dt|, 1, e^(nb*div))) / div)   (cust_op/test/relative_attn_bias/torch/utils.py:115-123)
+// evaluated with ATen's own CPU log so that the integer ids agree bit for bit with a torch evaluation
+// of that formula.  bounds[0] = 0, bounds[nb+1] = +inf.
+// ---------------------------------------------------------------------------------------------
+static at::Tensor bucket_of(const at::Tensor& x, int64_t nb, double div) {
+    float cmax = std::exp((float)(nb * div));
+    return at::log(at::clamp(x, 1.0, (double)cmax)).div((float)div).to(at::kLong);
+}
+
+at::Tensor hstu_time_bucket_bounds(int64_t num_buckets, double bucket_divisor) {
+    TORCH_CHECK(num_buckets >= 1 && num_buckets <= 4096, "num_buckets expect in [1, 4096], but value is ", num_buckets);
+    TORCH_CHECK(bucket_divisor > 0, "bucket_divisor must be positive");
+    const int64_t nb = num_buckets;
+    auto opt_i = at::TensorOptions().dtype(at::kInt);
+    // search over the bit patterns of positive floats (monotone as integers)
+    float one = 1.0f, big = std::numeric_limits<float>::max();
+    int32_t lo0, hi0;
+    std::memcpy(&lo0, &one, 4);
+    std::memcpy(&hi0, &big, 4);
+    auto target = at::arange(1, nb + 1, at::kLong);
+    auto lo = at::full({nb}, lo0, opt_i), hi = at::full({nb}, hi0, opt_i);
+    auto reach = bucket_of(hi.view(at::kFloat), nb, bucket_divisor).ge(target);  // bucket attainable at all
+    for (int it = 0; it < 34; ++it) {
+        auto mid = lo + (hi - lo).div(2, "floor").to(at::kInt);
+        auto ok = bucket_of(mid.view(at::kFloat), nb, bucket_divisor).ge(target);
+        hi = at::where(ok, mid, hi);
+        lo = at::where(ok, lo, at::minimum(mid + 1, hi));
+    }
+    auto b = hi.view(at::kFloat).clone();
+    b = at::where(reach, b, at::full_like(b, std::numeric_limits<float>::infinity()));
+    auto out = at::empty({nb + 2}, at::kFloat);
+    out[0] = 0.0f;
+    out.slice(0, 1, nb + 1).copy_(b);
+    out[nb + 1] = std::numeric_limits<float>::infinity();
+    return out;
+}
+
+static at::Tensor cached_bounds(int64_t nb, double div, const at::Device& dev) {
+    static std::mutex mu;
+    static std::vector<std::tuple<int64_t, double, at::Device, at::Tensor>> cache;
+    std::lock_guard<std::mutex> g(mu);
+    for (auto& e : cache)
+        if (std::get<0>(e) == nb && std::get<1>(e) == div && std::get<2>(e) == dev) return std::get<3>(e);
+    auto t = hstu_time_bucket_bounds(nb, div).to(dev);
+    cache.emplace_back(nb, div, dev, t);
+    return t;
+}
+
+// ---------------------------------------------------------------------------------------------
+// jagged (equal / delta) + table-bias extension
+// ---------------------------------------------------------------------------------------------
+struct Tables {
+    c10::optional<at::Tensor> pos_table, ts_table, timestamps;
+    double bucket_divisor = 0.301;
+};
+
+static at::Tensor jagged_forward_impl(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v,
+                                      const c10::optional<at::Tensor>& mask, const c10::optional<at::Tensor>& attn_bias,
+                                      int64_t mask_type, int64_t max_seq_len_q, int64_t max_seq_len_k, double silu_scale,
+                                      const at::Tensor& seq_offset, const at::Tensor& seq_offset_k,
+                                      const c10::optional<at::Tensor>& num_context,
+                                      const c10::optional<at::Tensor>& num_target,
+                                      const c10::optional<int64_t>& target_group_size, const c10::optional<double>& alpha,
+                                      bool deterministic, const Tables* tables, const char* op) {
+    TORCH_CHECK(q.dim() == 3, "The q should be 3D in jagged layout");
+    TORCH_CHECK(k.dim() == 3 && v.dim() == 3, "The k and v should be 3D in jagged layout");
+    TORCH_CHECK(seq_offset.defined() && seq_offset.dim() == 1 && seq_offset.size(0) >= 2,
+                "acSeqOffset params error should have at least two element.");
+    TORCH_CHECK(seq_offset_k.defined() && seq_offset_k.dim() == 1 && seq_offset_k.size(0) >= 2,
+                "acSeqOffsetK params error should have at least two element.");
+    TORCH_CHECK(seq_offset.scalar_type() == at::kInt || seq_offset.scalar_type() == at::kLong,
+                "seq_offset dtype expect int32 or int64, but get ", seq_offset.scalar_type());
+    TORCH_CHECK(seq_offset_k.size(0) == seq_offset.size(0), "seq_offset and seq_offset_k should have the same shape");
+    Holder h;
+    const auto it = seq_offset.scalar_type();
+    const int64_t batch = seq_offset.size(0) - 1;
+    auto off_q = h.same(seq_offset);
+    auto off_k = h.index(seq_offset_k, it, -1, "seq_offset_k");
+    auto dq = h.same(q), dk = h.same(k), dv = h.same(v);
+    auto ctx = h.index(num_context, it, batch, "num_context");
+    auto tgt = h.index(num_target, it, batch, "num_target");
+
+    max_seq_len_check(max_seq_len_q);
+    max_seq_len_check(max_seq_len_k);
+    const bool mask_defined = mask.has_value() && mask->defined();
+    mask_check(mask_type, mask_defined);
+
+    const int32_t dt = io_dtype(dq, "q");
+    TORCH_CHECK(dk.scalar_type() == dq.scalar_type() && dv.scalar_type() == dq.scalar_type(), "q, k, v dtype mismatch");
+    TORCH_CHECK(dk.size(0) == dv.size(0), "K, V seqLens mismatch");
+    TORCH_CHECK(dk.size(1) == dv.size(1), "K, V headNum mismatch");
+    TORCH_CHECK(dq.size(2) == dk.size(2), "Q, K, V headDIM Shape Check failed");
+
+    hstu_fwd_params p;
+    std::memset(&p, 0, sizeof(p));
+    p.struct_size = sizeof(p);
+    p.flags = deterministic ? HSTU_FLAG_DETERMINISTIC : 0u;
+    p.dtype = dt;
+    p.index_type = it == at::kLong ? HSTU_I64 : HSTU_I32;
+    p.total_q = dq.size(0);
+    p.total_k = dk.size(0);
+    p.batch = (int32_t)batch;
+    p.heads_q = (int32_t)dq.size(1);
+    p.heads_k = (int32_t)dk.size(1);
+    p.dim_qk = (int32_t)dq.size(2);
+    p.dim_v = (int32_t)dv.size(2);
+    p.mask_type = (int32_t)mask_type;
+    p.max_seq_len_q = (int32_t)max_seq_len_q;
+    p.max_seq_len_k = (int32_t)max_seq_len_k;
+    p.target_group_size = (int32_t)target_group_size.value_or(0);
+    p.silu_scale = (float)((silu_scale == 0.0) ? 1.0 / (double)max_seq_len_q : silu_scale);
+    p.alpha = (float)alpha.value_or(1.0);
+
+    at::Tensor dmask, dbias;
+    const std::vector<int64_t> full = {batch, dq.size(1), max_seq_len_q, max_seq_len_k};
+    if (mask_defined && mask_type == 3) {
+        dmask = h.same(*mask);
+        TORCH_CHECK(dmask.scalar_type() == dq.scalar_type(), "mask dtype must equal the q dtype");
+        TORCH_CHECK(dmask.sizes() == at::IntArrayRef(full), "mask shape expect [batch, heads, max_seq_len, max_seq_len_k], but get ", dmask.sizes());
+    }
+    if (attn_bias.has_value() && attn_bias->defined()) {
+        dbias = h.same(*attn_bias);
+        TORCH_CHECK(dbias.scalar_type() == dq.scalar_type(), "attn_bias dtype must equal the q dtype");
+        TORCH_CHECK(dbias.sizes() == at::IntArrayRef(full), "attn_bias shape expect [batch, heads, max_seq_len, max_seq_len_k], but get ", dbias.sizes());
+    }
+    at::Tensor pos, tst, tsb, tsv;
+    if (tables) {
+        if (tables->pos_table.has_value() && tables->pos_table->defined()) {
+            pos = h.same(tables->pos_table->to(at::kFloat));
+            TORCH_CHECK(pos.dim() == 1 && pos.size(0) == 2 * max_seq_len_k - 1, "pos_table expect 2*max_seq_len_k-1 = ",
+                        2 * max_seq_len_k - 1, " entries, but get ", pos.sizes());
+        }
+        if (tables->ts_table.has_value() && tables->ts_table->defined()) {
+            TORCH_CHECK(tables->timestamps.has_value() && tables->timestamps->defined(), "ts_table needs timestamps");
+            tst = h.same(tables->ts_table->to(at::kFloat));
+            tsv = h.same(tables->timestamps->to(at::kLong));
+            TORCH_CHECK(tst.dim() == 1 && tst.size(0) >= 2, "ts_table expect num_buckets+1 entries");
+            TORCH_CHECK(tsv.dim() == 1 && tsv.size(0) == dk.size(0), "timestamps expect one int64 per K row (", dk.size(0), "), but get ", tsv.sizes());
+            tsb = cached_bounds(tst.size(0) - 1, tables->bucket_divisor, dq.device());
+            p.num_buckets = (int32_t)(tst.size(0) - 1);
+        }
+    }
+    for (const at::Tensor* t : {&dk, &dv, &off_q, &off_k, &ctx, &tgt, &dmask, &dbias, &pos, &tst, &tsv})
+        TORCH_CHECK(!t->defined() || t->device() == dq.device(), "all tensors must be on the device of q");
+
+    auto out = at::empty({dq.size(0), dq.size(1), dv.size(2)}, dq.options());
+    p.q = dq.const_data_ptr();
+    p.k = dk.const_data_ptr();
+    p.v = dv.const_data_ptr();
+    p.out = out.data_ptr();
+    p.mask = ptr_or_null(dmask);
+    p.attn_bias = ptr_or_null(dbias);
+    p.seq_offset_q = off_q.const_data_ptr();
+    p.seq_offset_k = off_k.const_data_ptr();
+    p.num_context = ptr_or_null(ctx);
+    p.num_target = ptr_or_null(tgt);
+    p.pos_table = (const float*)ptr_or_null(pos);
+    p.ts_table = (const float*)ptr_or_null(tst);
+    p.ts_bounds = (const float*)ptr_or_null(tsb);
+    p.timestamps = (const int64_t*)ptr_or_null(tsv);
+    run_abi(hstu_hip_jagged_forward_get_workspace_size, hstu_hip_jagged_forward, p, dq, op);
+    return out;
+}
+
+at::Tensor hstu_jagged_equal(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v,
+                             const c10::optional<at::Tensor>& mask, const c10::optional<at::Tensor>& attn_bias,
+                             int64_t mask_type, int64_t max_seq_len, double silu_scale, const at::Tensor& seq_offset,
+                             const c10::optional<at::Tensor>& num_context, const c10::optional<at::Tensor>& num_target,
+                             c10::optional<int64_t> target_group_size, c10::optional<double> alpha, bool deterministic) {
+    return jagged_forward_impl(q, k, v, mask, attn_bias, mask_type, max_seq_len, max_seq_len, silu_scale, seq_offset,
+                               seq_offset, num_context, num_target, target_group_size, alpha, deterministic, nullptr,
+                               "hstu_jagged");
+}
+
+at::Tensor hstu_jagged_delta(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v,
+                             const c10::optional<at::Tensor>& mask, const c10::optional<at::Tensor>& attn_bias,
+                             int64_t mask_type, int64_t max_seq_len, int64_t max_seq_len_k, double silu_scale,
+                             const at::Tensor& seq_offset, const at::Tensor& seq_offset_k,
+                             const c10::optional<at::Tensor>& num_context, const c10::optional<at::Tensor>& num_target,
+                             c10::optional<int64_t> target_group_size, c10::optional<double> alpha, bool deterministic) {
+    return jagged_forward_impl(q, k, v, mask, attn_bias, mask_type, max_seq_len, max_seq_len_k, silu_scale, seq_offset,
+                               seq_offset_k, num_context, num_target, target_group_size, alpha, deterministic, nullptr,
+                               "hstu_jagged");
+}
+
+at::Tensor hstu_jagged_table_bias(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v,
+                                  const c10::optional<at::Tensor>& pos_table, const c10::optional<at::Tensor>& ts_table,
+                                  const c10::optional<at::Tensor>& timestamps, const c10::optional<at::Tensor>& attn_bias,
+                                  int64_t mask_type, int64_t max_seq_len, int64_t max_seq_len_k, double silu_scale,
+                                  const at::Tensor& seq_offset, const at::Tensor& seq_offset_k,
+                                  const c10::optional<at::Tensor>& num_context, const c10::optional<at::Tensor>& num_target,
+                                  c10::optional<int64_t> target_group_size, c10::optional<double> alpha,
+                                  double bucket_divisor) {
+    Tables t;
+    t.pos_table = pos_table;
+    t.ts_table = ts_table;
+    t.timestamps = timestamps;
+    t.bucket_divisor = bucket_divisor;
+    return jagged_forward_impl(q, k, v, c10::nullopt, attn_bias, mask_type, max_seq_len, max_seq_len_k, silu_scale,
+                               seq_offset, seq_offset_k, num_context, num_target, target_group_size, alpha, false, &t,
+                               "hstu_jagged_table_bias");
+}
+
+// ---------------------------------------------------------------------------------------------
+// paged (+ fp8 cache extension)
+// ---------------------------------------------------------------------------------------------
+static void check_non_empty(const at::Tensor& t, const char* name) {
+    TORCH_CHECK(t.defined() && t.numel() > 0, name, " must be a non-empty tensor");
+}
+
+static at::Tensor paged_forward_impl(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v,
+                                     const at::Tensor& kv_cache, const c10::optional<at::Tensor>& kv_scales,
+                                     const c10::optional<at::Tensor>& mask, const c10::optional<at::Tensor>& attn_bias,
+                                     int64_t mask_type, int64_t max_seq_len, int64_t max_seq_len_k, double silu_scale,
+                                     const at::Tensor& seq_offset, const at::Tensor& seq_offset_k,
+                                     const at::Tensor& seq_offset_t, const at::Tensor& page_offsets,
+                                     const at::Tensor& page_ids, const at::Tensor& last_page_len,
+                                     const at::Tensor& num_target, int64_t target_group_size,
+                                     const c10::optional<double>& alpha, bool deterministic, const char* op) {
+    check_non_empty(kv_cache, "kv_cache");
+    check_non_empty(page_ids, "page_ids");
+    check_non_empty(last_page_len, "last_page_len");
+    TORCH_CHECK(q.dim() == 3, "The q should be 3D in jagged layout");
+    TORCH_CHECK(k.dim() == 3 && v.dim() == 3, "The k and v should be 3D in jagged layout");
+    TORCH_CHECK(seq_offset.defined() && seq_offset.dim() == 1 && seq_offset.size(0) >= 2,
+                "acSeqOffsetq params error should have at least two element.");
+    TORCH_CHECK(seq_offset_k.defined() && seq_offset_k.dim() == 1 && seq_offset_k.size(0) >= 2,
+                "acSeqOffsetK params error should have at least two element.");
+    TORCH_CHECK(seq_offset_t.defined() && seq_offset_t.dim() == 1 && seq_offset_t.size(0) >= 2,
+                "acSeqOffsetT params error should have at least two element.");
+    TORCH_CHECK(seq_offset.scalar_type() == at::kInt || seq_offset.scalar_type() == at::kLong,
+                "seq_offset dtype expect int32 or int64, but get ", seq_offset.scalar_type());
+    TORCH_CHECK(seq_offset.size(0) == seq_offset_k.size(0) && seq_offset.size(0) == seq_offset_t.size(0),
+                "offsetsLenQ, offsetsLenK and offsetsLenT should have the same shape.");
+    Holder h;
+    const auto it = seq_offset.scalar_type();
+    const int64_t batch = seq_offset.size(0) - 1;
+    auto off_q = h.same(seq_offset);
+    auto off_k = h.index(seq_offset_k, it, -1, "seq_offset_k");
+    auto poff = h.index(page_offsets, it, batch + 1, "page_offsets");
+    auto pids = h.index(page_ids, it, -1, "page_ids");
+    auto plast = h.index(last_page_len, it, batch, "last_page_len");
+    auto dq = h.same(q), dk = h.same(k), dv = h.same(v), cache = h.same(kv_cache);
+
+    max_seq_len_check(max_seq_len);
+    max_seq_len_check(max_seq_len_k);
+    const bool mask_defined = mask.has_value() && mask->defined();
+    mask_check(mask_type, mask_defined);
+    TORCH_CHECK(!num_target.defined() || target_group_size > 0,
+                "targetGroupSize must be greater than 0 when numTarget is defined");
+    auto tgt = h.index(num_target, it, batch, "num_target");
+
+    const int32_t dt = io_dtype(dq, "q");
+    TORCH_CHECK(dk.scalar_type() == dq.scalar_type() && dv.scalar_type() == dq.scalar_type(), "q, k, v dtype mismatch");
+    TORCH_CHECK(dk.sizes() == dv.sizes(), "K, V shape mismatch");
+    TORCH_CHECK(dq.size(2) == dk.size(2), "Q, K, V headDIM Shape Check failed");
+    TORCH_CHECK(cache.dim() == 5 && cache.size(1) == 2, "kv_cache expect [pages, 2, page_size, heads, dim], but get ", cache.sizes());
+    TORCH_CHECK(cache.size(3) == dk.size(1) && cache.size(4) == dk.size(2), "kv_cache heads/dim must match k");
+
+    hstu_fwd_params p;
+    std::memset(&p, 0, sizeof(p));
+    p.struct_size = sizeof(p);
+    p.flags = deterministic ? HSTU_FLAG_DETERMINISTIC : 0u;
+    p.dtype = dt;
+    p.index_type = it == at::kLong ? HSTU_I64 : HSTU_I32;
+    p.total_q = dq.size(0);
+    p.total_k = dk.size(0);
+    p.batch = (int32_t)batch;
+    p.heads_q = (int32_t)dq.size(1);
+    p.heads_k = (int32_t)dk.size(1);
+    p.dim_qk = (int32_t)dq.size(2);
+    p.dim_v = (int32_t)dv.size(2);
+    p.mask_type = (int32_t)mask_type;
+    p.max_seq_len_q = (int32_t)max_seq_len;
+    p.max_seq_len_k = (int32_t)max_seq_len_k;
+    p.target_group_size = (int32_t)target_group_size;
+    p.silu_scale = (float)((silu_scale == 0.0) ? 1.0 / (double)max_seq_len : silu_scale);
+    p.alpha = (float)alpha.value_or(1.0);
+    p.num_pages = cache.size(0);
+    p.page_size = (int32_t)cache.size(2);
+
+    at::Tensor scales;
+    const bool fp8 = cache.scalar_type() == at::kFloat8_e4m3fn || cache.scalar_type() == at::kByte;
+    if (fp8) {
+        TORCH_CHECK(kv_scales.has_value() && kv_scales->defined(), "fp8 kv_cache needs kv_scales [pages, 2, heads]");
+        scales = h.same(kv_scales->to(at::kFloat));
+        TORCH_CHECK(scales.dim() == 3 && scales.size(0) == cache.size(0) && scales.size(1) == 2 && scales.size(2) == cache.size(3),
+                    "kv_scales expect [pages, 2, heads], but get ", scales.sizes());
+        p.cache_dtype = HSTU_FP8_E4M3;
+    } else {
+        TORCH_CHECK(cache.scalar_type() == dq.scalar_type(), "kv_cache dtype must equal the q dtype (or be float8_e4m3fn with kv_scales)");
+        p.cache_dtype = dt;
+    }
+    at::Tensor dmask, dbias;
+    const std::vector<int64_t> full = {batch, dq.size(1), max_seq_len, max_seq_len_k};
+    if (mask_defined && mask_type == 3) {
+        dmask = h.same(*mask);
+        TORCH_CHECK(dmask.scalar_type() == dq.scalar_type(), "mask dtype must equal the q dtype");
+        TORCH_CHECK(dmask.sizes() == at::IntArrayRef(full), "mask shape expect [batch, heads, max_seq_len, max_seq_len_k], but get ", dmask.sizes());
+    }
+    if (attn_bias.has_value() && attn_bias->defined()) {
+        dbias = h.same(*attn_bias);
+        TORCH_CHECK(dbias.scalar_type() == dq.scalar_type(), "attn_bias dtype must equal the q dtype");
+        TORCH_CHECK(dbias.sizes() == at::IntArrayRef(full), "attn_bias shape expect [batch, heads, max_seq_len, max_seq_len_k], but get ", dbias.sizes());
+    }
+    for (const at::Tensor* t : {&dk, &dv, &cache, &off_q, &off_k, &poff, &pids, &plast, &tgt, &dmask, &dbias, &scales})
+        TORCH_CHECK(!t->defined() || t->device() == dq.device(), "all tensors must be on the device of q");
+
+    auto out = at::empty_like(dq);
+    p.q = dq.const_data_ptr();
+    p.k = dk.const_data_ptr();
+    p.v = dv.const_data_ptr();
+    p.out = out.data_ptr();
+    p.mask = ptr_or_null(dmask);
+    p.attn_bias = ptr_or_null(dbias);
+    p.seq_offset_q = off_q.const_data_ptr();
+    p.seq_offset_k = off_k.const_data_ptr();
+    p.num_target = ptr_or_null(tgt);
+    p.kv_cache = cache.const_data_ptr();
+    p.page_offsets = poff.const_data_ptr();
+    p.page_ids = pids.const_data_ptr();
+    p.last_page_len = plast.const_data_ptr();
+    p.kv_scales = (const float*)ptr_or_null(scales);
+    run_abi(hstu_hip_paged_forward_get_workspace_size, hstu_hip_paged_forward, p, dq, op);
+    return out;
+}
+
+at::Tensor hstu_paged(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, const at::Tensor& kv_cache,
+                      const c10::optional<at::Tensor>& mask, const c10::optional<at::Tensor>& attn_bias, int64_t mask_type,
+                      int64_t max_seq_len, int64_t max_seq_len_k, double silu_scale, const at::Tensor& seq_offset,
+                      const at::Tensor& seq_offset_k, const at::Tensor& seq_offset_t, const at::Tensor& page_offsets,
+                      const at::Tensor& page_ids, const at::Tensor& last_page_len, const at::Tensor& num_target,
+                      int64_t target_group_size, c10::optional<double> alpha, bool deterministic) {
+    return paged_forward_impl(q, k, v, kv_cache, c10::nullopt, mask, attn_bias, mask_type, max_seq_len, max_seq_len_k,
+                              silu_scale, seq_offset, seq_offset_k, seq_offset_t, page_offsets, page_ids, last_page_len,
+                              num_target, target_group_size, alpha, deterministic, "hstu_paged");
+}
+
+at::Tensor hstu_paged_fp8(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, const at::Tensor& kv_cache,
+                          const at::Tensor& kv_scales, const c10::optional<at::Tensor>& mask,
+                          const c10::optional<at::Tensor>& attn_bias, int64_t mask_type, int64_t max_seq_len,
+                          int64_t max_seq_len_k, double silu_scale, const at::Tensor& seq_offset,
+                          const at::Tensor& seq_offset_k, const at::Tensor& seq_offset_t, const at::Tensor& page_offsets,
+                          const at::Tensor& page_ids, const at::Tensor& last_page_len, const at::Tensor& num_target,
+                          int64_t target_group_size, c10::optional<double> alpha, bool deterministic) {
+    TORCH_CHECK(kv_cache.defined() && (kv_cache.scalar_type() == at::kFloat8_e4m3fn || kv_cache.scalar_type() == at::kByte),
+                "hstu_paged_fp8 expects a float8_e4m3fn (or uint8 bit pattern) kv_cache");
+    return paged_forward_impl(q, k, v, kv_cache, kv_scales, mask, attn_bias, mask_type, max_seq_len, max_seq_len_k,
+                              silu_scale, seq_offset, seq_offset_k, seq_offset_t, page_offsets, page_ids, last_page_len,
+                              num_target, target_group_size, alpha, deterministic, "hstu_paged_fp8");
+}
+
+// ---------------------------------------------------------------------------------------------
+// dense
+// ---------------------------------------------------------------------------------------------
+at::Tensor hstu_dense(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, const c10::optional<at::Tensor>& mask,
+                      const c10::optional<at::Tensor>& attn_bias, int64_t mask_type, int64_t max_seq_len, double silu_scale) {
+    TORCH_CHECK(q.dim() == 4, "The q should be 4D in dense layout");
+    Holder h;
+    auto dq = h.same(q), dk = h.same(k), dv = h.same(v);
+    max_seq_len_check(max_seq_len);
+    const bool mask_defined = mask.has_value() && mask->defined();
+    mask_check(mask_type, mask_defined);
+    const int32_t dt = io_dtype(dq, "q");
+    TORCH_CHECK(dk.scalar_type() == dq.scalar_type() && dv.scalar_type() == dq.scalar_type(), "q, k, v dtype mismatch");
+    TORCH_CHECK(dq.sizes() == dk.sizes() && dq.sizes() == dv.sizes(), "dense layout needs q, k and v of one shape");
+    TORCH_CHECK(dq.size(1) == max_seq_len, "dense layout: max_seq_len must equal the sequence dimension of q (", dq.size(1), ")");
+
+    hstu_fwd_params p;
+    std::memset(&p, 0, sizeof(p));
+    p.struct_size = sizeof(p);
+    p.dtype = dt;
+    p.index_type = HSTU_I64;
+    p.batch = (int32_t)dq.size(0);
+    p.total_q = p.total_k = dq.size(0) * dq.size(1);
+    p.heads_q = p.heads_k = (int32_t)dq.size(2);
+    p.dim_qk = p.dim_v = (int32_t)dq.size(3);
+    p.mask_type = (int32_t)mask_type;
+    p.max_seq_len_q = p.max_seq_len_k = (int32_t)max_seq_len;
+    p.silu_scale = (float)((silu_scale == 0.0) ? 1.0 / (double)max_seq_len : silu_scale);
+    p.alpha = 1.0f;
+    at::Tensor dmask, dbias;
+    const std::vector<int64_t> full = {dq.size(0), dq.size(2), max_seq_len, max_seq_len};
+    if (mask_defined && mask_type == 3) {
+        dmask = h.same(*mask);
+        TORCH_CHECK(dmask.scalar_type() == dq.scalar_type(), "mask dtype must equal the q dtype");
+        TORCH_CHECK(dmask.sizes() == at::IntArrayRef(full), "mask shape expect [batch, heads, seq, seq], but get ", dmask.sizes());
+    }
+    if (attn_bias.has_value() && attn_bias->defined()) {
+        dbias = h.same(*attn_bias);
+        TORCH_CHECK(dbias.scalar_type() == dq.scalar_type(), "attn_bias dtype must equal the q dtype");
+        TORCH_CHECK(dbias.sizes() == at::IntArrayRef(full), "attn_bias shape expect [batch, heads, seq, seq], but get ", dbias.sizes());
+    }
+    auto out = at::empty_like(dq);
+    p.q = dq.const_data_ptr();
+    p.k = dk.const_data_ptr();
+    p.v = dv.const_data_ptr();
+    p.out = out.data_ptr();
+    p.mask = ptr_or_null(dmask);
+    p.attn_bias = ptr_or_null(dbias);
+    run_abi(hstu_hip_dense_forward_get_workspace_size, hstu_hip_dense_forward, p, dq, "hstu_dense");
+    return out;
+}
+
+TORCH_LIBRARY_FRAGMENT(mxrec, m) {
+    m.def("hstu_jagged.equal(Tensor q, "
+          "                  Tensor k, "
+          "                  Tensor v, "
+          "                  Tensor? mask=None, "
+          "                  Tensor? attn_bias=None, "
+          "                  int mask_type=0, "
+          "                  int max_seq_len=0, "
+          "                  float silu_scale=0.0, "
+          "                  Tensor seq_offset=None, "
+          "                  Tensor? num_context=None, "
+          "                  Tensor? num_target=None, "
+          "                  int? target_group_size=0, "
+          "                  float? alpha=1.0, "
+          "                  bool deterministic=False) -> Tensor");
+    m.def("hstu_jagged.delta(Tensor q, "
+          "                  Tensor k, "
+          "                  Tensor v, "
+          "                  Tensor? mask=None, "
+          "                  Tensor? attn_bias=None, "
+          "                  int mask_type=0, "
+          "                  int max_seq_len=0, "
+          "                  int max_seq_len_k=0, "
+          "                  float silu_scale=0.0, "
+          "                  Tensor seq_offset=None, "
+          "                  Tensor seq_offset_k=None, "
+          "                  Tensor? num_context=None, "
+          "                  Tensor? num_target=None, "
+          "                  int? target_group_size=0, "
+          "                  float? alpha=1.0, "
+          "                  bool deterministic=False) -> Tensor");
+    m.def("hstu_paged(Tensor q, "
+          "           Tensor k, "
+          "           Tensor v, "
+          "           Tensor kv_cache=None, "
+          "           Tensor? mask=None, "
+          "           Tensor? attn_bias=None,"
+          "           int mask_type=0, "
+          "           int max_seq_len=0, "
+          "           int max_seq_len_k=0, "
+          "           float silu_scale=0.0, "
+          "           Tensor seq_offset=None, "
+          "           Tensor seq_offset_k=None, "
+          "           Tensor seq_offset_t=None, "
+          "           Tensor page_offsets=None, "
+          "           Tensor page_ids=None, "
+          "           Tensor last_page_len=None, "
+          "           Tensor num_target=None, "
+          "           int target_group_size=0, "
+          "           float? alpha=1.0, "
+          "           bool deterministic=False) -> Tensor");
+    m.def("hstu_dense(Tensor q, "
+          "           Tensor k, "
+          "           Tensor v, "
+          "           Tensor? mask=None, "
+          "           Tensor? attn_bias=None, "
+          "           int mask_type=0, "
+          "           int max_seq_len=0, "
+          "           float silu_scale=0.0) -> Tensor");
+    // no counterpart in the reference:
+    m.def("hstu_jagged_table_bias(Tensor q, Tensor k, Tensor v, Tensor? pos_table=None, Tensor? ts_table=None, "
+          "Tensor? timestamps=None, Tensor? attn_bias=None, int mask_type=0, int max_seq_len=0, int max_seq_len_k=0, "
+          "float silu_scale=0.0, Tensor seq_offset=None, Tensor seq_offset_k=None, Tensor? num_context=None, "
+          "Tensor? num_target=None, int? target_group_size=0, float? alpha=1.0, float bucket_divisor=0.301) -> Tensor");
+    m.def("hstu_paged_fp8(Tensor q, Tensor k, Tensor v, Tensor kv_cache=None, Tensor kv_scales=None, Tensor? mask=None, "
+          "Tensor? attn_bias=None, int mask_type=0, int max_seq_len=0, int max_seq_len_k=0, float silu_scale=0.0, "
+          "Tensor seq_offset=None, Tensor seq_offset_k=None, Tensor seq_offset_t=None, Tensor page_offsets=None, "
+          "Tensor page_ids=None, Tensor last_page_len=None, Tensor num_target=None, int target_group_size=0, "
+          "float? alpha=1.0, bool deterministic=False) -> Tensor");
+    m.def("hstu_time_bucket_bounds(int num_buckets=128, float bucket_divisor=0.301) -> Tensor", &hstu_time_bucket_bounds);
+}
+
+#define HSTU_IMPLS(m)                                                         \
+    m.impl("hstu_jagged.equal", TORCH_FN(hstu_jagged_equal));                 \
+    m.impl("hstu_jagged.delta", TORCH_FN(hstu_jagged_delta));                 \
+    m.impl("hstu_paged", TORCH_FN(hstu_paged));                               \
+    m.impl("hstu_dense", TORCH_FN(hstu_dense));                               \
+    m.impl("hstu_jagged_table_bias", TORCH_FN(hstu_jagged_table_bias));       \
+    m.impl("hstu_paged_fp8", TORCH_FN(hstu_paged_fp8));
+
+// ROCm tensors dispatch on the CUDA key.  The CPU key runs the same host checks and then
+// reports that there is no CPU implementation.
+TORCH_LIBRARY_IMPL(mxrec, CUDA, m) { HSTU_IMPLS(m) }
+TORCH_LIBRARY_IMPL(mxrec, CPU, m) { HSTU_IMPLS(m) }
+
+}  // namespace mxrec_hstu

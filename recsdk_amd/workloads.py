@@ -1,0 +1,154 @@
+"""Synthetic workloads: the five benchmark configurations of the HSTU forward, built from
+``numpy.random.default_rng(seed)`` so that tests, smoke and bench see identical inputs.
+
+Each builder returns a dict of CPU tensors plus the scalar attributes of the call; ``to_device``
+moves the tensors.  Harness conventions follow the reference's test generators
+(test_hstu_jagged_forward.py:27-90: offsets = cat([0], cumsum(L)); test_hstu_paged_forward.py:324-390:
+pages allocated consecutively per user, partially filled last page zero padded).
+"""
+from __future__ import annotations
+
+import math
+from typing import Dict
+
+import numpy as np
+import torch
+
+FP8_MAX = 448.0
+
+
+def offsets(lengths, dtype=torch.int64) -> torch.Tensor:
+    o = np.zeros(len(lengths) + 1, dtype=np.int64)
+    o[1:] = np.cumsum(np.asarray(lengths, dtype=np.int64))
+    return torch.from_numpy(o).to(dtype)
+
+
+def _normal(rng, shape, dtype, std=0.5):
+    return torch.from_numpy(rng.normal(0.0, std, shape).astype(np.float32)).to(dtype)
+
+
+def causal_flops(lens_q, lens_k, heads, d_qk, d_v) -> float:
+    """FLOPs of both GEMMs over the causal-visible part: sum_b 2*Lq*Lk-ish; for Lq == Lk this is
+    the headline count sum_b 2*L^2*h*d (the two GEMMs, halved by the causal mask)."""
+    f = 0.0
+    for a, c in zip(lens_q, lens_k):
+        vis = a * (c - a) + a * (a + 1) / 2.0          # visible (row, col) pairs with delta = c - a
+        f += 2.0 * vis * heads * (d_qk + d_v)
+    return f
+
+
+def headline_flops(lens, heads, d) -> float:
+    return float(sum(2.0 * l * l * heads * d for l in lens))
+
+
+def jagged_config(seed, batch, heads, dim, lo, hi, dtype, max_seq_len=None, index_dtype=torch.int64) -> Dict:
+    rng = np.random.default_rng(seed)
+    lens = [int(x) for x in rng.integers(lo, hi + 1, batch)]
+    t = sum(lens)
+    return dict(q=_normal(rng, (t, heads, dim), dtype), k=_normal(rng, (t, heads, dim), dtype),
+                v=_normal(rng, (t, heads, dim), dtype), seq_offset=offsets(lens, index_dtype), lens=lens,
+                max_seq_len=max_seq_len or hi, alpha=1.0 / math.sqrt(dim), mask_type=0)
+
+
+def config1(seed=0):
+    """CPU plumbing case: B=4, h=2, d=32, L in [16,128], fp32."""
+    return jagged_config(seed, 4, 2, 32, 16, 128, torch.float32, max_seq_len=128)
+
+
+def config2(seed=0, dtype=torch.bfloat16):
+    """Headline: B=64, h=4, d=128, L in [256,1024], bf16, causal, no bias."""
+    return jagged_config(seed, 64, 4, 128, 256, 1024, dtype, max_seq_len=1024)
+
+
+def zipf_lengths(rng, n, lo, hi, s=1.2):
+    ks = np.arange(lo, hi + 1, dtype=np.float64)
+    pmf = ks ** (-s)
+    cdf = np.cumsum(pmf / pmf.sum())
+    u = rng.random(n)
+    return [int(lo + np.searchsorted(cdf, x)) for x in u]
+
+
+def config3(seed=0, dtype=torch.bfloat16):
+    """Skewed: B=16, h=8, d=128, truncated Zipf(1.2) lengths in [64,4096], rel-pos table of 2*4096-1."""
+    rng = np.random.default_rng(seed)
+    lens = zipf_lengths(rng, 16, 64, 4096)
+    t = sum(lens)
+    c = dict(q=_normal(rng, (t, 8, 128), dtype), k=_normal(rng, (t, 8, 128), dtype), v=_normal(rng, (t, 8, 128), dtype),
+             seq_offset=offsets(lens), lens=lens, max_seq_len=4096, alpha=1.0 / math.sqrt(128), mask_type=0)
+    c["pos_table"] = _normal(rng, (2 * 4096 - 1,), torch.float32, 0.02)
+    return c
+
+
+def config4(seed=0, dtype=torch.bfloat16, batch=128):
+    """Target-aware ranking: h=4, d=64, history in [128,768] + 64 targets, time + position tables."""
+    rng = np.random.default_rng(seed)
+    hist = [int(x) for x in rng.integers(128, 769, batch)]
+    lens = [h + 64 for h in hist]
+    t = sum(lens)
+    c = dict(q=_normal(rng, (t, 4, 64), dtype), k=_normal(rng, (t, 4, 64), dtype), v=_normal(rng, (t, 4, 64), dtype),
+             seq_offset=offsets(lens), lens=lens, max_seq_len=768 + 64, alpha=1.0 / math.sqrt(64), mask_type=0)
+    c["num_target"] = torch.full((batch,), 64, dtype=torch.int64)
+    c["target_group_size"] = 1
+    ts = []
+    for l in lens:
+        gaps = rng.exponential(600.0, l).astype(np.int64)
+        ts.append(1_700_000_000 + np.cumsum(gaps))
+    c["timestamps"] = torch.from_numpy(np.concatenate(ts))
+    c["ts_table"] = _normal(rng, (129,), torch.float32, 0.02)
+    c["pos_table"] = _normal(rng, (2 * c["max_seq_len"] - 1,), torch.float32, 0.02)
+    return c
+
+
+def quantize_pages_fp8(cache: torch.Tensor):
+    """[pages, 2, ps, heads, dim] -> (float8_e4m3fn cache, fp32 scales [pages, 2, heads]) with
+    scale = absmax/448 per (page, k|v, head)."""
+    x = cache.float()
+    amax = x.abs().amax(dim=(2, 4))
+    scales = torch.where(amax > 0, amax / FP8_MAX, torch.ones_like(amax))
+    q8 = (x / scales[:, :, None, :, None]).clamp(-FP8_MAX, FP8_MAX).to(torch.float8_e4m3fn)
+    return q8, scales
+
+
+def paged_config(seed, users, heads, dim, hist_lo, hist_hi, num_cand, page_size, dtype, new_hist=0, shuffle=True) -> Dict:
+    """Per user: ``new_hist`` new history rows + ``num_cand`` candidate rows as q/k/v input; a cached
+    history of uniform length in [hist_lo, hist_hi] (which includes the new history rows)."""
+    rng = np.random.default_rng(seed)
+    hist = [int(x) for x in rng.integers(hist_lo, hist_hi + 1, users)]
+    lq = [new_hist + num_cand] * users
+    t = sum(lq)
+    npages = [(h + page_size - 1) // page_size for h in hist]
+    total = sum(npages)
+    order = rng.permutation(total) if shuffle else np.arange(total)
+    cache = torch.zeros(total, 2, page_size, heads, dim, dtype=dtype)
+    page_ids, page_offsets, last = [], [0], []
+    pos = 0
+    for u, h in enumerate(hist):
+        kv = _normal(rng, (2, npages[u] * page_size, heads, dim), dtype)
+        kv[:, h:] = 0
+        ids = order[pos: pos + npages[u]]
+        pos += npages[u]
+        cache[torch.from_numpy(ids)] = kv.reshape(2, npages[u], page_size, heads, dim).transpose(0, 1)
+        page_ids += [int(i) for i in ids]
+        page_offsets.append(pos)
+        last.append(h % page_size or page_size)
+    lk = [h + num_cand for h in hist]
+    i32 = torch.int32
+    return dict(q=_normal(rng, (t, heads, dim), dtype), k=_normal(rng, (t, heads, dim), dtype),
+                v=_normal(rng, (t, heads, dim), dtype), kv_cache=cache, seq_offset=offsets(lq, i32),
+                seq_offset_k=offsets(lk, i32), seq_offset_t=offsets([num_cand] * users, i32),
+                page_offsets=torch.tensor(page_offsets, dtype=i32), page_ids=torch.tensor(page_ids, dtype=i32),
+                last_page_len=torch.tensor(last, dtype=i32), num_target=torch.full((users,), num_cand, dtype=i32),
+                target_group_size=1, hist=hist, lens_q=lq, lens_k=lk, max_seq_len=max(lq), max_seq_len_k=max(lk),
+                alpha=1.0 / math.sqrt(dim), mask_type=0)
+
+
+def config5(seed=0, users=32):
+    """Candidate scoring: 256 candidates per user against a cached history in [1024,4096];
+    fp8-e4m3 cache in 64-token pages with per-(page, k|v, head) scales."""
+    c = paged_config(seed, users, 4, 128, 1024, 4096, 256, 64, torch.bfloat16)
+    c["kv_cache_fp8"], c["kv_scales"] = quantize_pages_fp8(c["kv_cache"])
+    return c
+
+
+def to_device(cfg: Dict, device="cuda") -> Dict:
+    return {k: (v.to(device) if isinstance(v, torch.Tensor) else v) for k, v in cfg.items()}
