@@ -1,0 +1,149 @@
+#!/usr/bin/env python3
+"""Benchmark of the HSTU jagged attention forward on one MI355X.
+
+A step is one call of the hot path (``hstu_hip_jagged_forward`` / ``hstu_hip_paged_forward`` through
+the C ABI, on torch's current stream) over one synthetic batch whose inputs are already resident in
+HBM.  Default workload: the headline configuration (B=64, h=4, d=128, L~U[256,1024], bf16, causal,
+no bias, seed 0).  Prints ONE JSON line.
+
+FLOPs follow the metric's definition: sum over sequences of 2*L^2*h*d (both GEMMs, halved by the
+causal mask); for the paged workload 4*Lq*Lk*h*d (no causal halving: candidates see all history).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0
+
+
+def build_workload(name, torch, W):
+    if name == "config2":
+        c = W.config2()
+        flops = W.headline_flops(c["lens"], 4, 128)
+        t = sum(c["lens"])
+        desc = "config2 headline: B=64 h=4 d=128 L~U[256,1024] bf16 causal no-bias seed0"
+        return c, "jagged", flops, 4 * t * 4 * 128 * 2, desc
+    if name == "config3":
+        c = W.config3()
+        flops = W.headline_flops(c["lens"], 8, 128)
+        t = sum(c["lens"])
+        return c, "jagged", flops, 4 * t * 8 * 128 * 2 + 8191 * 4, "config3 skewed: B=16 h=8 d=128 Zipf(1.2) L in [64,4096] bf16 rel-pos table"
+    if name == "config4":
+        c = W.config4()
+        flops = W.headline_flops(c["lens"], 4, 64)
+        t = sum(c["lens"])
+        return c, "jagged", flops, 4 * t * 4 * 64 * 2 + t * 8, "config4 target-aware: B=128 h=4 d=64 hist~U[128,768]+64 targets bf16 time+pos tables"
+    if name == "config5":
+        c = W.config5()
+        c["use_fp8"] = True
+        flops = float(sum(4.0 * 256 * (h + 1) * 4 * 128 for h in c["hist"]))
+        kv = sum(c["hist"]) * 2 * 4 * 128
+        qo = 2 * 32 * 256 * 4 * 128 * 2
+        return c, "paged", flops, kv + 2 * qo, "config5 paged fp8-KV: 32 users x 256 candidates, hist~U[1024,4096], 64-token pages"
+    raise SystemExit(f"unknown workload {name}")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py: this build runs on ONE GPU (the path is single-device; see DESIGN.md for how it "
+                         "would shard). Run with --gpus 1.")
+    import torch
+    import recsdk_amd  # noqa: F401  (fails loudly if the HIP libraries are missing)
+    from recsdk_amd import _capi, workloads as W
+
+    assert torch.cuda.is_available(), "bench.py needs the MI355X"
+    cfg, op, flops, alg_bytes, desc = build_workload(args.workload, torch, W)
+    dev = W.to_device(cfg)
+    q, k, v = dev["q"], dev["k"], dev["v"]
+    out = torch.empty_like(q)
+    kw = dict(seq_offset_q=dev["seq_offset"], seq_offset_k=dev.get("seq_offset_k"), max_seq_len_q=cfg["max_seq_len"],
+              max_seq_len_k=cfg.get("max_seq_len_k"), mask_type=0, alpha=cfg["alpha"], num_target=dev.get("num_target"),
+              target_group_size=cfg.get("target_group_size", 0), pos_table=dev.get("pos_table"),
+              ts_table=dev.get("ts_table"), timestamps=dev.get("timestamps"))
+    if cfg.get("ts_table") is not None:
+        kw["ts_bounds"] = recsdk_amd.time_bucket_bounds(128, 0.301).cuda()
+    if op == "paged":
+        kw.update(kv_cache=dev["kv_cache_fp8"], kv_scales=dev["kv_scales"], page_offsets=dev["page_offsets"],
+                  page_ids=dev["page_ids"], last_page_len=dev["last_page_len"])
+    params, keep = _capi.make_params(q, k, v, out, **kw)
+    kernel = _capi.describe_kernel(params)
+    import ctypes as C
+    L = _capi.lib()
+    fn = getattr(L, f"hstu_hip_{op}_forward")
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    pref = C.byref(params)
+
+    def step():
+        rc = fn(pref, None, 0, stream)
+        if rc != 0:
+            raise RuntimeError(L.hstu_hip_last_error().decode())
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    kern_ms = e0.elapsed_time(e1) / args.steps        # HIP events on the launch stream: average launch duration
+    tflops = flops / (ms_per_step * 1e-3) / 1e12
+    kern_tflops = flops / (kern_ms * 1e-3) / 1e12
+
+    result = {
+        "metric": "hstu_jagged_attn_fwd_tflops", "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "us_per_call": round(ms_per_step * 1e3, 2), "pct_bf16_mfma_peak": round(100 * tflops / PEAK_BF16_TFLOPS, 2),
+        "config": {"workload": desc, "kernel": kernel, "flops_per_call": flops, "algorithmic_bytes_per_call": alg_bytes,
+                   "entry": f"hstu_hip_{op}_forward (C ABI)", "l2_flushed_between_calls": False},
+        "roofline": {"bound": "mfma", "achieved": round(kern_tflops, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(kern_tflops / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "kernel_us": round(kern_ms * 1e3, 2),
+                     "hbm_algorithmic_gbs": round(alg_bytes / (kern_ms * 1e-3) / 1e9, 1),
+                     "hbm_frac": round(alg_bytes / (kern_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)},
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(cfg, op, flops, torch)
+    print(json.dumps(result), flush=True)
+
+
+def cpu_baseline(cfg, op, flops, torch):
+    """The CPU oracle (a from-scratch port of the reference's PyTorch golden) timed on this box's host
+    cores over the same batch; one warm-up + the best of 2 runs."""
+    from tests import hstu_testlib as T
+    n = torch.get_num_threads()
+    f = (lambda: T.oracle_paged(cfg)) if op == "paged" else (lambda: T.oracle_jagged(cfg, mode="lowp"))
+    if op == "jagged" and (cfg.get("pos_table") is not None or cfg.get("ts_table") is not None):
+        return {"value": None, "unit": "TFLOP/s", "cores": n, "kind": "port",
+                "sample": "not timed: the dense-bias oracle of this workload needs tens of GB"}
+    f()
+    best = 1e30
+    for _ in range(2):
+        t0 = time.perf_counter()
+        f()
+        best = min(best, time.perf_counter() - t0)
+    return {"value": round(flops / best / 1e12, 4), "unit": "TFLOP/s", "cores": n, "kind": "port",
+            "sample": "the whole batch of this workload once (bf16 I/O, the golden's rounding points), "
+                      f"{best:.2f} s on {n} threads", "seconds_per_call": round(best, 3)}
+
+
+if __name__ == "__main__":
+    main()

@@ -1,6 +1,366 @@
-// placeholder until the MFMA kernels land
+// HSTU forward on the gfx950 matrix cores (bf16 / fp16 I/O, head dim 64 or 128).
+//
+// One workgroup (4 waves) owns a 128-row Q tile of one (sequence, head); wave w owns rows 32w..32w+31.
+// K and V tiles of 64 columns stream through LDS, double buffered, one barrier per tile.
+// Per tile and wave:
+//     S^T = K Q^T           v_mfma_f32_32x32x16 with A = K fragment (ds_read_b128), B = Q fragment (registers)
+//     P   = s*sigmoid(a*s)  in registers (v_exp_f32 + v_rcp_f32), mask/bias fused, packed to 16 bit
+//     O^T += V^T P^T        A = V^T fragment (ds_read_b64_tr_b16 transposing loads), B = P straight from
+//                           the S accumulator registers -- the accumulator layout of S^T is exactly the
+//                           B-operand layout PV needs, so the score matrix never leaves the registers.
+// alpha*silu_scale is applied once to the fp32 accumulator in the epilogue (it factors out of the sum).
+// Element-wise order follows the reference (vector_score_inter.h:299-323): x = alpha*(S+bias), SiLU,
+// then scale*mask; P is rounded to the I/O dtype before PV as there (vector_score_inter.h:177-184),
+// S itself stays in fp32.
 #include "hstu_device.h"
+
 namespace hstu {
-bool mfma_supported(const KArgs&, const char** name) { *name = nullptr; return false; }
-hipError_t launch_mfma(const KArgs&, hipStream_t) { return hipErrorNotSupported; }
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((ext_vector_type(8))) short s16x8;
+typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
+
+#define LDS_PTR(type, p) ((__attribute__((address_space(3))) type*)(p))
+
+template <typename T> struct MM;
+template <> struct MM<__bf16> {
+    typedef bf16x8 v8;
+    static __device__ __forceinline__ f32x16 mfma(v8 a, v8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+    static __device__ __forceinline__ unsigned pack2(float x, float y) {
+        bf16x2 r; r[0] = (__bf16)x; r[1] = (__bf16)y; return __builtin_bit_cast(unsigned, r);
+    }
+};
+template <> struct MM<_Float16> {
+    typedef f16x8 v8;
+    static __device__ __forceinline__ f32x16 mfma(v8 a, v8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+    static __device__ __forceinline__ unsigned pack2(float x, float y) {
+        f16x2 r; r[0] = (_Float16)x; r[1] = (_Float16)y; return __builtin_bit_cast(unsigned, r);
+    }
+};
+
+constexpr int BM = 128;  // Q rows per workgroup
+constexpr int BN = 64;   // K columns per step
+constexpr int NT = 256;  // threads
+
+template <int D> struct Tile {
+    static constexpr int KS = D + 8;    // K row stride in elements: +16 B keeps ds_read_b128 of 16 rows on distinct banks
+    static constexpr int VS = D + 32;   // V row stride: +64 B spreads the 4-row transposing reads over the banks
+    static constexpr int NCH = D / 32;  // 16-byte chunks per thread and tile
+    static constexpr int K_ELEMS = BN * KS;
+    static constexpr int V_ELEMS = BN * VS;
+    static constexpr int LDS_BYTES = 2 * (K_ELEMS + V_ELEMS) * 2;
+};
+
+// Source of one K or V row for the tile loader.
+template <typename T, bool PAGED>
+struct RowRef {
+    const void* ptr;  // NULL = zero row
+    float scale;
+    bool fp8;
+};
+
+template <typename T, bool PAGED>
+__device__ __forceinline__ RowRef<T, PAGED> kv_row_ref(const KArgs& a, const Seq& s, int which, int j, int hk, int D) {
+    const hstu_fwd_params& p = a.p;
+    RowRef<T, PAGED> r;
+    r.scale = 1.f;
+    r.fp8 = false;
+    if (PAGED && j < s.hist_k) {
+        const int is64 = p.index_type == HSTU_I64;
+        int64_t page = ld_idx(p.page_ids, s.page0 + j / p.page_size, is64);
+        int slot = j % p.page_size;
+        int64_t e = ((((page * 2 + which) * p.page_size) + slot) * p.heads_k + hk) * (int64_t)D;
+        if (p.cache_dtype == HSTU_FP8_E4M3) {
+            r.ptr = reinterpret_cast<const uint8_t*>(p.kv_cache) + e;
+            r.scale = p.kv_scales[(page * 2 + which) * p.heads_k + hk];
+            r.fp8 = true;
+        } else {
+            r.ptr = reinterpret_cast<const T*>(p.kv_cache) + e;
+        }
+    } else {
+        int64_t row = PAGED ? s.cand_row + (j - s.hist_k) : s.k_start + j;
+        r.ptr = reinterpret_cast<const T*>(which ? p.v : p.k) + (row * p.heads_k + hk) * (int64_t)D;
+    }
+    return r;
 }
+
+template <typename T, bool PAGED>
+__device__ __forceinline__ u32x4 load_chunk(const RowRef<T, PAGED>& r, int cc) {
+    if (PAGED && r.fp8) {
+        u32x2 raw = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint8_t*>(r.ptr) + cc * 8);
+        // e4m3 -> fp32 (exact), times the fp32 scale, rounded once to the I/O dtype.  The scaled
+        // pack-convert instruction only honours the exponent of its scale operand, so it is not used.
+        u32x4 o;
+#pragma unroll
+        for (int x = 0; x < 4; x++) {
+            f32x2 f = (x & 1) ? __builtin_amdgcn_cvt_pk_f32_fp8(raw[x >> 1], true) : __builtin_amdgcn_cvt_pk_f32_fp8(raw[x >> 1], false);
+            o[x] = MM<T>::pack2(f[0] * r.scale, f[1] * r.scale);
+        }
+        return o;
+    }
+    return *reinterpret_cast<const u32x4*>(reinterpret_cast<const T*>(r.ptr) + cc * 8);
+}
+
+// visibility class of a 32x32 block (rows r0.., columns c0..) under the built-in mask
+enum { BLK_ALL = 0, BLK_CAUSAL = 1, BLK_PRED = 2, BLK_SKIP = 3 };
+
+__device__ __forceinline__ int classify_block(const Seq& s, int tgs, int r0, int c0) {
+    const bool has_ctx = s.ctx > 0 && r0 < s.ctx;
+    const bool has_tgt = s.tgt > 0 && tgs > 0 && r0 + 31 >= s.hist_q && c0 + 31 >= s.hist_k;
+    if (!has_ctx && c0 > r0 + 31 + s.delta) return BLK_SKIP;
+    if (has_ctx || has_tgt) return BLK_PRED;
+    if (c0 + 31 <= r0 + s.delta) return BLK_ALL;
+    return BLK_CAUSAL;
+}
+
+template <typename T, int D, bool EXTRA, bool PAGED>
+__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void hstu_mfma_kernel(const KArgs a, const int ntiles_attr, const int nbh, const int nbh_pad) {
+    typedef Tile<D> TL;
+    typedef typename MM<T>::v8 v8;
+    const hstu_fwd_params& p = a.p;
+    __shared__ __attribute__((aligned(16))) T lds[2 * (TL::K_ELEMS + TL::V_ELEMS)];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, w = tid >> 6;
+    const int g = lane >> 5, l32 = lane & 31;
+
+    // blockIdx -> (slot, sequence, head).  Slots run from the last Q tile (largest K extent) to the
+    // first so that heavy tiles are dispatched first; nbh_pad is a multiple of 8 so that every tile of
+    // one (sequence, head) lands on the same XCD and its K/V stay in that XCD's L2.
+    const int slot = blockIdx.x / nbh_pad;
+    const int bh_raw = blockIdx.x - slot * nbh_pad;
+    const bool active = bh_raw < nbh;          // padding workgroups only help with the tail rows below
+    const int bh = active ? bh_raw : 0;
+    const int b = bh / p.heads_q, h = bh - b * p.heads_q;
+    const int hk = h / a.head_ratio;
+    const Seq s = load_seq(a, b);
+    const bool tril = p.mask_type == HSTU_MASK_TRIL;
+    const int tgs = p.target_group_size;
+    const T* qbase = reinterpret_cast<const T*>(p.q);
+    T* obase = reinterpret_cast<T*>(p.out);
+
+    // LDS layout: [K buffer 0][V buffer 0][K buffer 1][V buffer 1]
+    constexpr int BUF_ELEMS = TL::K_ELEMS + TL::V_ELEMS;
+
+    // the first slot also sweeps tiles beyond the max_seq_len attribute should a sequence exceed it
+    for (int tile = ntiles_attr - 1 - slot; active && tile * BM < s.lq; tile++) {
+        const int i0 = tile * BM;
+        const int kend = (s.lk > 0) ? k_extent(a, s, i0, min(i0 + BM, s.lq)) : 0;
+        const int ntk = (kend + BN - 1) / BN;
+        const int r0 = i0 + 32 * w;      // first row of this wave
+        const int qi = r0 + l32;         // this lane's Q row
+        const bool qvalid = qi < s.lq;
+
+        // Q fragment (B operand of S^T = K Q^T): column = Q row, k = head-dim index
+        v8 qf[D / 16];
+        {
+            const T* qp = qbase + ((s.q_start + qi) * p.heads_q + h) * (int64_t)D + 8 * g;
+#pragma unroll
+            for (int ds = 0; ds < D / 16; ds++) {
+                u32x4 z = {0, 0, 0, 0};
+                if (qvalid) z = *reinterpret_cast<const u32x4*>(qp + 16 * ds);
+                qf[ds] = __builtin_bit_cast(v8, z);
+            }
+        }
+        f32x16 oacc[D / 32];
+#pragma unroll
+        for (int db = 0; db < D / 32; db++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) oacc[db][r] = 0.f;
+
+        int64_t tq = 0;
+        if (EXTRA && p.ts_table && qvalid && qi + s.delta >= 0) tq = p.timestamps[s.k_start + qi + s.delta];
+
+        u32x4 kreg[TL::NCH], vreg[TL::NCH];
+        auto fetch = [&](int kt) {
+            const int k0 = kt * BN;
+#pragma unroll
+            for (int i = 0; i < TL::NCH; i++) {
+                const int c = tid + NT * i;
+                const int row = c / (D / 8), cc = c % (D / 8);
+                const int j = k0 + row;
+                u32x4 kz = {0, 0, 0, 0}, vz = {0, 0, 0, 0};
+                if (j < kend) {
+                    RowRef<T, PAGED> rk = kv_row_ref<T, PAGED>(a, s, 0, j, hk, D);
+                    RowRef<T, PAGED> rv = kv_row_ref<T, PAGED>(a, s, 1, j, hk, D);
+                    kz = load_chunk<T, PAGED>(rk, cc);
+                    vz = load_chunk<T, PAGED>(rv, cc);
+                }
+                kreg[i] = kz;
+                vreg[i] = vz;
+            }
+        };
+        auto stash = [&](int buf) {
+#pragma unroll
+            for (int i = 0; i < TL::NCH; i++) {
+                const int c = tid + NT * i;
+                const int row = c / (D / 8), cc = c % (D / 8);
+                *reinterpret_cast<u32x4*>(lds + buf * BUF_ELEMS + row * TL::KS + cc * 8) = kreg[i];
+                *reinterpret_cast<u32x4*>(lds + buf * BUF_ELEMS + TL::K_ELEMS + row * TL::VS + cc * 8) = vreg[i];
+            }
+        };
+
+        if (ntk > 0) {
+            fetch(0);
+            stash(0);
+        }
+        __syncthreads();
+
+        for (int kt = 0; kt < ntk; kt++) {
+            const int buf = kt & 1;
+            const int k0 = kt * BN;
+            const T* Kb = lds + buf * BUF_ELEMS;
+            const T* Vb = Kb + TL::K_ELEMS;
+            if (kt + 1 < ntk) fetch(kt + 1);
+
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++) {
+                const int c0 = k0 + 32 * kb;
+                const int cls = tril ? classify_block(s, tgs, r0, c0) : BLK_ALL;
+                if (cls == BLK_SKIP) continue;  // wave-uniform
+                // ---- S^T block: 32 keys x 32 Q rows
+                f32x16 sacc;
+#pragma unroll
+                for (int r = 0; r < 16; r++) sacc[r] = 0.f;
+                const T* kp = Kb + (32 * kb + l32) * TL::KS + 8 * g;
+#pragma unroll
+                for (int ds = 0; ds < D / 16; ds++) {
+                    v8 kf = *reinterpret_cast<const v8*>(kp + 16 * ds);
+                    sacc = MM<T>::mfma(kf, qf[ds], sacc);
+                }
+                // ---- P = s * sigmoid(alpha * s) (scale folded into the epilogue), masked
+                // accumulator register r holds key c0 + 8*(r/4) + 4*g + r%4 for Q row qi
+                float pf[16];
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    float x = sacc[r];
+                    const int j = c0 + 8 * (r >> 2) + 4 * g + (r & 3);
+                    float mval = 1.f;
+                    if (EXTRA) {
+                        const bool in_attr = qi < p.max_seq_len_q && j < p.max_seq_len_k;
+                        const int64_t bm = (((int64_t)b * p.heads_q + h) * p.max_seq_len_q + qi) * (int64_t)p.max_seq_len_k + j;
+                        if (p.attn_bias && in_attr) x += to_float(reinterpret_cast<const T*>(p.attn_bias)[bm]);
+                        if (p.pos_table) {
+                            const int idx = (p.max_seq_len_k - 1) + j - (qi + s.delta);
+                            if (idx >= 0 && idx < 2 * p.max_seq_len_k - 1) x += p.pos_table[idx];
+                        }
+                        if (p.ts_table && j < s.lk) {
+                            float dt = abs_dt_as_float(tq, p.timestamps[s.k_start + j]);
+                            x += p.ts_table[ts_bucket(p.ts_bounds, p.num_buckets, dt)];
+                        }
+                        if (p.mask_type == HSTU_MASK_CUSTOM) mval = in_attr ? to_float(reinterpret_cast<const T*>(p.mask)[bm]) : 0.f;
+                    }
+                    float e = __builtin_amdgcn_exp2f(x * a.exp_scale);
+                    float pv = x * __builtin_amdgcn_rcpf(1.0f + e);
+                    if (EXTRA) pv *= mval;
+                    pf[r] = pv;
+                }
+                if (cls == BLK_CAUSAL) {
+                    const int lim = qi + s.delta - (c0 + 4 * g);  // visible iff 8*(r/4) + r%4 <= lim
+#pragma unroll
+                    for (int r = 0; r < 16; r++) pf[r] = (8 * (r >> 2) + (r & 3) <= lim) ? pf[r] : 0.f;
+                } else if (cls == BLK_PRED) {
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const int j = c0 + 8 * (r >> 2) + 4 * g + (r & 3);
+                        pf[r] = builtin_visible(s, tgs, qi, j) ? pf[r] : 0.f;
+                    }
+                }
+                // ---- O^T += V^T P^T : two 16-key steps per block
+#pragma unroll
+                for (int hh = 0; hh < 2; hh++) {
+                    u32x4 pk;
+#pragma unroll
+                    for (int x = 0; x < 4; x++) pk[x] = MM<T>::pack2(pf[8 * hh + 2 * x], pf[8 * hh + 2 * x + 1]);
+                    const v8 pb = __builtin_bit_cast(v8, pk);
+                    // transposing LDS read: a 16-lane group reads 4 key rows x 16 columns and every lane
+                    // receives 4 consecutive keys of one column
+                    const T* vp = Vb + (32 * kb + 16 * hh + 4 * g + ((lane & 15) >> 2)) * TL::VS + 16 * (l32 >> 4) + 4 * (lane & 3);
+#pragma unroll
+                    for (int db = 0; db < D / 32; db++) {
+                        s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, vp + 32 * db));
+                        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, vp + 32 * db + 8 * TL::VS));
+                        s16x8 vv = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                        oacc[db] = MM<T>::mfma(__builtin_bit_cast(v8, vv), pb, oacc[db]);
+                    }
+                }
+            }
+
+            if (kt + 1 < ntk) stash(buf ^ 1);
+            __syncthreads();
+        }
+
+        // ---- epilogue: O^T accumulator register r of block db holds d = 32*db + 8*(r/4) + 4*g + r%4 for row qi
+        if (qvalid) {
+            T* op = obase + ((s.q_start + qi) * p.heads_q + h) * (int64_t)D + 4 * g;
+#pragma unroll
+            for (int db = 0; db < D / 32; db++) {
+#pragma unroll
+                for (int rr = 0; rr < 4; rr++) {
+                    u32x2 o;
+                    o[0] = MM<T>::pack2(oacc[db][4 * rr] * a.out_scale, oacc[db][4 * rr + 1] * a.out_scale);
+                    o[1] = MM<T>::pack2(oacc[db][4 * rr + 2] * a.out_scale, oacc[db][4 * rr + 3] * a.out_scale);
+                    *reinterpret_cast<u32x2*>(op + 32 * db + 8 * rr) = o;
+                }
+            }
+        }
+        __syncthreads();
+        if (slot != 0) break;
+    }
+
+    // rows past the last offset are zero (the reference zero-fills its output: hstu_jagged.cpp:56-59)
+    if (p.seq_offset_q) {
+        const int is64 = p.index_type == HSTU_I64;
+        const int64_t tail = ld_idx(p.seq_offset_q, p.batch, is64);
+        if (tail < p.total_q) {
+            const int64_t n = (p.total_q - tail) * p.heads_q * (int64_t)D;
+            T* o = obase + tail * p.heads_q * (int64_t)D;
+            for (int64_t e = (int64_t)blockIdx.x * NT + tid; e < n; e += (int64_t)gridDim.x * NT) o[e] = (T)0.f;
+        }
+    }
+}
+
+bool mfma_supported(const KArgs& a, const char** name) {
+    const hstu_fwd_params& p = a.p;
+    *name = nullptr;
+    if (p.dtype != HSTU_BF16 && p.dtype != HSTU_F16) return false;
+    if (p.dim_qk != p.dim_v || (p.dim_qk != 64 && p.dim_qk != 128)) return false;
+    const bool bf = p.dtype == HSTU_BF16;
+    if (p.dim_qk == 128) *name = bf ? "mfma_bf16_d128" : "mfma_f16_d128";
+    else *name = bf ? "mfma_bf16_d64" : "mfma_f16_d64";
+    return true;
+}
+
+template <typename T, int D>
+static hipError_t launch_td(const KArgs& a, hipStream_t stream) {
+    const hstu_fwd_params& p = a.p;
+    const int ntiles = (p.max_seq_len_q + BM - 1) / BM;
+    const int nbh = p.batch * p.heads_q;
+    const int nbh_pad = (nbh + 7) / 8 * 8;
+    const bool extra = p.attn_bias || p.pos_table || p.ts_table || p.mask_type == HSTU_MASK_CUSTOM;
+    const bool paged = a.op == OP_PAGED;
+    dim3 grid((unsigned)(ntiles * nbh_pad)), block(NT);
+    if (paged) {
+        if (extra) hipLaunchKernelGGL((hstu_mfma_kernel<T, D, true, true>), grid, block, 0, stream, a, ntiles, nbh, nbh_pad);
+        else hipLaunchKernelGGL((hstu_mfma_kernel<T, D, false, true>), grid, block, 0, stream, a, ntiles, nbh, nbh_pad);
+    } else {
+        if (extra) hipLaunchKernelGGL((hstu_mfma_kernel<T, D, true, false>), grid, block, 0, stream, a, ntiles, nbh, nbh_pad);
+        else hipLaunchKernelGGL((hstu_mfma_kernel<T, D, false, false>), grid, block, 0, stream, a, ntiles, nbh, nbh_pad);
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_mfma(const KArgs& a, hipStream_t stream) {
+    const hstu_fwd_params& p = a.p;
+    if (p.dtype == HSTU_BF16) return p.dim_qk == 128 ? launch_td<__bf16, 128>(a, stream) : launch_td<__bf16, 64>(a, stream);
+    return p.dim_qk == 128 ? launch_td<_Float16, 128>(a, stream) : launch_td<_Float16, 64>(a, stream);
+}
+
+}  // namespace hstu

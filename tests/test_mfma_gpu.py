@@ -1,0 +1,187 @@
+"""GPU parity tests of the MFMA kernels (bf16/fp16, head dim 64/128) against the CPU oracle and
+against the plain-FMA kernel, through the C ABI."""
+import math
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import hstu_oracle as O
+from recsdk_amd import workloads as W
+from tests import hstu_testlib as T
+from tests.test_parity_gpu import _jag, say, FORCE_GENERIC
+
+pytestmark = pytest.mark.gpu
+LOWP = [torch.bfloat16, torch.float16]
+
+
+def _check(cfg, dtype, what, op="jagged", oracle=None, tol=None, **kw):
+    ref = oracle if oracle is not None else T.oracle_jagged(cfg)
+    out, name = T.run_capi(cfg, op=op, **kw)
+    assert name.startswith("mfma_"), name
+    T.assert_parity(out, ref, dtype, what=what + " vs oracle", tol=tol)
+    gen, gname = T.run_capi(cfg, op=op, flags=FORCE_GENERIC, **kw)
+    assert gname.startswith("generic")
+    T.assert_parity(out, gen.float(), dtype, what=what + " vs generic kernel", tol=tol)
+    return out
+
+
+@pytest.mark.parametrize("dtype", LOWP)
+@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("lens", [[1], [31, 32, 33], [63, 64, 65, 127, 128, 129], [300, 0, 17, 0], [513, 257]])
+def test_mfma_causal_shapes(lens, d, dtype):
+    say("mfma_causal", dtype, d, lens)
+    cfg, _ = _jag(21, lens, 4, 4, d, d, dtype)
+    _check(cfg, dtype, f"causal d={d} lens={lens}")
+
+
+@pytest.mark.parametrize("dtype", LOWP)
+@pytest.mark.parametrize("d", [64, 128])
+def test_mfma_gqa_delta_int32_tail(d, dtype):
+    say("mfma_gqa_delta", dtype, d)
+    cfg, _ = _jag(22, [70, 200, 33], 8, 2, d, d, dtype, lens_k=[130, 200, 97], index_dtype=torch.int32, extra_rows=7)
+    out = _check(cfg, dtype, "gqa+delta")
+    assert torch.equal(out[-7:], torch.zeros_like(out[-7:]))
+    cfg["mask_type"] = 2
+    _check(cfg, dtype, "no mask")
+    # max_seq_len attribute smaller than the longest sequence: every row must still be produced
+    cfg2, _ = _jag(23, [300, 140], 2, 2, d, d, dtype)
+    cfg2["max_seq_len"] = 100
+    _check(cfg2, dtype, "short max_seq_len attr")
+
+
+@pytest.mark.parametrize("dtype", LOWP)
+@pytest.mark.parametrize("ctx,tgt,tgs", [(3, 0, 0), (0, 6, 1), (40, 70, 3), (2, 7, 0), (0, 64, 1), (33, 33, 33)])
+def test_mfma_builtin_masks(ctx, tgt, tgs, dtype):
+    say("mfma_masks", dtype, ctx, tgt, tgs)
+    cfg, _ = _jag(24, [140, 271, 129], 2, 2, 64, 64, dtype)
+    cfg["num_context"] = torch.tensor([ctx, ctx, ctx])
+    cfg["num_target"] = torch.tensor([tgt, tgt + 1 if tgt else 0, tgt])
+    cfg["target_group_size"] = tgs
+    _check(cfg, dtype, "builtin masks")
+    cfg2, _ = _jag(25, [90, 150], 2, 1, 128, 128, dtype, lens_k=[190, 150])
+    cfg2["num_target"] = torch.tensor([tgt, tgt]); cfg2["num_context"] = torch.tensor([ctx, ctx])
+    cfg2["target_group_size"] = tgs
+    _check(cfg2, dtype, "builtin masks + delta")
+
+
+@pytest.mark.parametrize("dtype", LOWP)
+def test_mfma_bias_and_custom_mask(dtype):
+    say("mfma_bias_mask", dtype)
+    lens = [137, 64, 290]
+    cfg, rng = _jag(26, lens, 2, 2, 64, 64, dtype)
+    b, n, m = 3, 2, max(lens)
+    cfg["attn_bias"] = torch.from_numpy(rng.random((b, n, m, m)).astype(np.float32)).to(dtype)
+    _check(cfg, dtype, "dense bias")
+    cfg["mask"] = torch.from_numpy(rng.integers(0, 2, (b, n, m, m)).astype(np.float32)).to(dtype)
+    cfg["mask_type"] = 3
+    _check(cfg, dtype, "dense bias + custom mask")
+
+
+@pytest.mark.parametrize("dtype", LOWP)
+@pytest.mark.parametrize("d", [64, 128])
+def test_mfma_table_bias(d, dtype):
+    say("mfma_tables", dtype, d)
+    rng = np.random.default_rng(27)
+    lens, lens_k = [150, 77, 320], [150, 190, 320]
+    cfg, _ = _jag(27, lens, 2, 2, d, d, dtype, lens_k=lens_k)
+    mk = cfg["max_seq_len_k"]
+    cfg["pos_table"] = torch.from_numpy(rng.normal(0, 0.5, 2 * mk - 1).astype(np.float32))
+    cfg["ts_table"] = torch.from_numpy(rng.normal(0, 0.5, 129).astype(np.float32))
+    ts = [1_700_000_000 + np.cumsum(rng.exponential(600.0, l).astype(np.int64)) for l in lens_k]
+    ts[1][5:9] = ts[1][5]
+    cfg["timestamps"] = torch.from_numpy(np.concatenate(ts))
+    cfg["num_target"] = torch.tensor([4, 4, 64]); cfg["target_group_size"] = 1
+    out = _check(cfg, dtype, "fused tables")
+    assert torch.equal(T.run_op(cfg, op="table"), out)
+
+
+@pytest.mark.parametrize("dtype", LOWP)
+@pytest.mark.parametrize("d,page_size,new_hist", [(64, 32, 0), (128, 64, 7), (128, 16, 130)])
+def test_mfma_paged(d, page_size, new_hist, dtype):
+    say("mfma_paged", dtype, d, page_size, new_hist)
+    cfg = W.paged_config(28, 5, 2, d, new_hist + 1, 400, 40, page_size, dtype, new_hist=new_hist)
+    out = _check(cfg, dtype, "paged", op="paged", oracle=T.oracle_paged(cfg))
+    assert torch.equal(T.run_op(cfg, op="paged"), out)
+
+
+@pytest.mark.parametrize("d", [64, 128])
+def test_mfma_paged_fp8(d):
+    """fp8 cache == the same kernel on the dequantised cache (bit for bit), <= 5e-2 from the unquantised oracle."""
+    say("mfma_paged_fp8", d)
+    cfg = W.paged_config(29, 4, 2, d, 100, 700, 48, 64, torch.bfloat16)
+    cfg["kv_cache_fp8"], cfg["kv_scales"] = W.quantize_pages_fp8(cfg["kv_cache"])
+    out8, name = T.run_capi(cfg, op="paged", use_fp8=True)
+    assert name.startswith("mfma_")
+    deq = O.dequantize_kv_cache_fp8(cfg["kv_cache_fp8"].view(torch.uint8), cfg["kv_scales"], torch.bfloat16)
+    out16, _ = T.run_capi(dict(cfg, kv_cache=deq), op="paged")
+    assert torch.equal(out8, out16)
+    T.assert_parity(out8, T.oracle_paged(cfg), torch.bfloat16, tol=5e-2, what="fp8 vs unquantised oracle")
+    assert torch.equal(T.run_op(cfg, op="paged_fp8"), out8)
+
+
+def test_mfma_dense_layout():
+    say("mfma_dense")
+    rng = np.random.default_rng(30)
+    b, s, n, d = 3, 200, 2, 64
+    mk = lambda: torch.from_numpy(rng.normal(0, 0.5, (b, s, n, d)).astype(np.float32)).to(torch.bfloat16)
+    cfg = dict(q=mk(), k=mk(), v=mk(), max_seq_len=s, mask_type=0)
+    ref = O.hstu_dense_forward(cfg["q"], cfg["k"], cfg["v"], max_seq_len=s)
+    out, name = T.run_capi(cfg, op="dense")
+    assert name == "mfma_bf16_d64"
+    T.assert_parity(out, ref, torch.bfloat16)
+
+
+# ---- BASELINE configurations at full size ---------------------------------------------------
+def test_config2_headline_full_size():
+    """B=64, h=4, d=128, L in [256,1024], bf16, causal, no bias: oracle parity + the reference's own
+    criteria (mismatch ratio test_common_utils.py:57-61; double benchmark pytorch_native_backend.py:199-229)."""
+    cfg = W.config2()
+    say("config2", sum(cfg["lens"]))
+    ref = T.oracle_jagged(cfg)
+    out, name = T.run_capi(cfg)
+    assert name == "mfma_bf16_d128"
+    T.assert_parity(out, ref, torch.bfloat16, what="config2")
+    lowp = T.oracle_jagged(cfg, mode="lowp")
+    assert O.mismatch_ratio_close(out, lowp, 5e-3, 5e-3)
+    assert O.double_benchmark_close(out, lowp, ref, multiplier=2)
+    assert torch.equal(T.run_op(cfg), out)
+    # size-independent properties: linear in V; causal (perturbing the tail of K/V leaves earlier rows alone)
+    v2 = (cfg["v"].float() * 2).to(torch.bfloat16)
+    out2, _ = T.run_capi(cfg, v=v2)
+    assert torch.allclose(out2.float(), 2 * out.float(), rtol=2e-2, atol=1e-6)
+    o = cfg["seq_offset"].tolist()
+    k3, v3 = cfg["k"].clone(), cfg["v"].clone()
+    k3[o[1] - 50: o[1]] += 1; v3[o[1] - 50: o[1]] -= 1
+    out3, _ = T.run_capi(cfg, k=k3, v=v3)
+    assert torch.equal(out3[: o[1] - 50], out[: o[1] - 50]) and torch.equal(out3[o[1]:], out[o[1]:])
+    assert not torch.equal(out3[o[1] - 50: o[1]], out[o[1] - 50: o[1]])
+
+
+def test_config3_skewed_with_pos_table():
+    cfg = W.config3()
+    say("config3", cfg["lens"])
+    ref = T.oracle_jagged(cfg)
+    out, name = T.run_capi(cfg)
+    assert name == "mfma_bf16_d128"
+    T.assert_parity(out, ref, torch.bfloat16, what="config3")
+
+
+def test_config4_target_aware():
+    cfg = W.config4(batch=32)   # quarter batch keeps the dense-bias oracle in seconds; bench runs B=128
+    say("config4", sum(cfg["lens"]))
+    ref = T.oracle_jagged(cfg)
+    out, name = T.run_capi(cfg)
+    assert name == "mfma_bf16_d64"
+    T.assert_parity(out, ref, torch.bfloat16, what="config4")
+
+
+def test_config5_paged_fp8():
+    cfg = W.config5(users=8)    # quarter batch for the oracle; bench runs 32 users
+    say("config5", cfg["hist"])
+    out8, name = T.run_capi(cfg, op="paged", use_fp8=True)
+    assert name == "mfma_bf16_d128"
+    deq = O.dequantize_kv_cache_fp8(cfg["kv_cache_fp8"].view(torch.uint8), cfg["kv_scales"], torch.bfloat16)
+    T.assert_parity(out8, T.oracle_paged(cfg, cache=deq), torch.bfloat16, what="config5 vs oracle on dequantised cache")
+    T.assert_parity(out8, T.oracle_paged(cfg), torch.bfloat16, tol=5e-2, what="config5 vs unquantised oracle")
