@@ -20,6 +20,9 @@ sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
+# HBM-side bytes per launch from rocprofv3 FETCH_SIZE/WRITE_SIZE, each scaled by what the same counter reads for the
+# plain 256 MiB copy of `--workload copy` (factors 2.000 and 1.000); see profiles/hstu_mfma_kernel_configs2-5.md
+MEASURED_TRAFFIC_BYTES = {"config2": 330.6e6}
 
 
 def build_workload(name, torch, W):
@@ -54,7 +57,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5"])
+    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "copy"],
+                    help="'copy' runs a plain 256 MiB device copy: the known-size kernel the FETCH_SIZE/WRITE_SIZE counters are scaled by")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -65,6 +69,8 @@ def main():
     from recsdk_amd import _capi, workloads as W
 
     assert torch.cuda.is_available(), "bench.py needs the MI355X"
+    if args.workload == "copy":
+        return copy_calibration(args, torch)
     cfg, op, flops, alg_bytes, desc = build_workload(args.workload, torch, W)
     dev = W.to_device(cfg)
     q, k, v = dev["q"], dev["k"], dev["v"]
@@ -115,7 +121,7 @@ def main():
         "config": {"workload": desc, "kernel": kernel, "flops_per_call": flops, "algorithmic_bytes_per_call": alg_bytes,
                    "entry": f"hstu_hip_{op}_forward (C ABI)", "l2_flushed_between_calls": False},
         "roofline": {"bound": "mfma", "achieved": round(kern_tflops, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(kern_tflops / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "frac": round(kern_tflops / PEAK_BF16_TFLOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
                      "kernel_us": round(kern_ms * 1e3, 2),
                      "hbm_algorithmic_gbs": round(alg_bytes / (kern_ms * 1e-3) / 1e9, 1),
                      "hbm_frac": round(alg_bytes / (kern_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)},
@@ -123,6 +129,25 @@ def main():
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(cfg, op, flops, torch)
     print(json.dumps(result), flush=True)
+
+
+def copy_calibration(args, torch):
+    n = 256 << 20
+    src = torch.randint(0, 255, (n,), dtype=torch.uint8, device="cuda")
+    dst = torch.empty_like(src)
+    for _ in range(args.warmup):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(args.steps):
+        dst.copy_(src)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / args.steps
+    print(json.dumps({"metric": "device_copy", "value": round(2 * n / (ms * 1e-3) / 1e9, 1), "unit": "GB/s", "n_gpus": 1,
+                      "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 5),
+                      "config": {"workload": "plain copy of 256 MiB (reads 262144 KiB, writes 262144 KiB per launch)"}}))
 
 
 def cpu_baseline(cfg, op, flops, torch):

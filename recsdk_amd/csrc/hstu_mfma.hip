@@ -12,6 +12,9 @@
 // Element-wise order follows the reference (vector_score_inter.h:299-323): x = alpha*(S+bias), SiLU,
 // then scale*mask; P is rounded to the I/O dtype before PV as there (vector_score_inter.h:177-184),
 // S itself stays in fp32.
+#include <cstdio>
+#include <cstdlib>
+
 #include "hstu_device.h"
 
 namespace hstu {
@@ -161,12 +164,12 @@ void hstu_mfma_kernel(const KArgs a, const int ntiles_attr, const int nbh, const
         // Q fragment (B operand of S^T = K Q^T): column = Q row, k = head-dim index
         v8 qf[D / 16];
         {
-            const T* qp = qbase + ((s.q_start + qi) * p.heads_q + h) * (int64_t)D + 8 * g;
+            const T* qp = qbase + ((s.q_start + min(qi, s.lq - 1)) * p.heads_q + h) * (int64_t)D + 8 * g;
 #pragma unroll
             for (int ds = 0; ds < D / 16; ds++) {
-                u32x4 z = {0, 0, 0, 0};
-                if (qvalid) z = *reinterpret_cast<const u32x4*>(qp + 16 * ds);
-                qf[ds] = __builtin_bit_cast(v8, z);
+                const u32x4 z = {0, 0, 0, 0};
+                const u32x4 x = *reinterpret_cast<const u32x4*>(qp + 16 * ds);
+                qf[ds] = __builtin_bit_cast(v8, qvalid ? x : z);
             }
         }
         f32x16 oacc[D / 32];
@@ -178,6 +181,9 @@ void hstu_mfma_kernel(const KArgs a, const int ntiles_attr, const int nbh, const
         int64_t tq = 0;
         if (EXTRA && p.ts_table && qvalid && qi + s.delta >= 0) tq = p.timestamps[s.k_start + qi + s.delta];
 
+        // Global -> register -> LDS staging.  Loads are unconditional (rows past the visible range are
+        // clamped to the last visible row and zeroed when written to LDS) so that they stay in straight-line
+        // code and only the LDS write waits for them.
         u32x4 kreg[TL::NCH], vreg[TL::NCH];
         auto fetch = [&](int kt) {
             const int k0 = kt * BN;
@@ -185,25 +191,24 @@ void hstu_mfma_kernel(const KArgs a, const int ntiles_attr, const int nbh, const
             for (int i = 0; i < TL::NCH; i++) {
                 const int c = tid + NT * i;
                 const int row = c / (D / 8), cc = c % (D / 8);
-                const int j = k0 + row;
-                u32x4 kz = {0, 0, 0, 0}, vz = {0, 0, 0, 0};
-                if (j < kend) {
-                    RowRef<T, PAGED> rk = kv_row_ref<T, PAGED>(a, s, 0, j, hk, D);
-                    RowRef<T, PAGED> rv = kv_row_ref<T, PAGED>(a, s, 1, j, hk, D);
-                    kz = load_chunk<T, PAGED>(rk, cc);
-                    vz = load_chunk<T, PAGED>(rv, cc);
-                }
-                kreg[i] = kz;
-                vreg[i] = vz;
+                const int j = min(k0 + row, kend - 1);
+                RowRef<T, PAGED> rk = kv_row_ref<T, PAGED>(a, s, 0, j, hk, D);
+                RowRef<T, PAGED> rv = kv_row_ref<T, PAGED>(a, s, 1, j, hk, D);
+                kreg[i] = load_chunk<T, PAGED>(rk, cc);
+                vreg[i] = load_chunk<T, PAGED>(rv, cc);
             }
         };
-        auto stash = [&](int buf) {
+        auto stash = [&](int kt) {
+            const int k0 = kt * BN;
+            const int buf = kt & 1;
 #pragma unroll
             for (int i = 0; i < TL::NCH; i++) {
                 const int c = tid + NT * i;
                 const int row = c / (D / 8), cc = c % (D / 8);
-                *reinterpret_cast<u32x4*>(lds + buf * BUF_ELEMS + row * TL::KS + cc * 8) = kreg[i];
-                *reinterpret_cast<u32x4*>(lds + buf * BUF_ELEMS + TL::K_ELEMS + row * TL::VS + cc * 8) = vreg[i];
+                const bool ok = k0 + row < kend;
+                const u32x4 z = {0, 0, 0, 0};
+                *reinterpret_cast<u32x4*>(lds + buf * BUF_ELEMS + row * TL::KS + cc * 8) = ok ? kreg[i] : z;
+                *reinterpret_cast<u32x4*>(lds + buf * BUF_ELEMS + TL::K_ELEMS + row * TL::VS + cc * 8) = ok ? vreg[i] : z;
             }
         };
 
@@ -225,15 +230,26 @@ void hstu_mfma_kernel(const KArgs a, const int ntiles_attr, const int nbh, const
                 const int c0 = k0 + 32 * kb;
                 const int cls = tril ? classify_block(s, tgs, r0, c0) : BLK_ALL;
                 if (cls == BLK_SKIP) continue;  // wave-uniform
-                // ---- S^T block: 32 keys x 32 Q rows
+                // ---- S^T block: 32 keys x 32 Q rows.  All K fragments are requested before the first
+                // MFMA so that the LDS latency is paid once per block, not once per instruction.
+                const T* kp = Kb + (32 * kb + l32) * TL::KS + 8 * g;
+                v8 kf[D / 16];
+#pragma unroll
+                for (int ds = 0; ds < D / 16; ds++) kf[ds] = *reinterpret_cast<const v8*>(kp + 16 * ds);
                 f32x16 sacc;
 #pragma unroll
                 for (int r = 0; r < 16; r++) sacc[r] = 0.f;
-                const T* kp = Kb + (32 * kb + l32) * TL::KS + 8 * g;
 #pragma unroll
-                for (int ds = 0; ds < D / 16; ds++) {
-                    v8 kf = *reinterpret_cast<const v8*>(kp + 16 * ds);
-                    sacc = MM<T>::mfma(kf, qf[ds], sacc);
+                for (int ds = 0; ds < D / 16; ds++) sacc = MM<T>::mfma(kf[ds], qf[ds], sacc);
+                // V^T fragments of the first 16-key step: requested now, consumed after the SiLU pass.
+                // Transposing LDS read: a 16-lane group reads 4 key rows x 16 columns and every lane
+                // receives 4 consecutive keys of one column.
+                const T* vp = Vb + (32 * kb + 4 * g + ((lane & 15) >> 2)) * TL::VS + 16 * (l32 >> 4) + 4 * (lane & 3);
+                s16x4 vlo[D / 32], vhi[D / 32];
+#pragma unroll
+                for (int db = 0; db < D / 32; db++) {
+                    vlo[db] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, vp + 32 * db));
+                    vhi[db] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, vp + 32 * db + 8 * TL::VS));
                 }
                 // ---- P = s * sigmoid(alpha * s) (scale folded into the epilogue), masked
                 // accumulator register r holds key c0 + 8*(r/4) + 4*g + r%4 for Q row qi
@@ -267,33 +283,44 @@ void hstu_mfma_kernel(const KArgs a, const int ntiles_attr, const int nbh, const
 #pragma unroll
                     for (int r = 0; r < 16; r++) pf[r] = (8 * (r >> 2) + (r & 3) <= lim) ? pf[r] : 0.f;
                 } else if (cls == BLK_PRED) {
+                    // branch-free form of builtin_visible(); j runs over this lane's 16 keys
+                    const bool ctx_row = s.ctx > 0 && qi < s.ctx;
+                    const bool tgt_row = tgs > 0 && s.tgt > 0 && qi >= s.hist_q;
+                    const int left = tgt_row ? s.hist_k + ((qi - s.hist_q) / tgs) * tgs : 0;  // first visible target column
+                    const int jmax = qi + s.delta;
 #pragma unroll
                     for (int r = 0; r < 16; r++) {
                         const int j = c0 + 8 * (r >> 2) + 4 * g + (r & 3);
-                        pf[r] = builtin_visible(s, tgs, qi, j) ? pf[r] : 0.f;
+                        const bool vis = (ctx_row & (j < s.hist_k)) | ((j <= jmax) & !(tgt_row & (j >= s.hist_k) & (j < left)));
+                        pf[r] = vis ? pf[r] : 0.f;
                     }
                 }
                 // ---- O^T += V^T P^T : two 16-key steps per block
+                u32x4 pk0, pk1;
 #pragma unroll
-                for (int hh = 0; hh < 2; hh++) {
-                    u32x4 pk;
+                for (int x = 0; x < 4; x++) {
+                    pk0[x] = MM<T>::pack2(pf[2 * x], pf[2 * x + 1]);
+                    pk1[x] = MM<T>::pack2(pf[8 + 2 * x], pf[8 + 2 * x + 1]);
+                }
+                s16x4 wlo[D / 32], whi[D / 32];
 #pragma unroll
-                    for (int x = 0; x < 4; x++) pk[x] = MM<T>::pack2(pf[8 * hh + 2 * x], pf[8 * hh + 2 * x + 1]);
-                    const v8 pb = __builtin_bit_cast(v8, pk);
-                    // transposing LDS read: a 16-lane group reads 4 key rows x 16 columns and every lane
-                    // receives 4 consecutive keys of one column
-                    const T* vp = Vb + (32 * kb + 16 * hh + 4 * g + ((lane & 15) >> 2)) * TL::VS + 16 * (l32 >> 4) + 4 * (lane & 3);
+                for (int db = 0; db < D / 32; db++) {   // second step's fragments fly while the first step multiplies
+                    wlo[db] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, vp + 32 * db + 16 * TL::VS));
+                    whi[db] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, vp + 32 * db + 24 * TL::VS));
+                }
 #pragma unroll
-                    for (int db = 0; db < D / 32; db++) {
-                        s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, vp + 32 * db));
-                        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, vp + 32 * db + 8 * TL::VS));
-                        s16x8 vv = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                        oacc[db] = MM<T>::mfma(__builtin_bit_cast(v8, vv), pb, oacc[db]);
-                    }
+                for (int db = 0; db < D / 32; db++) {
+                    s16x8 vv = {vlo[db][0], vlo[db][1], vlo[db][2], vlo[db][3], vhi[db][0], vhi[db][1], vhi[db][2], vhi[db][3]};
+                    oacc[db] = MM<T>::mfma(__builtin_bit_cast(v8, vv), __builtin_bit_cast(v8, pk0), oacc[db]);
+                }
+#pragma unroll
+                for (int db = 0; db < D / 32; db++) {
+                    s16x8 vv = {wlo[db][0], wlo[db][1], wlo[db][2], wlo[db][3], whi[db][0], whi[db][1], whi[db][2], whi[db][3]};
+                    oacc[db] = MM<T>::mfma(__builtin_bit_cast(v8, vv), __builtin_bit_cast(v8, pk1), oacc[db]);
                 }
             }
 
-            if (kt + 1 < ntk) stash(buf ^ 1);
+            if (kt + 1 < ntk) stash(kt + 1);
             __syncthreads();
         }
 
@@ -347,6 +374,11 @@ static hipError_t launch_td(const KArgs& a, hipStream_t stream) {
     const bool extra = p.attn_bias || p.pos_table || p.ts_table || p.mask_type == HSTU_MASK_CUSTOM;
     const bool paged = a.op == OP_PAGED;
     dim3 grid((unsigned)(ntiles * nbh_pad)), block(NT);
+    if (getenv("HSTU_HIP_DEBUG")) {
+        int nb = -1;
+        hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, hstu_mfma_kernel<T, D, false, false>, NT, 0);
+        fprintf(stderr, "[hstu_hip] mfma d=%d grid=%u workgroups/CU=%d (%s)\n", D, grid.x, nb, hipGetErrorString(e));
+    }
     if (paged) {
         if (extra) hipLaunchKernelGGL((hstu_mfma_kernel<T, D, true, true>), grid, block, 0, stream, a, ntiles, nbh, nbh_pad);
         else hipLaunchKernelGGL((hstu_mfma_kernel<T, D, false, true>), grid, block, 0, stream, a, ntiles, nbh, nbh_pad);

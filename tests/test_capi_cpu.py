@@ -1,0 +1,173 @@
+"""CPU-side checks of the boundary: the C-ABI library loads and exports every symbol that
+include/hstu_hip.h declares, the ctypes mirror of the argument block matches the C struct, argument
+validation speaks the reference's messages, and the torch op layer rejects what the reference rejects
+(test_hstu_jagged_forward.py:508-711).  No kernel is launched here."""
+import ctypes as C
+import os
+import re
+
+import pytest
+import torch
+
+import recsdk_amd
+from recsdk_amd import _capi
+from oracle import hstu_oracle as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_functions():
+    src = open(os.path.join(ROOT, "include", "hstu_hip.h")).read()
+    src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
+    return sorted(set(re.findall(r"\b(hstu_hip_\w+)\s*\(", src)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = _declared_functions()
+    assert len(names) >= 9
+    lib = _capi.lib()
+    for n in names:
+        assert hasattr(lib, n), f"{n} is declared in include/hstu_hip.h but not exported"
+    assert sorted(names) == sorted(_capi.EXPORTS)
+    assert lib.hstu_hip_abi_version() == 1
+
+
+def _params(**over):
+    p = _capi.HstuFwdParams()
+    p.struct_size = C.sizeof(_capi.HstuFwdParams)
+    p.dtype, p.index_type = _capi.HSTU_BF16, _capi.HSTU_I64
+    for f in ("q", "k", "v", "out", "seq_offset_q", "seq_offset_k"):
+        setattr(p, f, 0x1000)       # never dereferenced on the host
+    p.total_q = p.total_k = 100
+    p.batch, p.heads_q, p.heads_k, p.dim_qk, p.dim_v = 2, 4, 4, 128, 128
+    p.max_seq_len_q = p.max_seq_len_k = 64
+    p.silu_scale, p.alpha = 1 / 64, 0.1
+    for k, v in over.items():
+        setattr(p, k, v)
+    return p
+
+
+def _ws(p, op="jagged"):
+    n = C.c_uint64(123)
+    rc = getattr(_capi.lib(), f"hstu_hip_{op}_forward_get_workspace_size")(C.byref(p), C.byref(n))
+    return rc, n.value, _capi.lib().hstu_hip_last_error().decode()
+
+
+def test_struct_layout_matches_and_workspace_is_zero():
+    rc, n, msg = _ws(_params())
+    assert rc == 0 and n == 0, msg          # a size mismatch between ctypes and C would be rejected here
+    rc, _, msg = _ws(_params(struct_size=8))
+    assert rc == -1 and "size mismatch" in msg
+
+
+@pytest.mark.parametrize("over,needle", [
+    (dict(batch=0), "batchSize limit (0, 2048]"),
+    (dict(batch=2049), "batchSize limit (0, 2048]"),
+    (dict(max_seq_len_q=20481), "maxSeqLen expect in [1, 20480]"),
+    (dict(max_seq_len_k=0), "maxSeqLenK expect in [1, 20480]"),
+    (dict(heads_q=17, heads_k=17), "head num expect in [1, 16]"),
+    (dict(heads_q=3, heads_k=2), "divisible"),
+    (dict(dim_qk=513), "dim size expect in [1, 512]"),
+    (dict(dim_v=24), "multiple of 16"),
+    (dict(mask_type=1), "not support triu"),
+    (dict(mask_type=3), "use custom mask must have valid mask tensor"),
+    (dict(mask_type=4), "maskType expect in [0, 3]"),
+    (dict(dtype=7), "dtype expect"),
+    (dict(seq_offset_k=None), "seq_offset_q and seq_offset_k must not be NULL"),
+    (dict(kv_cache=0x1000), "only taken by the paged op"),
+])
+def test_validation_messages(over, needle):
+    rc, _, msg = _ws(_params(**over))
+    assert rc == -1 and needle in msg, msg
+
+
+def test_paged_and_dense_validation():
+    rc, _, msg = _ws(_params(), op="paged")
+    assert rc == -1 and "should not be nullptr" in msg
+    ok = _params(kv_cache=0x1000, page_offsets=0x1000, page_ids=0x1000, last_page_len=0x1000, page_size=64,
+                 cache_dtype=_capi.HSTU_BF16)
+    assert _ws(ok, op="paged")[0] == 0
+    rc, _, msg = _ws(_params(kv_cache=0x1000, page_offsets=0x1000, page_ids=0x1000, last_page_len=0x1000,
+                             page_size=64, cache_dtype=_capi.HSTU_FP8_E4M3), op="paged")
+    assert rc == -1 and "kv_scales" in msg
+    rc, _, msg = _ws(_params(), op="dense")
+    assert rc == -1 and "no sequence offsets" in msg
+    d = _params(seq_offset_q=None, seq_offset_k=None, total_q=128, total_k=128)
+    assert _ws(d, op="dense")[0] == 0
+
+
+def test_describe_kernel_selection():
+    buf = C.create_string_buffer(64)
+    lib = _capi.lib()
+    for over, want in [(dict(), "mfma_bf16_d128"), (dict(dim_qk=64, dim_v=64, dtype=_capi.HSTU_F16), "mfma_f16_d64"),
+                       (dict(dtype=_capi.HSTU_F32), "generic_f32"), (dict(dim_v=64), "generic_bf16"),
+                       (dict(flags=_capi.FLAG_FORCE_GENERIC), "generic_bf16")]:
+        p = _params(**over)
+        assert lib.hstu_hip_describe_kernel(C.byref(p), buf, 64) == 0
+        assert buf.value.decode() == want
+
+
+# ---- torch op layer: same checks, same messages, on CPU tensors ------------------------------
+def _call(q, off, mask_type=0, max_len=8, mask=None, **kw):
+    return torch.ops.mxrec.hstu_jagged(q, q, q, mask, None, mask_type, max_len, 0.0, off, **kw)
+
+
+def test_op_schemas_match_the_reference():
+    s = {str(x) for o in ("hstu_jagged", "hstu_paged", "hstu_dense") for x in
+         [torch._C._get_schema("mxrec::" + o, n) for n in (["equal", "delta"] if o == "hstu_jagged" else [""])]}
+    eq = next(x for x in s if "hstu_jagged.equal" in x)
+    assert "Tensor? mask=None, Tensor? attn_bias=None, int mask_type=0, int max_seq_len=0, float silu_scale=0." in eq
+    assert "Tensor? num_context=None, Tensor? num_target=None, int? target_group_size=0, float? alpha=1." in eq
+    assert "bool deterministic=False" in eq
+    de = next(x for x in s if "hstu_jagged.delta" in x)
+    assert "int max_seq_len=0, int max_seq_len_k=0, float silu_scale" in de and "Tensor seq_offset_k=None" in de
+    pg = next(x for x in s if "hstu_paged" in x)
+    for name in ("kv_cache", "seq_offset_t", "page_offsets", "page_ids", "last_page_len", "num_target"):
+        assert name in pg
+
+
+def test_op_error_messages():
+    q = torch.randn(10, 2, 32)
+    off = torch.tensor([0, 4, 10])
+    with pytest.raises(RuntimeError, match="The q should be 3D in jagged layout"):
+        _call(q[0], off)
+    with pytest.raises(RuntimeError, match=r"maxSeqLen expect in \[1, 20480\], but value is 20481"):
+        _call(q, off, max_len=20481)
+    with pytest.raises(RuntimeError, match="maskType current not support triu now"):
+        _call(q, off, mask_type=1)
+    with pytest.raises(RuntimeError, match="use custom mask must have valid mask tensor"):
+        _call(q, off, mask_type=3)
+    with pytest.raises(RuntimeError, match=r"maskType expect in \[0, 3\]"):
+        _call(q, off, mask_type=5)
+    with pytest.raises(RuntimeError, match="acSeqOffset params error should have at least two element"):
+        _call(q, off[:1])
+    with pytest.raises(RuntimeError, match="The length of num_context expect 2"):
+        _call(q, off, num_context=torch.tensor([1, 1, 1]))
+    with pytest.raises(RuntimeError, match="V dim size"):
+        x = torch.randn(10, 2, 24)
+        _call(x, off)
+    with pytest.raises(RuntimeError, match="head num expect"):
+        x = torch.randn(10, 17, 32)
+        _call(x, off)
+    with pytest.raises(RuntimeError, match="The q should be 4D in dense layout"):
+        torch.ops.mxrec.hstu_dense(q, q, q, None, None, 0, 8, 0.0)
+    # the overload is chosen by the type of the 8th positional argument, as in the reference's tests
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        torch.ops.mxrec.hstu_jagged(q, q, q, None, None, 0, 8, 8, 0.0, off, off)
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        _call(q, off)
+
+
+def test_time_bucket_bounds_reproduce_the_reference_formula():
+    """bucket(|dt|) from the bounds == trunc(log(clamp(|dt|,1,e^(128*0.301)))/0.301) in torch fp32
+    (cust_op/test/relative_attn_bias/torch/utils.py:115-123), exactly, for every integer up to 3e6,
+    powers of two and random 63-bit values."""
+    b = recsdk_amd.time_bucket_bounds(128, 0.301)
+    assert b.shape == (130,) and b[0] == 0 and torch.isinf(b[-1]) and torch.all(b[1:] >= b[:-1])
+    g = torch.Generator().manual_seed(0)
+    d = torch.cat([torch.arange(0, 3_000_000, dtype=torch.int64), 2 ** torch.arange(0, 63, dtype=torch.int64),
+                   torch.randint(0, 2 ** 62, (200000,), generator=g)])
+    want = O.time_bucket_ids(torch.zeros(1, dtype=torch.int64), d)[0]
+    got = torch.bucketize(d.to(torch.float32), b[1:-1], right=True)
+    assert torch.equal(want, got)
+    assert want.max() == 128 and want.min() == 0
