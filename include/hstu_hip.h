@@ -118,6 +118,9 @@ typedef struct hstu_fwd_params {
      *   timestamps [total_k] int64 on the K timeline; ts_table [num_buckets+1] float;
      *   ts_bounds [num_buckets+2] float, ascending, bounds[0] = 0, bounds[num_buckets+1] = +inf:
      *     bucket(i,j) = the b with bounds[b] <= (float)|t_i - t_j| < bounds[b+1];  bias += ts_table[bucket]
+     *   ts_log2_scale: optional search hint.  If non-zero, floor(log2(|dt|) * ts_log2_scale) must be within one
+     *     bucket of the answer (for the reference's log buckets: ln(2)/bucket_divisor); the result is always
+     *     decided by ts_bounds.  0 = no hint (binary search).
      * Added to attn_bias when both are given.
      */
     const float* pos_table;
@@ -125,7 +128,7 @@ typedef struct hstu_fwd_params {
     const float* ts_bounds;
     const int64_t* timestamps;
     int32_t num_buckets;
-    int32_t reserved0;
+    float ts_log2_scale;
 } hstu_fwd_params;
 
 /* replaces aclnnHstuJaggedForwardGetWorkspaceSize / aclnnHstuJaggedForward (hstu_jagged.cpp:63-65) */

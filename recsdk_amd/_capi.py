@@ -7,6 +7,7 @@ layer; torch tensors are only used here as owners of device memory (``data_ptr()
 from __future__ import annotations
 
 import ctypes as C
+import math
 import os
 from typing import Optional
 
@@ -42,7 +43,7 @@ class HstuFwdParams(C.Structure):
         ("last_page_len", C.c_void_p), ("kv_scales", C.c_void_p),
         ("num_pages", C.c_int64), ("page_size", C.c_int32), ("cache_dtype", C.c_int32),
         ("pos_table", C.c_void_p), ("ts_table", C.c_void_p), ("ts_bounds", C.c_void_p), ("timestamps", C.c_void_p),
-        ("num_buckets", C.c_int32), ("reserved0", C.c_int32),
+        ("num_buckets", C.c_int32), ("ts_log2_scale", C.c_float),
     ]
 
 
@@ -80,7 +81,7 @@ def make_params(q, k, v, out, *, seq_offset_q=None, seq_offset_k=None, max_seq_l
                 mask_type=MASK_TRIL, mask=None, attn_bias=None, silu_scale=0.0, alpha=1.0, num_context=None,
                 num_target=None, target_group_size=0, kv_cache=None, page_offsets=None, page_ids=None,
                 last_page_len=None, kv_scales=None, pos_table=None, ts_table=None, ts_bounds=None,
-                timestamps=None, flags=0, dense=False):
+                timestamps=None, bucket_divisor=0.301, flags=0, dense=False):
     """Fill an argument block from tensors.  Returns (params, keepalive list)."""
     p = HstuFwdParams()
     p.struct_size = C.sizeof(HstuFwdParams)
@@ -129,6 +130,7 @@ def make_params(q, k, v, out, *, seq_offset_q=None, seq_offset_k=None, max_seq_l
         p.kv_scales = _ptr(kv_scales)
     p.pos_table, p.ts_table, p.ts_bounds, p.timestamps = _ptr(pos_table), _ptr(ts_table), _ptr(ts_bounds), _ptr(timestamps)
     p.num_buckets = 0 if ts_table is None else ts_table.numel() - 1
+    p.ts_log2_scale = 0.0 if ts_table is None or not bucket_divisor else math.log(2.0) / bucket_divisor
     return p, keep
 
 

@@ -90,6 +90,8 @@ static int validate(const hstu_fwd_params* p, int op, KArgs* out) {
     if (p->ts_table) {
         if (!p->timestamps || !p->ts_bounds || p->num_buckets < 1)
             return fail(HSTU_ERR_INVALID_ARGUMENT, "ts_table needs timestamps, ts_bounds and num_buckets >= 1");
+        if (!std::isfinite(p->ts_log2_scale) || p->ts_log2_scale < 0)
+            return fail(HSTU_ERR_INVALID_ARGUMENT, "ts_log2_scale must be finite and non-negative");
     }
 
     out->p = *p;

@@ -122,13 +122,22 @@ __device__ __forceinline__ int classify_block(const Seq& s, int tgs, int r0, int
     return BLK_CAUSAL;
 }
 
-template <typename T, int D, bool EXTRA, bool PAGED>
+// EXTRA: 0 = no bias / built-in mask only, 1 = dense bias and/or custom mask (tables, if any, gathered from
+// global memory), 2 = bias tables only, gathered from LDS-resident copies
+template <typename T, int D, int EXTRA, bool PAGED>
 __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void hstu_mfma_kernel(const KArgs a, const int ntiles_attr, const int nbh, const int nbh_pad) {
     typedef Tile<D> TL;
     typedef typename MM<T>::v8 v8;
     const hstu_fwd_params& p = a.p;
     __shared__ __attribute__((aligned(16))) T lds[2 * (TL::K_ELEMS + TL::V_ELEMS)];
+    // table mode: per K tile a window of the position table and the key timestamps (double buffered with the
+    // K/V tiles), plus the whole time table and its bucket bounds as (lower, upper) pairs
+    constexpr int PW = BM + BN;   // window entries: (j - k0) - (qi - i0) + BM - 1 in [0, BM + BN - 2]
+    __shared__ float lds_pos[EXTRA == 2 ? 2 * PW : 1];
+    __shared__ __attribute__((aligned(8))) long long lds_tk[EXTRA == 2 ? 2 * BN : 1];
+    __shared__ __attribute__((aligned(8))) float lds_tsb[EXTRA == 2 ? 2 * 132 : 1];
+    __shared__ float lds_tst[EXTRA == 2 ? 132 : 1];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, w = tid >> 6;
@@ -180,6 +189,16 @@ void hstu_mfma_kernel(const KArgs a, const int ntiles_attr, const int nbh, const
 
         int64_t tq = 0;
         if (EXTRA && p.ts_table && qvalid && qi + s.delta >= 0) tq = p.timestamps[s.k_start + qi + s.delta];
+        const bool tab_pos = EXTRA == 2 && p.pos_table != nullptr;
+        const bool tab_ts = EXTRA == 2 && p.ts_table != nullptr && p.num_buckets <= 128 && p.ts_log2_scale > 0.f;
+        const bool glb_ts = EXTRA == 2 && p.ts_table != nullptr && !tab_ts;   // tables too large for LDS or no hint
+        if (tab_ts && tid <= p.num_buckets) {
+            lds_tst[tid] = p.ts_table[tid];
+            lds_tsb[2 * tid] = p.ts_bounds[tid];
+            lds_tsb[2 * tid + 1] = p.ts_bounds[tid + 1];
+        }
+        float pw_reg = 0.f;
+        long long tk_reg = 0;
 
         // Global -> register -> LDS staging.  Loads are unconditional (rows past the visible range are
         // clamped to the last visible row and zeroed when written to LDS) so that they stay in straight-line
@@ -197,6 +216,14 @@ void hstu_mfma_kernel(const KArgs a, const int ntiles_attr, const int nbh, const
                 kreg[i] = load_chunk<T, PAGED>(rk, cc);
                 vreg[i] = load_chunk<T, PAGED>(rv, cc);
             }
+            if (EXTRA == 2) {
+                if (tab_pos && tid < PW - 1) {
+                    // window entry e holds pos_table[(max_k - 1) + (k0 + e - (BM - 1) - i0) - delta]
+                    const int idx = (p.max_seq_len_k - 1) + k0 + tid - (BM - 1) - i0 - s.delta;
+                    pw_reg = (idx >= 0 && idx < 2 * p.max_seq_len_k - 1) ? p.pos_table[idx] : 0.f;
+                }
+                if (tab_ts && tid < BN) tk_reg = p.timestamps[s.k_start + min(k0 + tid, s.lk - 1)];
+            }
         };
         auto stash = [&](int kt) {
             const int k0 = kt * BN;
@@ -209,6 +236,10 @@ void hstu_mfma_kernel(const KArgs a, const int ntiles_attr, const int nbh, const
                 const u32x4 z = {0, 0, 0, 0};
                 *reinterpret_cast<u32x4*>(lds + buf * BUF_ELEMS + row * TL::KS + cc * 8) = ok ? kreg[i] : z;
                 *reinterpret_cast<u32x4*>(lds + buf * BUF_ELEMS + TL::K_ELEMS + row * TL::VS + cc * 8) = ok ? vreg[i] : z;
+            }
+            if (EXTRA == 2) {
+                if (tab_pos && tid < PW - 1) lds_pos[buf * PW + tid] = pw_reg;
+                if (tab_ts && tid < BN) lds_tk[buf * BN + tid] = tk_reg;
             }
         };
 
@@ -259,7 +290,7 @@ void hstu_mfma_kernel(const KArgs a, const int ntiles_attr, const int nbh, const
                     float x = sacc[r];
                     const int j = c0 + 8 * (r >> 2) + 4 * g + (r & 3);
                     float mval = 1.f;
-                    if (EXTRA) {
+                    if (EXTRA == 1) {
                         const bool in_attr = qi < p.max_seq_len_q && j < p.max_seq_len_k;
                         const int64_t bm = (((int64_t)b * p.heads_q + h) * p.max_seq_len_q + qi) * (int64_t)p.max_seq_len_k + j;
                         if (p.attn_bias && in_attr) x += to_float(reinterpret_cast<const T*>(p.attn_bias)[bm]);
@@ -273,9 +304,26 @@ void hstu_mfma_kernel(const KArgs a, const int ntiles_attr, const int nbh, const
                         }
                         if (p.mask_type == HSTU_MASK_CUSTOM) mval = in_attr ? to_float(reinterpret_cast<const T*>(p.mask)[bm]) : 0.f;
                     }
+                    if (EXTRA == 2) {
+                        const int jj = 32 * kb + 8 * (r >> 2) + 4 * g + (r & 3);        // j - k0
+                        if (tab_pos) x += lds_pos[buf * PW + jj - (32 * w + l32) + (BM - 1)];
+                        if (tab_ts) {
+                            const float dt = abs_dt_as_float(tq, lds_tk[buf * BN + jj]);
+                            // estimate from log2, then let the bounds decide (the estimate is within one bucket)
+                            int bk = (int)(__builtin_amdgcn_logf(fmaxf(dt, 1.0f)) * p.ts_log2_scale);
+                            bk = min(max(bk, 0), p.num_buckets);
+                            const float lo = lds_tsb[2 * bk], hi = lds_tsb[2 * bk + 1];
+                            bk += (dt >= hi ? 1 : 0) - (dt < lo ? 1 : 0);
+                            x += lds_tst[bk];
+                        } else if (glb_ts && 32 * kb + 8 * (r >> 2) + 4 * g + (r & 3) + k0 < s.lk) {
+                            // no search hint or a table too large for LDS: binary search over the bounds in global memory
+                            float dt = abs_dt_as_float(tq, p.timestamps[s.k_start + j]);
+                            x += p.ts_table[ts_bucket(p.ts_bounds, p.num_buckets, dt)];
+                        }
+                    }
                     float e = __builtin_amdgcn_exp2f(x * a.exp_scale);
                     float pv = x * __builtin_amdgcn_rcpf(1.0f + e);
-                    if (EXTRA) pv *= mval;
+                    if (EXTRA == 1) pv *= mval;
                     pf[r] = pv;
                 }
                 if (cls == BLK_CAUSAL) {
@@ -371,21 +419,26 @@ static hipError_t launch_td(const KArgs& a, hipStream_t stream) {
     const int ntiles = (p.max_seq_len_q + BM - 1) / BM;
     const int nbh = p.batch * p.heads_q;
     const int nbh_pad = (nbh + 7) / 8 * 8;
-    const bool extra = p.attn_bias || p.pos_table || p.ts_table || p.mask_type == HSTU_MASK_CUSTOM;
+    const bool dense_extra = p.attn_bias || p.mask_type == HSTU_MASK_CUSTOM;
+    const bool tables = p.pos_table || p.ts_table;
+    const int extra = dense_extra ? 1 : (tables ? 2 : 0);
     const bool paged = a.op == OP_PAGED;
     dim3 grid((unsigned)(ntiles * nbh_pad)), block(NT);
     if (getenv("HSTU_HIP_DEBUG")) {
         int nb = -1;
-        hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, hstu_mfma_kernel<T, D, false, false>, NT, 0);
+        hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, hstu_mfma_kernel<T, D, 0, false>, NT, 0);
         fprintf(stderr, "[hstu_hip] mfma d=%d grid=%u workgroups/CU=%d (%s)\n", D, grid.x, nb, hipGetErrorString(e));
     }
+#define HSTU_LAUNCH(E, P) hipLaunchKernelGGL((hstu_mfma_kernel<T, D, E, P>), grid, block, 0, stream, a, ntiles, nbh, nbh_pad)
     if (paged) {
-        if (extra) hipLaunchKernelGGL((hstu_mfma_kernel<T, D, true, true>), grid, block, 0, stream, a, ntiles, nbh, nbh_pad);
-        else hipLaunchKernelGGL((hstu_mfma_kernel<T, D, false, true>), grid, block, 0, stream, a, ntiles, nbh, nbh_pad);
+        if (extra == 0) HSTU_LAUNCH(0, true);
+        else HSTU_LAUNCH(1, true);      // paged + bias: the general gather path
     } else {
-        if (extra) hipLaunchKernelGGL((hstu_mfma_kernel<T, D, true, false>), grid, block, 0, stream, a, ntiles, nbh, nbh_pad);
-        else hipLaunchKernelGGL((hstu_mfma_kernel<T, D, false, false>), grid, block, 0, stream, a, ntiles, nbh, nbh_pad);
+        if (extra == 0) HSTU_LAUNCH(0, false);
+        else if (extra == 1) HSTU_LAUNCH(1, false);
+        else HSTU_LAUNCH(2, false);
     }
+#undef HSTU_LAUNCH
     return hipGetLastError();
 }
 

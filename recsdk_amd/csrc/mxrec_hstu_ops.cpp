@@ -223,6 +223,7 @@ static at::Tensor jagged_forward_impl(const at::Tensor& q, const at::Tensor& k, 
             TORCH_CHECK(tsv.dim() == 1 && tsv.size(0) == dk.size(0), "timestamps expect one int64 per K row (", dk.size(0), "), but get ", tsv.sizes());
             tsb = cached_bounds(tst.size(0) - 1, tables->bucket_divisor, dq.device());
             p.num_buckets = (int32_t)(tst.size(0) - 1);
+            p.ts_log2_scale = (float)(std::log(2.0) / tables->bucket_divisor);
         }
     }
     for (const at::Tensor* t : {&dk, &dv, &off_q, &off_k, &ctx, &tgt, &dmask, &dbias, &pos, &tst, &tsv})
