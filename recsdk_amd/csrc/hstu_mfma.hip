@@ -63,51 +63,71 @@ template <int D> struct Tile {
 // Source of one K or V row for the tile loader.
 template <typename T, bool PAGED>
 struct RowRef {
-    const void* ptr;  // NULL = zero row
+    const void* ptr;
     float scale;
     bool fp8;
 };
 
+constexpr int MAXP = 320;  // pages of one user whose ids (and fp8 scales) are kept in LDS; later pages are looked up in global memory
+
 template <typename T, bool PAGED>
-__device__ __forceinline__ RowRef<T, PAGED> kv_row_ref(const KArgs& a, const Seq& s, int which, int j, int hk, int D) {
+__device__ __forceinline__ RowRef<T, PAGED> kv_row_ref(const KArgs& a, const Seq& s, int which, int j, int hk, int D,
+                                                       const int* lds_pid, const float* lds_psc) {
     const hstu_fwd_params& p = a.p;
     RowRef<T, PAGED> r;
     r.scale = 1.f;
     r.fp8 = false;
-    if (PAGED && j < s.hist_k) {
-        const int is64 = p.index_type == HSTU_I64;
-        int64_t page = ld_idx(p.page_ids, s.page0 + j / p.page_size, is64);
-        int slot = j % p.page_size;
-        int64_t e = ((((page * 2 + which) * p.page_size) + slot) * p.heads_k + hk) * (int64_t)D;
-        if (p.cache_dtype == HSTU_FP8_E4M3) {
-            r.ptr = reinterpret_cast<const uint8_t*>(p.kv_cache) + e;
-            r.scale = p.kv_scales[(page * 2 + which) * p.heads_k + hk];
-            r.fp8 = true;
-        } else {
-            r.ptr = reinterpret_cast<const T*>(p.kv_cache) + e;
-        }
-    } else {
-        int64_t row = PAGED ? s.cand_row + (j - s.hist_k) : s.k_start + j;
-        r.ptr = reinterpret_cast<const T*>(which ? p.v : p.k) + (row * p.heads_k + hk) * (int64_t)D;
+    if (!PAGED) {
+        r.ptr = reinterpret_cast<const T*>(which ? p.v : p.k) + ((s.k_start + j) * p.heads_k + hk) * (int64_t)D;
+        return r;
     }
+    // Branch-free: both sources are addressed and one is selected, so the loads that follow stay in
+    // straight-line code.  Page ids (and fp8 scales) come from the LDS copy made at the start of the tile;
+    // the host only selects this kernel when every page index of a sequence fits that copy.
+    const int ps = p.page_size;
+    const bool pow2 = (ps & (ps - 1)) == 0;
+    const bool hist = j < s.hist_k;
+    const int jh = hist ? j : 0;
+    const int pidx = pow2 ? (jh >> (31 - __builtin_clz(ps))) : jh / ps;
+    const int slot = pow2 ? (jh & (ps - 1)) : jh - pidx * ps;
+    const int pc = min(pidx, MAXP - 1);
+    const int64_t page = lds_pid[pc];
+    // one 64-bit multiply per row: page * (elements per page); everything inside a page is 32-bit
+    const unsigned plane = (unsigned)ps * p.heads_k * D;  // elements of the K (or V) half of a page
+    const int64_t e = page * (int64_t)(2u * plane) + (unsigned)(which * plane + (slot * p.heads_k + hk) * D);
+    const bool fp8 = p.cache_dtype == HSTU_FP8_E4M3;
+    const char* cache_ptr = reinterpret_cast<const char*>(p.kv_cache) + (fp8 ? e : e * (int64_t)sizeof(T));
+    const int64_t row = s.cand_row + (j - s.hist_k);
+    const char* in_ptr = reinterpret_cast<const char*>(which ? p.v : p.k) + ((row * p.heads_k + hk) * (int64_t)D) * (int64_t)sizeof(T);
+    r.ptr = hist ? cache_ptr : in_ptr;
+    r.fp8 = hist && fp8;
+    r.scale = r.fp8 ? lds_psc[2 * pc + which] : 1.f;
     return r;
 }
 
+// Issue the load of one 8-element chunk.  fp8 rows are fetched raw (8 bytes) and converted when they are
+// written to LDS, so that nothing waits on the load here.
 template <typename T, bool PAGED>
 __device__ __forceinline__ u32x4 load_chunk(const RowRef<T, PAGED>& r, int cc) {
     if (PAGED && r.fp8) {
         u32x2 raw = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint8_t*>(r.ptr) + cc * 8);
-        // e4m3 -> fp32 (exact), times the fp32 scale, rounded once to the I/O dtype.  The scaled
-        // pack-convert instruction only honours the exponent of its scale operand, so it is not used.
-        u32x4 o;
-#pragma unroll
-        for (int x = 0; x < 4; x++) {
-            f32x2 f = (x & 1) ? __builtin_amdgcn_cvt_pk_f32_fp8(raw[x >> 1], true) : __builtin_amdgcn_cvt_pk_f32_fp8(raw[x >> 1], false);
-            o[x] = MM<T>::pack2(f[0] * r.scale, f[1] * r.scale);
-        }
+        u32x4 o = {raw[0], raw[1], 0u, 0u};
         return o;
     }
     return *reinterpret_cast<const u32x4*>(reinterpret_cast<const T*>(r.ptr) + cc * 8);
+}
+
+// e4m3 -> fp32 (exact), times the fp32 scale, rounded once to the I/O dtype.  The scaled pack-convert
+// instruction only honours the exponent of its scale operand, so it is not used.
+template <typename T>
+__device__ __forceinline__ u32x4 dequant_chunk(u32x4 raw, float scale) {
+    u32x4 o;
+#pragma unroll
+    for (int x = 0; x < 4; x++) {
+        f32x2 f = (x & 1) ? __builtin_amdgcn_cvt_pk_f32_fp8(raw[x >> 1], true) : __builtin_amdgcn_cvt_pk_f32_fp8(raw[x >> 1], false);
+        o[x] = MM<T>::pack2(f[0] * scale, f[1] * scale);
+    }
+    return o;
 }
 
 // visibility class of a 32x32 block (rows r0.., columns c0..) under the built-in mask
@@ -138,6 +158,9 @@ void hstu_mfma_kernel(const KArgs a, const int ntiles_attr, const int nbh, const
     __shared__ __attribute__((aligned(8))) long long lds_tk[EXTRA == 2 ? 2 * BN : 1];
     __shared__ __attribute__((aligned(8))) float lds_tsb[EXTRA == 2 ? 2 * 132 : 1];
     __shared__ float lds_tst[EXTRA == 2 ? 132 : 1];
+    // paged: page ids of this user and, for an fp8 cache, the (K, V) scales of this kv head
+    __shared__ int lds_pid[PAGED ? MAXP : 1];
+    __shared__ float lds_psc[PAGED ? 2 * MAXP : 1];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, w = tid >> 6;
@@ -199,6 +222,21 @@ void hstu_mfma_kernel(const KArgs a, const int ntiles_attr, const int nbh, const
         }
         float pw_reg = 0.f;
         long long tk_reg = 0;
+        if (PAGED) {
+            const int is64 = p.index_type == HSTU_I64;
+            const int np = min((s.hist_k + p.page_size - 1) / p.page_size, MAXP);
+            for (int i = tid; i < np; i += NT) {
+                const int64_t page = ld_idx(p.page_ids, s.page0 + i, is64);
+                lds_pid[i] = (int)page;
+                if (p.cache_dtype == HSTU_FP8_E4M3) {
+                    lds_psc[2 * i] = p.kv_scales[(page * 2 + 0) * p.heads_k + hk];
+                    lds_psc[2 * i + 1] = p.kv_scales[(page * 2 + 1) * p.heads_k + hk];
+                }
+            }
+            __syncthreads();
+        }
+        float kscale[TL::NCH], vscale[TL::NCH];
+        unsigned fp8mask = 0;
 
         // Global -> register -> LDS staging.  Loads are unconditional (rows past the visible range are
         // clamped to the last visible row and zeroed when written to LDS) so that they stay in straight-line
@@ -211,10 +249,15 @@ void hstu_mfma_kernel(const KArgs a, const int ntiles_attr, const int nbh, const
                 const int c = tid + NT * i;
                 const int row = c / (D / 8), cc = c % (D / 8);
                 const int j = min(k0 + row, kend - 1);
-                RowRef<T, PAGED> rk = kv_row_ref<T, PAGED>(a, s, 0, j, hk, D);
-                RowRef<T, PAGED> rv = kv_row_ref<T, PAGED>(a, s, 1, j, hk, D);
+                RowRef<T, PAGED> rk = kv_row_ref<T, PAGED>(a, s, 0, j, hk, D, lds_pid, lds_psc);
+                RowRef<T, PAGED> rv = kv_row_ref<T, PAGED>(a, s, 1, j, hk, D, lds_pid, lds_psc);
                 kreg[i] = load_chunk<T, PAGED>(rk, cc);
                 vreg[i] = load_chunk<T, PAGED>(rv, cc);
+                if (PAGED) {
+                    kscale[i] = rk.scale;
+                    vscale[i] = rv.scale;
+                    fp8mask = (fp8mask & ~(1u << i)) | ((rk.fp8 ? 1u : 0u) << i);
+                }
             }
             if (EXTRA == 2) {
                 if (tab_pos && tid < PW - 1) {
@@ -234,8 +277,13 @@ void hstu_mfma_kernel(const KArgs a, const int ntiles_attr, const int nbh, const
                 const int row = c / (D / 8), cc = c % (D / 8);
                 const bool ok = k0 + row < kend;
                 const u32x4 z = {0, 0, 0, 0};
-                *reinterpret_cast<u32x4*>(lds + buf * BUF_ELEMS + row * TL::KS + cc * 8) = ok ? kreg[i] : z;
-                *reinterpret_cast<u32x4*>(lds + buf * BUF_ELEMS + TL::K_ELEMS + row * TL::VS + cc * 8) = ok ? vreg[i] : z;
+                u32x4 kx = kreg[i], vx = vreg[i];
+                if (PAGED && ((fp8mask >> i) & 1)) {
+                    kx = dequant_chunk<T>(kx, kscale[i]);
+                    vx = dequant_chunk<T>(vx, vscale[i]);
+                }
+                *reinterpret_cast<u32x4*>(lds + buf * BUF_ELEMS + row * TL::KS + cc * 8) = ok ? kx : z;
+                *reinterpret_cast<u32x4*>(lds + buf * BUF_ELEMS + TL::K_ELEMS + row * TL::VS + cc * 8) = ok ? vx : z;
             }
             if (EXTRA == 2) {
                 if (tab_pos && tid < PW - 1) lds_pos[buf * PW + tid] = pw_reg;
@@ -407,6 +455,7 @@ bool mfma_supported(const KArgs& a, const char** name) {
     *name = nullptr;
     if (p.dtype != HSTU_BF16 && p.dtype != HSTU_F16) return false;
     if (p.dim_qk != p.dim_v || (p.dim_qk != 64 && p.dim_qk != 128)) return false;
+    if (a.op == OP_PAGED && (p.max_seq_len_k + p.page_size - 1) / p.page_size > MAXP) return false;  // page ids of a user must fit the LDS copy
     const bool bf = p.dtype == HSTU_BF16;
     if (p.dim_qk == 128) *name = bf ? "mfma_bf16_d128" : "mfma_f16_d128";
     else *name = bf ? "mfma_bf16_d64" : "mfma_f16_d64";
