@@ -91,9 +91,15 @@ def main():
     fn = getattr(L, f"hstu_hip_{op}_forward")
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
     pref = C.byref(params)
+    # two-phase call like the reference's aclnn entry points: size query once, workspace allocated outside the timed region
+    nws = C.c_uint64(0)
+    if getattr(L, f"hstu_hip_{op}_forward_get_workspace_size")(pref, C.byref(nws)) != 0:
+        raise RuntimeError(L.hstu_hip_last_error().decode())
+    ws = torch.empty(max(int(nws.value), 4), dtype=torch.uint8, device="cuda")
+    ws_ptr = C.c_void_p(ws.data_ptr())
 
     def step():
-        rc = fn(pref, None, 0, stream)
+        rc = fn(pref, ws_ptr, nws.value, stream)
         if rc != 0:
             raise RuntimeError(L.hstu_hip_last_error().decode())
 

@@ -103,8 +103,6 @@ static int validate(const hstu_fwd_params* p, int op, KArgs* out) {
 }
 
 static int run(const hstu_fwd_params* p, int op, void* workspace, uint64_t workspace_bytes, void* stream) {
-    (void)workspace;
-    (void)workspace_bytes;
     KArgs a;
     int rc = validate(p, op, &a);
     if (rc != HSTU_OK) return rc;
@@ -113,7 +111,11 @@ static int run(const hstu_fwd_params* p, int op, void* workspace, uint64_t works
     const char* name = nullptr;
     hipError_t e;
     if (!(p->flags & HSTU_FLAG_FORCE_GENERIC) && mfma_supported(a, &name)) {
-        e = launch_mfma(a, st);
+        const uint64_t need = mfma_workspace_bytes(a);
+        if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 3))
+            return fail(HSTU_ERR_WORKSPACE, "workspace of %llu bytes (4-byte aligned) needed, got %llu at %p",
+                        (unsigned long long)need, (unsigned long long)workspace_bytes, workspace);
+        e = launch_mfma(a, workspace, st);
     } else {
         e = launch_generic(a, st);
     }
@@ -126,7 +128,10 @@ static int ws_size(const hstu_fwd_params* p, int op, uint64_t* bytes) {
     KArgs a;
     int rc = validate(p, op, &a);
     if (rc != HSTU_OK) return rc;
-    *bytes = 0;  // every output row has exactly one producing workgroup: no partials, no flags
+    // every output row has exactly one producing workgroup: no partials, no flags; the MFMA kernels keep
+    // their work list here
+    const char* name = nullptr;
+    *bytes = (!(p->flags & HSTU_FLAG_FORCE_GENERIC) && mfma_supported(a, &name)) ? mfma_workspace_bytes(a) : 0;
     return HSTU_OK;
 }
 

@@ -21,6 +21,8 @@ struct KArgs {
 // launchers (defined next to their kernels); return hipError_t of the launch
 hipError_t launch_generic(const KArgs& a, hipStream_t stream);
 bool mfma_supported(const KArgs& a, const char** name);
-hipError_t launch_mfma(const KArgs& a, hipStream_t stream);
+// bytes of device workspace the MFMA path needs for its work list; the buffer needs no initialisation
+uint64_t mfma_workspace_bytes(const KArgs& a);
+hipError_t launch_mfma(const KArgs& a, void* workspace, hipStream_t stream);
 
 }  // namespace hstu

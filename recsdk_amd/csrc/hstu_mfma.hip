@@ -142,11 +142,128 @@ __device__ __forceinline__ int classify_block(const Seq& s, int tgs, int r0, int
     return BLK_CAUSAL;
 }
 
+// ---- work list ------------------------------------------------------------------------------------------
+// The hardware dispatches workgroups in index order and a workgroup that finds no work still costs a slot, so
+// the grid is driven by a list that a one-workgroup kernel builds first from the sequence lengths:
+//   * one item = one 128-row Q tile of one (sequence, head), packed as  seq | head << 12 | tile << 16 | sweep << 24
+//   * sequences are sorted by K length (longest first) and their (sequence, head) groups are dealt to the
+//     8 XCDs in snake order; a group's tiles sit next to each other in its XCD's list, last tile first, so that
+//     the workgroups that share one K/V run at the same time on CUs that share one L2
+//   * workgroup i runs on XCD i % 8 and takes entry i / 8 of that XCD's list: list[i]
+//   * items beyond a list's capacity go to an overflow list that workgroups with an empty slot drain
+// Layout of the workspace (uint32): [0] overflow count, [1] overflow taken, [16 .. 16 + 8*cap) interleaved lists,
+// then the overflow list.
+constexpr unsigned ITEM_EMPTY = 0xffffffffu;
+constexpr int SCHED_NT = 1024;
+constexpr int WS_HEADER = 16;
+
+struct SchedDims {
+    int ntiles_attr;   // Q tiles the max_seq_len_q attribute covers
+    unsigned cap;      // entries per XCD list
+    unsigned bound;    // upper bound of the number of items (= entries of the overflow list)
+};
+
+static SchedDims sched_dims(const hstu_fwd_params& p) {
+    SchedDims d;
+    d.ntiles_attr = (p.max_seq_len_q + BM - 1) / BM;
+    // sum over sequences of min(ceil(lq / BM), ntiles_attr) <= min(total_q / BM + batch, batch * ntiles_attr)
+    const int64_t by_rows = p.total_q / BM + p.batch, by_attr = (int64_t)p.batch * d.ntiles_attr;
+    d.bound = (unsigned)((by_rows < by_attr ? by_rows : by_attr) * p.heads_q);
+    d.cap = (d.bound + 7) / 8 + (unsigned)d.ntiles_attr;
+    return d;
+}
+
+uint64_t mfma_workspace_bytes(const KArgs& a) {
+    const SchedDims d = sched_dims(a.p);
+    return (uint64_t)(WS_HEADER + 8 * (uint64_t)d.cap + d.bound) * sizeof(uint32_t);
+}
+
+__device__ __forceinline__ int xcd_of_group(unsigned r) { return (r & 8) ? 7 - (int)(r & 7) : (int)(r & 7); }
+
+__global__ __launch_bounds__(SCHED_NT)
+void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict__ ws) {
+    const hstu_fwd_params& p = a.p;
+    __shared__ unsigned short s_tiles[HSTU_MAX_BATCH];    // tiles of a sequence, by batch index
+    __shared__ unsigned short s_order[HSTU_MAX_BATCH];    // batch index, by rank
+    __shared__ unsigned char s_key[HSTU_MAX_BATCH];
+    __shared__ unsigned char s_sweep[HSTU_MAX_BATCH];
+    __shared__ unsigned s_hist[256], s_base[256];
+    __shared__ unsigned s_val[SCHED_NT], s_scan[SCHED_NT];
+    __shared__ unsigned s_cbase[16], s_ovf;
+    const int tid = threadIdx.x;
+    unsigned* list = ws + WS_HEADER;
+    unsigned* ovf = list + 8 * (size_t)d.cap;
+
+    for (size_t i = tid; i < 8 * (size_t)d.cap; i += SCHED_NT) list[i] = ITEM_EMPTY;
+    if (tid < 256) s_hist[tid] = 0;
+    if (tid < 16) s_cbase[tid] = 0;
+    if (tid == 0) s_ovf = 0;
+    __syncthreads();
+    // sort key: number of 64-column K tiles (work of a Q tile grows with it), longest first
+    for (int b = tid; b < p.batch; b += SCHED_NT) {
+        const Seq s = load_seq(a, b);
+        const int t = (s.lq + BM - 1) / BM;
+        s_tiles[b] = (unsigned short)min(t, d.ntiles_attr);
+        s_sweep[b] = t > d.ntiles_attr;
+        const int key = 255 - min(255, (s.lk + BN - 1) / BN);
+        s_key[b] = (unsigned char)key;
+        atomicAdd(&s_hist[key], 1u);
+    }
+    __syncthreads();
+    // exclusive scan of the 256 key counts (Hillis-Steele in LDS)
+    if (tid < 256) s_base[tid] = s_hist[tid];
+    __syncthreads();
+    for (int off = 1; off < 256; off <<= 1) {
+        const unsigned add = (tid < 256 && tid >= off) ? s_base[tid - off] : 0u;
+        __syncthreads();
+        if (tid < 256) s_base[tid] += add;
+        __syncthreads();
+    }
+    if (tid < 256) s_base[tid] -= s_hist[tid];
+    __syncthreads();
+    for (int b = tid; b < p.batch; b += SCHED_NT) s_order[atomicAdd(&s_base[s_key[b]], 1u)] = (unsigned short)b;
+    __syncthreads();
+
+    // groups r = rank * heads + head; exclusive prefix of the tile counts inside each XCD's list.  A chunk of
+    // 1024 consecutive groups is scanned with stride 16 (one scan per residue class r % 16); XCD x owns the
+    // classes x and 15 - x, class x first.
+    const unsigned H = (unsigned)p.heads_q, G = (unsigned)p.batch * H;
+    for (unsigned c0 = 0; c0 < G; c0 += SCHED_NT) {
+        const unsigned r = c0 + tid;
+        const unsigned rank = r / H, h = r - rank * H;
+        const int b = r < G ? (int)s_order[rank] : 0;
+        const unsigned v = r < G ? s_tiles[b] : 0u;
+        s_val[tid] = v;
+        s_scan[tid] = v;
+        __syncthreads();
+        for (int off = 16; off < SCHED_NT; off <<= 1) {
+            const unsigned add = tid >= off ? s_scan[tid - off] : 0u;
+            __syncthreads();
+            s_scan[tid] += add;
+            __syncthreads();
+        }
+        const int j = tid & 15, tp = (tid & ~15) | (15 - j);
+        unsigned pos = s_cbase[j] + s_cbase[15 - j] + (s_scan[tid] - v);
+        pos += j < 8 ? s_scan[tp] - s_val[tp] : s_scan[tp];
+        const int x = xcd_of_group(r);
+        for (unsigned i = 0; i < v; i++) {
+            const unsigned tile = v - 1 - i;
+            const unsigned item = (unsigned)b | h << 12 | tile << 16 | ((i == 0 && s_sweep[b]) ? 1u << 24 : 0u);
+            if (pos + i < d.cap) list[8 * (size_t)(pos + i) + x] = item;
+            else ovf[atomicAdd(&s_ovf, 1u)] = item;
+        }
+        __syncthreads();
+        if (tid < 16) s_cbase[tid] += s_scan[SCHED_NT - 16 + tid];
+        __syncthreads();
+    }
+    if (tid == 0) { ws[0] = s_ovf; ws[1] = 0; }
+}
+
 // EXTRA: 0 = no bias / built-in mask only, 1 = dense bias and/or custom mask (tables, if any, gathered from
 // global memory), 2 = bias tables only, gathered from LDS-resident copies
 template <typename T, int D, int EXTRA, bool PAGED>
 __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2)))
-void hstu_mfma_kernel(const KArgs a, const int ntiles_attr, const int nbh, const int nbh_pad) {
+void hstu_mfma_kernel(const KArgs a, unsigned* __restrict__ ws) {
     typedef Tile<D> TL;
     typedef typename MM<T>::v8 v8;
     const hstu_fwd_params& p = a.p;
@@ -166,14 +283,21 @@ void hstu_mfma_kernel(const KArgs a, const int ntiles_attr, const int nbh, const
     const int lane = tid & 63, w = tid >> 6;
     const int g = lane >> 5, l32 = lane & 31;
 
-    // blockIdx -> (slot, sequence, head).  Slots run from the last Q tile (largest K extent) to the
-    // first so that heavy tiles are dispatched first; nbh_pad is a multiple of 8 so that every tile of
-    // one (sequence, head) lands on the same XCD and its K/V stay in that XCD's L2.
-    const int slot = blockIdx.x / nbh_pad;
-    const int bh_raw = blockIdx.x - slot * nbh_pad;
-    const bool active = bh_raw < nbh;          // padding workgroups only help with the tail rows below
-    const int bh = active ? bh_raw : 0;
-    const int b = bh / p.heads_q, h = bh - b * p.heads_q;
+    // blockIdx -> item of the work list (see above); a workgroup whose slot is empty looks into the overflow list
+    __shared__ unsigned s_item;
+    unsigned item = ws[WS_HEADER + blockIdx.x];
+    if (item == ITEM_EMPTY && ws[0] != 0) {
+        if (tid == 0) {
+            const unsigned k = atomicAdd(&ws[1], 1u);
+            s_item = k < ws[0] ? ws[WS_HEADER + gridDim.x + k] : ITEM_EMPTY;
+        }
+        __syncthreads();
+        item = __builtin_amdgcn_readfirstlane(s_item);
+    }
+    const bool active = item != ITEM_EMPTY;
+    const int b = active ? (int)(item & 0xfff) : 0, h = active ? (int)((item >> 12) & 0xf) : 0;
+    const int tile0 = (int)((item >> 16) & 0xff);
+    const bool sweep = (item >> 24) & 1;   // last tile the max_seq_len_q attribute covers of a sequence that is longer
     const int hk = h / a.head_ratio;
     const Seq s = load_seq(a, b);
     const bool tril = p.mask_type == HSTU_MASK_TRIL;
@@ -184,8 +308,7 @@ void hstu_mfma_kernel(const KArgs a, const int ntiles_attr, const int nbh, const
     // LDS layout: [K buffer 0][V buffer 0][K buffer 1][V buffer 1]
     constexpr int BUF_ELEMS = TL::K_ELEMS + TL::V_ELEMS;
 
-    // the first slot also sweeps tiles beyond the max_seq_len attribute should a sequence exceed it
-    for (int tile = ntiles_attr - 1 - slot; active && tile * BM < s.lq; tile++) {
+    for (int tile = tile0; active && tile * BM < s.lq; tile++) {
         const int i0 = tile * BM;
         const int kend = (s.lk > 0) ? k_extent(a, s, i0, min(i0 + BM, s.lq)) : 0;
         const int ntk = (kend + BN - 1) / BN;
@@ -435,7 +558,7 @@ void hstu_mfma_kernel(const KArgs a, const int ntiles_attr, const int nbh, const
             }
         }
         __syncthreads();
-        if (slot != 0) break;
+        if (!sweep) break;
     }
 
     // rows past the last offset are zero (the reference zero-fills its output: hstu_jagged.cpp:56-59)
@@ -463,22 +586,23 @@ bool mfma_supported(const KArgs& a, const char** name) {
 }
 
 template <typename T, int D>
-static hipError_t launch_td(const KArgs& a, hipStream_t stream) {
+static hipError_t launch_td(const KArgs& a, unsigned* ws, hipStream_t stream) {
     const hstu_fwd_params& p = a.p;
-    const int ntiles = (p.max_seq_len_q + BM - 1) / BM;
-    const int nbh = p.batch * p.heads_q;
-    const int nbh_pad = (nbh + 7) / 8 * 8;
+    const SchedDims d = sched_dims(p);
     const bool dense_extra = p.attn_bias || p.mask_type == HSTU_MASK_CUSTOM;
     const bool tables = p.pos_table || p.ts_table;
     const int extra = dense_extra ? 1 : (tables ? 2 : 0);
     const bool paged = a.op == OP_PAGED;
-    dim3 grid((unsigned)(ntiles * nbh_pad)), block(NT);
+    hipLaunchKernelGGL(hstu_schedule_kernel, dim3(1), dim3(SCHED_NT), 0, stream, a, d, ws);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    dim3 grid(8 * d.cap), block(NT);   // the overflow list starts at entry gridDim.x of the lists
     if (getenv("HSTU_HIP_DEBUG")) {
         int nb = -1;
-        hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, hstu_mfma_kernel<T, D, 0, false>, NT, 0);
+        e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, hstu_mfma_kernel<T, D, 0, false>, NT, 0);
         fprintf(stderr, "[hstu_hip] mfma d=%d grid=%u workgroups/CU=%d (%s)\n", D, grid.x, nb, hipGetErrorString(e));
     }
-#define HSTU_LAUNCH(E, P) hipLaunchKernelGGL((hstu_mfma_kernel<T, D, E, P>), grid, block, 0, stream, a, ntiles, nbh, nbh_pad)
+#define HSTU_LAUNCH(E, P) hipLaunchKernelGGL((hstu_mfma_kernel<T, D, E, P>), grid, block, 0, stream, a, ws)
     if (paged) {
         if (extra == 0) HSTU_LAUNCH(0, true);
         else HSTU_LAUNCH(1, true);      // paged + bias: the general gather path
@@ -491,10 +615,11 @@ static hipError_t launch_td(const KArgs& a, hipStream_t stream) {
     return hipGetLastError();
 }
 
-hipError_t launch_mfma(const KArgs& a, hipStream_t stream) {
+hipError_t launch_mfma(const KArgs& a, void* workspace, hipStream_t stream) {
     const hstu_fwd_params& p = a.p;
-    if (p.dtype == HSTU_BF16) return p.dim_qk == 128 ? launch_td<__bf16, 128>(a, stream) : launch_td<__bf16, 64>(a, stream);
-    return p.dim_qk == 128 ? launch_td<_Float16, 128>(a, stream) : launch_td<_Float16, 64>(a, stream);
+    unsigned* ws = reinterpret_cast<unsigned*>(workspace);
+    if (p.dtype == HSTU_BF16) return p.dim_qk == 128 ? launch_td<__bf16, 128>(a, ws, stream) : launch_td<__bf16, 64>(a, ws, stream);
+    return p.dim_qk == 128 ? launch_td<_Float16, 128>(a, ws, stream) : launch_td<_Float16, 64>(a, ws, stream);
 }
 
 }  // namespace hstu

@@ -53,9 +53,20 @@ def _ws(p, op="jagged"):
     return rc, n.value, _capi.lib().hstu_hip_last_error().decode()
 
 
-def test_struct_layout_matches_and_workspace_is_zero():
+def test_struct_layout_matches_and_workspace_size():
     rc, n, msg = _ws(_params())
-    assert rc == 0 and n == 0, msg          # a size mismatch between ctypes and C would be rejected here
+    # a size mismatch between ctypes and C would be rejected here.  MFMA kernels keep their work list in the
+    # workspace: 16 header words + 8 XCD lists of cap entries + an overflow list of `bound` entries, with
+    # bound = min(total_q // 128 + batch, batch * ceil(max_seq_len_q / 128)) * heads_q, cap = ceil(bound / 8) + tiles
+    assert rc == 0 and n == 4 * (16 + 8 * 2 + 8), msg
+    rc, n, msg = _ws(_params(dtype=_capi.HSTU_F32))
+    assert rc == 0 and n == 0, msg          # the generic kernel needs none
+    rc, n, msg = _ws(_params(flags=_capi.FLAG_FORCE_GENERIC))
+    assert rc == 0 and n == 0, msg
+    # a call without the workspace is refused before anything is launched
+    pp = _params()
+    rc = _capi.lib().hstu_hip_jagged_forward(C.byref(pp), None, 0, None)
+    assert rc == -3 and "workspace" in _capi.lib().hstu_hip_last_error().decode()
     rc, _, msg = _ws(_params(struct_size=8))
     assert rc == -1 and "size mismatch" in msg
 
