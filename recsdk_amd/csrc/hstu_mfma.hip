@@ -267,7 +267,18 @@ void hstu_mfma_kernel(const KArgs a, unsigned* __restrict__ ws) {
     typedef Tile<D> TL;
     typedef typename MM<T>::v8 v8;
     const hstu_fwd_params& p = a.p;
-    __shared__ __attribute__((aligned(16))) T lds[2 * (TL::K_ELEMS + TL::V_ELEMS)];
+    // K/V tiles of head dim 128 that come straight from q-like [rows, heads, D] tensors are copied global -> LDS
+    // by buffer loads with the LDS destination (no register staging).  One wave instruction fills 1024
+    // contiguous LDS bytes = 4 rows, so a tile is a sequence of 4-row blocks (K blocks padded by 64 B); inside
+    // a block row rho keeps its 16-byte chunk c at position (c + rho) % 16 (K) or (c + 4 rho) % 16 (V), which
+    // spreads the fragment reads below over all banks.  Everything else goes through registers into padded rows.
+    constexpr bool DMA = !PAGED && D == 128;
+    constexpr int KBLK = 1088, VBLK = 1024;              // bytes per 4-row block
+    constexpr int K_BYTES = DMA ? 16 * KBLK : TL::K_ELEMS * 2;
+    constexpr int STAGE_BYTES = DMA ? 16 * KBLK + 16 * VBLK : (TL::K_ELEMS + TL::V_ELEMS) * 2;
+    // two separate arrays: reads of one tile are then independent of the copy in flight into the other
+    __shared__ __attribute__((aligned(1024))) char lds0[STAGE_BYTES];
+    __shared__ __attribute__((aligned(1024))) char lds1[STAGE_BYTES];
     // table mode: per K tile a window of the position table and the key timestamps (double buffered with the
     // K/V tiles), plus the whole time table and its bucket bounds as (lower, upper) pairs
     constexpr int PW = BM + BN;   // window entries: (j - k0) - (qi - i0) + BM - 1 in [0, BM + BN - 2]
@@ -280,7 +291,8 @@ void hstu_mfma_kernel(const KArgs a, unsigned* __restrict__ ws) {
     __shared__ float lds_psc[PAGED ? 2 * MAXP : 1];
 
     const int tid = threadIdx.x;
-    const int lane = tid & 63, w = tid >> 6;
+    const int lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave index, kept in a scalar register
     const int g = lane >> 5, l32 = lane & 31;
 
     // blockIdx -> item of the work list (see above); a workgroup whose slot is empty looks into the overflow list
@@ -305,8 +317,18 @@ void hstu_mfma_kernel(const KArgs a, unsigned* __restrict__ ws) {
     const T* qbase = reinterpret_cast<const T*>(p.q);
     T* obase = reinterpret_cast<T*>(p.out);
 
-    // LDS layout: [K buffer 0][V buffer 0][K buffer 1][V buffer 1]
-    constexpr int BUF_ELEMS = TL::K_ELEMS + TL::V_ELEMS;
+    // loop-invariant per-lane byte offsets of the direct-copy layout
+    const unsigned rowstride = (unsigned)p.heads_k * D * 2;   // bytes between consecutive K (or V) rows
+    const int lrho = lane >> 4, lpos = lane & 15;             // loader: lane L fills slot L of a 4-row block
+    const unsigned ldK = lrho * rowstride + (((lpos - lrho) & 15) << 4);
+    const unsigned ldV = lrho * rowstride + (((lpos - 4 * lrho) & 15) << 4);
+    const int krho = l32 & 3;                                 // K fragment: row l32 of a 32-key block
+    const int kfrag_off = (l32 >> 2) * KBLK + krho * 256;
+    const int q4 = (lane & 15) >> 2, u16 = l32 >> 4, piece = lane & 3;   // V transposing reads
+    int voff[4];
+#pragma unroll
+    for (int db = 0; db < 4; db++)
+        voff[db] = 16 * KBLK + g * VBLK + q4 * 256 + ((4 * ((db + q4) & 3) + 2 * u16 + (piece >> 1)) << 4) + 8 * (piece & 1);
 
     for (int tile = tile0; active && tile * BM < s.lq; tile++) {
         const int i0 = tile * BM;
@@ -361,25 +383,42 @@ void hstu_mfma_kernel(const KArgs a, unsigned* __restrict__ ws) {
         float kscale[TL::NCH], vscale[TL::NCH];
         unsigned fp8mask = 0;
 
-        // Global -> register -> LDS staging.  Loads are unconditional (rows past the visible range are
-        // clamped to the last visible row and zeroed when written to LDS) so that they stay in straight-line
-        // code and only the LDS write waits for them.
-        u32x4 kreg[TL::NCH], vreg[TL::NCH];
-        auto fetch = [&](int kt) {
+        // Loader.  Register path: loads are unconditional (rows past the visible range are clamped to the last
+        // visible row and zeroed when written to LDS) so that they stay in straight-line code and only the LDS
+        // write waits for them.  Direct path: a buffer view of this (sequence, kv head) that ends with the last
+        // visible row, so rows past it read as zeros.
+        u32x4 kreg[DMA ? 1 : TL::NCH], vreg[DMA ? 1 : TL::NCH];
+        const char* kview = reinterpret_cast<const char*>(p.k) + ((int64_t)s.k_start * p.heads_k + hk) * D * 2;
+        const char* vview = reinterpret_cast<const char*>(p.v) + ((int64_t)s.k_start * p.heads_k + hk) * D * 2;
+        const unsigned view_bytes = kend > 0 ? (unsigned)(kend - 1) * rowstride + D * 2 : 0;
+        auto fetch = [&](int kt, char* dst) __attribute__((always_inline)) {
             const int k0 = kt * BN;
+            if constexpr (DMA) {
+                const unsigned tile_off = (unsigned)k0 * rowstride;
+                __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc((void*)(kview + tile_off), 0, (int)(view_bytes - tile_off), 0x00020000);
+                __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc((void*)(vview + tile_off), 0, (int)(view_bytes - tile_off), 0x00020000);
 #pragma unroll
-            for (int i = 0; i < TL::NCH; i++) {
-                const int c = tid + NT * i;
-                const int row = c / (D / 8), cc = c % (D / 8);
-                const int j = min(k0 + row, kend - 1);
-                RowRef<T, PAGED> rk = kv_row_ref<T, PAGED>(a, s, 0, j, hk, D, lds_pid, lds_psc);
-                RowRef<T, PAGED> rv = kv_row_ref<T, PAGED>(a, s, 1, j, hk, D, lds_pid, lds_psc);
-                kreg[i] = load_chunk<T, PAGED>(rk, cc);
-                vreg[i] = load_chunk<T, PAGED>(rv, cc);
-                if (PAGED) {
-                    kscale[i] = rk.scale;
-                    vscale[i] = rv.scale;
-                    fp8mask = (fp8mask & ~(1u << i)) | ((rk.fp8 ? 1u : 0u) << i);
+                for (int i = 0; i < 4; i++) {
+                    const int blk = 4 * w + i;
+                    const unsigned so = (unsigned)(4 * blk) * rowstride;
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, LDS_PTR(void, dst + blk * KBLK), 16, ldK + so, 0, 0, 0);
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, LDS_PTR(void, dst + 16 * KBLK + blk * VBLK), 16, ldV + so, 0, 0, 0);
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < TL::NCH; i++) {
+                    const int c = tid + NT * i;
+                    const int row = c / (D / 8), cc = c % (D / 8);
+                    const int j = min(k0 + row, kend - 1);
+                    RowRef<T, PAGED> rk = kv_row_ref<T, PAGED>(a, s, 0, j, hk, D, lds_pid, lds_psc);
+                    RowRef<T, PAGED> rv = kv_row_ref<T, PAGED>(a, s, 1, j, hk, D, lds_pid, lds_psc);
+                    kreg[i] = load_chunk<T, PAGED>(rk, cc);
+                    vreg[i] = load_chunk<T, PAGED>(rv, cc);
+                    if (PAGED) {
+                        kscale[i] = rk.scale;
+                        vscale[i] = rv.scale;
+                        fp8mask = (fp8mask & ~(1u << i)) | ((rk.fp8 ? 1u : 0u) << i);
+                    }
                 }
             }
             if (EXTRA == 2) {
@@ -391,41 +430,61 @@ void hstu_mfma_kernel(const KArgs a, unsigned* __restrict__ ws) {
                 if (tab_ts && tid < BN) tk_reg = p.timestamps[s.k_start + min(k0 + tid, s.lk - 1)];
             }
         };
-        auto stash = [&](int kt) {
+        // second half of the register path, and the table windows; ends with the tile being complete in LDS
+        auto stash = [&](int kt, char* dst) __attribute__((always_inline)) {
             const int k0 = kt * BN;
             const int buf = kt & 1;
+            if (!DMA && k0 < kend) {
+                T* dk = reinterpret_cast<T*>(dst);
+                T* dv = dk + TL::K_ELEMS;
 #pragma unroll
-            for (int i = 0; i < TL::NCH; i++) {
-                const int c = tid + NT * i;
-                const int row = c / (D / 8), cc = c % (D / 8);
-                const bool ok = k0 + row < kend;
-                const u32x4 z = {0, 0, 0, 0};
-                u32x4 kx = kreg[i], vx = vreg[i];
-                if (PAGED && ((fp8mask >> i) & 1)) {
-                    kx = dequant_chunk<T>(kx, kscale[i]);
-                    vx = dequant_chunk<T>(vx, vscale[i]);
+                for (int i = 0; i < TL::NCH; i++) {
+                    const int c = tid + NT * i;
+                    const int row = c / (D / 8), cc = c % (D / 8);
+                    const bool ok = k0 + row < kend;
+                    const u32x4 z = {0, 0, 0, 0};
+                    u32x4 kx = kreg[i], vx = vreg[i];
+                    if (PAGED && ((fp8mask >> i) & 1)) {
+                        kx = dequant_chunk<T>(kx, kscale[i]);
+                        vx = dequant_chunk<T>(vx, vscale[i]);
+                    }
+                    *reinterpret_cast<u32x4*>(dk + row * TL::KS + cc * 8) = ok ? kx : z;
+                    *reinterpret_cast<u32x4*>(dv + row * TL::VS + cc * 8) = ok ? vx : z;
                 }
-                *reinterpret_cast<u32x4*>(lds + buf * BUF_ELEMS + row * TL::KS + cc * 8) = ok ? kx : z;
-                *reinterpret_cast<u32x4*>(lds + buf * BUF_ELEMS + TL::K_ELEMS + row * TL::VS + cc * 8) = ok ? vx : z;
             }
             if (EXTRA == 2) {
                 if (tab_pos && tid < PW - 1) lds_pos[buf * PW + tid] = pw_reg;
                 if (tab_ts && tid < BN) lds_tk[buf * BN + tid] = tk_reg;
             }
+            if constexpr (DMA) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+        };
+        // fragment reads
+        auto read_kf = [&](const char* cur, int kb, int ds) __attribute__((always_inline)) -> v8 {
+            if constexpr (DMA) {
+                const int pos = (2 * ds + g + krho) & 15;   // chunk 2*ds + g of row l32, rotated by the row's rho
+                return *reinterpret_cast<const v8*>(cur + kb * 8 * KBLK + kfrag_off + (pos << 4));
+            } else {
+                return *reinterpret_cast<const v8*>(reinterpret_cast<const T*>(cur) + (32 * kb + l32) * TL::KS + 8 * g + 16 * ds);
+            }
+        };
+        // 4 keys (rows 32*kb + 8*part + 4*g ..+3) of column 32*db + l32 % 32 for this lane
+        auto read_vf = [&](const char* cur, int kb, int db, int part) __attribute__((always_inline)) -> s16x4 {
+            if constexpr (DMA) {
+                return __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, cur + (8 * kb + 2 * part) * VBLK + voff[db]));
+            } else {
+                const T* vp = reinterpret_cast<const T*>(cur) + TL::K_ELEMS + (32 * kb + 8 * part + 4 * g + ((lane & 15) >> 2)) * TL::VS + 16 * (l32 >> 4) + 4 * (lane & 3);
+                return __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, vp + 32 * db));
+            }
         };
 
-        if (ntk > 0) {
-            fetch(0);
-            stash(0);
-        }
-        __syncthreads();
+        if (ntk > 0) fetch(0, lds0);
+        stash(0, lds0);
 
-        for (int kt = 0; kt < ntk; kt++) {
+        auto iteration = [&](int kt, const char* cur, char* nxt) __attribute__((always_inline)) {
             const int buf = kt & 1;
             const int k0 = kt * BN;
-            const T* Kb = lds + buf * BUF_ELEMS;
-            const T* Vb = Kb + TL::K_ELEMS;
-            if (kt + 1 < ntk) fetch(kt + 1);
+            if (kt + 1 < ntk) fetch(kt + 1, nxt);
 
 #pragma unroll
             for (int kb = 0; kb < 2; kb++) {
@@ -434,10 +493,9 @@ void hstu_mfma_kernel(const KArgs a, unsigned* __restrict__ ws) {
                 if (cls == BLK_SKIP) continue;  // wave-uniform
                 // ---- S^T block: 32 keys x 32 Q rows.  All K fragments are requested before the first
                 // MFMA so that the LDS latency is paid once per block, not once per instruction.
-                const T* kp = Kb + (32 * kb + l32) * TL::KS + 8 * g;
                 v8 kf[D / 16];
 #pragma unroll
-                for (int ds = 0; ds < D / 16; ds++) kf[ds] = *reinterpret_cast<const v8*>(kp + 16 * ds);
+                for (int ds = 0; ds < D / 16; ds++) kf[ds] = read_kf(cur, kb, ds);
                 f32x16 sacc;
 #pragma unroll
                 for (int r = 0; r < 16; r++) sacc[r] = 0.f;
@@ -446,12 +504,11 @@ void hstu_mfma_kernel(const KArgs a, unsigned* __restrict__ ws) {
                 // V^T fragments of the first 16-key step: requested now, consumed after the SiLU pass.
                 // Transposing LDS read: a 16-lane group reads 4 key rows x 16 columns and every lane
                 // receives 4 consecutive keys of one column.
-                const T* vp = Vb + (32 * kb + 4 * g + ((lane & 15) >> 2)) * TL::VS + 16 * (l32 >> 4) + 4 * (lane & 3);
                 s16x4 vlo[D / 32], vhi[D / 32];
 #pragma unroll
                 for (int db = 0; db < D / 32; db++) {
-                    vlo[db] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, vp + 32 * db));
-                    vhi[db] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, vp + 32 * db + 8 * TL::VS));
+                    vlo[db] = read_vf(cur, kb, db, 0);
+                    vhi[db] = read_vf(cur, kb, db, 1);
                 }
                 // ---- P = s * sigmoid(alpha * s) (scale folded into the epilogue), masked
                 // accumulator register r holds key c0 + 8*(r/4) + 4*g + r%4 for Q row qi
@@ -524,8 +581,8 @@ void hstu_mfma_kernel(const KArgs a, unsigned* __restrict__ ws) {
                 s16x4 wlo[D / 32], whi[D / 32];
 #pragma unroll
                 for (int db = 0; db < D / 32; db++) {   // second step's fragments fly while the first step multiplies
-                    wlo[db] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, vp + 32 * db + 16 * TL::VS));
-                    whi[db] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, vp + 32 * db + 24 * TL::VS));
+                    wlo[db] = read_vf(cur, kb, db, 2);
+                    whi[db] = read_vf(cur, kb, db, 3);
                 }
 #pragma unroll
                 for (int db = 0; db < D / 32; db++) {
@@ -539,8 +596,11 @@ void hstu_mfma_kernel(const KArgs a, unsigned* __restrict__ ws) {
                 }
             }
 
-            if (kt + 1 < ntk) stash(kt + 1);
-            __syncthreads();
+            stash(kt + 1, nxt);
+        };
+        for (int kt = 0; kt < ntk; kt += 2) {
+            iteration(kt, lds0, lds1);
+            if (kt + 1 < ntk) iteration(kt + 1, lds1, lds0);
         }
 
         // ---- epilogue: O^T accumulator register r of block db holds d = 32*db + 8*(r/4) + 4*g + r%4 for row qi
