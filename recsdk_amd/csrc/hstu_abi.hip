@@ -112,8 +112,8 @@ static int run(const hstu_fwd_params* p, int op, void* workspace, uint64_t works
     hipError_t e;
     if (!(p->flags & HSTU_FLAG_FORCE_GENERIC) && mfma_supported(a, &name)) {
         const uint64_t need = mfma_workspace_bytes(a);
-        if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 3))
-            return fail(HSTU_ERR_WORKSPACE, "workspace of %llu bytes (4-byte aligned) needed, got %llu at %p",
+        if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 15))
+            return fail(HSTU_ERR_WORKSPACE, "workspace of %llu bytes (16-byte aligned) needed, got %llu at %p",
                         (unsigned long long)need, (unsigned long long)workspace_bytes, workspace);
         e = launch_mfma(a, workspace, st);
     } else {

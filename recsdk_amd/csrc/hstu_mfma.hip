@@ -145,17 +145,20 @@ __device__ __forceinline__ int classify_block(const Seq& s, int tgs, int r0, int
 // ---- work list ------------------------------------------------------------------------------------------
 // The hardware dispatches workgroups in index order and a workgroup that finds no work still costs a slot, so
 // the grid is driven by a list that a one-workgroup kernel builds first from the sequence lengths:
-//   * one item = one 128-row Q tile of one (sequence, head), packed as  seq | head << 12 | tile << 16 | sweep << 24
+//   * one item = one 128-row Q tile of one (sequence, head): a record of 8 words -- seq | head << 12 | tile << 16
+//     | sweep << 24, then the sequence's geometry (q_start, lq, k_start, lk, num_context, num_target, first page
+//     entry), so that a workgroup needs one scalar load to know its work
 //   * sequences are sorted by K length (longest first) and their (sequence, head) groups are dealt to the
 //     8 XCDs in snake order; a group's tiles sit next to each other in its XCD's list, last tile first, so that
 //     the workgroups that share one K/V run at the same time on CUs that share one L2
-//   * workgroup i runs on XCD i % 8 and takes entry i / 8 of that XCD's list: list[i]
+//   * workgroup i runs on XCD i % 8 and takes entry i / 8 of that XCD's list: record i
 //   * items beyond a list's capacity go to an overflow list that workgroups with an empty slot drain
-// Layout of the workspace (uint32): [0] overflow count, [1] overflow taken, [16 .. 16 + 8*cap) interleaved lists,
-// then the overflow list.
+// Layout of the workspace (uint32): [0] overflow count, [1] overflow taken, from word 16 the 8*cap records of the
+// interleaved lists, then the records of the overflow list.
 constexpr unsigned ITEM_EMPTY = 0xffffffffu;
 constexpr int SCHED_NT = 1024;
 constexpr int WS_HEADER = 16;
+constexpr int REC = 8;   // words per record
 
 struct SchedDims {
     int ntiles_attr;   // Q tiles the max_seq_len_q attribute covers
@@ -175,7 +178,7 @@ static SchedDims sched_dims(const hstu_fwd_params& p) {
 
 uint64_t mfma_workspace_bytes(const KArgs& a) {
     const SchedDims d = sched_dims(a.p);
-    return (uint64_t)(WS_HEADER + 8 * (uint64_t)d.cap + d.bound) * sizeof(uint32_t);
+    return (uint64_t)(WS_HEADER + REC * (8 * (uint64_t)d.cap + d.bound)) * sizeof(uint32_t);
 }
 
 __device__ __forceinline__ int xcd_of_group(unsigned r) { return (r & 8) ? 7 - (int)(r & 7) : (int)(r & 7); }
@@ -190,18 +193,22 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
     __shared__ unsigned s_hist[256], s_base[256];
     __shared__ unsigned s_val[SCHED_NT], s_scan[SCHED_NT];
     __shared__ unsigned s_cbase[16], s_ovf;
+    __shared__ int s_geo[7][HSTU_MAX_BATCH];              // q_start, lq, k_start, lk, ctx, tgt, first page entry
     const int tid = threadIdx.x;
+    const int nthr = blockDim.x;   // 256, 512 or 1024: small batches run with fewer waves (cheaper barriers)
     unsigned* list = ws + WS_HEADER;
-    unsigned* ovf = list + 8 * (size_t)d.cap;
+    unsigned* ovf = list + REC * 8 * (size_t)d.cap;
 
-    for (size_t i = tid; i < 8 * (size_t)d.cap; i += SCHED_NT) list[i] = ITEM_EMPTY;
+    for (size_t i = tid; i < 8 * (size_t)d.cap; i += nthr) list[REC * i] = ITEM_EMPTY;
     if (tid < 256) s_hist[tid] = 0;
     if (tid < 16) s_cbase[tid] = 0;
     if (tid == 0) s_ovf = 0;
     __syncthreads();
     // sort key: number of 64-column K tiles (work of a Q tile grows with it), longest first
-    for (int b = tid; b < p.batch; b += SCHED_NT) {
+    for (int b = tid; b < p.batch; b += nthr) {
         const Seq s = load_seq(a, b);
+        s_geo[0][b] = (int)s.q_start; s_geo[1][b] = s.lq; s_geo[2][b] = (int)s.k_start; s_geo[3][b] = s.lk;
+        s_geo[4][b] = s.ctx; s_geo[5][b] = s.tgt; s_geo[6][b] = (int)s.page0;
         const int t = (s.lq + BM - 1) / BM;
         s_tiles[b] = (unsigned short)min(t, d.ntiles_attr);
         s_sweep[b] = t > d.ntiles_attr;
@@ -221,14 +228,14 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
     }
     if (tid < 256) s_base[tid] -= s_hist[tid];
     __syncthreads();
-    for (int b = tid; b < p.batch; b += SCHED_NT) s_order[atomicAdd(&s_base[s_key[b]], 1u)] = (unsigned short)b;
+    for (int b = tid; b < p.batch; b += nthr) s_order[atomicAdd(&s_base[s_key[b]], 1u)] = (unsigned short)b;
     __syncthreads();
 
     // groups r = rank * heads + head; exclusive prefix of the tile counts inside each XCD's list.  A chunk of
     // 1024 consecutive groups is scanned with stride 16 (one scan per residue class r % 16); XCD x owns the
     // classes x and 15 - x, class x first.
     const unsigned H = (unsigned)p.heads_q, G = (unsigned)p.batch * H;
-    for (unsigned c0 = 0; c0 < G; c0 += SCHED_NT) {
+    for (unsigned c0 = 0; c0 < G; c0 += nthr) {
         const unsigned r = c0 + tid;
         const unsigned rank = r / H, h = r - rank * H;
         const int b = r < G ? (int)s_order[rank] : 0;
@@ -236,7 +243,7 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
         s_val[tid] = v;
         s_scan[tid] = v;
         __syncthreads();
-        for (int off = 16; off < SCHED_NT; off <<= 1) {
+        for (int off = 16; off < nthr; off <<= 1) {
             const unsigned add = tid >= off ? s_scan[tid - off] : 0u;
             __syncthreads();
             s_scan[tid] += add;
@@ -249,11 +256,14 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
         for (unsigned i = 0; i < v; i++) {
             const unsigned tile = v - 1 - i;
             const unsigned item = (unsigned)b | h << 12 | tile << 16 | ((i == 0 && s_sweep[b]) ? 1u << 24 : 0u);
-            if (pos + i < d.cap) list[8 * (size_t)(pos + i) + x] = item;
-            else ovf[atomicAdd(&s_ovf, 1u)] = item;
+            unsigned* rec = pos + i < d.cap ? list + REC * (8 * (size_t)(pos + i) + x) : ovf + REC * (size_t)atomicAdd(&s_ovf, 1u);
+            const u32x4 lo = {item, (unsigned)s_geo[0][b], (unsigned)s_geo[1][b], (unsigned)s_geo[2][b]};
+            const u32x4 hi = {(unsigned)s_geo[3][b], (unsigned)s_geo[4][b], (unsigned)s_geo[5][b], (unsigned)s_geo[6][b]};
+            *reinterpret_cast<u32x4*>(rec) = lo;
+            *reinterpret_cast<u32x4*>(rec + 4) = hi;
         }
         __syncthreads();
-        if (tid < 16) s_cbase[tid] += s_scan[SCHED_NT - 16 + tid];
+        if (tid < 16) s_cbase[tid] += s_scan[nthr - 16 + tid];
         __syncthreads();
     }
     if (tid == 0) { ws[0] = s_ovf; ws[1] = 0; }
@@ -297,21 +307,24 @@ void hstu_mfma_kernel(const KArgs a, unsigned* __restrict__ ws) {
 
     // blockIdx -> item of the work list (see above); a workgroup whose slot is empty looks into the overflow list
     __shared__ unsigned s_item;
-    unsigned item = ws[WS_HEADER + blockIdx.x];
-    if (item == ITEM_EMPTY && ws[0] != 0) {
-        if (tid == 0) {
-            const unsigned k = atomicAdd(&ws[1], 1u);
-            s_item = k < ws[0] ? ws[WS_HEADER + gridDim.x + k] : ITEM_EMPTY;
-        }
+    const unsigned* rec = ws + WS_HEADER + REC * (size_t)blockIdx.x;
+    if (rec[0] == ITEM_EMPTY && ws[0] != 0) {
+        if (tid == 0) s_item = atomicAdd(&ws[1], 1u);
         __syncthreads();
-        item = __builtin_amdgcn_readfirstlane(s_item);
+        const unsigned k = __builtin_amdgcn_readfirstlane(s_item);
+        if (k < ws[0]) rec = ws + WS_HEADER + REC * ((size_t)gridDim.x + k);
     }
+    const unsigned item = rec[0];
     const bool active = item != ITEM_EMPTY;
     const int b = active ? (int)(item & 0xfff) : 0, h = active ? (int)((item >> 12) & 0xf) : 0;
     const int tile0 = (int)((item >> 16) & 0xff);
     const bool sweep = (item >> 24) & 1;   // last tile the max_seq_len_q attribute covers of a sequence that is longer
     const int hk = h / a.head_ratio;
-    const Seq s = load_seq(a, b);
+    Seq s;
+    s.q_start = active ? (int)rec[1] : 0; s.lq = active ? (int)rec[2] : 0;
+    s.k_start = active ? (int)rec[3] : 0; s.lk = active ? (int)rec[4] : 0;
+    s.ctx = active ? (int)rec[5] : 0; s.tgt = active ? (int)rec[6] : 0; s.page0 = active ? (int)rec[7] : 0;
+    s.delta = s.lk - s.lq; s.hist_q = s.lq - s.tgt; s.hist_k = s.lk - s.tgt; s.cand_row = s.q_start + s.hist_q;
     const bool tril = p.mask_type == HSTU_MASK_TRIL;
     const int tgs = p.target_group_size;
     const T* qbase = reinterpret_cast<const T*>(p.q);
@@ -486,29 +499,58 @@ void hstu_mfma_kernel(const KArgs a, unsigned* __restrict__ ws) {
             const int k0 = kt * BN;
             if (kt + 1 < ntk) fetch(kt + 1, nxt);
 
+            // LDS latency is kept off the MFMA chains: the K fragments of a block are requested one stage ahead
+            // (block 0 at the top, block 1 while block 0 runs its SiLU pass) and the V^T fragments fly under the
+            // S chain.  Transposing LDS read: a 16-lane group reads 4 key rows x 16 columns and every lane
+            // receives 4 consecutive keys of one column.
+            // (Only where registers allow: the variants with bias tables or paged rows read each fragment set
+            // right before its use.)
+            constexpr bool AHEAD = DMA && EXTRA == 0;
+            int cls2[2];
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++) cls2[kb] = tril ? classify_block(s, tgs, r0, k0 + 32 * kb) : BLK_ALL;
+            v8 kf[D / 16];
+            if (AHEAD && cls2[0] != BLK_SKIP) {
+#pragma unroll
+                for (int ds = 0; ds < D / 16; ds++) kf[ds] = read_kf(cur, 0, ds);
+            }
 #pragma unroll
             for (int kb = 0; kb < 2; kb++) {
                 const int c0 = k0 + 32 * kb;
-                const int cls = tril ? classify_block(s, tgs, r0, c0) : BLK_ALL;
+                const int cls = cls2[kb];
                 if (cls == BLK_SKIP) continue;  // wave-uniform
-                // ---- S^T block: 32 keys x 32 Q rows.  All K fragments are requested before the first
-                // MFMA so that the LDS latency is paid once per block, not once per instruction.
-                v8 kf[D / 16];
+                if (!AHEAD || (kb == 1 && cls2[0] == BLK_SKIP)) {
 #pragma unroll
-                for (int ds = 0; ds < D / 16; ds++) kf[ds] = read_kf(cur, kb, ds);
+                    for (int ds = 0; ds < D / 16; ds++) kf[ds] = read_kf(cur, kb, ds);
+                }
+                s16x4 vlo[D / 32], vhi[D / 32], wlo[D / 32], whi[D / 32];
+                if (AHEAD) {
+#pragma unroll
+                    for (int db = 0; db < D / 32; db++) {
+                        vlo[db] = read_vf(cur, kb, db, 0);
+                        vhi[db] = read_vf(cur, kb, db, 1);
+                        wlo[db] = read_vf(cur, kb, db, 2);
+                        whi[db] = read_vf(cur, kb, db, 3);
+                    }
+                }
+                // ---- S^T block: 32 keys x 32 Q rows
                 f32x16 sacc;
 #pragma unroll
                 for (int r = 0; r < 16; r++) sacc[r] = 0.f;
 #pragma unroll
                 for (int ds = 0; ds < D / 16; ds++) sacc = MM<T>::mfma(kf[ds], qf[ds], sacc);
-                // V^T fragments of the first 16-key step: requested now, consumed after the SiLU pass.
-                // Transposing LDS read: a 16-lane group reads 4 key rows x 16 columns and every lane
-                // receives 4 consecutive keys of one column.
-                s16x4 vlo[D / 32], vhi[D / 32];
+                if (AHEAD) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (kb == 0 && cls2[1] != BLK_SKIP) {
 #pragma unroll
-                for (int db = 0; db < D / 32; db++) {
-                    vlo[db] = read_vf(cur, kb, db, 0);
-                    vhi[db] = read_vf(cur, kb, db, 1);
+                        for (int ds = 0; ds < D / 16; ds++) kf[ds] = read_kf(cur, 1, ds);
+                    }
+                } else {
+#pragma unroll
+                    for (int db = 0; db < D / 32; db++) {
+                        vlo[db] = read_vf(cur, kb, db, 0);
+                        vhi[db] = read_vf(cur, kb, db, 1);
+                    }
                 }
                 // ---- P = s * sigmoid(alpha * s) (scale folded into the epilogue), masked
                 // accumulator register r holds key c0 + 8*(r/4) + 4*g + r%4 for Q row qi
@@ -578,11 +620,12 @@ void hstu_mfma_kernel(const KArgs a, unsigned* __restrict__ ws) {
                     pk0[x] = MM<T>::pack2(pf[2 * x], pf[2 * x + 1]);
                     pk1[x] = MM<T>::pack2(pf[8 + 2 * x], pf[8 + 2 * x + 1]);
                 }
-                s16x4 wlo[D / 32], whi[D / 32];
+                if (!AHEAD) {
 #pragma unroll
-                for (int db = 0; db < D / 32; db++) {   // second step's fragments fly while the first step multiplies
-                    wlo[db] = read_vf(cur, kb, db, 2);
-                    whi[db] = read_vf(cur, kb, db, 3);
+                    for (int db = 0; db < D / 32; db++) {   // second step's fragments fly while the first step multiplies
+                        wlo[db] = read_vf(cur, kb, db, 2);
+                        whi[db] = read_vf(cur, kb, db, 3);
+                    }
                 }
 #pragma unroll
                 for (int db = 0; db < D / 32; db++) {
@@ -653,7 +696,9 @@ static hipError_t launch_td(const KArgs& a, unsigned* ws, hipStream_t stream) {
     const bool tables = p.pos_table || p.ts_table;
     const int extra = dense_extra ? 1 : (tables ? 2 : 0);
     const bool paged = a.op == OP_PAGED;
-    hipLaunchKernelGGL(hstu_schedule_kernel, dim3(1), dim3(SCHED_NT), 0, stream, a, d, ws);
+    const int groups = p.batch * p.heads_q;
+    const int sched_threads = groups <= 256 ? 256 : (groups <= 512 ? 512 : SCHED_NT);
+    hipLaunchKernelGGL(hstu_schedule_kernel, dim3(1), dim3(sched_threads), 0, stream, a, d, ws);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     dim3 grid(8 * d.cap), block(NT);   // the overflow list starts at entry gridDim.x of the lists

@@ -185,3 +185,32 @@ def test_config5_paged_fp8():
     deq = O.dequantize_kv_cache_fp8(cfg["kv_cache_fp8"].view(torch.uint8), cfg["kv_scales"], torch.bfloat16)
     T.assert_parity(out8, T.oracle_paged(cfg, cache=deq), torch.bfloat16, what="config5 vs oracle on dequantised cache")
     T.assert_parity(out8, T.oracle_paged(cfg), torch.bfloat16, tol=5e-2, what="config5 vs unquantised oracle")
+
+
+# ---- work list (schedule kernel) -----------------------------------------------------------------
+def test_work_list_overflow_path():
+    """Sequences sorted by K length but with very uneven Q lengths: one XCD list gets more tiles than its
+    capacity, the surplus goes through the overflow list and every row is still produced exactly once."""
+    say("work_list_overflow")
+    dtype = torch.bfloat16
+    lens_q = [1024] + [16] * 14 + [1024]
+    lens_k = [2048] + [1500 - i for i in range(14)] + [1024]      # ranks 0 and 15 land on the same XCD
+    cfg, _ = _jag(31, lens_q, 1, 1, 128, 128, dtype, lens_k=lens_k)
+    _check(cfg, dtype, "overflow list")
+
+
+@pytest.mark.parametrize("nseq,heads", [(300, 3), (2048, 2), (1, 16), (37, 16)])
+def test_work_list_many_sequences(nseq, heads):
+    """More (sequence, head) groups than one scan chunk; ragged lengths including empty sequences."""
+    say("work_list_many", nseq, heads)
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(nseq)
+    lens = torch.randint(0, 160, (nseq,), generator=g).tolist()
+    lens[0] = 257
+    cfg, _ = _jag(32, lens, heads, heads, 64, 64, dtype)
+    out, name = T.run_capi(cfg)
+    assert name.startswith("mfma_"), name
+    gen, _ = T.run_capi(cfg, flags=FORCE_GENERIC)
+    T.assert_parity(out, gen.float(), dtype, what=f"many sequences {nseq}x{heads} vs generic kernel")
+    if nseq <= 300:
+        T.assert_parity(out, T.oracle_jagged(cfg), dtype, what=f"many sequences {nseq}x{heads} vs oracle")
