@@ -499,58 +499,29 @@ void hstu_mfma_kernel(const KArgs a, unsigned* __restrict__ ws) {
             const int k0 = kt * BN;
             if (kt + 1 < ntk) fetch(kt + 1, nxt);
 
-            // LDS latency is kept off the MFMA chains: the K fragments of a block are requested one stage ahead
-            // (block 0 at the top, block 1 while block 0 runs its SiLU pass) and the V^T fragments fly under the
-            // S chain.  Transposing LDS read: a 16-lane group reads 4 key rows x 16 columns and every lane
-            // receives 4 consecutive keys of one column.
-            // (Only where registers allow: the variants with bias tables or paged rows read each fragment set
-            // right before its use.)
-            constexpr bool AHEAD = DMA && EXTRA == 0;
-            int cls2[2];
-#pragma unroll
-            for (int kb = 0; kb < 2; kb++) cls2[kb] = tril ? classify_block(s, tgs, r0, k0 + 32 * kb) : BLK_ALL;
-            v8 kf[D / 16];
-            if (AHEAD && cls2[0] != BLK_SKIP) {
-#pragma unroll
-                for (int ds = 0; ds < D / 16; ds++) kf[ds] = read_kf(cur, 0, ds);
-            }
 #pragma unroll
             for (int kb = 0; kb < 2; kb++) {
                 const int c0 = k0 + 32 * kb;
-                const int cls = cls2[kb];
+                const int cls = tril ? classify_block(s, tgs, r0, c0) : BLK_ALL;
                 if (cls == BLK_SKIP) continue;  // wave-uniform
-                if (!AHEAD || (kb == 1 && cls2[0] == BLK_SKIP)) {
+                // ---- S^T block: 32 keys x 32 Q rows.  All K fragments are requested before the first
+                // MFMA so that the LDS latency is paid once per block, not once per instruction.
+                v8 kf[D / 16];
 #pragma unroll
-                    for (int ds = 0; ds < D / 16; ds++) kf[ds] = read_kf(cur, kb, ds);
-                }
-                s16x4 vlo[D / 32], vhi[D / 32], wlo[D / 32], whi[D / 32];
-                if (AHEAD) {
-#pragma unroll
-                    for (int db = 0; db < D / 32; db++) {
-                        vlo[db] = read_vf(cur, kb, db, 0);
-                        vhi[db] = read_vf(cur, kb, db, 1);
-                        wlo[db] = read_vf(cur, kb, db, 2);
-                        whi[db] = read_vf(cur, kb, db, 3);
-                    }
-                }
-                // ---- S^T block: 32 keys x 32 Q rows
+                for (int ds = 0; ds < D / 16; ds++) kf[ds] = read_kf(cur, kb, ds);
                 f32x16 sacc;
 #pragma unroll
                 for (int r = 0; r < 16; r++) sacc[r] = 0.f;
 #pragma unroll
                 for (int ds = 0; ds < D / 16; ds++) sacc = MM<T>::mfma(kf[ds], qf[ds], sacc);
-                if (AHEAD) {
-                    __builtin_amdgcn_sched_barrier(0);
-                    if (kb == 0 && cls2[1] != BLK_SKIP) {
+                // V^T fragments of the first 16-key step: requested now, consumed after the SiLU pass.
+                // Transposing LDS read: a 16-lane group reads 4 key rows x 16 columns and every lane
+                // receives 4 consecutive keys of one column.
+                s16x4 vlo[D / 32], vhi[D / 32], wlo[D / 32], whi[D / 32];
 #pragma unroll
-                        for (int ds = 0; ds < D / 16; ds++) kf[ds] = read_kf(cur, 1, ds);
-                    }
-                } else {
-#pragma unroll
-                    for (int db = 0; db < D / 32; db++) {
-                        vlo[db] = read_vf(cur, kb, db, 0);
-                        vhi[db] = read_vf(cur, kb, db, 1);
-                    }
+                for (int db = 0; db < D / 32; db++) {
+                    vlo[db] = read_vf(cur, kb, db, 0);
+                    vhi[db] = read_vf(cur, kb, db, 1);
                 }
                 // ---- P = s * sigmoid(alpha * s) (scale folded into the epilogue), masked
                 // accumulator register r holds key c0 + 8*(r/4) + 4*g + r%4 for Q row qi
@@ -620,12 +591,10 @@ void hstu_mfma_kernel(const KArgs a, unsigned* __restrict__ ws) {
                     pk0[x] = MM<T>::pack2(pf[2 * x], pf[2 * x + 1]);
                     pk1[x] = MM<T>::pack2(pf[8 + 2 * x], pf[8 + 2 * x + 1]);
                 }
-                if (!AHEAD) {
 #pragma unroll
-                    for (int db = 0; db < D / 32; db++) {   // second step's fragments fly while the first step multiplies
-                        wlo[db] = read_vf(cur, kb, db, 2);
-                        whi[db] = read_vf(cur, kb, db, 3);
-                    }
+                for (int db = 0; db < D / 32; db++) {   // second step's fragments fly while the first step multiplies
+                    wlo[db] = read_vf(cur, kb, db, 2);
+                    whi[db] = read_vf(cur, kb, db, 3);
                 }
 #pragma unroll
                 for (int db = 0; db < D / 32; db++) {
