@@ -49,6 +49,10 @@ enum { HSTU_MASK_TRIL = 0, HSTU_MASK_TRIU = 1, HSTU_MASK_NONE = 2, HSTU_MASK_CUS
 /* flags */
 #define HSTU_FLAG_DETERMINISTIC 1u /* accepted; every output row has one producer, so results never depend on it */
 #define HSTU_FLAG_FORCE_GENERIC 2u /* run the plain fp32-FMA kernel even where an MFMA kernel exists (testing) */
+/* The workspace still holds the work list an earlier call built for the same sequence offsets, num_context,
+ * num_target, page offsets, shapes and attributes (e.g. the other layers of one model on one batch): do not
+ * rebuild it.  Only q/k/v/out/bias/table contents may differ between such calls. */
+#define HSTU_FLAG_REUSE_WORKSPACE 4u
 
 /*
  * One argument block for the three forward ops.  Pointers are device pointers unless stated.
@@ -131,7 +135,9 @@ typedef struct hstu_fwd_params {
     float ts_log2_scale;
 } hstu_fwd_params;
 
-/* replaces aclnnHstuJaggedForwardGetWorkspaceSize / aclnnHstuJaggedForward (hstu_jagged.cpp:63-65) */
+/* replaces aclnnHstuJaggedForwardGetWorkspaceSize / aclnnHstuJaggedForward (hstu_jagged.cpp:63-65).
+ * The workspace needs no initialisation; the MFMA kernels keep their work list (tiles sorted by length, grouped
+ * per XCD) in it, the plain kernel needs none.  It must be 16-byte aligned. */
 int hstu_hip_jagged_forward_get_workspace_size(const hstu_fwd_params* p, uint64_t* workspace_bytes);
 int hstu_hip_jagged_forward(const hstu_fwd_params* p, void* workspace, uint64_t workspace_bytes, void* stream);
 

@@ -152,9 +152,10 @@ __device__ __forceinline__ int classify_block(const Seq& s, int tgs, int r0, int
 //     8 XCDs in snake order; a group's tiles sit next to each other in its XCD's list, last tile first, so that
 //     the workgroups that share one K/V run at the same time on CUs that share one L2
 //   * workgroup i runs on XCD i % 8 and takes entry i / 8 of that XCD's list: record i
-//   * items beyond a list's capacity go to an overflow list that workgroups with an empty slot drain
-// Layout of the workspace (uint32): [0] overflow count, [1] overflow taken, from word 16 the 8*cap records of the
-// interleaved lists, then the records of the overflow list.
+//   * items beyond a list's capacity are parked in an overflow list and then moved to the free slots at the end
+//     of the other lists
+// Layout of the workspace (uint32): [0] number of items that were moved, from word 16 the 8*cap records of the
+// interleaved lists, then the parking area of the overflow list.  The main kernel only reads it.
 constexpr unsigned ITEM_EMPTY = 0xffffffffu;
 constexpr int SCHED_NT = 1024;
 constexpr int WS_HEADER = 16;
@@ -266,14 +267,29 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
         if (tid < 16) s_cbase[tid] += s_scan[nthr - 16 + tid];
         __syncthreads();
     }
-    if (tid == 0) { ws[0] = s_ovf; ws[1] = 0; }
+    // items that did not fit their XCD's list move to the free slots at the end of the other lists
+    const unsigned novf = s_ovf;
+    for (unsigned i = tid; i < novf; i += nthr) {
+        unsigned k = i;
+        for (int x = 0; x < 8; x++) {
+            const unsigned len = min(s_cbase[x] + s_cbase[15 - x], d.cap), free = d.cap - len;
+            if (k < free) {
+                unsigned* rec = list + REC * (8 * (size_t)(len + k) + x);
+                *reinterpret_cast<u32x4*>(rec) = *reinterpret_cast<const u32x4*>(ovf + REC * (size_t)i);
+                *reinterpret_cast<u32x4*>(rec + 4) = *reinterpret_cast<const u32x4*>(ovf + REC * (size_t)i + 4);
+                break;
+            }
+            k -= free;
+        }
+    }
+    if (tid == 0) ws[0] = novf;
 }
 
 // EXTRA: 0 = no bias / built-in mask only, 1 = dense bias and/or custom mask (tables, if any, gathered from
 // global memory), 2 = bias tables only, gathered from LDS-resident copies
 template <typename T, int D, int EXTRA, bool PAGED>
 __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2)))
-void hstu_mfma_kernel(const KArgs a, unsigned* __restrict__ ws) {
+void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws) {
     typedef Tile<D> TL;
     typedef typename MM<T>::v8 v8;
     const hstu_fwd_params& p = a.p;
@@ -305,25 +321,23 @@ void hstu_mfma_kernel(const KArgs a, unsigned* __restrict__ ws) {
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave index, kept in a scalar register
     const int g = lane >> 5, l32 = lane & 31;
 
-    // blockIdx -> item of the work list (see above); a workgroup whose slot is empty looks into the overflow list
-    __shared__ unsigned s_item;
-    const unsigned* rec = ws + WS_HEADER + REC * (size_t)blockIdx.x;
-    if (rec[0] == ITEM_EMPTY && ws[0] != 0) {
-        if (tid == 0) s_item = atomicAdd(&ws[1], 1u);
-        __syncthreads();
-        const unsigned k = __builtin_amdgcn_readfirstlane(s_item);
-        if (k < ws[0]) rec = ws + WS_HEADER + REC * ((size_t)gridDim.x + k);
+    // blockIdx -> record of the work list (see above)
+    unsigned rw[REC];
+    {
+        const unsigned* rec = ws + WS_HEADER + REC * (size_t)blockIdx.x;
+#pragma unroll
+        for (int i = 0; i < REC; i++) rw[i] = rec[i];
     }
-    const unsigned item = rec[0];
+    const unsigned item = rw[0];
     const bool active = item != ITEM_EMPTY;
     const int b = active ? (int)(item & 0xfff) : 0, h = active ? (int)((item >> 12) & 0xf) : 0;
     const int tile0 = (int)((item >> 16) & 0xff);
     const bool sweep = (item >> 24) & 1;   // last tile the max_seq_len_q attribute covers of a sequence that is longer
     const int hk = h / a.head_ratio;
     Seq s;
-    s.q_start = active ? (int)rec[1] : 0; s.lq = active ? (int)rec[2] : 0;
-    s.k_start = active ? (int)rec[3] : 0; s.lk = active ? (int)rec[4] : 0;
-    s.ctx = active ? (int)rec[5] : 0; s.tgt = active ? (int)rec[6] : 0; s.page0 = active ? (int)rec[7] : 0;
+    s.q_start = active ? (int)rw[1] : 0; s.lq = active ? (int)rw[2] : 0;
+    s.k_start = active ? (int)rw[3] : 0; s.lk = active ? (int)rw[4] : 0;
+    s.ctx = active ? (int)rw[5] : 0; s.tgt = active ? (int)rw[6] : 0; s.page0 = active ? (int)rw[7] : 0;
     s.delta = s.lk - s.lq; s.hist_q = s.lq - s.tgt; s.hist_k = s.lk - s.tgt; s.cand_row = s.q_start + s.hist_q;
     const bool tril = p.mask_type == HSTU_MASK_TRIL;
     const int tgs = p.target_group_size;
@@ -667,9 +681,12 @@ static hipError_t launch_td(const KArgs& a, unsigned* ws, hipStream_t stream) {
     const bool paged = a.op == OP_PAGED;
     const int groups = p.batch * p.heads_q;
     const int sched_threads = groups <= 256 ? 256 : (groups <= 512 ? 512 : SCHED_NT);
-    hipLaunchKernelGGL(hstu_schedule_kernel, dim3(1), dim3(sched_threads), 0, stream, a, d, ws);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return e;
+    hipError_t e = hipSuccess;
+    if (!(p.flags & HSTU_FLAG_REUSE_WORKSPACE)) {
+        hipLaunchKernelGGL(hstu_schedule_kernel, dim3(1), dim3(sched_threads), 0, stream, a, d, ws);
+        e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
     dim3 grid(8 * d.cap), block(NT);   // the overflow list starts at entry gridDim.x of the lists
     if (getenv("HSTU_HIP_DEBUG")) {
         int nb = -1;

@@ -11,8 +11,11 @@ def _dev(t):
     return None if t is None else (t.cuda() if isinstance(t, torch.Tensor) else t)
 
 
-def run_capi(cfg, *, op="jagged", flags=0, **over):
-    """Call hstu_hip_<op>_forward through ctypes.  Returns the output on the CPU."""
+def run_capi(cfg, *, op="jagged", flags=0, reuse_from=None, **over):
+    """Call hstu_hip_<op>_forward through ctypes.  Returns the output on the CPU.
+
+    ``reuse_from``: a configuration with the same geometry; it is run first and its workspace (work list) is then
+    handed to the call for ``cfg`` with HSTU_FLAG_REUSE_WORKSPACE set."""
     from recsdk_amd import _capi
     c = dict(cfg)
     c.update(over)
@@ -39,7 +42,17 @@ def run_capi(cfg, *, op="jagged", flags=0, **over):
                   last_page_len=_dev(c["last_page_len"]), kv_scales=_dev(c["kv_scales"]) if c.get("use_fp8") else None)
     p, keep = _capi.make_params(q, k, v, out, **kw)
     name = _capi.describe_kernel(p)
-    _capi.run(op, p)
+    if reuse_from is not None:
+        import ctypes as C
+        r = dict(reuse_from)
+        p0, keep0 = _capi.make_params(_dev(r["q"]), _dev(r["k"]), _dev(r["v"]), torch.empty_like(out), **kw)
+        ws = _capi.run(op, p0)
+        torch.cuda.synchronize()
+        p.flags |= _capi.FLAG_REUSE_WORKSPACE
+        rc = getattr(_capi.lib(), f"hstu_hip_{op}_forward")(C.byref(p), ws.data_ptr(), ws.numel(), None)
+        assert rc == 0, _capi.lib().hstu_hip_last_error().decode()
+    else:
+        _capi.run(op, p)
     torch.cuda.synchronize()
     return out.cpu(), name
 

@@ -59,6 +59,8 @@ def test_struct_layout_matches_and_workspace_size():
     # workspace: 16 header words + 8-word records: 8 XCD lists of cap records + an overflow list of `bound` records, with
     # bound = min(total_q // 128 + batch, batch * ceil(max_seq_len_q / 128)) * heads_q, cap = ceil(bound / 8) + tiles
     assert rc == 0 and n == 4 * (16 + 8 * (8 * 2 + 8)), msg
+    rc, n, msg = _ws(_params(batch=257, total_q=25700))
+    assert rc == 0 and n == 4 * (16 + 8 * (8 * (129 + 1) + 257 * 4)), msg
     rc, n, msg = _ws(_params(dtype=_capi.HSTU_F32))
     assert rc == 0 and n == 0, msg          # the generic kernel needs none
     rc, n, msg = _ws(_params(flags=_capi.FLAG_FORCE_GENERIC))

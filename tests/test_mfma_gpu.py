@@ -214,3 +214,16 @@ def test_work_list_many_sequences(nseq, heads):
     T.assert_parity(out, gen.float(), dtype, what=f"many sequences {nseq}x{heads} vs generic kernel")
     if nseq <= 300:
         T.assert_parity(out, T.oracle_jagged(cfg), dtype, what=f"many sequences {nseq}x{heads} vs oracle")
+
+
+def test_work_list_reuse_across_calls():
+    """Second call on the same batch geometry with other q/k/v reuses the work list of the first one."""
+    say("work_list_reuse")
+    dtype = torch.bfloat16
+    cfg_a, _ = _jag(33, [300, 40, 513, 129], 4, 2, 128, 128, dtype)
+    cfg_b, _ = _jag(34, [300, 40, 513, 129], 4, 2, 128, 128, dtype)
+    out, name = T.run_capi(cfg_b, reuse_from=cfg_a)
+    assert name.startswith("mfma_"), name
+    fresh, _ = T.run_capi(cfg_b)
+    assert torch.equal(out, fresh)
+    T.assert_parity(out, T.oracle_jagged(cfg_b), dtype, what="reused work list vs oracle")
