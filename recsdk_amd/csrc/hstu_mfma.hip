@@ -287,10 +287,24 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
 
 // EXTRA: 0 = no bias / built-in mask only, 1 = dense bias and/or custom mask (tables, if any, gathered from
 // global memory), 2 = bias tables only, gathered from LDS-resident copies
+// The plain variant (head dim 128, built-in mask, no bias, rows straight from k/v) fits 168 registers and 34 KB of
+// LDS with 32-column K/V tiles: three workgroups per CU (3 waves/SIMD), which overlaps the MFMA, SiLU and LDS phases of
+// the waves better than two (measured -8 %).  Every other variant runs 64-column tiles at two workgroups per CU.
+template <int D, int EXTRA, bool PAGED> struct Shape {
+    static constexpr bool DMA = !PAGED && D == 128;
+    static constexpr bool LEAN = DMA && EXTRA == 0;
+    static constexpr int BNT = LEAN ? 32 : 64;     // K columns per step
+    static constexpr int WAVES = LEAN ? 3 : 2;     // waves per SIMD
+};
+
 template <typename T, int D, int EXTRA, bool PAGED>
-__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2)))
+__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(Shape<D, EXTRA, PAGED>::WAVES, Shape<D, EXTRA, PAGED>::WAVES)))
 void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws) {
     typedef Tile<D> TL;
+    typedef Shape<D, EXTRA, PAGED> SH;
+    constexpr int BNT = SH::BNT;
+    constexpr bool LEAN = SH::LEAN;
+    constexpr int NBLK4 = BNT / 4;                 // 4-row blocks per tile
     typedef typename MM<T>::v8 v8;
     const hstu_fwd_params& p = a.p;
     // K/V tiles of head dim 128 that come straight from q-like [rows, heads, D] tensors are copied global -> LDS
@@ -298,10 +312,9 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws) {
     // contiguous LDS bytes = 4 rows, so a tile is a sequence of 4-row blocks (K blocks padded by 64 B); inside
     // a block row rho keeps its 16-byte chunk c at position (c + rho) % 16 (K) or (c + 4 rho) % 16 (V), which
     // spreads the fragment reads below over all banks.  Everything else goes through registers into padded rows.
-    constexpr bool DMA = !PAGED && D == 128;
+    constexpr bool DMA = SH::DMA;
     constexpr int KBLK = 1088, VBLK = 1024;              // bytes per 4-row block
-    constexpr int K_BYTES = DMA ? 16 * KBLK : TL::K_ELEMS * 2;
-    constexpr int STAGE_BYTES = DMA ? 16 * KBLK + 16 * VBLK : (TL::K_ELEMS + TL::V_ELEMS) * 2;
+    constexpr int STAGE_BYTES = DMA ? NBLK4 * (KBLK + VBLK) : (TL::K_ELEMS + TL::V_ELEMS) * 2;
     // two separate arrays: reads of one tile are then independent of the copy in flight into the other
     __shared__ __attribute__((aligned(1024))) char lds0[STAGE_BYTES];
     __shared__ __attribute__((aligned(1024))) char lds1[STAGE_BYTES];
@@ -355,12 +368,12 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws) {
     int voff[4];
 #pragma unroll
     for (int db = 0; db < 4; db++)
-        voff[db] = 16 * KBLK + g * VBLK + q4 * 256 + ((4 * ((db + q4) & 3) + 2 * u16 + (piece >> 1)) << 4) + 8 * (piece & 1);
+        voff[db] = NBLK4 * KBLK + g * VBLK + q4 * 256 + ((4 * ((db + q4) & 3) + 2 * u16 + (piece >> 1)) << 4) + 8 * (piece & 1);
 
     for (int tile = tile0; active && tile * BM < s.lq; tile++) {
         const int i0 = tile * BM;
         const int kend = (s.lk > 0) ? k_extent(a, s, i0, min(i0 + BM, s.lq)) : 0;
-        const int ntk = (kend + BN - 1) / BN;
+        const int ntk = (kend + BNT - 1) / BNT;
         const int r0 = i0 + 32 * w;      // first row of this wave
         const int qi = r0 + l32;         // this lane's Q row
         const bool qvalid = qi < s.lq;
@@ -419,17 +432,17 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws) {
         const char* vview = reinterpret_cast<const char*>(p.v) + ((int64_t)s.k_start * p.heads_k + hk) * D * 2;
         const unsigned view_bytes = kend > 0 ? (unsigned)(kend - 1) * rowstride + D * 2 : 0;
         auto fetch = [&](int kt, char* dst) __attribute__((always_inline)) {
-            const int k0 = kt * BN;
+            const int k0 = kt * BNT;
             if constexpr (DMA) {
                 const unsigned tile_off = (unsigned)k0 * rowstride;
                 __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc((void*)(kview + tile_off), 0, (int)(view_bytes - tile_off), 0x00020000);
                 __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc((void*)(vview + tile_off), 0, (int)(view_bytes - tile_off), 0x00020000);
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const int blk = 4 * w + i;
+                for (int i = 0; i < NBLK4 / 4; i++) {
+                    const int blk = (NBLK4 / 4) * w + i;
                     const unsigned so = (unsigned)(4 * blk) * rowstride;
                     __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, LDS_PTR(void, dst + blk * KBLK), 16, ldK + so, 0, 0, 0);
-                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, LDS_PTR(void, dst + 16 * KBLK + blk * VBLK), 16, ldV + so, 0, 0, 0);
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, LDS_PTR(void, dst + NBLK4 * KBLK + blk * VBLK), 16, ldV + so, 0, 0, 0);
                 }
             } else {
 #pragma unroll
@@ -459,7 +472,7 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws) {
         };
         // second half of the register path, and the table windows; ends with the tile being complete in LDS
         auto stash = [&](int kt, char* dst) __attribute__((always_inline)) {
-            const int k0 = kt * BN;
+            const int k0 = kt * BNT;
             const int buf = kt & 1;
             if (!DMA && k0 < kend) {
                 T* dk = reinterpret_cast<T*>(dst);
@@ -510,11 +523,11 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws) {
 
         auto iteration = [&](int kt, const char* cur, char* nxt) __attribute__((always_inline)) {
             const int buf = kt & 1;
-            const int k0 = kt * BN;
+            const int k0 = kt * BNT;
             if (kt + 1 < ntk) fetch(kt + 1, nxt);
 
 #pragma unroll
-            for (int kb = 0; kb < 2; kb++) {
+            for (int kb = 0; kb < BNT / 32; kb++) {
                 const int c0 = k0 + 32 * kb;
                 const int cls = tril ? classify_block(s, tgs, r0, c0) : BLK_ALL;
                 if (cls == BLK_SKIP) continue;  // wave-uniform
@@ -532,10 +545,12 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws) {
                 // Transposing LDS read: a 16-lane group reads 4 key rows x 16 columns and every lane
                 // receives 4 consecutive keys of one column.
                 s16x4 vlo[D / 32], vhi[D / 32], wlo[D / 32], whi[D / 32];
+                if (!LEAN) {
 #pragma unroll
-                for (int db = 0; db < D / 32; db++) {
-                    vlo[db] = read_vf(cur, kb, db, 0);
-                    vhi[db] = read_vf(cur, kb, db, 1);
+                    for (int db = 0; db < D / 32; db++) {
+                        vlo[db] = read_vf(cur, kb, db, 0);
+                        vhi[db] = read_vf(cur, kb, db, 1);
+                    }
                 }
                 // ---- P = s * sigmoid(alpha * s) (scale folded into the epilogue), masked
                 // accumulator register r holds key c0 + 8*(r/4) + 4*g + r%4 for Q row qi
@@ -605,15 +620,32 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws) {
                     pk0[x] = MM<T>::pack2(pf[2 * x], pf[2 * x + 1]);
                     pk1[x] = MM<T>::pack2(pf[8 + 2 * x], pf[8 + 2 * x + 1]);
                 }
+                if (LEAN) {   // fewer live registers: fragments are read right before the step that uses them
+                    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int db = 0; db < D / 32; db++) {   // second step's fragments fly while the first step multiplies
-                    wlo[db] = read_vf(cur, kb, db, 2);
-                    whi[db] = read_vf(cur, kb, db, 3);
+                    for (int db = 0; db < D / 32; db++) {
+                        vlo[db] = read_vf(cur, kb, db, 0);
+                        vhi[db] = read_vf(cur, kb, db, 1);
+                    }
+                } else {
+#pragma unroll
+                    for (int db = 0; db < D / 32; db++) {   // second step's fragments fly while the first step multiplies
+                        wlo[db] = read_vf(cur, kb, db, 2);
+                        whi[db] = read_vf(cur, kb, db, 3);
+                    }
                 }
 #pragma unroll
                 for (int db = 0; db < D / 32; db++) {
                     s16x8 vv = {vlo[db][0], vlo[db][1], vlo[db][2], vlo[db][3], vhi[db][0], vhi[db][1], vhi[db][2], vhi[db][3]};
                     oacc[db] = MM<T>::mfma(__builtin_bit_cast(v8, vv), __builtin_bit_cast(v8, pk0), oacc[db]);
+                }
+                if (LEAN) {
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int db = 0; db < D / 32; db++) {
+                        wlo[db] = read_vf(cur, kb, db, 2);
+                        whi[db] = read_vf(cur, kb, db, 3);
+                    }
                 }
 #pragma unroll
                 for (int db = 0; db < D / 32; db++) {
