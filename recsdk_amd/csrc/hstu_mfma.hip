@@ -286,7 +286,8 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
 }
 
 // EXTRA: 0 = no bias / built-in mask only, 1 = dense bias and/or custom mask (tables, if any, gathered from
-// global memory), 2 = bias tables only, gathered from LDS-resident copies
+// global memory), 2 / 3 / 4 = bias tables only, gathered from LDS-resident copies: position table / time table /
+// both (compile-time so that the per-score code is branch-free)
 // The plain variant (head dim 128, built-in mask, no bias, rows straight from k/v) fits 168 registers and 34 KB of
 // LDS with 32-column K/V tiles: three workgroups per CU (3 waves/SIMD), which overlaps the MFMA, SiLU and LDS phases of
 // the waves better than two (measured -8 %).  Every other variant runs 64-column tiles at two workgroups per CU.
@@ -321,10 +322,11 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws) {
     // table mode: per K tile a window of the position table and the key timestamps (double buffered with the
     // K/V tiles), plus the whole time table and its bucket bounds as (lower, upper) pairs
     constexpr int PW = BM + BN;   // window entries: (j - k0) - (qi - i0) + BM - 1 in [0, BM + BN - 2]
-    __shared__ float lds_pos[EXTRA == 2 ? 2 * PW : 1];
-    __shared__ __attribute__((aligned(8))) long long lds_tk[EXTRA == 2 ? 2 * BN : 1];
-    __shared__ __attribute__((aligned(8))) float lds_tsb[EXTRA == 2 ? 2 * 132 : 1];
-    __shared__ float lds_tst[EXTRA == 2 ? 132 : 1];
+    constexpr bool TAB = EXTRA >= 2, tab_pos = EXTRA == 2 || EXTRA == 4, tab_ts = EXTRA == 3 || EXTRA == 4;
+    __shared__ float lds_pos[tab_pos ? 2 * PW : 1];
+    __shared__ __attribute__((aligned(8))) long long lds_tk[tab_ts ? 2 * BN : 1];
+    __shared__ __attribute__((aligned(8))) float lds_tsb[tab_ts ? 2 * 132 : 1];
+    __shared__ float lds_tst[tab_ts ? 132 : 1];
     // paged: page ids of this user and, for an fp8 cache, the (K, V) scales of this kv head
     __shared__ int lds_pid[PAGED ? MAXP : 1];
     __shared__ float lds_psc[PAGED ? 2 * MAXP : 1];
@@ -397,9 +399,6 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws) {
 
         int64_t tq = 0;
         if (EXTRA && p.ts_table && qvalid && qi + s.delta >= 0) tq = p.timestamps[s.k_start + qi + s.delta];
-        const bool tab_pos = EXTRA == 2 && p.pos_table != nullptr;
-        const bool tab_ts = EXTRA == 2 && p.ts_table != nullptr && p.num_buckets <= 128 && p.ts_log2_scale > 0.f;
-        const bool glb_ts = EXTRA == 2 && p.ts_table != nullptr && !tab_ts;   // tables too large for LDS or no hint
         if (tab_ts && tid <= p.num_buckets) {
             lds_tst[tid] = p.ts_table[tid];
             lds_tsb[2 * tid] = p.ts_bounds[tid];
@@ -461,7 +460,7 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws) {
                     }
                 }
             }
-            if (EXTRA == 2) {
+            if (TAB) {
                 if (tab_pos && tid < PW - 1) {
                     // window entry e holds pos_table[(max_k - 1) + (k0 + e - (BM - 1) - i0) - delta]
                     const int idx = (p.max_seq_len_k - 1) + k0 + tid - (BM - 1) - i0 - s.delta;
@@ -492,7 +491,7 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws) {
                     *reinterpret_cast<u32x4*>(dv + row * TL::VS + cc * 8) = ok ? vx : z;
                 }
             }
-            if (EXTRA == 2) {
+            if (TAB) {
                 if (tab_pos && tid < PW - 1) lds_pos[buf * PW + tid] = pw_reg;
                 if (tab_ts && tid < BN) lds_tk[buf * BN + tid] = tk_reg;
             }
@@ -574,7 +573,7 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws) {
                         }
                         if (p.mask_type == HSTU_MASK_CUSTOM) mval = in_attr ? to_float(reinterpret_cast<const T*>(p.mask)[bm]) : 0.f;
                     }
-                    if (EXTRA == 2) {
+                    if (TAB) {
                         const int jj = 32 * kb + 8 * (r >> 2) + 4 * g + (r & 3);        // j - k0
                         if (tab_pos) x += lds_pos[buf * PW + jj - (32 * w + l32) + (BM - 1)];
                         if (tab_ts) {
@@ -585,10 +584,6 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws) {
                             const float lo = lds_tsb[2 * bk], hi = lds_tsb[2 * bk + 1];
                             bk += (dt >= hi ? 1 : 0) - (dt < lo ? 1 : 0);
                             x += lds_tst[bk];
-                        } else if (glb_ts && 32 * kb + 8 * (r >> 2) + 4 * g + (r & 3) + k0 < s.lk) {
-                            // no search hint or a table too large for LDS: binary search over the bounds in global memory
-                            float dt = abs_dt_as_float(tq, p.timestamps[s.k_start + j]);
-                            x += p.ts_table[ts_bucket(p.ts_bounds, p.num_buckets, dt)];
                         }
                     }
                     float e = __builtin_amdgcn_exp2f(x * a.exp_scale);
@@ -708,8 +703,14 @@ static hipError_t launch_td(const KArgs& a, unsigned* ws, hipStream_t stream) {
     const hstu_fwd_params& p = a.p;
     const SchedDims d = sched_dims(p);
     const bool dense_extra = p.attn_bias || p.mask_type == HSTU_MASK_CUSTOM;
-    const bool tables = p.pos_table || p.ts_table;
-    const int extra = dense_extra ? 1 : (tables ? 2 : 0);
+    // the time table is used from LDS when it fits and the search hint is there; else the general path searches the
+    // bounds in global memory
+    const bool ts_in_lds = p.ts_table && p.num_buckets <= 128 && p.ts_log2_scale > 0.f;
+    int extra = 0;
+    if (dense_extra || (p.ts_table && !ts_in_lds)) extra = 1;
+    else if (p.pos_table && p.ts_table) extra = 4;
+    else if (p.ts_table) extra = 3;
+    else if (p.pos_table) extra = 2;
     const bool paged = a.op == OP_PAGED;
     const int groups = p.batch * p.heads_q;
     const int sched_threads = groups <= 256 ? 256 : (groups <= 512 ? 512 : SCHED_NT);
@@ -732,7 +733,9 @@ static hipError_t launch_td(const KArgs& a, unsigned* ws, hipStream_t stream) {
     } else {
         if (extra == 0) HSTU_LAUNCH(0, false);
         else if (extra == 1) HSTU_LAUNCH(1, false);
-        else HSTU_LAUNCH(2, false);
+        else if (extra == 2) HSTU_LAUNCH(2, false);
+        else if (extra == 3) HSTU_LAUNCH(3, false);
+        else HSTU_LAUNCH(4, false);
     }
 #undef HSTU_LAUNCH
     return hipGetLastError();
