@@ -124,7 +124,8 @@ typedef struct hstu_fwd_params {
      *     bucket(i,j) = the b with bounds[b] <= (float)|t_i - t_j| < bounds[b+1];  bias += ts_table[bucket]
      *   ts_log2_scale: optional search hint.  If non-zero, floor(log2(|dt|) * ts_log2_scale) must be within one
      *     bucket of the answer (for the reference's log buckets: ln(2)/bucket_divisor); the result is always
-     *     decided by ts_bounds.  0 = no hint (binary search).
+     *     decided by ts_bounds.  0 = no hint (binary search).  With the hint the kernel takes |dt| from timestamps
+ *     held as doubles relative to the sequence's first one: exact while one sequence spans less than 2^53 ticks.
      * Added to attn_bias when both are given.
      */
     const float* pos_table;

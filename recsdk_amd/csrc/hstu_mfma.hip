@@ -324,7 +324,7 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws) {
     constexpr int PW = BM + BN;   // window entries: (j - k0) - (qi - i0) + BM - 1 in [0, BM + BN - 2]
     constexpr bool TAB = EXTRA >= 2, tab_pos = EXTRA == 2 || EXTRA == 4, tab_ts = EXTRA == 3 || EXTRA == 4;
     __shared__ float lds_pos[tab_pos ? 2 * PW : 1];
-    __shared__ __attribute__((aligned(8))) long long lds_tk[tab_ts ? 2 * BN : 1];
+    __shared__ __attribute__((aligned(8))) double lds_tk[tab_ts ? 2 * BN : 1];
     __shared__ __attribute__((aligned(8))) float lds_tsb[tab_ts ? 2 * 132 : 1];
     __shared__ float lds_tst[tab_ts ? 132 : 1];
     // paged: page ids of this user and, for an fp8 cache, the (K, V) scales of this kv head
@@ -399,13 +399,19 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws) {
 
         int64_t tq = 0;
         if (EXTRA && p.ts_table && qvalid && qi + s.delta >= 0) tq = p.timestamps[s.k_start + qi + s.delta];
+        // LDS-table mode works on timestamps relative to the first one of the sequence, held as doubles: the
+        // difference of two of them and its rounding to fp32 equal (float)|t_i - t_j| of the int64 values as long as
+        // the timestamps of one sequence span less than 2^53
+        int64_t tbase = 0;
+        if (tab_ts && s.lk > 0) tbase = p.timestamps[s.k_start];
+        const double tqd = (double)(tq - tbase);
         if (tab_ts && tid <= p.num_buckets) {
             lds_tst[tid] = p.ts_table[tid];
             lds_tsb[2 * tid] = p.ts_bounds[tid];
             lds_tsb[2 * tid + 1] = p.ts_bounds[tid + 1];
         }
         float pw_reg = 0.f;
-        long long tk_reg = 0;
+        double tk_reg = 0;
         if (PAGED) {
             const int is64 = p.index_type == HSTU_I64;
             const int np = min((s.hist_k + p.page_size - 1) / p.page_size, MAXP);
@@ -466,7 +472,7 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws) {
                     const int idx = (p.max_seq_len_k - 1) + k0 + tid - (BM - 1) - i0 - s.delta;
                     pw_reg = (idx >= 0 && idx < 2 * p.max_seq_len_k - 1) ? p.pos_table[idx] : 0.f;
                 }
-                if (tab_ts && tid < BN) tk_reg = p.timestamps[s.k_start + min(k0 + tid, s.lk - 1)];
+                if (tab_ts && tid < BN) tk_reg = (double)(p.timestamps[s.k_start + min(k0 + tid, s.lk - 1)] - tbase);
             }
         };
         // second half of the register path, and the table windows; ends with the tile being complete in LDS
@@ -577,7 +583,7 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws) {
                         const int jj = 32 * kb + 8 * (r >> 2) + 4 * g + (r & 3);        // j - k0
                         if (tab_pos) x += lds_pos[buf * PW + jj - (32 * w + l32) + (BM - 1)];
                         if (tab_ts) {
-                            const float dt = abs_dt_as_float(tq, lds_tk[buf * BN + jj]);
+                            const float dt = (float)__builtin_fabs(tqd - lds_tk[buf * BN + jj]);
                             // estimate from log2, then let the bounds decide (the estimate is within one bucket)
                             int bk = (int)(__builtin_amdgcn_logf(fmaxf(dt, 1.0f)) * p.ts_log2_scale);
                             bk = min(max(bk, 0), p.num_buckets);
