@@ -24,6 +24,7 @@ typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) short s16x4;
 typedef __attribute__((ext_vector_type(8))) short s16x8;
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
@@ -145,8 +146,8 @@ __device__ __forceinline__ int classify_block(const Seq& s, int tgs, int r0, int
 // ---- work list ------------------------------------------------------------------------------------------
 // The hardware dispatches workgroups in index order and a workgroup that finds no work still costs a slot, so
 // the grid is driven by a list that a one-workgroup kernel builds first from the sequence lengths:
-//   * one item = one 128-row Q tile of one (sequence, head): a record of 8 words -- seq | head << 12 | tile << 16
-//     | sweep << 24, then the sequence's geometry (q_start, lq, k_start, lk, num_context, num_target, first page
+//   * one item = one 128-row Q tile of one (sequence, head) (or one of its 2-4 K ranges, see sched_dims): a record
+//     of 8 words -- seq | head << 12 | tile << 16 | sweep << 24 | K range << 25 | ranges << 28, then the sequence's geometry (q_start, lq, k_start, lk, num_context, num_target, first page
 //     entry), so that a workgroup needs one scalar load to know its work
 //   * sequences are sorted by K length (longest first) and their (sequence, head) groups are dealt to the
 //     8 XCDs in snake order; a group's tiles sit next to each other in its XCD's list, last tile first, so that
@@ -165,6 +166,7 @@ struct SchedDims {
     int ntiles_attr;   // Q tiles the max_seq_len_q attribute covers
     unsigned cap;      // entries per XCD list
     unsigned bound;    // upper bound of the number of items (= entries of the overflow list)
+    int nsplit;        // K ranges per Q tile (1 = none); each range is an item of its own
 };
 
 static SchedDims sched_dims(const hstu_fwd_params& p) {
@@ -173,13 +175,32 @@ static SchedDims sched_dims(const hstu_fwd_params& p) {
     // sum over sequences of min(ceil(lq / BM), ntiles_attr) <= min(total_q / BM + batch, batch * ntiles_attr)
     const int64_t by_rows = p.total_q / BM + p.batch, by_attr = (int64_t)p.batch * d.ntiles_attr;
     d.bound = (unsigned)((by_rows < by_attr ? by_rows : by_attr) * p.heads_q);
-    d.cap = (d.bound + 7) / 8 + (unsigned)d.ntiles_attr;
+    // Few Q tiles but long K (serving: a handful of users, candidates against a long history): split the K range of
+    // every tile over up to 4 workgroups so that the CUs hold 2-3 of them; the partial sums (HSTU has no softmax, so
+    // they simply add up) go through the workspace and a small reduction kernel.
+    d.nsplit = 1;
+    const int ktiles = (p.max_seq_len_k + BN - 1) / BN;
+    if (d.bound < 384 && ktiles >= 16) {
+        int s = 768 / (int)(d.bound ? d.bound : 1);
+        if (s > 4) s = 4;
+        if (s > ktiles / 4) s = ktiles / 4;
+        if (s > 1) d.nsplit = s;
+    }
+    d.bound *= (unsigned)d.nsplit;
+    d.cap = (d.bound + 7) / 8 + (unsigned)(d.ntiles_attr * d.nsplit);
     return d;
+}
+
+static uint64_t list_bytes(const SchedDims& d) {
+    const uint64_t b = (uint64_t)(WS_HEADER + REC * (8 * (uint64_t)d.cap + d.bound)) * sizeof(uint32_t);
+    return (b + 255) / 256 * 256;
 }
 
 uint64_t mfma_workspace_bytes(const KArgs& a) {
     const SchedDims d = sched_dims(a.p);
-    return (uint64_t)(WS_HEADER + REC * (8 * (uint64_t)d.cap + d.bound)) * sizeof(uint32_t);
+    uint64_t b = list_bytes(d);
+    if (d.nsplit > 1) b += (uint64_t)d.nsplit * a.p.total_q * a.p.heads_q * a.p.dim_v * sizeof(float);   // partial sums
+    return b;
 }
 
 __device__ __forceinline__ int xcd_of_group(unsigned r) { return (r & 8) ? 7 - (int)(r & 7) : (int)(r & 7); }
@@ -240,7 +261,8 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
         const unsigned r = c0 + tid;
         const unsigned rank = r / H, h = r - rank * H;
         const int b = r < G ? (int)s_order[rank] : 0;
-        const unsigned v = r < G ? s_tiles[b] : 0u;
+        const unsigned ns = (unsigned)d.nsplit;
+        const unsigned v = r < G ? s_tiles[b] * ns : 0u;   // entries of this group: (tile, K range) pairs
         s_val[tid] = v;
         s_scan[tid] = v;
         __syncthreads();
@@ -255,8 +277,8 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
         pos += j < 8 ? s_scan[tp] - s_val[tp] : s_scan[tp];
         const int x = xcd_of_group(r);
         for (unsigned i = 0; i < v; i++) {
-            const unsigned tile = v - 1 - i;
-            const unsigned item = (unsigned)b | h << 12 | tile << 16 | ((i == 0 && s_sweep[b]) ? 1u << 24 : 0u);
+            const unsigned tile = (v - 1 - i) / ns, part = i % ns;
+            const unsigned item = (unsigned)b | h << 12 | tile << 16 | ((i < ns && s_sweep[b]) ? 1u << 24 : 0u) | part << 25 | ns << 28;
             unsigned* rec = pos + i < d.cap ? list + REC * (8 * (size_t)(pos + i) + x) : ovf + REC * (size_t)atomicAdd(&s_ovf, 1u);
             const u32x4 lo = {item, (unsigned)s_geo[0][b], (unsigned)s_geo[1][b], (unsigned)s_geo[2][b]};
             const u32x4 hi = {(unsigned)s_geo[3][b], (unsigned)s_geo[4][b], (unsigned)s_geo[5][b], (unsigned)s_geo[6][b]};
@@ -300,7 +322,7 @@ template <int D, int EXTRA, bool PAGED> struct Shape {
 
 template <typename T, int D, int EXTRA, bool PAGED>
 __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(Shape<D, EXTRA, PAGED>::WAVES, Shape<D, EXTRA, PAGED>::WAVES)))
-void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws) {
+void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const float* part_base) {
     typedef Tile<D> TL;
     typedef Shape<D, EXTRA, PAGED> SH;
     constexpr int BNT = SH::BNT;
@@ -348,6 +370,7 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws) {
     const int b = active ? (int)(item & 0xfff) : 0, h = active ? (int)((item >> 12) & 0xf) : 0;
     const int tile0 = (int)((item >> 16) & 0xff);
     const bool sweep = (item >> 24) & 1;   // last tile the max_seq_len_q attribute covers of a sequence that is longer
+    const int part = active ? (int)((item >> 25) & 7) : 0, nsplit = active ? (int)((item >> 28) & 7) : 1;
     const int hk = h / a.head_ratio;
     Seq s;
     s.q_start = active ? (int)rw[1] : 0; s.lq = active ? (int)rw[2] : 0;
@@ -523,13 +546,16 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws) {
             }
         };
 
-        if (ntk > 0) fetch(0, lds0);
-        stash(0, lds0);
+        // K range of this workgroup: all tiles, or its share of them when the tile is split
+        const int per = (ntk + nsplit - 1) / nsplit;
+        const int kt0 = part * per, kt1 = min(ntk, kt0 + per);
+        if (kt0 < kt1) fetch(kt0, lds0);
+        stash(kt0, lds0);
 
         auto iteration = [&](int kt, const char* cur, char* nxt) __attribute__((always_inline)) {
             const int buf = kt & 1;
             const int k0 = kt * BNT;
-            if (kt + 1 < ntk) fetch(kt + 1, nxt);
+            if (kt + 1 < kt1) fetch(kt + 1, nxt);
 
 #pragma unroll
             for (int kb = 0; kb < BNT / 32; kb++) {
@@ -657,13 +683,13 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws) {
 
             stash(kt + 1, nxt);
         };
-        for (int kt = 0; kt < ntk; kt += 2) {
+        for (int kt = kt0; kt < kt1; kt += 2) {
             iteration(kt, lds0, lds1);
-            if (kt + 1 < ntk) iteration(kt + 1, lds1, lds0);
+            if (kt + 1 < kt1) iteration(kt + 1, lds1, lds0);
         }
 
         // ---- epilogue: O^T accumulator register r of block db holds d = 32*db + 8*(r/4) + 4*g + r%4 for row qi
-        if (qvalid) {
+        if (qvalid && nsplit == 1) {
             T* op = obase + ((s.q_start + qi) * p.heads_q + h) * (int64_t)D + 4 * g;
 #pragma unroll
             for (int db = 0; db < D / 32; db++) {
@@ -673,6 +699,17 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws) {
                     o[0] = MM<T>::pack2(oacc[db][4 * rr] * a.out_scale, oacc[db][4 * rr + 1] * a.out_scale);
                     o[1] = MM<T>::pack2(oacc[db][4 * rr + 2] * a.out_scale, oacc[db][4 * rr + 3] * a.out_scale);
                     *reinterpret_cast<u32x2*>(op + 32 * db + 8 * rr) = o;
+                }
+            }
+        } else if (qvalid) {
+            // partial sums of this K range, unscaled fp32, [range][row][head][D] behind the work list
+            float* pp = const_cast<float*>(part_base) + (((int64_t)part * p.total_q + s.q_start + qi) * p.heads_q + h) * (int64_t)D + 4 * g;
+#pragma unroll
+            for (int db = 0; db < D / 32; db++) {
+#pragma unroll
+                for (int rr = 0; rr < 4; rr++) {
+                    const f32x4 o = {oacc[db][4 * rr], oacc[db][4 * rr + 1], oacc[db][4 * rr + 2], oacc[db][4 * rr + 3]};
+                    *reinterpret_cast<f32x4*>(pp + 32 * db + 8 * rr) = o;
                 }
             }
         }
@@ -689,6 +726,29 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws) {
             T* o = obase + tail * p.heads_q * (int64_t)D;
             for (int64_t e = (int64_t)blockIdx.x * NT + tid; e < n; e += (int64_t)gridDim.x * NT) o[e] = (T)0.f;
         }
+    }
+}
+
+// out = (sum over the K ranges of the partial sums) * alpha * silu_scale, for the rows the sequences own
+template <typename T>
+__global__ __launch_bounds__(256)
+void hstu_reduce_kernel(const KArgs a, const float* __restrict__ part, const int nsplit) {
+    const hstu_fwd_params& p = a.p;
+    const int is64 = p.index_type == HSTU_I64;
+    const int64_t rows = p.seq_offset_q ? ld_idx(p.seq_offset_q, p.batch, is64) : p.total_q;
+    const int64_t per_range = p.total_q * p.heads_q * (int64_t)p.dim_v;
+    const int64_t n4 = rows * p.heads_q * (int64_t)p.dim_v / 4;
+    T* out = reinterpret_cast<T*>(p.out);
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (int64_t)gridDim.x * 256) {
+        f32x4 acc = *reinterpret_cast<const f32x4*>(part + 4 * i);
+        for (int r = 1; r < nsplit; r++) {
+            const f32x4 x = *reinterpret_cast<const f32x4*>(part + r * per_range + 4 * i);
+            acc[0] += x[0]; acc[1] += x[1]; acc[2] += x[2]; acc[3] += x[3];
+        }
+        u32x2 o;
+        o[0] = MM<T>::pack2(acc[0] * a.out_scale, acc[1] * a.out_scale);
+        o[1] = MM<T>::pack2(acc[2] * a.out_scale, acc[3] * a.out_scale);
+        *reinterpret_cast<u32x2*>(out + 4 * i) = o;
     }
 }
 
@@ -727,12 +787,13 @@ static hipError_t launch_td(const KArgs& a, unsigned* ws, hipStream_t stream) {
         if (e != hipSuccess) return e;
     }
     dim3 grid(8 * d.cap), block(NT);   // the overflow list starts at entry gridDim.x of the lists
+    const float* part = reinterpret_cast<const float*>(reinterpret_cast<const char*>(ws) + list_bytes(d));
     if (getenv("HSTU_HIP_DEBUG")) {
         int nb = -1;
         e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, hstu_mfma_kernel<T, D, 0, false>, NT, 0);
         fprintf(stderr, "[hstu_hip] mfma d=%d grid=%u workgroups/CU=%d (%s)\n", D, grid.x, nb, hipGetErrorString(e));
     }
-#define HSTU_LAUNCH(E, P) hipLaunchKernelGGL((hstu_mfma_kernel<T, D, E, P>), grid, block, 0, stream, a, ws)
+#define HSTU_LAUNCH(E, P) hipLaunchKernelGGL((hstu_mfma_kernel<T, D, E, P>), grid, block, 0, stream, a, ws, part)
     if (paged) {
         if (extra == 0) HSTU_LAUNCH(0, true);
         else HSTU_LAUNCH(1, true);      // paged + bias: the general gather path
@@ -744,6 +805,11 @@ static hipError_t launch_td(const KArgs& a, unsigned* ws, hipStream_t stream) {
         else HSTU_LAUNCH(4, false);
     }
 #undef HSTU_LAUNCH
+    e = hipGetLastError();
+    if (e != hipSuccess || d.nsplit == 1) return e;
+    const int64_t n4 = p.total_q * p.heads_q * (int64_t)p.dim_v / 4;
+    const unsigned rgrid = (unsigned)((n4 + 255) / 256 < 2048 ? (n4 + 255) / 256 : 2048);
+    hipLaunchKernelGGL(hstu_reduce_kernel<T>, dim3(rgrid ? rgrid : 1), dim3(256), 0, stream, a, part, d.nsplit);
     return hipGetLastError();
 }
 

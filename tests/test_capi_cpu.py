@@ -58,9 +58,12 @@ def test_struct_layout_matches_and_workspace_size():
     # a size mismatch between ctypes and C would be rejected here.  MFMA kernels keep their work list in the
     # workspace: 16 header words + 8-word records: 8 XCD lists of cap records + an overflow list of `bound` records, with
     # bound = min(total_q // 128 + batch, batch * ceil(max_seq_len_q / 128)) * heads_q, cap = ceil(bound / 8) + tiles
-    assert rc == 0 and n == 4 * (16 + 8 * (8 * 2 + 8)), msg
+    assert rc == 0 and n == 1024, msg                     # 4 * (16 + 8 * (8 * 2 + 8)) = 832, rounded up to 256
     rc, n, msg = _ws(_params(batch=257, total_q=25700))
-    assert rc == 0 and n == 4 * (16 + 8 * (8 * (129 + 1) + 257 * 4)), msg
+    assert rc == 0 and n == 66304, msg                    # 4 * (16 + 8 * (8 * 130 + 1028)) = 66240, rounded up
+    # few Q tiles, long K: the K range is split over 4 workgroups per tile and the fp32 partial sums follow the list
+    rc, n, msg = _ws(_params(max_seq_len_k=4096))
+    assert rc == 0 and n == 4 * (16 + 8 * (8 * (4 + 4) + 32)) // 256 * 256 + 256 + 4 * 100 * 4 * 128 * 4, msg
     rc, n, msg = _ws(_params(dtype=_capi.HSTU_F32))
     assert rc == 0 and n == 0, msg          # the generic kernel needs none
     rc, n, msg = _ws(_params(flags=_capi.FLAG_FORCE_GENERIC))

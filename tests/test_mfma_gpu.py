@@ -227,3 +227,18 @@ def test_work_list_reuse_across_calls():
     fresh, _ = T.run_capi(cfg_b)
     assert torch.equal(out, fresh)
     T.assert_parity(out, T.oracle_jagged(cfg_b), dtype, what="reused work list vs oracle")
+
+
+@pytest.mark.parametrize("dtype", LOWP)
+@pytest.mark.parametrize("d", [64, 128])
+def test_split_k_ranges(d, dtype):
+    """Few Q tiles against long K: each tile's K range is split over several workgroups, partial sums are reduced by
+    a second kernel.  Causal (early tiles have empty ranges), delta-q with targets, and a tail of unused rows."""
+    say("split_k", dtype, d)
+    cfg, _ = _jag(41, [2048, 700], 2, 2, d, d, dtype, extra_rows=5)
+    out = _check(cfg, dtype, f"split-K causal d={d}")
+    assert torch.equal(out[-5:], torch.zeros_like(out[-5:]))
+    cfg, _ = _jag(42, [100, 128, 37], 2, 1, d, d, dtype, lens_k=[2100, 1500, 1037])
+    cfg["num_target"] = torch.tensor([40, 128, 0])
+    cfg["target_group_size"] = 1
+    _check(cfg, dtype, f"split-K delta-q d={d}")
