@@ -122,10 +122,11 @@ typedef struct hstu_fwd_params {
      *   timestamps [total_k] int64 on the K timeline; ts_table [num_buckets+1] float;
      *   ts_bounds [num_buckets+2] float, ascending, bounds[0] = 0, bounds[num_buckets+1] = +inf:
      *     bucket(i,j) = the b with bounds[b] <= (float)|t_i - t_j| < bounds[b+1];  bias += ts_table[bucket]
-     *   ts_log2_scale: optional search hint.  If non-zero, floor(log2(|dt|) * ts_log2_scale) must be within one
-     *     bucket of the answer (for the reference's log buckets: ln(2)/bucket_divisor); the result is always
-     *     decided by ts_bounds.  0 = no hint (binary search).  With the hint the kernel takes |dt| from timestamps
- *     held as doubles relative to the sequence's first one: exact while one sequence spans less than 2^53 ticks.
+     *   ts_log2_scale: optional search hint.  If non-zero, bounds[b] must sit near 2^(b / ts_log2_scale): the kernel
+     *     rounds log2(|dt|) * ts_log2_scale to the nearest integer f and lets bounds[f] decide between bucket f and
+     *     f - 1, so the estimate only has to be within half a bucket (for the reference's log buckets the scale is
+     *     ln(2)/bucket_divisor).  0 = no hint (binary search over ts_bounds).  With the hint the kernel takes |dt| from
+     *     timestamps held as doubles relative to the sequence's first one: exact while one sequence spans < 2^53 ticks.
      * Added to attn_bias when both are given.
      */
     const float* pos_table;

@@ -347,8 +347,9 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
     constexpr bool TAB = EXTRA >= 2, tab_pos = EXTRA == 2 || EXTRA == 4, tab_ts = EXTRA == 3 || EXTRA == 4;
     __shared__ float lds_pos[tab_pos ? 2 * PW : 1];
     __shared__ __attribute__((aligned(8))) double lds_tk[tab_ts ? 2 * BN : 1];
-    __shared__ __attribute__((aligned(8))) float lds_tsb[tab_ts ? 2 * 132 : 1];
-    __shared__ float lds_tst[tab_ts ? 132 : 1];
+    // entry f of the time table: {bounds[f], table[f - 1], table[f]}: a score whose rounded log estimate is f sits in
+    // bucket f or f - 1, and the exact bound decides which
+    __shared__ __attribute__((aligned(16))) float lds_tsq[tab_ts ? 4 * 132 : 4];
     // paged: page ids of this user and, for an fp8 cache, the (K, V) scales of this kv head
     __shared__ int lds_pid[PAGED ? MAXP : 1];
     __shared__ float lds_psc[PAGED ? 2 * MAXP : 1];
@@ -428,10 +429,9 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
         int64_t tbase = 0;
         if (tab_ts && s.lk > 0) tbase = p.timestamps[s.k_start];
         const double tqd = (double)(tq - tbase);
-        if (tab_ts && tid <= p.num_buckets) {
-            lds_tst[tid] = p.ts_table[tid];
-            lds_tsb[2 * tid] = p.ts_bounds[tid];
-            lds_tsb[2 * tid + 1] = p.ts_bounds[tid + 1];
+        if (tab_ts && tid <= p.num_buckets + 1) {
+            const f32x4 entry = {p.ts_bounds[tid], p.ts_table[max(tid - 1, 0)], p.ts_table[min(tid, p.num_buckets)], 0.f};
+            *reinterpret_cast<f32x4*>(lds_tsq + 4 * tid) = entry;
         }
         float pw_reg = 0.f;
         double tk_reg = 0;
@@ -610,12 +610,11 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                         if (tab_pos) x += lds_pos[buf * PW + jj - (32 * w + l32) + (BM - 1)];
                         if (tab_ts) {
                             const float dt = (float)__builtin_fabs(tqd - lds_tk[buf * BN + jj]);
-                            // estimate from log2, then let the bounds decide (the estimate is within one bucket)
-                            int bk = (int)(__builtin_amdgcn_logf(fmaxf(dt, 1.0f)) * p.ts_log2_scale);
-                            bk = min(max(bk, 0), p.num_buckets);
-                            const float lo = lds_tsb[2 * bk], hi = lds_tsb[2 * bk + 1];
-                            bk += (dt >= hi ? 1 : 0) - (dt < lo ? 1 : 0);
-                            x += lds_tst[bk];
+                            // f = log estimate rounded to the nearest bucket boundary; the bucket is f or f - 1 and
+                            // the exact fp32 bound of f decides (the estimate only has to be within half a bucket)
+                            const int f = min((int)(__builtin_amdgcn_logf(fmaxf(dt, 1.0f)) * p.ts_log2_scale + 0.5f), p.num_buckets + 1);
+                            const f32x4 entry = *reinterpret_cast<const f32x4*>(lds_tsq + 4 * f);
+                            x += dt >= entry[0] ? entry[2] : entry[1];
                         }
                     }
                     float e = __builtin_amdgcn_exp2f(x * a.exp_scale);
