@@ -312,12 +312,13 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
 // both (compile-time so that the per-score code is branch-free)
 // The plain variant (head dim 128, built-in mask, no bias, rows straight from k/v) fits 168 registers and 34 KB of
 // LDS with 32-column K/V tiles: three workgroups per CU (3 waves/SIMD), which overlaps the MFMA, SiLU and LDS phases of
-// the waves better than two (measured -8 %).  Every other variant runs 64-column tiles at two workgroups per CU.
+// the waves better than two (measured -8 %).  The head-dim-64 variants other than the dense-bias one fit three per CU
+// with 64-column tiles (-10..15 %).  The rest run 64-column tiles at two workgroups per CU.
 template <int D, int EXTRA, bool PAGED> struct Shape {
     static constexpr bool DMA = !PAGED && D == 128;
     static constexpr bool LEAN = DMA && EXTRA == 0;
     static constexpr int BNT = LEAN ? 32 : 64;     // K columns per step
-    static constexpr int WAVES = LEAN ? 3 : 2;     // waves per SIMD
+    static constexpr int WAVES = (LEAN || (D == 64 && EXTRA != 1)) ? 3 : 2;     // waves per SIMD
 };
 
 template <typename T, int D, int EXTRA, bool PAGED>
@@ -326,7 +327,7 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
     typedef Tile<D> TL;
     typedef Shape<D, EXTRA, PAGED> SH;
     constexpr int BNT = SH::BNT;
-    constexpr bool LEAN = SH::LEAN;
+    constexpr bool LEAN = SH::WAVES == 3;          // register-tight variants read V fragments right before use
     constexpr int NBLK4 = BNT / 4;                 // 4-row blocks per tile
     typedef typename MM<T>::v8 v8;
     const hstu_fwd_params& p = a.p;
