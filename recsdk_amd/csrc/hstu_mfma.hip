@@ -473,6 +473,36 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                     __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, LDS_PTR(void, dst + blk * KBLK), 16, ldK + so, 0, 0, 0);
                     __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, LDS_PTR(void, dst + NBLK4 * KBLK + blk * VBLK), 16, ldV + so, 0, 0, 0);
                 }
+            } else if (PAGED && p.page_size % BNT == 0 && k0 + BNT <= s.hist_k) {
+                // the whole tile lies in one page of the history (pages hold a multiple of the tile's columns and the
+                // history starts at column 0): one page lookup for the tile, rows at a fixed stride
+                const int ps = p.page_size;
+                const int pidx = min(k0 / ps, MAXP - 1);
+                const int64_t page = __builtin_amdgcn_readfirstlane(lds_pid[pidx]);
+                const bool fp8 = p.cache_dtype == HSTU_FP8_E4M3;
+                const unsigned esz = fp8 ? 1u : (unsigned)sizeof(T);
+                const unsigned plane = (unsigned)ps * p.heads_k * D;   // elements of the K (or V) half of a page
+                const unsigned rowb = (unsigned)p.heads_k * D * esz;   // bytes between consecutive rows of a page
+                const char* kb = reinterpret_cast<const char*>(p.kv_cache) + (page * (int64_t)(2u * plane) + (unsigned)(((k0 % ps) * p.heads_k + hk) * D)) * esz;
+                const char* vb = kb + (size_t)plane * esz;
+                const float ks = fp8 ? lds_psc[2 * pidx] : 1.f, vs = fp8 ? lds_psc[2 * pidx + 1] : 1.f;
+                fp8mask = fp8 ? (1u << TL::NCH) - 1u : 0u;
+#pragma unroll
+                for (int i = 0; i < TL::NCH; i++) {
+                    const int c = tid + NT * i;
+                    const int row = c / (D / 8), cc = c % (D / 8);
+                    const unsigned off = row * rowb + cc * (fp8 ? 8u : 16u);
+                    if (fp8) {
+                        const u32x2 kr = *reinterpret_cast<const u32x2*>(kb + off), vr = *reinterpret_cast<const u32x2*>(vb + off);
+                        kreg[i] = (u32x4){kr[0], kr[1], 0u, 0u};
+                        vreg[i] = (u32x4){vr[0], vr[1], 0u, 0u};
+                    } else {
+                        kreg[i] = *reinterpret_cast<const u32x4*>(kb + off);
+                        vreg[i] = *reinterpret_cast<const u32x4*>(vb + off);
+                    }
+                    kscale[i] = ks;
+                    vscale[i] = vs;
+                }
             } else {
 #pragma unroll
                 for (int i = 0; i < TL::NCH; i++) {
