@@ -195,3 +195,45 @@ def test_time_bucket_bounds_reproduce_the_reference_formula():
     got = torch.bucketize(d.to(torch.float32), b[1:-1], right=True)
     assert torch.equal(want, got)
     assert want.max() == 128 and want.min() == 0
+
+
+def test_header_is_plain_c_and_links(tmp_path):
+    """The boundary header compiles as C99 (no C++-isms) and a C program can call the library through it."""
+    import os
+    import shutil
+    import subprocess
+    from recsdk_amd import _build
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no gcc")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    src = tmp_path / "abi.c"
+    src.write_text(r'''
+#include <stdio.h>
+#include <string.h>
+#include <dlfcn.h>
+#include "hstu_hip.h"
+int main(int argc, char** argv) {
+    void* h = dlopen(argv[1], RTLD_NOW | RTLD_GLOBAL);
+    if (!h) { printf("dlopen: %s\n", dlerror()); return 2; }
+    int (*ver)(void) = (int (*)(void))dlsym(h, "hstu_hip_abi_version");
+    int (*wsz)(const hstu_fwd_params*, uint64_t*) = (int (*)(const hstu_fwd_params*, uint64_t*))dlsym(h, "hstu_hip_jagged_forward_get_workspace_size");
+    const char* (*err)(void) = (const char* (*)(void))dlsym(h, "hstu_hip_last_error");
+    if (!ver || !wsz || !err) return 3;
+    hstu_fwd_params p;
+    memset(&p, 0, sizeof p);
+    p.struct_size = 8;                       /* wrong on purpose */
+    uint64_t n = 0;
+    int rc = wsz(&p, &n);
+    printf("%d %d %d %s\n", ver(), (int)sizeof(hstu_fwd_params), rc, err());
+    return 0;
+}
+''')
+    exe = tmp_path / "abi"
+    subprocess.run([gcc, "-std=c99", "-Wall", "-Werror", "-I", os.path.join(root, "include"), str(src), "-o", str(exe), "-ldl"],
+                   check=True)
+    _capi.lib()   # make sure the library exists; its HIP runtime dependency resolves through torch's copy
+    import torch
+    env = dict(os.environ, LD_LIBRARY_PATH=os.path.join(os.path.dirname(torch.__file__), "lib") + ":/opt/rocm/lib:" + os.environ.get("LD_LIBRARY_PATH", ""))
+    out = subprocess.run([str(exe), _build.hip_lib_path()], check=True, capture_output=True, text=True, env=env).stdout.split(None, 3)
+    assert out[0] == "1" and int(out[1]) == C.sizeof(_capi.HstuFwdParams) and out[2] == "-1" and "size mismatch" in out[3]
