@@ -213,7 +213,7 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
     __shared__ unsigned char s_key[HSTU_MAX_BATCH];
     __shared__ unsigned char s_sweep[HSTU_MAX_BATCH];
     __shared__ unsigned s_hist[256], s_base[256];
-    __shared__ unsigned s_val[SCHED_NT], s_scan[SCHED_NT];
+    __shared__ unsigned s_val[SCHED_NT], s_scan[SCHED_NT], s_gpos[SCHED_NT];
     __shared__ unsigned s_cbase[16], s_ovf;
     __shared__ int s_geo[7][HSTU_MAX_BATCH];              // q_start, lq, k_start, lk, ctx, tgt, first page entry
     const int tid = threadIdx.x;
@@ -221,6 +221,12 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
     unsigned* list = ws + WS_HEADER;
     unsigned* ovf = list + REC * 8 * (size_t)d.cap;
 
+#ifdef HSTU_SCHED_TIMING
+    unsigned long long ts0 = __builtin_amdgcn_s_memrealtime(), ts1 = 0, ts2 = 0, ts3 = 0, ts4 = 0;
+#define SST(x) x = __builtin_amdgcn_s_memrealtime()
+#else
+#define SST(x)
+#endif
     for (size_t i = tid; i < 8 * (size_t)d.cap; i += nthr) list[REC * i] = ITEM_EMPTY;
     if (tid < 256) s_hist[tid] = 0;
     if (tid < 16) s_cbase[tid] = 0;
@@ -239,20 +245,36 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
         atomicAdd(&s_hist[key], 1u);
     }
     __syncthreads();
-    // exclusive scan of the 256 key counts (Hillis-Steele in LDS)
-    if (tid < 256) s_base[tid] = s_hist[tid];
-    __syncthreads();
-    for (int off = 1; off < 256; off <<= 1) {
-        const unsigned add = (tid < 256 && tid >= off) ? s_base[tid - off] : 0u;
+    SST(ts1);
+    if (p.batch <= 32) {
+        // small batch: rank by counting (ties by batch index, so the order is reproducible), one barrier
+        if (tid < p.batch) {
+            const unsigned mine = s_key[tid];
+            unsigned rank = 0;
+            for (int i = 0; i < p.batch; i++) {
+                const unsigned k = s_key[i];
+                rank += (k < mine) || (k == mine && i < tid);
+            }
+            s_order[rank] = (unsigned short)tid;
+        }
         __syncthreads();
-        if (tid < 256) s_base[tid] += add;
+    } else {
+        // exclusive scan of the 256 key counts (Hillis-Steele in LDS)
+        if (tid < 256) s_base[tid] = s_hist[tid];
+        __syncthreads();
+        for (int off = 1; off < 256; off <<= 1) {
+            const unsigned add = (tid < 256 && tid >= off) ? s_base[tid - off] : 0u;
+            __syncthreads();
+            if (tid < 256) s_base[tid] += add;
+            __syncthreads();
+        }
+        if (tid < 256) s_base[tid] -= s_hist[tid];
+        __syncthreads();
+        for (int b = tid; b < p.batch; b += nthr) s_order[atomicAdd(&s_base[s_key[b]], 1u)] = (unsigned short)b;
         __syncthreads();
     }
-    if (tid < 256) s_base[tid] -= s_hist[tid];
-    __syncthreads();
-    for (int b = tid; b < p.batch; b += nthr) s_order[atomicAdd(&s_base[s_key[b]], 1u)] = (unsigned short)b;
-    __syncthreads();
 
+    SST(ts2);
     // groups r = rank * heads + head; exclusive prefix of the tile counts inside each XCD's list.  A chunk of
     // 1024 consecutive groups is scanned with stride 16 (one scan per residue class r % 16); XCD x owns the
     // classes x and 15 - x, class x first.
@@ -275,20 +297,34 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
         const int j = tid & 15, tp = (tid & ~15) | (15 - j);
         unsigned pos = s_cbase[j] + s_cbase[15 - j] + (s_scan[tid] - v);
         pos += j < 8 ? s_scan[tp] - s_val[tp] : s_scan[tp];
-        const int x = xcd_of_group(r);
-        for (unsigned i = 0; i < v; i++) {
-            const unsigned tile = (v - 1 - i) / ns, part = i % ns;
-            const unsigned item = (unsigned)b | h << 12 | tile << 16 | ((i < ns && s_sweep[b]) ? 1u << 24 : 0u) | part << 25 | ns << 28;
-            unsigned* rec = pos + i < d.cap ? list + REC * (8 * (size_t)(pos + i) + x) : ovf + REC * (size_t)atomicAdd(&s_ovf, 1u);
-            const u32x4 lo = {item, (unsigned)s_geo[0][b], (unsigned)s_geo[1][b], (unsigned)s_geo[2][b]};
-            const u32x4 hi = {(unsigned)s_geo[3][b], (unsigned)s_geo[4][b], (unsigned)s_geo[5][b], (unsigned)s_geo[6][b]};
-            *reinterpret_cast<u32x4*>(rec) = lo;
-            *reinterpret_cast<u32x4*>(rec + 4) = hi;
+        // the records of a group are written by `sub` threads side by side (a group has up to 160 * 4 of them)
+        s_gpos[tid] = pos;
+        __syncthreads();
+        const unsigned gcount = min((unsigned)nthr, G - c0);
+        unsigned sub = 1;
+        while (sub * 2 * gcount <= (unsigned)nthr) sub *= 2;
+        const unsigned gi = tid / sub, first = tid - gi * sub;
+        if (gi < gcount) {
+            const unsigned gr = c0 + gi, grank = gr / H, gh = gr - grank * H;
+            const int gb = (int)s_order[grank];
+            const unsigned gv = s_val[gi], gpos = s_gpos[gi];
+            const int x = xcd_of_group(gr);
+            const u32x4 hi = {(unsigned)s_geo[3][gb], (unsigned)s_geo[4][gb], (unsigned)s_geo[5][gb], (unsigned)s_geo[6][gb]};
+            u32x4 lo = {0u, (unsigned)s_geo[0][gb], (unsigned)s_geo[1][gb], (unsigned)s_geo[2][gb]};
+            const bool sw = s_sweep[gb];
+            for (unsigned i = first; i < gv; i += sub) {
+                const unsigned tile = (gv - 1 - i) / ns, part = i % ns;
+                lo[0] = (unsigned)gb | gh << 12 | tile << 16 | ((i < ns && sw) ? 1u << 24 : 0u) | part << 25 | ns << 28;
+                unsigned* rec = gpos + i < d.cap ? list + REC * (8 * (size_t)(gpos + i) + x) : ovf + REC * (size_t)atomicAdd(&s_ovf, 1u);
+                *reinterpret_cast<u32x4*>(rec) = lo;
+                *reinterpret_cast<u32x4*>(rec + 4) = hi;
+            }
         }
         __syncthreads();
         if (tid < 16) s_cbase[tid] += s_scan[nthr - 16 + tid];
         __syncthreads();
     }
+    SST(ts3);
     // items that did not fit their XCD's list move to the free slots at the end of the other lists
     const unsigned novf = s_ovf;
     for (unsigned i = tid; i < novf; i += nthr) {
@@ -305,6 +341,10 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
         }
     }
     if (tid == 0) ws[0] = novf;
+#ifdef HSTU_SCHED_TIMING
+    SST(ts4);
+    if (tid == 0) { ws[2] = (unsigned)(ts1 - ts0); ws[3] = (unsigned)(ts2 - ts1); ws[4] = (unsigned)(ts3 - ts2); ws[5] = (unsigned)(ts4 - ts3); }
+#endif
 }
 
 // EXTRA: 0 = no bias / built-in mask only, 1 = dense bias and/or custom mask (tables, if any, gathered from
@@ -809,7 +849,7 @@ static hipError_t launch_td(const KArgs& a, unsigned* ws, hipStream_t stream) {
     else if (p.pos_table) extra = 2;
     const bool paged = a.op == OP_PAGED;
     const int groups = p.batch * p.heads_q;
-    const int sched_threads = groups <= 256 ? 256 : (groups <= 512 ? 512 : SCHED_NT);
+    const int sched_threads = groups <= 256 ? 256 : (groups <= 512 ? 512 : SCHED_NT);   // spare threads write a group's records side by side
     hipError_t e = hipSuccess;
     if (!(p.flags & HSTU_FLAG_REUSE_WORKSPACE)) {
         hipLaunchKernelGGL(hstu_schedule_kernel, dim3(1), dim3(sched_threads), 0, stream, a, d, ws);
