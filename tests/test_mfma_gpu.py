@@ -242,3 +242,23 @@ def test_split_k_ranges(d, dtype):
     cfg["num_target"] = torch.tensor([40, 128, 0])
     cfg["target_group_size"] = 1
     _check(cfg, dtype, f"split-K delta-q d={d}")
+
+
+def test_limits_longest_sequence_and_most_groups():
+    """The reference's limits: one sequence of 20480 rows (160 Q tiles, 640 K tiles) and 2048 sequences x 16 heads
+    (32768 groups: 32 chunks of the schedule kernel's scan).  Cross-checked against the plain-FMA kernel."""
+    say("limits")
+    dtype = torch.bfloat16
+    cfg, _ = _jag(51, [20480], 1, 1, 128, 128, dtype)
+    out, name = T.run_capi(cfg)
+    assert name.startswith("mfma_"), name
+    gen, _ = T.run_capi(cfg, flags=FORCE_GENERIC)
+    T.assert_parity(out, gen.float(), dtype, what="L=20480 vs generic kernel")
+    g = torch.Generator().manual_seed(7)
+    lens = torch.randint(0, 4, (2048,), generator=g).tolist()
+    lens[1000] = 130
+    cfg, _ = _jag(52, lens, 16, 16, 64, 64, dtype)
+    out, name = T.run_capi(cfg)
+    assert name.startswith("mfma_"), name
+    gen, _ = T.run_capi(cfg, flags=FORCE_GENERIC)
+    T.assert_parity(out, gen.float(), dtype, what="2048 x 16 groups vs generic kernel")
