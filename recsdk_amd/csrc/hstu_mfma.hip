@@ -155,7 +155,8 @@ __device__ __forceinline__ int classify_block(const Seq& s, int tgs, int r0, int
 //   * workgroup i runs on XCD i % 8 and takes entry i / 8 of that XCD's list: record i
 //   * items beyond a list's capacity are parked in an overflow list and then moved to the free slots at the end
 //     of the other lists
-// Layout of the workspace (uint32): [0] number of items that were moved, from word 16 the 8*cap records of the
+// Layout of the workspace (uint32): [0] number of items that were moved, [2..3] rows the sequences own (int64),
+// from word 16 the 8*cap records of the
 // interleaved lists, then the parking area of the overflow list.  The main kernel only reads it.
 constexpr unsigned ITEM_EMPTY = 0xffffffffu;
 constexpr int SCHED_NT = 1024;
@@ -340,12 +341,28 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
             k -= free;
         }
     }
-    if (tid == 0) ws[0] = novf;
+    if (tid == 0) {
+        ws[0] = novf;
+        // rows the sequences own (the main kernel zero-fills the rows behind them)
+        const int64_t owned = p.seq_offset_q ? ld_idx(p.seq_offset_q, p.batch, p.index_type == HSTU_I64) : p.total_q;
+        *reinterpret_cast<int64_t*>(ws + 2) = owned;
+    }
 #ifdef HSTU_SCHED_TIMING
     SST(ts4);
-    if (tid == 0) { ws[2] = (unsigned)(ts1 - ts0); ws[3] = (unsigned)(ts2 - ts1); ws[4] = (unsigned)(ts3 - ts2); ws[5] = (unsigned)(ts4 - ts3); }
+    if (tid == 0) { ws[8] = (unsigned)(ts1 - ts0); ws[9] = (unsigned)(ts2 - ts1); ws[10] = (unsigned)(ts3 - ts2); ws[11] = (unsigned)(ts4 - ts3); }
 #endif
 }
+
+#ifdef HSTU_ITEM_TIMING
+// Development aid (not part of the normal build): per workgroup of the main kernel {start, time to the first tile in
+// LDS, time to the end, hardware id, K tiles}, in 10 ns ticks of the constant clock.
+__device__ unsigned g_item_times[8 * 32768];
+}  // namespace hstu
+extern "C" int hstu_hip_debug_item_times(void* dst, size_t bytes) {
+    return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(hstu::g_item_times), bytes);
+}
+namespace hstu {
+#endif
 
 // EXTRA: 0 = no bias / built-in mask only, 1 = dense bias and/or custom mask (tables, if any, gathered from
 // global memory), 2 / 3 / 4 = bias tables only, gathered from LDS-resident copies: position table / time table /
@@ -368,6 +385,10 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
     typedef Shape<D, EXTRA, PAGED> SH;
     constexpr int BNT = SH::BNT;
     constexpr bool LEAN = SH::WAVES == 3;          // register-tight variants read V fragments right before use
+#ifndef HSTU_PARK_OUT
+#define HSTU_PARK_OUT LEAN
+#endif
+    constexpr bool PARK_OUT = HSTU_PARK_OUT;
     constexpr int NBLK4 = BNT / 4;                 // 4-row blocks per tile
     typedef typename MM<T>::v8 v8;
     const hstu_fwd_params& p = a.p;
@@ -400,6 +421,11 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave index, kept in a scalar register
     const int g = lane >> 5, l32 = lane & 31;
 
+#ifdef HSTU_ITEM_TIMING
+    const unsigned long long it0 = __builtin_amdgcn_s_memrealtime();
+    unsigned long long it1 = it0, it_loop = it0;
+    int it_ntk = 0;
+#endif
     // blockIdx -> record of the work list (see above)
     unsigned rw[REC];
     {
@@ -407,6 +433,9 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
 #pragma unroll
         for (int i = 0; i < REC; i++) rw[i] = rec[i];
     }
+    // rows the sequences own, for the zero fill at the end: requested here so that nothing waits for it there
+    int64_t owned_rows = *reinterpret_cast<const int64_t*>(ws + 2);
+    asm volatile("" : "+s"(owned_rows));
     const unsigned item = rw[0];
     const bool active = item != ITEM_EMPTY;
     const int b = active ? (int)(item & 0xfff) : 0, h = active ? (int)((item >> 12) & 0xf) : 0;
@@ -622,6 +651,10 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
         const int kt0 = part * per, kt1 = min(ntk, kt0 + per);
         if (kt0 < kt1) fetch(kt0, lds0);
         stash(kt0, lds0);
+#ifdef HSTU_ITEM_TIMING
+        it1 = __builtin_amdgcn_s_memrealtime();
+        it_ntk += kt1 - kt0;
+#endif
 
         auto iteration = [&](int kt, const char* cur, char* nxt) __attribute__((always_inline)) {
             const int buf = kt & 1;
@@ -758,8 +791,40 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
             if (kt + 1 < kt1) iteration(kt + 1, lds1, lds0);
         }
 
+#ifdef HSTU_ITEM_TIMING
+        it_loop = __builtin_amdgcn_s_memrealtime();
+#endif
         // ---- epilogue: O^T accumulator register r of block db holds d = 32*db + 8*(r/4) + 4*g + r%4 for row qi
-        if (qvalid && nsplit == 1) {
+        if (PARK_OUT && nsplit == 1) {
+            // Through LDS, so that the stores are whole rows: each wave parks its 32 x D tile in the K/V stage that
+            // is free now (every wave is past the last barrier of the K loop), row stride 2*D + 8 bytes, and writes
+            // it out 16 bytes per lane, 64 / (D / 8) rows per instruction.
+            constexpr int ORS = 2 * D + 8;
+            static_assert(2 * 32 * ORS <= STAGE_BYTES, "two waves park their output tile in one stage");
+            char* park = ((w & 2) ? lds1 : lds0) + (w & 1) * (32 * ORS);
+#pragma unroll
+            for (int db = 0; db < D / 32; db++) {
+#pragma unroll
+                for (int rr = 0; rr < 4; rr++) {
+                    u32x2 o;
+                    o[0] = MM<T>::pack2(oacc[db][4 * rr] * a.out_scale, oacc[db][4 * rr + 1] * a.out_scale);
+                    o[1] = MM<T>::pack2(oacc[db][4 * rr + 2] * a.out_scale, oacc[db][4 * rr + 3] * a.out_scale);
+                    *reinterpret_cast<u32x2*>(park + l32 * ORS + (32 * db + 8 * rr + 4 * g) * 2) = o;
+                }
+            }
+            __builtin_amdgcn_wave_barrier();
+            constexpr int CPR = D / 8, RPI = 64 / CPR;   // 16-byte chunks per row, rows per instruction
+            int elane = lane;
+            asm volatile("" : "+v"(elane));   // keeps the address arithmetic below out of the K loop's live ranges
+            const int orow = elane / CPR, ochunk = elane % CPR;
+#pragma unroll
+            for (int i = 0; i < 32 / RPI; i++) {
+                const int row = RPI * i + orow;
+                const u32x4 x = *reinterpret_cast<const u32x4*>(park + row * ORS + ochunk * 16);
+                if (r0 + row < s.lq)
+                    *reinterpret_cast<u32x4*>(obase + ((s.q_start + r0 + row) * p.heads_q + h) * (int64_t)D + ochunk * 8) = x;
+            }
+        } else if (qvalid && nsplit == 1) {
             T* op = obase + ((s.q_start + qi) * p.heads_q + h) * (int64_t)D + 4 * g;
 #pragma unroll
             for (int db = 0; db < D / 32; db++) {
@@ -783,19 +848,25 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                 }
             }
         }
-        __syncthreads();
         if (!sweep) break;
+        __syncthreads();   // the next tile's loads overwrite the stages the output tiles were parked in
     }
 
+#ifdef HSTU_ITEM_TIMING
+    if (tid == 0 && blockIdx.x < 32768) {
+        const unsigned long long it2 = __builtin_amdgcn_s_memrealtime();
+        unsigned* o = g_item_times + 8 * blockIdx.x;
+        o[0] = (unsigned)it0; o[1] = (unsigned)(it1 - it0); o[2] = (unsigned)(it2 - it0);
+        o[3] = __builtin_amdgcn_s_getreg((31 << 11) | 4);     // HW_ID: CU 11:8, SH 12, SE 14:13
+        o[4] = (unsigned)it_ntk; o[5] = item; o[7] = (unsigned)(it_loop - it0);
+        o[6] = __builtin_amdgcn_s_getreg((3 << 11) | 20);     // XCC_ID
+    }
+#endif
     // rows past the last offset are zero (the reference zero-fills its output: hstu_jagged.cpp:56-59)
-    if (p.seq_offset_q) {
-        const int is64 = p.index_type == HSTU_I64;
-        const int64_t tail = ld_idx(p.seq_offset_q, p.batch, is64);
-        if (tail < p.total_q) {
-            const int64_t n = (p.total_q - tail) * p.heads_q * (int64_t)D;
-            T* o = obase + tail * p.heads_q * (int64_t)D;
-            for (int64_t e = (int64_t)blockIdx.x * NT + tid; e < n; e += (int64_t)gridDim.x * NT) o[e] = (T)0.f;
-        }
+    if (owned_rows < p.total_q) {
+        const int64_t n = (p.total_q - owned_rows) * p.heads_q * (int64_t)D;
+        T* o = obase + owned_rows * p.heads_q * (int64_t)D;
+        for (int64_t e = (int64_t)blockIdx.x * NT + tid; e < n; e += (int64_t)gridDim.x * NT) o[e] = (T)0.f;
     }
 }
 
