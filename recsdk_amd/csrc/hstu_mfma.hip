@@ -214,10 +214,11 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
     __shared__ unsigned char s_key[HSTU_MAX_BATCH];
     __shared__ unsigned char s_sweep[HSTU_MAX_BATCH];
     __shared__ unsigned s_hist[256], s_base[256];
-    __shared__ unsigned s_val[SCHED_NT], s_scan[SCHED_NT], s_gpos[SCHED_NT];
-    __shared__ unsigned s_cbase[16], s_ovf;
+    __shared__ unsigned s_val[SCHED_NT], s_gpos[SCHED_NT];
+    __shared__ unsigned s_wtot[(SCHED_NT / 64) * 16];   // per wave: entries of each residue class (group index % 16)
+    __shared__ unsigned s_w4[4], s_len[8], s_ovf;
     __shared__ int s_geo[7][HSTU_MAX_BATCH];              // q_start, lq, k_start, lk, ctx, tgt, first page entry
-    const int tid = threadIdx.x;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int nthr = blockDim.x;   // 256, 512 or 1024: small batches run with fewer waves (cheaper barriers)
     unsigned* list = ws + WS_HEADER;
     unsigned* ovf = list + REC * 8 * (size_t)d.cap;
@@ -230,7 +231,6 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
 #endif
     for (size_t i = tid; i < 8 * (size_t)d.cap; i += nthr) list[REC * i] = ITEM_EMPTY;
     if (tid < 256) s_hist[tid] = 0;
-    if (tid < 16) s_cbase[tid] = 0;
     if (tid == 0) s_ovf = 0;
     __syncthreads();
     // sort key: number of 64-column K tiles (work of a Q tile grows with it), longest first
@@ -260,16 +260,24 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
         }
         __syncthreads();
     } else {
-        // exclusive scan of the 256 key counts (Hillis-Steele in LDS)
-        if (tid < 256) s_base[tid] = s_hist[tid];
-        __syncthreads();
-        for (int off = 1; off < 256; off <<= 1) {
-            const unsigned add = (tid < 256 && tid >= off) ? s_base[tid - off] : 0u;
-            __syncthreads();
-            if (tid < 256) s_base[tid] += add;
-            __syncthreads();
+        // exclusive scan of the 256 key counts: shuffles inside each of the first four waves, then the waves' totals
+        unsigned hcount = 0, hincl = 0;
+        if (tid < 256) {
+            hcount = s_hist[tid];
+            hincl = hcount;
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) {
+                const unsigned t = __shfl_up(hincl, off, 64);
+                if (lane >= off) hincl += t;
+            }
+            if (lane == 63) s_w4[wave] = hincl;
         }
-        if (tid < 256) s_base[tid] -= s_hist[tid];
+        __syncthreads();
+        if (tid < 256) {
+            unsigned before = 0;
+            for (int ww = 0; ww < wave; ww++) before += s_w4[ww];
+            s_base[tid] = before + hincl - hcount;
+        }
         __syncthreads();
         for (int b = tid; b < p.batch; b += nthr) s_order[atomicAdd(&s_base[s_key[b]], 1u)] = (unsigned short)b;
         __syncthreads();
@@ -280,26 +288,37 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
     // 1024 consecutive groups is scanned with stride 16 (one scan per residue class r % 16); XCD x owns the
     // classes x and 15 - x, class x first.
     const unsigned H = (unsigned)p.heads_q, G = (unsigned)p.batch * H;
+    const int j = tid & 15, nwaves = nthr >> 6;
+    unsigned cb = 0;   // entries of the classes j and 15 - j in the chunks before this one
     for (unsigned c0 = 0; c0 < G; c0 += nthr) {
         const unsigned r = c0 + tid;
         const unsigned rank = r / H, h = r - rank * H;
         const int b = r < G ? (int)s_order[rank] : 0;
         const unsigned ns = (unsigned)d.nsplit;
         const unsigned v = r < G ? s_tiles[b] * ns : 0u;   // entries of this group: (tile, K range) pairs
-        s_val[tid] = v;
-        s_scan[tid] = v;
+        // inclusive scan with stride 16: two shuffles inside the wave, then the totals of the waves before
+        unsigned incl = v;
+        unsigned t = __shfl_up(incl, 16, 64);
+        if (lane >= 16) incl += t;
+        t = __shfl_up(incl, 32, 64);
+        if (lane >= 32) incl += t;
+        if (lane >= 48) s_wtot[wave * 16 + (lane - 48)] = incl;
         __syncthreads();
-        for (int off = 16; off < nthr; off <<= 1) {
-            const unsigned add = tid >= off ? s_scan[tid - off] : 0u;
-            __syncthreads();
-            s_scan[tid] += add;
-            __syncthreads();
+        unsigned before = 0, chunk = 0;
+        for (int ww = 0; ww < nwaves; ww++) {
+            const unsigned mine = s_wtot[ww * 16 + j], other = s_wtot[ww * 16 + 15 - j];
+            if (ww < wave) before += mine;
+            chunk += mine + other;
         }
-        const int j = tid & 15, tp = (tid & ~15) | (15 - j);
-        unsigned pos = s_cbase[j] + s_cbase[15 - j] + (s_scan[tid] - v);
-        pos += j < 8 ? s_scan[tp] - s_val[tp] : s_scan[tp];
+        incl += before;
+        const int tp = (lane & ~15) | (15 - j);
+        const unsigned pincl = __shfl(incl, tp, 64), pv = __shfl(v, tp, 64);
+        unsigned pos = cb + (incl - v);
+        pos += j < 8 ? pincl - pv : pincl;
+        cb += chunk;
         // the records of a group are written by `sub` threads side by side (a group has up to 160 * 4 of them)
         s_gpos[tid] = pos;
+        s_val[tid] = v;
         __syncthreads();
         const unsigned gcount = min((unsigned)nthr, G - c0);
         unsigned sub = 1;
@@ -321,17 +340,16 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
                 *reinterpret_cast<u32x4*>(rec + 4) = hi;
             }
         }
-        __syncthreads();
-        if (tid < 16) s_cbase[tid] += s_scan[nthr - 16 + tid];
-        __syncthreads();
     }
+    if (tid < 8) s_len[tid] = cb;   // entries of list x = classes x and 15 - x
+    __syncthreads();
     SST(ts3);
     // items that did not fit their XCD's list move to the free slots at the end of the other lists
     const unsigned novf = s_ovf;
     for (unsigned i = tid; i < novf; i += nthr) {
         unsigned k = i;
         for (int x = 0; x < 8; x++) {
-            const unsigned len = min(s_cbase[x] + s_cbase[15 - x], d.cap), free = d.cap - len;
+            const unsigned len = min(s_len[x], d.cap), free = d.cap - len;
             if (k < free) {
                 unsigned* rec = list + REC * (8 * (size_t)(len + k) + x);
                 *reinterpret_cast<u32x4*>(rec) = *reinterpret_cast<const u32x4*>(ovf + REC * (size_t)i);
