@@ -744,21 +744,25 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                     if (EXTRA == 1) pv *= mval;
                     pf[r] = pv;
                 }
-                if (cls == BLK_CAUSAL) {
-                    const int lim = qi + s.delta - (c0 + 4 * g);  // visible iff 8*(r/4) + r%4 <= lim
+                // The built-in mask: the two-per-CU variants zero the fp32 values; the register-tight ones mask the packed
+                // pairs instead (fewer operations, and a fully visible block then needs no copies at the join)
+                if (!LEAN) {
+                    if (cls == BLK_CAUSAL) {
+                        const int lim = qi + s.delta - (c0 + 4 * g);  // visible iff 8*(r/4) + r%4 <= lim
 #pragma unroll
-                    for (int r = 0; r < 16; r++) pf[r] = (8 * (r >> 2) + (r & 3) <= lim) ? pf[r] : 0.f;
-                } else if (cls == BLK_PRED) {
-                    // branch-free form of builtin_visible(); j runs over this lane's 16 keys
-                    const bool ctx_row = s.ctx > 0 && qi < s.ctx;
-                    const bool tgt_row = tgs > 0 && s.tgt > 0 && qi >= s.hist_q;
-                    const int left = tgt_row ? s.hist_k + ((qi - s.hist_q) / tgs) * tgs : 0;  // first visible target column
-                    const int jmax = qi + s.delta;
+                        for (int r = 0; r < 16; r++) pf[r] = (8 * (r >> 2) + (r & 3) <= lim) ? pf[r] : 0.f;
+                    } else if (cls == BLK_PRED) {
+                        // branch-free form of builtin_visible(); j runs over this lane's 16 keys
+                        const bool ctx_row = s.ctx > 0 && qi < s.ctx;
+                        const bool tgt_row = tgs > 0 && s.tgt > 0 && qi >= s.hist_q;
+                        const int left = tgt_row ? s.hist_k + ((qi - s.hist_q) / tgs) * tgs : 0;  // first visible target column
+                        const int jmax = qi + s.delta;
 #pragma unroll
-                    for (int r = 0; r < 16; r++) {
-                        const int j = c0 + 8 * (r >> 2) + 4 * g + (r & 3);
-                        const bool vis = (ctx_row & (j < s.hist_k)) | ((j <= jmax) & !(tgt_row & (j >= s.hist_k) & (j < left)));
-                        pf[r] = vis ? pf[r] : 0.f;
+                        for (int r = 0; r < 16; r++) {
+                            const int j = c0 + 8 * (r >> 2) + 4 * g + (r & 3);
+                            const bool vis = (ctx_row & (j < s.hist_k)) | ((j <= jmax) & !(tgt_row & (j >= s.hist_k) & (j < left)));
+                            pf[r] = vis ? pf[r] : 0.f;
+                        }
                     }
                 }
                 // ---- O^T += V^T P^T : two 16-key steps per block
@@ -767,6 +771,33 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                 for (int x = 0; x < 4; x++) {
                     pk0[x] = MM<T>::pack2(pf[2 * x], pf[2 * x + 1]);
                     pk1[x] = MM<T>::pack2(pf[8 + 2 * x], pf[8 + 2 * x + 1]);
+                }
+                if (LEAN) {
+                    // pair x of the first step holds this lane's key offsets 8*(x/2) + 2*(x%2) and + 1, the second step 16 more
+                    if (cls == BLK_CAUSAL) {
+                        const int lim = qi + s.delta - (c0 + 4 * g);  // key offset o of this lane is visible iff o <= lim
+#pragma unroll
+                        for (int x = 0; x < 4; x++) {
+                            const int o = 8 * (x >> 1) + 2 * (x & 1);
+                            pk0[x] &= o + 1 <= lim ? 0xffffffffu : (o <= lim ? 0xffffu : 0u);
+                            pk1[x] &= o + 17 <= lim ? 0xffffffffu : (o + 16 <= lim ? 0xffffu : 0u);
+                        }
+                    } else if (cls == BLK_PRED) {
+                        // branch-free form of builtin_visible() for this lane's 16 keys
+                        const bool ctx_row = s.ctx > 0 && qi < s.ctx;
+                        const bool tgt_row = tgs > 0 && s.tgt > 0 && qi >= s.hist_q;
+                        const int left = tgt_row ? s.hist_k + ((qi - s.hist_q) / tgs) * tgs : 0;  // first visible target column
+                        const int jmax = qi + s.delta;
+                        auto vis = [&](int r) __attribute__((always_inline)) -> bool {
+                            const int j = c0 + 8 * (r >> 2) + 4 * g + (r & 3);
+                            return (ctx_row & (j < s.hist_k)) | ((j <= jmax) & !(tgt_row & (j >= s.hist_k) & (j < left)));
+                        };
+#pragma unroll
+                        for (int x = 0; x < 4; x++) {
+                            pk0[x] &= (vis(2 * x) ? 0xffffu : 0u) | (vis(2 * x + 1) ? 0xffff0000u : 0u);
+                            pk1[x] &= (vis(8 + 2 * x) ? 0xffffu : 0u) | (vis(9 + 2 * x) ? 0xffff0000u : 0u);
+                        }
+                    }
                 }
                 if (LEAN) {   // fewer live registers: fragments are read right before the step that uses them
                     __builtin_amdgcn_sched_barrier(0);
