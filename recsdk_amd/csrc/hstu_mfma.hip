@@ -149,6 +149,8 @@ __device__ __forceinline__ int classify_block(const Seq& s, int tgs, int r0, int
 //   * one item = one 128-row Q tile of one (sequence, head) (or one of its 2-4 K ranges, see sched_dims): a record
 //     of 8 words -- seq | head << 12 | tile << 16 | sweep << 24 | K range << 25 | ranges << 28, then the sequence's geometry (q_start, lq, k_start, lk, num_context, num_target, first page
 //     entry), so that a workgroup needs one scalar load to know its work
+//   * the first two Q tiles of a long sequence are one item (bits 25..27 of an unsplit item count the further tiles
+//     it covers): they see few K columns and would mostly pay a workgroup's start and end
 //   * sequences are sorted by K length (longest first) and their (sequence, head) groups are dealt to the
 //     8 XCDs in snake order; a group's tiles sit next to each other in its XCD's list, last tile first, so that
 //     the workgroups that share one K/V run at the same time on CUs that share one L2
@@ -212,7 +214,7 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
     __shared__ unsigned short s_tiles[HSTU_MAX_BATCH];    // tiles of a sequence, by batch index
     __shared__ unsigned short s_order[HSTU_MAX_BATCH];    // batch index, by rank
     __shared__ unsigned char s_key[HSTU_MAX_BATCH];
-    __shared__ unsigned char s_sweep[HSTU_MAX_BATCH];
+    __shared__ unsigned char s_sweep[HSTU_MAX_BATCH];     // bit 0: the last item sweeps the tiles behind the attribute; bit 1: tiles 0 and 1 are one item
     __shared__ unsigned s_hist[256], s_base[256];
     __shared__ unsigned s_val[SCHED_NT], s_gpos[SCHED_NT];
     __shared__ unsigned s_wtot[(SCHED_NT / 64) * 16];   // per wave: entries of each residue class (group index % 16)
@@ -239,8 +241,17 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
         s_geo[0][b] = (int)s.q_start; s_geo[1][b] = s.lq; s_geo[2][b] = (int)s.k_start; s_geo[3][b] = s.lk;
         s_geo[4][b] = s.ctx; s_geo[5][b] = s.tgt; s_geo[6][b] = (int)s.page0;
         const int t = (s.lq + BM - 1) / BM;
-        s_tiles[b] = (unsigned short)min(t, d.ntiles_attr);
-        s_sweep[b] = t > d.ntiles_attr;
+        const int nt = min(t, d.ntiles_attr);
+        s_tiles[b] = (unsigned short)nt;
+        // The two first Q tiles of a long sequence see few K columns; as items of their own they mostly pay the start and
+        // end of a workgroup.  They become one item when together they stay under 70 % of the sequence's last tile.
+        bool pair = false;
+        if (d.nsplit == 1 && t == nt && nt >= 3) {
+            const int c0 = (k_extent(a, s, 0, BM) + 63) / 64, c1 = (k_extent(a, s, BM, min(2 * BM, s.lq)) + 63) / 64;
+            const int ctop = (k_extent(a, s, (nt - 1) * BM, s.lq) + 63) / 64;
+            pair = 10 * (c0 + c1) <= 7 * ctop;
+        }
+        s_sweep[b] = (t > d.ntiles_attr ? 1 : 0) | (pair ? 2 : 0);
         const int key = 255 - min(255, (s.lk + BN - 1) / BN);
         s_key[b] = (unsigned char)key;
         atomicAdd(&s_hist[key], 1u);
@@ -295,7 +306,7 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
         const unsigned rank = r / H, h = r - rank * H;
         const int b = r < G ? (int)s_order[rank] : 0;
         const unsigned ns = (unsigned)d.nsplit;
-        const unsigned v = r < G ? s_tiles[b] * ns : 0u;   // entries of this group: (tile, K range) pairs
+        const unsigned v = r < G ? (s_tiles[b] - ((s_sweep[b] >> 1) & 1)) * ns : 0u;   // entries of this group: (tile, K range) pairs
         // inclusive scan with stride 16: two shuffles inside the wave, then the totals of the waves before
         unsigned incl = v;
         unsigned t = __shfl_up(incl, 16, 64);
@@ -331,9 +342,12 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
             const int x = xcd_of_group(gr);
             const u32x4 hi = {(unsigned)s_geo[3][gb], (unsigned)s_geo[4][gb], (unsigned)s_geo[5][gb], (unsigned)s_geo[6][gb]};
             u32x4 lo = {0u, (unsigned)s_geo[0][gb], (unsigned)s_geo[1][gb], (unsigned)s_geo[2][gb]};
-            const bool sw = s_sweep[gb];
+            const bool sw = s_sweep[gb] & 1, pair = s_sweep[gb] & 2;   // pair implies ns == 1
             for (unsigned i = first; i < gv; i += sub) {
-                const unsigned tile = (gv - 1 - i) / ns, part = i % ns;
+                // last tile first; with `pair` the last entry is tile 0 and covers one more tile (the field that numbers the
+                // K ranges of a split tile then holds the count of further tiles)
+                const bool both = pair && i == gv - 1;
+                const unsigned tile = both ? 0u : (gv - 1 - i) / ns + (pair ? 1u : 0u), part = both ? 1u : i % ns;
                 lo[0] = (unsigned)gb | gh << 12 | tile << 16 | ((i < ns && sw) ? 1u << 24 : 0u) | part << 25 | ns << 28;
                 unsigned* rec = gpos + i < d.cap ? list + REC * (8 * (size_t)(gpos + i) + x) : ovf + REC * (size_t)atomicAdd(&s_ovf, 1u);
                 *reinterpret_cast<u32x4*>(rec) = lo;
@@ -459,7 +473,12 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
     const int b = active ? (int)(item & 0xfff) : 0, h = active ? (int)((item >> 12) & 0xf) : 0;
     const int tile0 = (int)((item >> 16) & 0xff);
     const bool sweep = (item >> 24) & 1;   // last tile the max_seq_len_q attribute covers of a sequence that is longer
-    const int part = active ? (int)((item >> 25) & 7) : 0, nsplit = active ? (int)((item >> 28) & 7) : 1;
+    // bits 25..27: K range of the tile when it is split (bits 28..30 = ranges > 1), else further tiles of the sequence that
+    // this item covers after its first one
+    const int nsplit = active ? (int)((item >> 28) & 7) : 1;
+    const int pfield = active ? (int)((item >> 25) & 7) : 0;
+    const int part = nsplit > 1 ? pfield : 0;
+    const int tile_last = sweep ? 0x7fffff : tile0 + (nsplit > 1 ? 0 : pfield);
     const int hk = h / a.head_ratio;
     Seq s;
     s.q_start = active ? (int)rw[1] : 0; s.lq = active ? (int)rw[2] : 0;
@@ -897,7 +916,7 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                 }
             }
         }
-        if (!sweep) break;
+        if (tile >= tile_last) break;
         __syncthreads();   // the next tile's loads overwrite the stages the output tiles were parked in
     }
 
