@@ -988,7 +988,7 @@ static hipError_t launch_td(const KArgs& a, unsigned* ws, hipStream_t stream) {
     else if (p.pos_table) extra = 2;
     const bool paged = a.op == OP_PAGED;
     const int groups = p.batch * p.heads_q;
-    const int sched_threads = groups <= 256 ? 256 : (groups <= 512 ? 512 : SCHED_NT);   // spare threads write a group's records side by side
+    const int sched_threads = groups <= 128 ? 256 : (groups <= 512 ? 512 : SCHED_NT);   // spare threads write a group's records side by side
     hipError_t e = hipSuccess;
     if (!(p.flags & HSTU_FLAG_REUSE_WORKSPACE)) {
         hipLaunchKernelGGL(hstu_schedule_kernel, dim3(1), dim3(sched_threads), 0, stream, a, d, ws);
