@@ -1,5 +1,5 @@
 /*
- * hstu_hip.h -- C ABI of the MI355X (gfx950) HSTU fused attention forward.
+ * hstu_hip.h -- C ABI of the MI355X (gfx950) HSTU fused attention forward (and the jagged backward).
  *
  * out = (SiLU(alpha * (Q K^T + bias)) * silu_scale * mask) V   over packed ("jagged") sequences,
  * no softmax, no materialised score matrix.
@@ -151,6 +151,33 @@ int hstu_hip_paged_forward(const hstu_fwd_params* p, void* workspace, uint64_t w
  * q/k/v are [batch, max_seq_len_q, heads, dim]; seq_offset_* must be NULL */
 int hstu_hip_dense_forward_get_workspace_size(const hstu_fwd_params* p, uint64_t* workspace_bytes);
 int hstu_hip_dense_forward(const hstu_fwd_params* p, void* workspace, uint64_t workspace_bytes, void* stream);
+
+/*
+ * Backward of the jagged op (the .equal and .delta overloads; seq_offset_k == seq_offset_q for .equal).
+ * replaces aclnnHstuJaggedBackwardGetWorkspaceSize / aclnnHstuJaggedBackward (hstu_jagged.cpp:69-138):
+ *     x  = alpha * (Q K^T + bias)        P  = silu(x) * silu_scale * mask
+ *     dS = (dO V^T) * silu_scale * mask * sigmoid(x) * (1 + x * (1 - sigmoid(x))) * alpha
+ *     dQ = dS K     dK = dS^T Q     dV = P^T dO     dBias = dS
+ * (golden: build/presmoke/hstu/hstu_common.py:387-476).  `fwd` holds the arguments of the forward call; its `out`
+ * is not read and may be NULL.  Only what the reference's backward takes is accepted: dense attn_bias (no bias
+ * tables), built-in or custom mask, no paged cache.  P and dS are rounded to the I/O dtype before the second
+ * GEMMs like P in the forward; every gradient element has one producing workgroup and a fixed summation order
+ * (deterministic, no atomics).  With GQA, grad_k / grad_v sum over the query heads of a K/V head.
+ */
+typedef struct hstu_bwd_params {
+    uint32_t struct_size;   /* sizeof(hstu_bwd_params) */
+    uint32_t reserved;
+    hstu_fwd_params fwd;
+    const void* grad_out;   /* [total_q, heads_q, dim_v]   upstream gradient, I/O dtype */
+    void* grad_q;           /* [total_q, heads_q, dim_qk]  every row is written (rows past the last offset: zeros) */
+    void* grad_k;           /* [total_k, heads_k, dim_qk] */
+    void* grad_v;           /* [total_k, heads_k, dim_v] */
+    void* grad_bias;        /* [batch, heads_q, max_seq_len_q, max_seq_len_k] or NULL; required iff fwd.attn_bias;
+                             * written completely (zeros outside the sequences and where the mask is 0) */
+} hstu_bwd_params;
+
+int hstu_hip_jagged_backward_get_workspace_size(const hstu_bwd_params* p, uint64_t* workspace_bytes);
+int hstu_hip_jagged_backward(const hstu_bwd_params* p, void* workspace, uint64_t workspace_bytes, void* stream);
 
 /* replaces aclGetRecentErrMsg() (pytorch_npu_helper.hpp:510-543): message of the last failing call on this thread */
 const char* hstu_hip_last_error(void);

@@ -29,6 +29,8 @@ Definition followed (reference file:line):
 * bias formulas: time buckets -- cust_op/test/relative_attn_bias/torch/utils.py:26-27,99-129;
   Toeplitz relative position -- utils.py:38-51
 
+* backward: explicit gradient formulas of the reference golden -- build/presmoke/hstu/hstu_common.py:387-476
+
 Pinning status (what fixes each function independently of this file's own
 formulas; the checks live in tests/test_oracle_*.py):
 
@@ -42,6 +44,10 @@ formulas; the checks live in tests/test_oracle_*.py):
   repeat_interleave).                                                     PINNED
 * ``hstu_paged_forward``: equivalence with the delta-q jagged op on the
   de-paged K/V.                                                           PINNED
+* ``hstu_jagged_backward``: torch.autograd of ``hstu_jagged_forward`` in
+  float64 (an independent derivation: no gradient formula is shared), central
+  finite differences on tiny inputs, and the GQA sum against explicitly
+  repeated K/V heads (tests/test_oracle_backward.py).                     PINNED
 * ``time_bucket_ids`` / ``rel_pos_bias``: closed forms with the reference's
   constants; integer ids compared exactly against a float64 evaluation away
   from bucket edges and at the documented edge cases.                    PINNED
@@ -263,6 +269,73 @@ def hstu_jagged_forward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, seq_o
     if out_dtype is not None:
         out = out.to(out_dtype)
     return out
+
+
+def hstu_jagged_backward(grad: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                         seq_offset_q: torch.Tensor, seq_offset_k: Optional[torch.Tensor] = None, *,
+                         max_seq_len_q: int, max_seq_len_k: Optional[int] = None, mask_type: int = MASK_TRIL,
+                         mask: Optional[torch.Tensor] = None, attn_bias: Optional[torch.Tensor] = None,
+                         silu_scale: float = 0.0, alpha: float = 1.0,
+                         num_context: Optional[Sequence[int]] = None, num_target: Optional[Sequence[int]] = None,
+                         target_group_size: int = 0, compute_dtype: torch.dtype = torch.float64):
+    """Gradients of ``hstu_jagged_forward`` for an upstream gradient ``grad`` ``[Tq, Nq, Dv]``.
+
+    Restates the reference golden ``hstu_bwd_gold`` (build/presmoke/hstu/hstu_common.py:387-476) per sequence,
+    without the padding to dense tensors and without intermediate rounding:
+
+        x  = alpha * (Q K^T + bias)          P  = silu(x) * silu_scale * mask
+        dS = (dO V^T) * silu_scale * mask * sigmoid(x) * (1 + x * (1 - sigmoid(x))) * alpha
+        dQ = dS K      dK = dS^T Q      dV = P^T dO      dBias = dS
+
+    With GQA the K/V gradients of the query heads that share a K/V head are summed (hstu_common.py:457-463).
+    Returns ``(dq, dk, dv, dbias)`` in ``compute_dtype``; ``dbias`` is ``None`` without ``attn_bias`` and is zero
+    outside the sequences' own ``[:lq, :lk]`` corners (the op allocates it with zeros, hstu_jagged.cpp:121-123).
+    """
+    if seq_offset_k is None:
+        seq_offset_k = seq_offset_q
+    if max_seq_len_k is None:
+        max_seq_len_k = max_seq_len_q
+    cd = compute_dtype
+    nq, nk = q.shape[1], k.shape[1]
+    ratio = nq // nk
+    scale = (1.0 / max_seq_len_q) if silu_scale == 0.0 else silu_scale
+    oq, okk = seq_offset_q.tolist(), seq_offset_k.tolist()
+    nb = len(oq) - 1
+    ctx = [0] * nb if num_context is None else [int(x) for x in num_context]
+    tgt = [0] * nb if num_target is None else [int(x) for x in num_target]
+    dq = torch.zeros(q.shape, dtype=cd)
+    dk = torch.zeros(k.shape, dtype=cd)
+    dv = torch.zeros(v.shape, dtype=cd)
+    dbias = None if attn_bias is None else torch.zeros(attn_bias.shape, dtype=cd)
+    for b in range(nb):
+        lq, lk = int(oq[b + 1] - oq[b]), int(okk[b + 1] - okk[b])
+        if lq == 0 or lk == 0:
+            continue
+        qb = q[oq[b]: oq[b] + lq].to(cd).permute(1, 0, 2)                                   # [Nq, lq, D]
+        gb = grad[oq[b]: oq[b] + lq].to(cd).permute(1, 0, 2)                                # [Nq, lq, Dv]
+        kb = k[okk[b]: okk[b] + lk].to(cd).repeat_interleave(ratio, dim=1).permute(1, 0, 2)  # [Nq, lk, D]
+        vb = v[okk[b]: okk[b] + lk].to(cd).repeat_interleave(ratio, dim=1).permute(1, 0, 2)
+        if mask_type == MASK_TRIL:
+            m = builtin_mask(lq, lk, ctx[b], tgt[b], target_group_size).to(cd)
+        elif mask_type == MASK_CUSTOM:
+            m = mask[b, :, :lq, :lk].to(cd)
+        else:
+            m = torch.ones(lq, lk, dtype=cd)
+        x = torch.matmul(qb, kb.transpose(1, 2))
+        if attn_bias is not None:
+            x = x + attn_bias[b, :, :lq, :lk].to(cd)
+        x = x * alpha
+        sg = torch.sigmoid(x)
+        p = x * sg * scale * m
+        ds = torch.matmul(gb, vb.transpose(1, 2)) * scale * m * sg * (1 + x * (1 - sg)) * alpha
+        dq[oq[b]: oq[b] + lq] = torch.matmul(ds, kb).permute(1, 0, 2)
+        dkb = torch.matmul(ds.transpose(1, 2), qb)                                          # [Nq, lk, D]
+        dvb = torch.matmul(p.transpose(1, 2), gb)
+        dk[okk[b]: okk[b] + lk] = dkb.reshape(nk, ratio, lk, -1).sum(1).permute(1, 0, 2)
+        dv[okk[b]: okk[b] + lk] = dvb.reshape(nk, ratio, lk, -1).sum(1).permute(1, 0, 2)
+        if dbias is not None:
+            dbias[b, :, :lq, :lk] = ds
+    return dq, dk, dv, dbias
 
 
 def hstu_dense_forward(q, k, v, *, max_seq_len: int, mask_type: int = MASK_TRIL, mask=None, attn_bias=None,

@@ -24,6 +24,7 @@ EXPORTS = [
     "hstu_hip_jagged_forward_get_workspace_size", "hstu_hip_jagged_forward",
     "hstu_hip_paged_forward_get_workspace_size", "hstu_hip_paged_forward",
     "hstu_hip_dense_forward_get_workspace_size", "hstu_hip_dense_forward",
+    "hstu_hip_jagged_backward_get_workspace_size", "hstu_hip_jagged_backward",
     "hstu_hip_last_error", "hstu_hip_describe_kernel", "hstu_hip_abi_version",
 ]
 
@@ -47,6 +48,14 @@ class HstuFwdParams(C.Structure):
     ]
 
 
+class HstuBwdParams(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32), ("reserved", C.c_uint32), ("fwd", HstuFwdParams),
+        ("grad_out", C.c_void_p), ("grad_q", C.c_void_p), ("grad_k", C.c_void_p), ("grad_v", C.c_void_p),
+        ("grad_bias", C.c_void_p),
+    ]
+
+
 _lib: Optional[C.CDLL] = None
 
 
@@ -66,6 +75,8 @@ def lib() -> C.CDLL:
         for n in ("jagged", "paged", "dense"):
             getattr(_lib, f"hstu_hip_{n}_forward").argtypes = [C.POINTER(HstuFwdParams), C.c_void_p, C.c_uint64, C.c_void_p]
             getattr(_lib, f"hstu_hip_{n}_forward_get_workspace_size").argtypes = [C.POINTER(HstuFwdParams), C.POINTER(C.c_uint64)]
+        _lib.hstu_hip_jagged_backward.argtypes = [C.POINTER(HstuBwdParams), C.c_void_p, C.c_uint64, C.c_void_p]
+        _lib.hstu_hip_jagged_backward_get_workspace_size.argtypes = [C.POINTER(HstuBwdParams), C.POINTER(C.c_uint64)]
         _lib.hstu_hip_describe_kernel.argtypes = [C.POINTER(HstuFwdParams), C.c_char_p, C.c_size_t]
     return _lib
 
@@ -150,6 +161,26 @@ def run(op: str, params: HstuFwdParams, stream=None):
     _check(getattr(L, f"hstu_hip_{op}_forward_get_workspace_size")(C.byref(params), C.byref(n)))
     ws = torch.empty(n.value, dtype=torch.uint8, device="cuda") if n.value else None
     _check(getattr(L, f"hstu_hip_{op}_forward")(C.byref(params), _ptr(ws), n.value, stream if stream is not None else _stream()))
+    return ws
+
+
+def make_backward_params(fwd: HstuFwdParams, grad_out, grad_q, grad_k, grad_v, grad_bias=None) -> HstuBwdParams:
+    """Argument block of the jagged backward around the forward call's block (whose ``out`` is not read)."""
+    p = HstuBwdParams()
+    p.struct_size = C.sizeof(HstuBwdParams)
+    p.fwd = fwd
+    p.grad_out, p.grad_q, p.grad_k, p.grad_v = grad_out.data_ptr(), grad_q.data_ptr(), grad_k.data_ptr(), grad_v.data_ptr()
+    p.grad_bias = _ptr(grad_bias)
+    return p
+
+
+def run_backward(params: HstuBwdParams, stream=None):
+    """Two-phase call of the jagged backward."""
+    L = lib()
+    n = C.c_uint64(0)
+    _check(L.hstu_hip_jagged_backward_get_workspace_size(C.byref(params), C.byref(n)))
+    ws = torch.empty(n.value, dtype=torch.uint8, device="cuda") if n.value else None
+    _check(L.hstu_hip_jagged_backward(C.byref(params), _ptr(ws), n.value, stream if stream is not None else _stream()))
     return ws
 
 

@@ -25,7 +25,7 @@ static int fail(int code, const char* fmt, ...) {
 
 static bool in_range(int64_t v, int64_t lo, int64_t hi) { return v >= lo && v <= hi; }
 
-static int validate(const hstu_fwd_params* p, int op, KArgs* out) {
+static int validate(const hstu_fwd_params* p, int op, KArgs* out, bool need_out = true) {
     if (!p) return fail(HSTU_ERR_INVALID_ARGUMENT, "params is NULL");
     if (p->struct_size != sizeof(hstu_fwd_params))
         return fail(HSTU_ERR_INVALID_ARGUMENT, "hstu_fwd_params size mismatch: caller %u, library %zu (ABI version %d)",
@@ -34,7 +34,7 @@ static int validate(const hstu_fwd_params* p, int op, KArgs* out) {
         return fail(HSTU_ERR_INVALID_ARGUMENT, "dtype expect float32, float16 or bfloat16, but value is %d", p->dtype);
     if (p->index_type != HSTU_I32 && p->index_type != HSTU_I64)
         return fail(HSTU_ERR_INVALID_ARGUMENT, "index_type expect int32 or int64, but value is %d", p->index_type);
-    if (!p->q || !p->k || !p->v || !p->out) return fail(HSTU_ERR_INVALID_ARGUMENT, "q, k, v and out must not be NULL");
+    if (!p->q || !p->k || !p->v || (need_out && !p->out)) return fail(HSTU_ERR_INVALID_ARGUMENT, "q, k, v and out must not be NULL");
     if (p->batch == 0 || p->batch > HSTU_MAX_BATCH || p->batch < 0)
         return fail(HSTU_ERR_INVALID_ARGUMENT, "batchSize limit (0, %d], but get %d", HSTU_MAX_BATCH, p->batch);
     if (!in_range(p->max_seq_len_q, 1, HSTU_MAX_SEQ_LEN))
@@ -135,6 +135,28 @@ static int ws_size(const hstu_fwd_params* p, int op, uint64_t* bytes) {
     return HSTU_OK;
 }
 
+// the jagged backward: the forward's checks plus what the reference's backward does not take
+static int validate_backward(const hstu_bwd_params* p, BArgs* out) {
+    if (!p) return fail(HSTU_ERR_INVALID_ARGUMENT, "params is NULL");
+    if (p->struct_size != sizeof(hstu_bwd_params))
+        return fail(HSTU_ERR_INVALID_ARGUMENT, "hstu_bwd_params size mismatch: caller %u, library %zu (ABI version %d)",
+                    p->struct_size, sizeof(hstu_bwd_params), HSTU_HIP_ABI_VERSION);
+    int rc = validate(&p->fwd, OP_JAGGED, &out->f, false);
+    if (rc != HSTU_OK) return rc;
+    if (p->fwd.pos_table || p->fwd.ts_table)
+        return fail(HSTU_ERR_UNSUPPORTED, "the backward takes a dense attn_bias only (no bias tables)");
+    if (!p->grad_out || !p->grad_q || !p->grad_k || !p->grad_v)
+        return fail(HSTU_ERR_INVALID_ARGUMENT, "grad_out, grad_q, grad_k and grad_v must not be NULL");
+    if ((p->fwd.attn_bias != nullptr) != (p->grad_bias != nullptr))
+        return fail(HSTU_ERR_INVALID_ARGUMENT, "grad_bias must be given exactly when attn_bias is");
+    out->grad_out = p->grad_out;
+    out->grad_q = p->grad_q;
+    out->grad_k = p->grad_k;
+    out->grad_v = p->grad_v;
+    out->grad_bias = p->grad_bias;
+    return HSTU_OK;
+}
+
 }  // namespace hstu
 
 using namespace hstu;
@@ -147,6 +169,27 @@ int hstu_hip_paged_forward_get_workspace_size(const hstu_fwd_params* p, uint64_t
 int hstu_hip_paged_forward(const hstu_fwd_params* p, void* ws, uint64_t n, void* s) { return run(p, OP_PAGED, ws, n, s); }
 int hstu_hip_dense_forward_get_workspace_size(const hstu_fwd_params* p, uint64_t* b) { return ws_size(p, OP_DENSE, b); }
 int hstu_hip_dense_forward(const hstu_fwd_params* p, void* ws, uint64_t n, void* s) { return run(p, OP_DENSE, ws, n, s); }
+
+int hstu_hip_jagged_backward_get_workspace_size(const hstu_bwd_params* p, uint64_t* bytes) {
+    if (!bytes) return fail(HSTU_ERR_INVALID_ARGUMENT, "workspace_bytes is NULL");
+    BArgs a;
+    int rc = validate_backward(p, &a);
+    if (rc != HSTU_OK) return rc;
+    *bytes = 0;   // every gradient element has one producing workgroup: nothing to stage
+    return HSTU_OK;
+}
+
+int hstu_hip_jagged_backward(const hstu_bwd_params* p, void* workspace, uint64_t workspace_bytes, void* stream) {
+    (void)workspace;
+    (void)workspace_bytes;
+    BArgs a;
+    int rc = validate_backward(p, &a);
+    if (rc != HSTU_OK) return rc;
+    if (p->fwd.total_q == 0 && p->fwd.total_k == 0) return HSTU_OK;
+    hipError_t e = launch_backward_generic(a, reinterpret_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString(e));
+    return HSTU_OK;
+}
 
 const char* hstu_hip_last_error(void) { return g_last_error.c_str(); }
 

@@ -25,4 +25,15 @@ bool mfma_supported(const KArgs& a, const char** name);
 uint64_t mfma_workspace_bytes(const KArgs& a);
 hipError_t launch_mfma(const KArgs& a, void* workspace, hipStream_t stream);
 
+// Backward of the jagged op: the forward's argument block plus the gradient buffers.
+struct BArgs {
+    KArgs f;
+    const void* grad_out;
+    void* grad_q;
+    void* grad_k;
+    void* grad_v;
+    void* grad_bias;
+};
+hipError_t launch_backward_generic(const BArgs& a, hipStream_t stream);
+
 }  // namespace hstu

@@ -1,0 +1,113 @@
+"""GPU parity of the jagged backward (through the C ABI) against the oracle's float64 restatement of the reference
+golden (build/presmoke/hstu/hstu_common.py:387-476) on the same seeded inputs."""
+import math
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import hstu_oracle as O
+from recsdk_amd import workloads as W
+from tests import hstu_testlib as T
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print("[case]", *a, flush=True)
+    sys.stdout.flush()
+
+
+def _case(seed, lens_q, nq, nk, dqk, dv, dtype, lens_k=None, bias=False, ctx=None, tgt=None, tgs=0, mask=None,
+          index_dtype=torch.int64, extra_rows=0):
+    rng = np.random.default_rng(seed)
+    lens_k = lens_q if lens_k is None else lens_k
+    tq, tk = sum(lens_q) + extra_rows, sum(lens_k) + extra_rows
+    mk = lambda shape, std=0.5: torch.from_numpy(rng.normal(0, std, shape).astype(np.float32)).to(dtype)
+    mq, mkk = max(max(lens_q), 1), max(max(lens_k), 1)
+    c = dict(q=mk((tq, nq, dqk)), k=mk((tk, nk, dqk)), v=mk((tk, nk, dv)), seq_offset=W.offsets(lens_q, index_dtype),
+             seq_offset_k=W.offsets(lens_k, index_dtype), max_seq_len=mq, max_seq_len_k=mkk, alpha=1.0 / math.sqrt(dqk),
+             mask_type=0, silu_scale=1.0 / 8)
+    if bias:
+        c["attn_bias"] = mk((len(lens_q), nq, mq, mkk), 0.3)
+    if ctx is not None:
+        c["num_context"] = torch.tensor(ctx, dtype=index_dtype)
+        c["num_target"] = torch.tensor(tgt, dtype=index_dtype)
+        c["target_group_size"] = tgs
+    if mask == "custom":
+        c["mask_type"] = 3
+        c["mask"] = (torch.from_numpy(rng.random((len(lens_q), nq, mq, mkk))) < 0.6).to(dtype)
+    elif mask == "none":
+        c["mask_type"] = 2
+    grad = mk((tq, nq, dv), 1.0)
+    return c, grad
+
+
+def _oracle(c, grad):
+    return O.hstu_jagged_backward(grad, c["q"], c["k"], c["v"], c["seq_offset"], c["seq_offset_k"],
+                                  max_seq_len_q=c["max_seq_len"], max_seq_len_k=c["max_seq_len_k"], mask_type=c["mask_type"],
+                                  mask=c.get("mask"), attn_bias=c.get("attn_bias"), silu_scale=c["silu_scale"], alpha=c["alpha"],
+                                  num_context=c.get("num_context"), num_target=c.get("num_target"),
+                                  target_group_size=c.get("target_group_size", 0))
+
+
+def _check(c, grad, dtype, what):
+    got = T.run_capi_backward(c, grad)
+    want = _oracle(c, grad)
+    nq_rows, nk_rows = int(c["seq_offset"][-1]), int(c["seq_offset_k"][-1])
+    for name, g, w in zip(("dq", "dk", "dv", "dbias"), got, want):
+        if w is None:
+            assert g is None
+            continue
+        T.assert_parity(g, w, dtype, what=f"{what} {name}")
+    # rows past the last offset carry zeros
+    assert float(got[0][nq_rows:].abs().max() if got[0][nq_rows:].numel() else 0.0) == 0.0
+    assert float(got[1][nk_rows:].abs().max() if got[1][nk_rows:].numel() else 0.0) == 0.0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_backward_plain_causal(dtype):
+    say("backward causal", dtype)
+    c, grad = _case(1, [37, 5, 64, 0, 129], 2, 2, 32, 32, dtype)
+    _check(c, grad, dtype, "causal")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_backward_delta_q_gqa_bias(dtype):
+    say("backward delta-q gqa bias", dtype)
+    c, grad = _case(2, [20, 7, 33], 4, 2, 64, 48, dtype, lens_k=[52, 30, 33], bias=True)
+    _check(c, grad, dtype, "delta-q gqa bias")
+
+
+def test_backward_context_and_targets_with_bias():
+    say("backward ctx/tgt")
+    c, grad = _case(3, [70, 40], 2, 1, 32, 16, torch.float32, bias=True, ctx=[3, 0], tgt=[9, 6], tgs=3)
+    _check(c, grad, torch.float32, "ctx/tgt")
+
+
+@pytest.mark.parametrize("mask", ["custom", "none"])
+def test_backward_custom_and_no_mask(mask):
+    say("backward mask", mask)
+    c, grad = _case(4, [33, 18], 2, 2, 16, 16, torch.float32, mask=mask, bias=(mask == "custom"))
+    _check(c, grad, torch.float32, mask)
+
+
+def test_backward_large_head_dim_int32_offsets_and_tail_rows():
+    say("backward d=256, int32 offsets, rows past the last offset")
+    c, grad = _case(5, [50, 31], 2, 2, 256, 128, torch.bfloat16, index_dtype=torch.int32, extra_rows=5)
+    _check(c, grad, torch.bfloat16, "d=256")
+
+
+def test_backward_matches_autograd_of_our_forward_oracle_at_training_shape():
+    """A slice of the headline shape (d=128, 4 heads, bf16) against torch.autograd of the forward oracle in float64."""
+    say("backward headline slice")
+    c, grad = _case(6, [300, 257, 512], 4, 4, 128, 128, torch.bfloat16)
+    got = T.run_capi_backward(c, grad)
+    leaves = [c[n].double().requires_grad_(True) for n in ("q", "k", "v")]
+    out = O.hstu_jagged_forward(leaves[0], leaves[1], leaves[2], c["seq_offset"], c["seq_offset_k"], max_seq_len_q=c["max_seq_len"],
+                                max_seq_len_k=c["max_seq_len_k"], silu_scale=c["silu_scale"], alpha=c["alpha"], mode="exact",
+                                compute_dtype=torch.float64)
+    auto = torch.autograd.grad(out, leaves, grad_outputs=grad.double())
+    for name, g, w in zip(("dq", "dk", "dv"), got, auto):
+        T.assert_parity(g, w, torch.bfloat16, what=f"headline slice {name}")
