@@ -146,7 +146,9 @@ static at::Tensor jagged_forward_impl(const at::Tensor& q, const at::Tensor& k, 
                                       const c10::optional<at::Tensor>& num_context,
                                       const c10::optional<at::Tensor>& num_target,
                                       const c10::optional<int64_t>& target_group_size, const c10::optional<double>& alpha,
-                                      bool deterministic, const Tables* tables, const char* op) {
+                                      bool deterministic, const Tables* tables, const char* op,
+                                      const at::Tensor* grad = nullptr,
+                                      std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor>* grads = nullptr) {
     TORCH_CHECK(q.dim() == 3, "The q should be 3D in jagged layout");
     TORCH_CHECK(k.dim() == 3 && v.dim() == 3, "The k and v should be 3D in jagged layout");
     TORCH_CHECK(seq_offset.defined() && seq_offset.dim() == 1 && seq_offset.size(0) >= 2,
@@ -229,11 +231,12 @@ static at::Tensor jagged_forward_impl(const at::Tensor& q, const at::Tensor& k, 
     for (const at::Tensor* t : {&dk, &dv, &off_q, &off_k, &ctx, &tgt, &dmask, &dbias, &pos, &tst, &tsv})
         TORCH_CHECK(!t->defined() || t->device() == dq.device(), "all tensors must be on the device of q");
 
-    auto out = at::empty({dq.size(0), dq.size(1), dv.size(2)}, dq.options());
+    at::Tensor out;
+    if (!grad) out = at::empty({dq.size(0), dq.size(1), dv.size(2)}, dq.options());
     p.q = dq.const_data_ptr();
     p.k = dk.const_data_ptr();
     p.v = dv.const_data_ptr();
-    p.out = out.data_ptr();
+    p.out = grad ? nullptr : out.data_ptr();
     p.mask = ptr_or_null(dmask);
     p.attn_bias = ptr_or_null(dbias);
     p.seq_offset_q = off_q.const_data_ptr();
@@ -244,6 +247,38 @@ static at::Tensor jagged_forward_impl(const at::Tensor& q, const at::Tensor& k, 
     p.ts_table = (const float*)ptr_or_null(tst);
     p.ts_bounds = (const float*)ptr_or_null(tsb);
     p.timestamps = (const int64_t*)ptr_or_null(tsv);
+    if (grad) {
+        // the backward of the same call (reference: hstu_deltaq_backward_impl_npu, hstu_jagged.cpp:69-138): gradients
+        // shaped like q, k, v, and like attn_bias when there is one (every element is written by the kernels)
+        auto dgrad = h.same(*grad);
+        TORCH_CHECK(dgrad.dim() == 3 && dgrad.size(0) == dq.size(0) && dgrad.size(1) == dq.size(1) && dgrad.size(2) == dv.size(2),
+                    "grad shape expect [total_q, heads_q, dim_v], but get ", dgrad.sizes());
+        TORCH_CHECK(dgrad.scalar_type() == dq.scalar_type() && dgrad.device() == dq.device(), "grad must have the dtype and device of q");
+        hstu_bwd_params b;
+        std::memset(&b, 0, sizeof(b));
+        b.struct_size = sizeof(b);
+        b.fwd = p;
+        auto gq = at::empty_like(dq), gk = at::empty_like(dk), gv = at::empty_like(dv);
+        at::Tensor gb;
+        if (dbias.defined()) gb = at::empty_like(dbias);
+        b.grad_out = dgrad.const_data_ptr();
+        b.grad_q = gq.data_ptr();
+        b.grad_k = gk.data_ptr();
+        b.grad_v = gv.data_ptr();
+        b.grad_bias = gb.defined() ? gb.data_ptr() : nullptr;
+        uint64_t ws_bytes = 0;
+        int rc = hstu_hip_jagged_backward_get_workspace_size(&b, &ws_bytes);
+        TORCH_CHECK(rc == HSTU_OK, "mxrec::", op, ": ", hstu_hip_last_error());
+        require_gpu(dq, op);
+        at::Tensor ws;
+        if (ws_bytes) ws = at::empty({(int64_t)ws_bytes}, dq.options().dtype(at::kByte));
+        c10::hip::OptionalHIPGuardMasqueradingAsCUDA guard(dq.device());
+        auto stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA();
+        rc = hstu_hip_jagged_backward(&b, ws_bytes ? ws.data_ptr() : nullptr, ws_bytes, (void*)stream.stream());
+        TORCH_CHECK(rc == HSTU_OK, "mxrec::", op, ": ", hstu_hip_last_error());
+        *grads = std::make_tuple(gq, gk, gv, gb);
+        return at::Tensor();
+    }
     run_abi(hstu_hip_jagged_forward_get_workspace_size, hstu_hip_jagged_forward, p, dq, op);
     return out;
 }
@@ -267,6 +302,31 @@ at::Tensor hstu_jagged_delta(const at::Tensor& q, const at::Tensor& k, const at:
     return jagged_forward_impl(q, k, v, mask, attn_bias, mask_type, max_seq_len, max_seq_len_k, silu_scale, seq_offset,
                                seq_offset_k, num_context, num_target, target_group_size, alpha, deterministic, nullptr,
                                "hstu_jagged");
+}
+
+using GradTuple = std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor>;
+
+GradTuple hstu_jagged_backward_equal(const at::Tensor& grad, const at::Tensor& q, const at::Tensor& k, const at::Tensor& v,
+                                     const c10::optional<at::Tensor>& mask, const c10::optional<at::Tensor>& attn_bias,
+                                     int64_t mask_type, int64_t max_seq_len, double silu_scale, const at::Tensor& seq_offset,
+                                     const c10::optional<at::Tensor>& num_context, const c10::optional<at::Tensor>& num_target,
+                                     c10::optional<int64_t> target_group_size, c10::optional<double> alpha) {
+    GradTuple g;
+    jagged_forward_impl(q, k, v, mask, attn_bias, mask_type, max_seq_len, max_seq_len, silu_scale, seq_offset, seq_offset,
+                        num_context, num_target, target_group_size, alpha, false, nullptr, "hstu_jagged_backward", &grad, &g);
+    return g;
+}
+
+GradTuple hstu_jagged_backward_delta(const at::Tensor& grad, const at::Tensor& q, const at::Tensor& k, const at::Tensor& v,
+                                     const c10::optional<at::Tensor>& mask, const c10::optional<at::Tensor>& attn_bias,
+                                     int64_t mask_type, int64_t max_seq_len, int64_t max_seq_len_k, double silu_scale,
+                                     const at::Tensor& seq_offset, const at::Tensor& seq_offset_k,
+                                     const c10::optional<at::Tensor>& num_context, const c10::optional<at::Tensor>& num_target,
+                                     c10::optional<int64_t> target_group_size, c10::optional<double> alpha) {
+    GradTuple g;
+    jagged_forward_impl(q, k, v, mask, attn_bias, mask_type, max_seq_len, max_seq_len_k, silu_scale, seq_offset, seq_offset_k,
+                        num_context, num_target, target_group_size, alpha, false, nullptr, "hstu_jagged_backward", &grad, &g);
+    return g;
 }
 
 at::Tensor hstu_jagged_table_bias(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v,
@@ -519,6 +579,37 @@ TORCH_LIBRARY_FRAGMENT(mxrec, m) {
           "                  int? target_group_size=0, "
           "                  float? alpha=1.0, "
           "                  bool deterministic=False) -> Tensor");
+    // schemas of hstu_jagged.cpp:202-215,232-247
+    m.def("hstu_jagged_backward.equal(Tensor grad, "
+          "                           Tensor q, "
+          "                           Tensor k, "
+          "                           Tensor v, "
+          "                           Tensor? mask=None, "
+          "                           Tensor? attn_bias=None, "
+          "                           int mask_type=0, "
+          "                           int max_seq_len=0, "
+          "                           float silu_scale=0.0, "
+          "                           Tensor seq_offset=None, "
+          "                           Tensor? num_context=None, "
+          "                           Tensor? num_target=None, "
+          "                           int? target_group_size=0,"
+          "                           float? alpha=1.0) -> (Tensor, Tensor, Tensor, Tensor)");
+    m.def("hstu_jagged_backward.delta(Tensor grad, "
+          "                           Tensor q, "
+          "                           Tensor k, "
+          "                           Tensor v, "
+          "                           Tensor? mask=None, "
+          "                           Tensor? attn_bias=None, "
+          "                           int mask_type=0, "
+          "                           int max_seq_len=0, "
+          "                           int max_seq_len_k=0, "
+          "                           float silu_scale=0.0, "
+          "                           Tensor seq_offset=None, "
+          "                           Tensor seq_offset_k=None, "
+          "                           Tensor? num_context=None, "
+          "                           Tensor? num_target=None, "
+          "                           int? target_group_size=0,"
+          "                           float? alpha=1.0) -> (Tensor, Tensor, Tensor, Tensor)");
     m.def("hstu_paged(Tensor q, "
           "           Tensor k, "
           "           Tensor v, "
@@ -563,6 +654,8 @@ TORCH_LIBRARY_FRAGMENT(mxrec, m) {
 #define HSTU_IMPLS(m)                                                         \
     m.impl("hstu_jagged.equal", TORCH_FN(hstu_jagged_equal));                 \
     m.impl("hstu_jagged.delta", TORCH_FN(hstu_jagged_delta));                 \
+    m.impl("hstu_jagged_backward.equal", TORCH_FN(hstu_jagged_backward_equal)); \
+    m.impl("hstu_jagged_backward.delta", TORCH_FN(hstu_jagged_backward_delta)); \
     m.impl("hstu_paged", TORCH_FN(hstu_paged));                               \
     m.impl("hstu_dense", TORCH_FN(hstu_dense));                               \
     m.impl("hstu_jagged_table_bias", TORCH_FN(hstu_jagged_table_bias));       \

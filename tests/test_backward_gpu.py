@@ -111,3 +111,24 @@ def test_backward_matches_autograd_of_our_forward_oracle_at_training_shape():
     auto = torch.autograd.grad(out, leaves, grad_outputs=grad.double())
     for name, g, w in zip(("dq", "dk", "dv"), got, auto):
         T.assert_parity(g, w, torch.bfloat16, what=f"headline slice {name}")
+
+
+def test_backward_torch_ops_equal_and_delta_overloads():
+    """The drop-in entries: torch.ops.mxrec.hstu_jagged_backward with the reference's two schemas."""
+    say("backward torch ops")
+    import recsdk_amd  # noqa: F401
+    dev = lambda t: None if t is None else t.cuda()
+    c, grad = _case(7, [40, 23], 2, 2, 64, 64, torch.bfloat16, bias=True)
+    want = T.run_capi_backward(c, grad)
+    got = torch.ops.mxrec.hstu_jagged_backward(dev(grad), dev(c["q"]), dev(c["k"]), dev(c["v"]), None, dev(c["attn_bias"]), 0,
+                                               c["max_seq_len"], c["silu_scale"], dev(c["seq_offset"]), None, None, 0, c["alpha"])
+    for g, w in zip(got, want):
+        assert torch.equal(g.cpu(), w)
+    c, grad = _case(8, [12, 9], 4, 2, 32, 32, torch.float32, lens_k=[30, 9])
+    want = T.run_capi_backward(c, grad)
+    got = torch.ops.mxrec.hstu_jagged_backward(dev(grad), dev(c["q"]), dev(c["k"]), dev(c["v"]), None, None, 0, c["max_seq_len"],
+                                               c["max_seq_len_k"], c["silu_scale"], dev(c["seq_offset"]), dev(c["seq_offset_k"]),
+                                               None, None, 0, c["alpha"])
+    for g, w in zip(got[:3], want[:3]):
+        assert torch.equal(g.cpu(), w)
+    assert got[3] is None or got[3].numel() == 0
