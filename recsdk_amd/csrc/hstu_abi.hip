@@ -186,7 +186,9 @@ int hstu_hip_jagged_backward(const hstu_bwd_params* p, void* workspace, uint64_t
     int rc = validate_backward(p, &a);
     if (rc != HSTU_OK) return rc;
     if (p->fwd.total_q == 0 && p->fwd.total_k == 0) return HSTU_OK;
-    hipError_t e = launch_backward_generic(a, reinterpret_cast<hipStream_t>(stream));
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    const bool mfma = !(p->fwd.flags & HSTU_FLAG_FORCE_GENERIC) && mfma_backward_supported(a);
+    hipError_t e = mfma ? launch_backward_mfma(a, st) : launch_backward_generic(a, st);
     if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString(e));
     return HSTU_OK;
 }

@@ -35,5 +35,7 @@ struct BArgs {
     void* grad_bias;
 };
 hipError_t launch_backward_generic(const BArgs& a, hipStream_t stream);
+bool mfma_backward_supported(const BArgs& a);
+hipError_t launch_backward_mfma(const BArgs& a, hipStream_t stream);
 
 }  // namespace hstu

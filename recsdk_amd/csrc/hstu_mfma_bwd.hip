@@ -1,0 +1,280 @@
+// Jagged HSTU backward on the gfx950 matrix cores (bf16 / fp16, head dim 64 or 128, built-in mask, no bias).
+//
+// Three kernels from one template, each a variation of the forward kernel's scheme: the rows a wave owns sit in
+// registers as B operands, the other side streams through LDS in 64-row tiles, the 32x32 score block is produced by
+// MFMAs with the owned rows as columns, so that its accumulator layout is the B-operand layout of the GEMM that
+// follows and the block never leaves the registers:
+//   MODE_DQ  owns 128 Q rows (and their dO rows); streams K, V:   S^T = K Q^T, G^T = V dO^T, dS^T = f(S^T, G^T),
+//                                                                  dQ^T += K^T dS^T
+//   MODE_DK  owns 128 K rows (and their V rows); streams Q, dO:   S = Q K^T, G = dO V^T, dS = f(S, G), dK^T += Q^T dS
+//   MODE_DV  owns 128 K rows; streams Q, dO:                      S = Q K^T, P = silu(S), dV^T += dO^T P
+// with f = G * sigmoid(x) * (1 + x * (1 - sigmoid(x))), x = alpha * S (golden: build/presmoke/hstu/hstu_common.py:446-452).
+// alpha * silu_scale factors out of the sums and is applied once to the fp32 accumulators; P and dS are rounded to the
+// I/O dtype when they are packed for the second GEMM, as P in the forward.  Every gradient element has one producing
+// workgroup (with GQA the K-side kernels loop over the query heads of their K/V head): no atomics, deterministic.
+#include "hstu_device.h"
+
+namespace hstu {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 b_bf16x8;
+typedef __attribute__((ext_vector_type(8))) _Float16 b_f16x8;
+typedef __attribute__((ext_vector_type(2))) __bf16 b_bf16x2;
+typedef __attribute__((ext_vector_type(2))) _Float16 b_f16x2;
+typedef __attribute__((ext_vector_type(16))) float b_f32x16;
+typedef __attribute__((ext_vector_type(4))) short b_s16x4;
+typedef __attribute__((ext_vector_type(8))) short b_s16x8;
+typedef __attribute__((ext_vector_type(4))) unsigned int b_u32x4;
+typedef __attribute__((ext_vector_type(2))) unsigned int b_u32x2;
+
+#define BWD_LDS_PTR(type, p) ((__attribute__((address_space(3))) type*)(p))
+
+template <typename T> struct BMM;
+template <> struct BMM<__bf16> {
+    typedef b_bf16x8 v8;
+    static __device__ __forceinline__ b_f32x16 mfma(v8 a, v8 b, b_f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+    static __device__ __forceinline__ unsigned pack2(float x, float y) {
+        b_bf16x2 r; r[0] = (__bf16)x; r[1] = (__bf16)y; return __builtin_bit_cast(unsigned, r);
+    }
+};
+template <> struct BMM<_Float16> {
+    typedef b_f16x8 v8;
+    static __device__ __forceinline__ b_f32x16 mfma(v8 a, v8 b, b_f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+    static __device__ __forceinline__ unsigned pack2(float x, float y) {
+        b_f16x2 r; r[0] = (_Float16)x; r[1] = (_Float16)y; return __builtin_bit_cast(unsigned, r);
+    }
+};
+
+enum { MODE_DQ = 0, MODE_DK = 1, MODE_DV = 2 };
+constexpr int WBM = 128;   // rows a workgroup owns
+constexpr int WBN = 64;    // rows of the other side per step
+
+template <typename T, int D, int MODE>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void hstu_bwd_mfma_kernel(const BArgs a) {
+    typedef typename BMM<T>::v8 v8;
+    const hstu_fwd_params& p = a.f.p;
+    constexpr int TS = D + 8;            // row stride of the LDS tiles in elements
+    constexpr int NCH = D / 32;          // 16-byte chunks per thread and tile
+    constexpr bool TWO = MODE != MODE_DV;   // a second score-shaped GEMM (dO V^T)
+    __shared__ __attribute__((aligned(16))) T t1[WBN * TS];
+    __shared__ __attribute__((aligned(16))) T t2[WBN * TS];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int g = lane >> 5, l32 = lane & 31;
+    const int b = blockIdx.z, ho = blockIdx.y;
+    const Seq s = load_seq(a.f, b);
+    const int ratio = a.f.head_ratio;
+    const bool tril = p.mask_type == HSTU_MASK_TRIL;
+    const int tgs = p.target_group_size;
+    const T* qb = reinterpret_cast<const T*>(p.q);
+    const T* kb_ = reinterpret_cast<const T*>(p.k);
+    const T* vb = reinterpret_cast<const T*>(p.v);
+    const T* gb = reinterpret_cast<const T*>(a.grad_out);
+
+    const int own_len = MODE == MODE_DQ ? s.lq : s.lk;
+    // tiles beyond the grid (sequences longer than the max_seq_len attribute) are taken by the same workgroups
+    for (int tile = blockIdx.x; tile * WBM < own_len; tile += gridDim.x) {
+        const int o0 = tile * WBM;
+        const int r0 = o0 + 32 * w, orow = r0 + l32;
+        const bool ovalid = orow < own_len;
+        const int hk = MODE == MODE_DQ ? ho / ratio : ho;
+        // owned rows as B operands: column = owned row, k = head-dim index
+        v8 xf[D / 16], yf[TWO ? D / 16 : 1];
+        {
+            const int rr = min(orow, own_len - 1);
+            const T* xp = MODE == MODE_DQ ? qb + ((s.q_start + rr) * p.heads_q + ho) * (int64_t)D : kb_ + ((s.k_start + rr) * p.heads_k + hk) * (int64_t)D;
+            const T* yp = MODE == MODE_DQ ? gb + ((s.q_start + rr) * p.heads_q + ho) * (int64_t)D : vb + ((s.k_start + rr) * p.heads_k + hk) * (int64_t)D;
+            const b_u32x4 z = {0, 0, 0, 0};
+#pragma unroll
+            for (int ds = 0; ds < D / 16; ds++) {
+                const b_u32x4 x = *reinterpret_cast<const b_u32x4*>(xp + 16 * ds + 8 * g);
+                xf[ds] = __builtin_bit_cast(v8, ovalid ? x : z);
+                if (TWO) {
+                    const b_u32x4 y = *reinterpret_cast<const b_u32x4*>(yp + 16 * ds + 8 * g);
+                    yf[ds] = __builtin_bit_cast(v8, ovalid ? y : z);
+                }
+            }
+        }
+        b_f32x16 oacc[D / 32];
+#pragma unroll
+        for (int db = 0; db < D / 32; db++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) oacc[db][r] = 0.f;
+
+        // range of the streamed side
+        int t_begin = 0, t_end;
+        if (MODE == MODE_DQ) {
+            t_end = s.lk > 0 ? k_extent(a.f, s, o0, min(o0 + WBM, s.lq)) : 0;
+        } else {
+            t_end = s.lq;
+            // first Q row that can see one of these K rows: causal -> j <= i + delta; context rows see the whole history
+            if (tril && s.ctx <= 0) t_begin = max(0, o0 - s.delta) / WBN * WBN;
+        }
+        const int nheads = MODE == MODE_DQ ? 1 : ratio;
+        for (int hq = 0; hq < nheads; hq++) {
+            const int h = MODE == MODE_DQ ? ho : ho * ratio + hq;
+            for (int t0 = t_begin; t0 < t_end; t0 += WBN) {
+                __syncthreads();
+                // the two tiles of this step: rows t0.. of (K, V) or (Q, dO); rows past the end are zeros
+#pragma unroll
+                for (int i = 0; i < NCH; i++) {
+                    const int c = tid + 256 * i;
+                    const int row = c / (D / 8), cc = c % (D / 8);
+                    const bool ok = t0 + row < t_end;
+                    const int64_t grow = (MODE == MODE_DQ ? s.k_start : s.q_start) + min(t0 + row, t_end - 1);
+                    const int64_t e = MODE == MODE_DQ ? (grow * p.heads_k + hk) * (int64_t)D : (grow * p.heads_q + h) * (int64_t)D;
+                    const b_u32x4 z = {0, 0, 0, 0};
+                    const b_u32x4 x1 = *reinterpret_cast<const b_u32x4*>((MODE == MODE_DQ ? kb_ : qb) + e + cc * 8);
+                    const b_u32x4 x2 = *reinterpret_cast<const b_u32x4*>((MODE == MODE_DQ ? vb : gb) + e + cc * 8);
+                    *reinterpret_cast<b_u32x4*>(t1 + row * TS + cc * 8) = ok ? x1 : z;
+                    *reinterpret_cast<b_u32x4*>(t2 + row * TS + cc * 8) = ok ? x2 : z;
+                }
+                __syncthreads();
+#pragma unroll
+                for (int kb = 0; kb < WBN / 32; kb++) {
+                    const int c0 = t0 + 32 * kb;   // first streamed row of this block
+                    // Q rows [i_lo, i_lo + 32) against K rows [j_lo, j_lo + 32) of this block (wave-uniform)
+                    const int i_lo = MODE == MODE_DQ ? r0 : c0, j_lo = MODE == MODE_DQ ? c0 : r0;
+                    bool pred = false;
+                    if (tril) {
+                        const bool has_ctx = s.ctx > 0 && i_lo < s.ctx;
+                        const bool has_tgt = s.tgt > 0 && tgs > 0 && i_lo + 31 >= s.hist_q && j_lo + 31 >= s.hist_k;
+                        if (!has_ctx && j_lo > i_lo + 31 + s.delta) continue;   // nothing visible
+                        pred = has_ctx || has_tgt || j_lo + 31 > i_lo + s.delta;
+                    }
+                    if (c0 >= t_end) continue;
+                    b_f32x16 sacc, gacc;
+#pragma unroll
+                    for (int r = 0; r < 16; r++) { sacc[r] = 0.f; gacc[r] = 0.f; }
+#pragma unroll
+                    for (int ds = 0; ds < D / 16; ds++) {
+                        const v8 f1 = *reinterpret_cast<const v8*>(t1 + (32 * kb + l32) * TS + 8 * g + 16 * ds);
+                        sacc = BMM<T>::mfma(f1, xf[ds], sacc);
+                    }
+                    if (TWO) {
+#pragma unroll
+                        for (int ds = 0; ds < D / 16; ds++) {
+                            const v8 f2 = *reinterpret_cast<const v8*>(t2 + (32 * kb + l32) * TS + 8 * g + 16 * ds);
+                            gacc = BMM<T>::mfma(f2, yf[ds], gacc);
+                        }
+                    }
+                    // accumulator register r holds streamed row c0 + 8*(r/4) + 4*g + r%4 for the owned row of this lane
+                    float wv[16];
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const float sv = sacc[r];
+                        const float e = __builtin_amdgcn_exp2f(sv * a.f.exp_scale);
+                        const float sg = __builtin_amdgcn_rcpf(1.0f + e);
+                        if (TWO) {
+                            const float x = sv * p.alpha;
+                            wv[r] = gacc[r] * sg * __builtin_fmaf(x, 1.0f - sg, 1.0f);
+                        } else {
+                            wv[r] = sv * sg;
+                        }
+                    }
+                    b_u32x4 pk0, pk1;
+#pragma unroll
+                    for (int x = 0; x < 4; x++) {
+                        pk0[x] = BMM<T>::pack2(wv[2 * x], wv[2 * x + 1]);
+                        pk1[x] = BMM<T>::pack2(wv[8 + 2 * x], wv[8 + 2 * x + 1]);
+                    }
+                    if (pred) {
+                        // branch-free form of builtin_visible() for this lane's 16 elements
+                        auto vis = [&](int r) __attribute__((always_inline)) -> bool {
+                            const int t = c0 + 8 * (r >> 2) + 4 * g + (r & 3);
+                            const int i = MODE == MODE_DQ ? orow : t, j = MODE == MODE_DQ ? t : orow;
+                            const bool ctx_row = s.ctx > 0 && i < s.ctx;
+                            const bool tgt_row = tgs > 0 && s.tgt > 0 && i >= s.hist_q;
+                            const int left = tgt_row ? s.hist_k + ((i - s.hist_q) / tgs) * tgs : 0;
+                            return (ctx_row & (j < s.hist_k)) | ((j <= i + s.delta) & !(tgt_row & (j >= s.hist_k) & (j < left)));
+                        };
+#pragma unroll
+                        for (int x = 0; x < 4; x++) {
+                            pk0[x] &= (vis(2 * x) ? 0xffffu : 0u) | (vis(2 * x + 1) ? 0xffff0000u : 0u);
+                            pk1[x] &= (vis(8 + 2 * x) ? 0xffffu : 0u) | (vis(9 + 2 * x) ? 0xffff0000u : 0u);
+                        }
+                    }
+                    // OUT^T += (tile)^T W: transposing LDS reads, 4 streamed rows of one head-dim column per lane
+                    const T* tt = MODE == MODE_DV ? t2 : t1;
+#pragma unroll
+                    for (int db = 0; db < D / 32; db++) {
+                        const T* vp = tt + (32 * kb + 4 * g + ((lane & 15) >> 2)) * TS + 16 * (l32 >> 4) + 4 * (lane & 3) + 32 * db;
+                        const b_s16x4 a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(BWD_LDS_PTR(b_s16x4, vp));
+                        const b_s16x4 a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(BWD_LDS_PTR(b_s16x4, vp + 8 * TS));
+                        const b_s16x4 a2 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(BWD_LDS_PTR(b_s16x4, vp + 16 * TS));
+                        const b_s16x4 a3 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(BWD_LDS_PTR(b_s16x4, vp + 24 * TS));
+                        const b_s16x8 lo = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+                        const b_s16x8 hi = {a2[0], a2[1], a2[2], a2[3], a3[0], a3[1], a3[2], a3[3]};
+                        oacc[db] = BMM<T>::mfma(__builtin_bit_cast(v8, lo), __builtin_bit_cast(v8, pk0), oacc[db]);
+                        oacc[db] = BMM<T>::mfma(__builtin_bit_cast(v8, hi), __builtin_bit_cast(v8, pk1), oacc[db]);
+                    }
+                }
+            }
+        }
+        // accumulator register r of block db holds head-dim index 32*db + 8*(r/4) + 4*g + r%4 for the owned row
+        if (ovalid) {
+            T* out;
+            if (MODE == MODE_DQ) out = reinterpret_cast<T*>(a.grad_q) + ((s.q_start + orow) * p.heads_q + ho) * (int64_t)D;
+            else if (MODE == MODE_DK) out = reinterpret_cast<T*>(a.grad_k) + ((s.k_start + orow) * p.heads_k + ho) * (int64_t)D;
+            else out = reinterpret_cast<T*>(a.grad_v) + ((s.k_start + orow) * p.heads_k + ho) * (int64_t)D;
+            const float sc = a.f.out_scale;   // alpha * silu_scale
+#pragma unroll
+            for (int db = 0; db < D / 32; db++) {
+#pragma unroll
+                for (int rr = 0; rr < 4; rr++) {
+                    b_u32x2 o;
+                    o[0] = BMM<T>::pack2(oacc[db][4 * rr] * sc, oacc[db][4 * rr + 1] * sc);
+                    o[1] = BMM<T>::pack2(oacc[db][4 * rr + 2] * sc, oacc[db][4 * rr + 3] * sc);
+                    *reinterpret_cast<b_u32x2*>(out + 32 * db + 8 * rr + 4 * g) = o;
+                }
+            }
+        }
+    }
+
+    // rows past the last offset carry no gradient
+    {
+        const int is64 = p.index_type == HSTU_I64;
+        const int64_t total = MODE == MODE_DQ ? p.total_q : p.total_k;
+        const int heads = MODE == MODE_DQ ? p.heads_q : p.heads_k;
+        const int64_t tail = ld_idx(MODE == MODE_DQ ? p.seq_offset_q : p.seq_offset_k, p.batch, is64);
+        if (tail < total) {
+            T* o = reinterpret_cast<T*>(MODE == MODE_DQ ? a.grad_q : (MODE == MODE_DK ? a.grad_k : a.grad_v)) + tail * heads * (int64_t)D;
+            const int64_t n = (total - tail) * heads * (int64_t)D;
+            const int64_t nblk = (int64_t)gridDim.x * gridDim.y * gridDim.z;
+            const int64_t blk = ((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+            for (int64_t e = blk * 256 + tid; e < n; e += nblk * 256) o[e] = (T)0.f;
+        }
+    }
+}
+
+bool mfma_backward_supported(const BArgs& a) {
+    const hstu_fwd_params& p = a.f.p;
+    if (p.dtype != HSTU_BF16 && p.dtype != HSTU_F16) return false;
+    if (p.dim_qk != p.dim_v || (p.dim_qk != 64 && p.dim_qk != 128)) return false;
+    if (p.attn_bias || p.mask_type == HSTU_MASK_CUSTOM) return false;
+    return true;
+}
+
+template <typename T, int D>
+static hipError_t launch_bwd_td(const BArgs& a, hipStream_t stream) {
+    const hstu_fwd_params& p = a.f.p;
+    // sequences longer than the max_seq_len attributes are covered as well: tiles over the larger of attribute and rows
+    const int qt = (int)((p.max_seq_len_q + WBM - 1) / WBM), kt = (int)((p.max_seq_len_k + WBM - 1) / WBM);
+    hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DQ>), dim3(qt, p.heads_q, p.batch), dim3(256), 0, stream, a);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DK>), dim3(kt, p.heads_k, p.batch), dim3(256), 0, stream, a);
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DV>), dim3(kt, p.heads_k, p.batch), dim3(256), 0, stream, a);
+    return hipGetLastError();
+}
+
+hipError_t launch_backward_mfma(const BArgs& a, hipStream_t stream) {
+    const hstu_fwd_params& p = a.f.p;
+    if (p.dtype == HSTU_BF16) return p.dim_qk == 128 ? launch_bwd_td<__bf16, 128>(a, stream) : launch_bwd_td<__bf16, 64>(a, stream);
+    return p.dim_qk == 128 ? launch_bwd_td<_Float16, 128>(a, stream) : launch_bwd_td<_Float16, 64>(a, stream);
+}
+
+}  // namespace hstu

@@ -57,7 +57,7 @@ def run_capi(cfg, *, op="jagged", flags=0, reuse_from=None, **over):
     return out.cpu(), name
 
 
-def run_capi_backward(cfg, grad, **over):
+def run_capi_backward(cfg, grad, flags=0, **over):
     """Call hstu_hip_jagged_backward through ctypes.  Returns (dq, dk, dv, dbias or None) on the CPU."""
     from recsdk_amd import _capi
     c = dict(cfg)
@@ -68,7 +68,7 @@ def run_capi_backward(cfg, grad, **over):
               mask=_dev(c.get("mask")), attn_bias=bias, silu_scale=c.get("silu_scale", 0.0), alpha=c.get("alpha", 1.0),
               num_context=_dev(c.get("num_context")), num_target=_dev(c.get("num_target")),
               target_group_size=c.get("target_group_size", 0), seq_offset_q=_dev(c["seq_offset"]),
-              seq_offset_k=_dev(c.get("seq_offset_k")))
+              seq_offset_k=_dev(c.get("seq_offset_k")), flags=flags)
     fwd, keep = _capi.make_params(q, k, v, q, **kw)     # the forward's `out` is not read by the backward
     fwd.out = None
     nan = float("nan")

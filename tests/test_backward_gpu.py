@@ -132,3 +132,39 @@ def test_backward_torch_ops_equal_and_delta_overloads():
     for g, w in zip(got[:3], want[:3]):
         assert torch.equal(g.cpu(), w)
     assert got[3] is None or got[3].numel() == 0
+
+
+MFMA_CASES = [
+    # lens_q, nq, nk, d, dtype, extras
+    dict(lens_q=[300, 129, 64, 1, 0, 257], nq=2, nk=2, d=128, dtype=torch.bfloat16),
+    dict(lens_q=[200, 77], nq=4, nk=2, d=64, dtype=torch.float16),                                    # GQA
+    dict(lens_q=[130, 40], nq=2, nk=1, d=128, dtype=torch.bfloat16, lens_k=[333, 40]),                 # delta-q + GQA
+    dict(lens_q=[260, 150], nq=2, nk=2, d=64, dtype=torch.bfloat16, ctx=[5, 0], tgt=[40, 17], tgs=3),  # context rows + target groups
+    dict(lens_q=[190, 33], nq=1, nk=1, d=128, dtype=torch.float16, mask="none"),
+    dict(lens_q=[515], nq=2, nk=2, d=64, dtype=torch.bfloat16, ctx=[130], tgt=[0], tgs=1),             # context rows across tiles
+]
+
+
+@pytest.mark.parametrize("c", MFMA_CASES)
+def test_backward_mfma_kernels(c):
+    say("backward mfma", {k: v for k, v in c.items() if k != "dtype"}, c["dtype"])
+    c = dict(c)
+    dtype, d = c.pop("dtype"), c.pop("d")
+    cfg, grad = _case(11, c.pop("lens_q"), c.pop("nq"), c.pop("nk"), d, d, dtype, **c)
+    got = T.run_capi_backward(cfg, grad)
+    want = _oracle(cfg, grad)
+    gen = T.run_capi_backward(cfg, grad, flags=2)   # the plain-FMA kernels
+    for name, g, w, x in zip(("dq", "dk", "dv"), got, want, gen):
+        T.assert_parity(g, w, dtype, what=f"mfma backward {name}")
+        T.assert_parity(g, x.double(), dtype, what=f"mfma vs plain kernels {name}")
+
+
+def test_backward_mfma_sequences_longer_than_the_attribute():
+    """max_seq_len smaller than the longest sequence: the tiles behind the attribute are still covered."""
+    say("backward mfma, rows behind max_seq_len")
+    cfg, grad = _case(12, [400, 90], 2, 2, 64, 64, torch.bfloat16)
+    cfg["max_seq_len"] = cfg["max_seq_len_k"] = 128
+    got = T.run_capi_backward(cfg, grad)
+    want = _oracle(cfg, grad)
+    for name, g, w in zip(("dq", "dk", "dv"), got, want):
+        T.assert_parity(g, w, torch.bfloat16, what=f"long {name}")
