@@ -57,7 +57,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=1000)
-    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "copy"],
+    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "config2_bwd", "copy"],
                     help="'copy' runs a plain 256 MiB device copy: the known-size kernel the FETCH_SIZE/WRITE_SIZE counters are scaled by")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
@@ -71,6 +71,8 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs the MI355X"
     if args.workload == "copy":
         return copy_calibration(args, torch)
+    if args.workload == "config2_bwd":
+        return backward_bench(args, torch, W, _capi)
     cfg, op, flops, alg_bytes, desc = build_workload(args.workload, torch, W)
     dev = W.to_device(cfg)
     q, k, v = dev["q"], dev["k"], dev["v"]
@@ -150,6 +152,56 @@ def main():
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(cfg, op, flops, torch)
     print(json.dumps(result), flush=True)
+
+
+def backward_bench(args, torch, W, _capi):
+    """The jagged backward (dQ, dK, dV) on the headline configuration: five GEMM-shaped products of L^2 * h * d
+    multiply-adds each under the causal mask (S, dO V^T, dV, dK, dQ) = 2.5 x the forward's FLOPs."""
+    import ctypes as C
+    cfg = W.config2()
+    dev = W.to_device(cfg)
+    q, k, v = dev["q"], dev["k"], dev["v"]
+    g = torch.Generator(device="cuda").manual_seed(1)
+    grad = torch.randn(q.shape, generator=g, device="cuda", dtype=torch.float32).to(q.dtype)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    fwd, keep = _capi.make_params(q, k, v, q, seq_offset_q=dev["seq_offset"], max_seq_len_q=cfg["max_seq_len"], alpha=cfg["alpha"])
+    fwd.out = None
+    p = _capi.make_backward_params(fwd, grad, dq, dk, dv)
+    L = _capi.lib()
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    flops = 2.5 * W.headline_flops(cfg["lens"], 4, 128)
+
+    def step():
+        if L.hstu_hip_jagged_backward(C.byref(p), None, 0, stream) != 0:
+            raise RuntimeError(L.hstu_hip_last_error().decode())
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms = wall * 1e3 / args.steps
+    kern_ms = e0.elapsed_time(e1) / args.steps
+    tflops = flops / (ms * 1e-3) / 1e12
+    t = sum(cfg["lens"])
+    alg_bytes = 7 * t * 4 * 128 * 2   # Q, K, V, dO read once; dQ, dK, dV written once
+    print(json.dumps({
+        "metric": "hstu_jagged_attn_bwd_tflops", "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic", "us_per_call": round(ms * 1e3, 2),
+        "pct_bf16_mfma_peak": round(100 * tflops / PEAK_BF16_TFLOPS, 2),
+        "config": {"workload": "config2 shapes, backward: B=64 h=4 d=128 L~U[256,1024] bf16 causal no-bias seed0",
+                   "flops_per_call": flops, "algorithmic_bytes_per_call": alg_bytes, "entry": "hstu_hip_jagged_backward (C ABI)"},
+        "roofline": {"bound": "mfma", "achieved": round(flops / (kern_ms * 1e-3) / 1e12, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(flops / (kern_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "kernel_us": round(kern_ms * 1e3, 2)},
+    }), flush=True)
 
 
 def copy_calibration(args, torch):
