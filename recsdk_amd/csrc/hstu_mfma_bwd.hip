@@ -53,11 +53,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void hstu_bwd_mfma_kernel(const BArgs a) {
     typedef typename BMM<T>::v8 v8;
     const hstu_fwd_params& p = a.f.p;
-    constexpr int TS = D + 8;            // row stride of the LDS tiles in elements
+    // row strides of the LDS tiles in elements: +16 bytes keeps the 16-byte row-wise reads of 16 rows on distinct banks,
+    // +64 bytes does the same for the 4-row transposing reads; a tile that is read both ways (K for dQ, Q for dK) takes
+    // the second and pays a two-way conflict on its row-wise reads
+    constexpr int TS1 = MODE == MODE_DV ? D + 8 : D + 32;
+    constexpr int TS2 = MODE == MODE_DV ? D + 32 : D + 8;
     constexpr int NCH = D / 32;          // 16-byte chunks per thread and tile
     constexpr bool TWO = MODE != MODE_DV;   // a second score-shaped GEMM (dO V^T)
-    __shared__ __attribute__((aligned(16))) T t1[WBN * TS];
-    __shared__ __attribute__((aligned(16))) T t2[WBN * TS];
+    // two stages: the tiles of the next step are fetched into registers while this step computes, and written to the
+    // other stage afterwards (one barrier per step)
+    __shared__ __attribute__((aligned(16))) T t1s[2][WBN * TS1];
+    __shared__ __attribute__((aligned(16))) T t2s[2][WBN * TS2];
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -74,7 +80,8 @@ void hstu_bwd_mfma_kernel(const BArgs a) {
 
     const int own_len = MODE == MODE_DQ ? s.lq : s.lk;
     // tiles beyond the grid (sequences longer than the max_seq_len attribute) are taken by the same workgroups
-    for (int tile = blockIdx.x; tile * WBM < own_len; tile += gridDim.x) {
+    for (int tl = blockIdx.x; tl * WBM < own_len; tl += gridDim.x) {
+        const int tile = tl;
         const int o0 = tile * WBM;
         const int r0 = o0 + 32 * w, orow = r0 + l32;
         const bool ovalid = orow < own_len;
@@ -114,34 +121,54 @@ void hstu_bwd_mfma_kernel(const BArgs a) {
         const int nheads = MODE == MODE_DQ ? 1 : ratio;
         for (int hq = 0; hq < nheads; hq++) {
             const int h = MODE == MODE_DQ ? ho : ho * ratio + hq;
-            for (int t0 = t_begin; t0 < t_end; t0 += WBN) {
-                __syncthreads();
-                // the two tiles of this step: rows t0.. of (K, V) or (Q, dO); rows past the end are zeros
+            b_u32x4 n1[NCH], n2[NCH];
+            auto fetch = [&](int t0) __attribute__((always_inline)) {
+#pragma unroll
+                for (int i = 0; i < NCH; i++) {
+                    const int c = tid + 256 * i;
+                    const int row = c / (D / 8), cc = c % (D / 8);
+                    const int64_t grow = (MODE == MODE_DQ ? s.k_start : s.q_start) + min(t0 + row, t_end - 1);
+                    const int64_t e = MODE == MODE_DQ ? (grow * p.heads_k + hk) * (int64_t)D : (grow * p.heads_q + h) * (int64_t)D;
+                    // nothing here waits for the data: rows past the end are zeroed when the tile is written to LDS
+                    n1[i] = *reinterpret_cast<const b_u32x4*>((MODE == MODE_DQ ? kb_ : qb) + e + cc * 8);
+                    n2[i] = *reinterpret_cast<const b_u32x4*>((MODE == MODE_DQ ? vb : gb) + e + cc * 8);
+                }
+            };
+            auto stash = [&](int t0, int stage) __attribute__((always_inline)) {
 #pragma unroll
                 for (int i = 0; i < NCH; i++) {
                     const int c = tid + 256 * i;
                     const int row = c / (D / 8), cc = c % (D / 8);
                     const bool ok = t0 + row < t_end;
-                    const int64_t grow = (MODE == MODE_DQ ? s.k_start : s.q_start) + min(t0 + row, t_end - 1);
-                    const int64_t e = MODE == MODE_DQ ? (grow * p.heads_k + hk) * (int64_t)D : (grow * p.heads_q + h) * (int64_t)D;
                     const b_u32x4 z = {0, 0, 0, 0};
-                    const b_u32x4 x1 = *reinterpret_cast<const b_u32x4*>((MODE == MODE_DQ ? kb_ : qb) + e + cc * 8);
-                    const b_u32x4 x2 = *reinterpret_cast<const b_u32x4*>((MODE == MODE_DQ ? vb : gb) + e + cc * 8);
-                    *reinterpret_cast<b_u32x4*>(t1 + row * TS + cc * 8) = ok ? x1 : z;
-                    *reinterpret_cast<b_u32x4*>(t2 + row * TS + cc * 8) = ok ? x2 : z;
+                    *reinterpret_cast<b_u32x4*>(t1s[stage] + row * TS1 + cc * 8) = ok ? n1[i] : z;
+                    *reinterpret_cast<b_u32x4*>(t2s[stage] + row * TS2 + cc * 8) = ok ? n2[i] : z;
                 }
-                __syncthreads();
+            };
+            __syncthreads();   // every wave is done with the stages of the previous head / tile
+            if (t_begin < t_end) {
+                fetch(t_begin);
+                stash(t_begin, 0);
+            }
+            __syncthreads();
+            int stage = 0;
+            for (int t0 = t_begin; t0 < t_end; t0 += WBN, stage ^= 1) {
+                const T* t1 = t1s[stage];
+                const T* t2 = t2s[stage];
+                const bool more = t0 + WBN < t_end;
+                if (more) fetch(t0 + WBN);
 #pragma unroll
                 for (int kb = 0; kb < WBN / 32; kb++) {
                     const int c0 = t0 + 32 * kb;   // first streamed row of this block
                     // Q rows [i_lo, i_lo + 32) against K rows [j_lo, j_lo + 32) of this block (wave-uniform)
                     const int i_lo = MODE == MODE_DQ ? r0 : c0, j_lo = MODE == MODE_DQ ? c0 : r0;
-                    bool pred = false;
+                    bool pred = false, diag = false;   // full predicate (context rows / targets) or only the causal compare
                     if (tril) {
                         const bool has_ctx = s.ctx > 0 && i_lo < s.ctx;
                         const bool has_tgt = s.tgt > 0 && tgs > 0 && i_lo + 31 >= s.hist_q && j_lo + 31 >= s.hist_k;
                         if (!has_ctx && j_lo > i_lo + 31 + s.delta) continue;   // nothing visible
-                        pred = has_ctx || has_tgt || j_lo + 31 > i_lo + s.delta;
+                        pred = has_ctx || has_tgt;
+                        diag = !pred && j_lo + 31 > i_lo + s.delta;
                     }
                     if (c0 >= t_end) continue;
                     b_f32x16 sacc, gacc;
@@ -149,13 +176,13 @@ void hstu_bwd_mfma_kernel(const BArgs a) {
                     for (int r = 0; r < 16; r++) { sacc[r] = 0.f; gacc[r] = 0.f; }
 #pragma unroll
                     for (int ds = 0; ds < D / 16; ds++) {
-                        const v8 f1 = *reinterpret_cast<const v8*>(t1 + (32 * kb + l32) * TS + 8 * g + 16 * ds);
+                        const v8 f1 = *reinterpret_cast<const v8*>(t1 + (32 * kb + l32) * TS1 + 8 * g + 16 * ds);
                         sacc = BMM<T>::mfma(f1, xf[ds], sacc);
                     }
                     if (TWO) {
 #pragma unroll
                         for (int ds = 0; ds < D / 16; ds++) {
-                            const v8 f2 = *reinterpret_cast<const v8*>(t2 + (32 * kb + l32) * TS + 8 * g + 16 * ds);
+                            const v8 f2 = *reinterpret_cast<const v8*>(t2 + (32 * kb + l32) * TS2 + 8 * g + 16 * ds);
                             gacc = BMM<T>::mfma(f2, yf[ds], gacc);
                         }
                     }
@@ -179,7 +206,18 @@ void hstu_bwd_mfma_kernel(const BArgs a) {
                         pk0[x] = BMM<T>::pack2(wv[2 * x], wv[2 * x + 1]);
                         pk1[x] = BMM<T>::pack2(wv[8 + 2 * x], wv[8 + 2 * x + 1]);
                     }
-                    if (pred) {
+                    if (diag) {
+                        // visible iff j <= i + delta; t runs over this lane's 16 streamed rows
+                        auto vis = [&](int r) __attribute__((always_inline)) -> bool {
+                            const int t = c0 + 8 * (r >> 2) + 4 * g + (r & 3);
+                            return MODE == MODE_DQ ? t <= orow + s.delta : orow <= t + s.delta;
+                        };
+#pragma unroll
+                        for (int x = 0; x < 4; x++) {
+                            pk0[x] &= (vis(2 * x) ? 0xffffu : 0u) | (vis(2 * x + 1) ? 0xffff0000u : 0u);
+                            pk1[x] &= (vis(8 + 2 * x) ? 0xffffu : 0u) | (vis(9 + 2 * x) ? 0xffff0000u : 0u);
+                        }
+                    } else if (pred) {
                         // branch-free form of builtin_visible() for this lane's 16 elements
                         auto vis = [&](int r) __attribute__((always_inline)) -> bool {
                             const int t = c0 + 8 * (r >> 2) + 4 * g + (r & 3);
@@ -197,19 +235,22 @@ void hstu_bwd_mfma_kernel(const BArgs a) {
                     }
                     // OUT^T += (tile)^T W: transposing LDS reads, 4 streamed rows of one head-dim column per lane
                     const T* tt = MODE == MODE_DV ? t2 : t1;
+                    constexpr int TT = MODE == MODE_DV ? TS2 : TS1;
 #pragma unroll
                     for (int db = 0; db < D / 32; db++) {
-                        const T* vp = tt + (32 * kb + 4 * g + ((lane & 15) >> 2)) * TS + 16 * (l32 >> 4) + 4 * (lane & 3) + 32 * db;
+                        const T* vp = tt + (32 * kb + 4 * g + ((lane & 15) >> 2)) * TT + 16 * (l32 >> 4) + 4 * (lane & 3) + 32 * db;
                         const b_s16x4 a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(BWD_LDS_PTR(b_s16x4, vp));
-                        const b_s16x4 a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(BWD_LDS_PTR(b_s16x4, vp + 8 * TS));
-                        const b_s16x4 a2 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(BWD_LDS_PTR(b_s16x4, vp + 16 * TS));
-                        const b_s16x4 a3 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(BWD_LDS_PTR(b_s16x4, vp + 24 * TS));
+                        const b_s16x4 a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(BWD_LDS_PTR(b_s16x4, vp + 8 * TT));
+                        const b_s16x4 a2 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(BWD_LDS_PTR(b_s16x4, vp + 16 * TT));
+                        const b_s16x4 a3 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(BWD_LDS_PTR(b_s16x4, vp + 24 * TT));
                         const b_s16x8 lo = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
                         const b_s16x8 hi = {a2[0], a2[1], a2[2], a2[3], a3[0], a3[1], a3[2], a3[3]};
                         oacc[db] = BMM<T>::mfma(__builtin_bit_cast(v8, lo), __builtin_bit_cast(v8, pk0), oacc[db]);
                         oacc[db] = BMM<T>::mfma(__builtin_bit_cast(v8, hi), __builtin_bit_cast(v8, pk1), oacc[db]);
                     }
                 }
+                if (more) stash(t0 + WBN, stage ^ 1);
+                __syncthreads();
             }
         }
         // accumulator register r of block db holds head-dim index 32*db + 8*(r/4) + 4*g + r%4 for the owned row
