@@ -50,7 +50,7 @@ constexpr int WBN = 64;    // rows of the other side per step
 
 template <typename T, int D, int MODE>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
-void hstu_bwd_mfma_kernel(const BArgs a) {
+void hstu_bwd_mfma_kernel(const BArgs a, const int ntiles_grid) {
     typedef typename BMM<T>::v8 v8;
     const hstu_fwd_params& p = a.f.p;
     // row strides of the LDS tiles in elements: +16 bytes keeps the 16-byte row-wise reads of 16 rows on distinct banks,
@@ -68,7 +68,16 @@ void hstu_bwd_mfma_kernel(const BArgs a) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int g = lane >> 5, l32 = lane & 31;
-    const int b = blockIdx.z, ho = blockIdx.y;
+    // Workgroup -> (sequence, head, tile).  Workgroup i runs on XCD i % 8: the (sequence, head) groups are dealt to the
+    // XCDs round robin and all tiles of a group follow each other on one XCD, so that the tiles that stream the same
+    // rows share an L2 and no XCD collects the heavy tiles of every group.
+    const int heads_own = MODE == MODE_DQ ? p.heads_q : p.heads_k;
+    const int ngroups = p.batch * heads_own;
+    const int slot = blockIdx.x >> 3;
+    const int gi = 8 * (slot / ntiles_grid) + (blockIdx.x & 7);
+    const int tl0 = slot % ntiles_grid;
+    const bool idle = gi >= ngroups;
+    const int b = idle ? 0 : gi / heads_own, ho = idle ? 0 : gi % heads_own;
     const Seq s = load_seq(a.f, b);
     const int ratio = a.f.head_ratio;
     const bool tril = p.mask_type == HSTU_MASK_TRIL;
@@ -80,8 +89,10 @@ void hstu_bwd_mfma_kernel(const BArgs a) {
 
     const int own_len = MODE == MODE_DQ ? s.lq : s.lk;
     // tiles beyond the grid (sequences longer than the max_seq_len attribute) are taken by the same workgroups
-    for (int tl = blockIdx.x; tl * WBM < own_len; tl += gridDim.x) {
-        const int tile = tl;
+    for (int tl = tl0; !idle && tl * WBM < own_len; tl += ntiles_grid) {
+        // heavy tiles first: the last Q tile sees the most K columns, the first K tile is seen by the most Q rows
+        const int ntl = (own_len + WBM - 1) / WBM;
+        const int tile = MODE == MODE_DQ ? ntl - 1 - tl : tl;
         const int o0 = tile * WBM;
         const int r0 = o0 + 32 * w, orow = r0 + l32;
         const bool ovalid = orow < own_len;
@@ -282,9 +293,7 @@ void hstu_bwd_mfma_kernel(const BArgs a) {
         if (tail < total) {
             T* o = reinterpret_cast<T*>(MODE == MODE_DQ ? a.grad_q : (MODE == MODE_DK ? a.grad_k : a.grad_v)) + tail * heads * (int64_t)D;
             const int64_t n = (total - tail) * heads * (int64_t)D;
-            const int64_t nblk = (int64_t)gridDim.x * gridDim.y * gridDim.z;
-            const int64_t blk = ((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
-            for (int64_t e = blk * 256 + tid; e < n; e += nblk * 256) o[e] = (T)0.f;
+            for (int64_t e = (int64_t)blockIdx.x * 256 + tid; e < n; e += (int64_t)gridDim.x * 256) o[e] = (T)0.f;
         }
     }
 }
@@ -302,13 +311,14 @@ static hipError_t launch_bwd_td(const BArgs& a, hipStream_t stream) {
     const hstu_fwd_params& p = a.f.p;
     // sequences longer than the max_seq_len attributes are covered as well: tiles over the larger of attribute and rows
     const int qt = (int)((p.max_seq_len_q + WBM - 1) / WBM), kt = (int)((p.max_seq_len_k + WBM - 1) / WBM);
-    hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DQ>), dim3(qt, p.heads_q, p.batch), dim3(256), 0, stream, a);
+    const unsigned gq = 8u * (unsigned)((p.batch * p.heads_q + 7) / 8) * qt, gk = 8u * (unsigned)((p.batch * p.heads_k + 7) / 8) * kt;
+    hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DQ>), dim3(gq), dim3(256), 0, stream, a, qt);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DK>), dim3(kt, p.heads_k, p.batch), dim3(256), 0, stream, a);
+    hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DK>), dim3(gk), dim3(256), 0, stream, a, kt);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DV>), dim3(kt, p.heads_k, p.batch), dim3(256), 0, stream, a);
+    hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DV>), dim3(gk), dim3(256), 0, stream, a, kt);
     return hipGetLastError();
 }
 
