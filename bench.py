@@ -171,8 +171,14 @@ def backward_bench(args, torch, W, _capi):
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
     flops = 2.5 * W.headline_flops(cfg["lens"], 4, 128)
 
+    nws = C.c_uint64(0)
+    if L.hstu_hip_jagged_backward_get_workspace_size(C.byref(p), C.byref(nws)) != 0:
+        raise RuntimeError(L.hstu_hip_last_error().decode())
+    ws = torch.empty(max(int(nws.value), 16), dtype=torch.uint8, device="cuda")
+    ws_ptr = C.c_void_p(ws.data_ptr())
+
     def step():
-        if L.hstu_hip_jagged_backward(C.byref(p), None, 0, stream) != 0:
+        if L.hstu_hip_jagged_backward(C.byref(p), ws_ptr, nws.value, stream) != 0:
             raise RuntimeError(L.hstu_hip_last_error().decode())
 
     for _ in range(args.warmup):

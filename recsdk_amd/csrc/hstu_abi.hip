@@ -175,20 +175,26 @@ int hstu_hip_jagged_backward_get_workspace_size(const hstu_bwd_params* p, uint64
     BArgs a;
     int rc = validate_backward(p, &a);
     if (rc != HSTU_OK) return rc;
-    *bytes = 0;   // every gradient element has one producing workgroup: nothing to stage
+    // every gradient element has one producing workgroup: no partial sums; the MFMA kernels keep their two work lists here
+    const bool mfma = !(p->fwd.flags & HSTU_FLAG_FORCE_GENERIC) && mfma_backward_supported(a);
+    *bytes = mfma ? mfma_backward_workspace_bytes(a) : 0;
     return HSTU_OK;
 }
 
 int hstu_hip_jagged_backward(const hstu_bwd_params* p, void* workspace, uint64_t workspace_bytes, void* stream) {
-    (void)workspace;
-    (void)workspace_bytes;
     BArgs a;
     int rc = validate_backward(p, &a);
     if (rc != HSTU_OK) return rc;
     if (p->fwd.total_q == 0 && p->fwd.total_k == 0) return HSTU_OK;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     const bool mfma = !(p->fwd.flags & HSTU_FLAG_FORCE_GENERIC) && mfma_backward_supported(a);
-    hipError_t e = mfma ? launch_backward_mfma(a, st) : launch_backward_generic(a, st);
+    if (mfma) {
+        const uint64_t need = mfma_backward_workspace_bytes(a);
+        if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 15))
+            return fail(HSTU_ERR_WORKSPACE, "workspace of %llu bytes (16-byte aligned) needed, got %llu at %p",
+                        (unsigned long long)need, (unsigned long long)workspace_bytes, workspace);
+    }
+    hipError_t e = mfma ? launch_backward_mfma(a, workspace, st) : launch_backward_generic(a, st);
     if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString(e));
     return HSTU_OK;
 }

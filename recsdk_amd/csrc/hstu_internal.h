@@ -25,6 +25,20 @@ bool mfma_supported(const KArgs& a, const char** name);
 uint64_t mfma_workspace_bytes(const KArgs& a);
 hipError_t launch_mfma(const KArgs& a, void* workspace, hipStream_t stream);
 
+// The device-built work list of the MFMA kernels, for kernels outside hstu_mfma.hip.  Layout (uint32 words): 16 header
+// words ([2..3] = rows the sequences own, int64), then `grid` records of 8 words, read by workgroup index:
+// seq | head << 12 | tile << 16 | sweep << 24 | further tiles << 25 | 1 << 28, then q_start, lq, k_start, lk,
+// num_context, num_target, first page entry of the sequence; 0xffffffff in word 0 = no work.  `sweep`: the item also
+// covers every later tile of its sequence (rows behind the max_seq_len attribute).
+struct WorkList {
+    unsigned grid;     // workgroups to launch = records
+    uint64_t bytes;    // workspace bytes of the list
+};
+constexpr unsigned WORK_ITEM_EMPTY = 0xffffffffu;
+constexpr int WORK_HEADER_WORDS = 16, WORK_RECORD_WORDS = 8;
+WorkList work_list_shape(const hstu_fwd_params& p);
+hipError_t launch_work_list(const KArgs& a, unsigned* ws, bool pair, hipStream_t stream);
+
 // Backward of the jagged op: the forward's argument block plus the gradient buffers.
 struct BArgs {
     KArgs f;
@@ -36,6 +50,7 @@ struct BArgs {
 };
 hipError_t launch_backward_generic(const BArgs& a, hipStream_t stream);
 bool mfma_backward_supported(const BArgs& a);
-hipError_t launch_backward_mfma(const BArgs& a, hipStream_t stream);
+uint64_t mfma_backward_workspace_bytes(const BArgs& a);
+hipError_t launch_backward_mfma(const BArgs& a, void* workspace, hipStream_t stream);
 
 }  // namespace hstu

@@ -170,10 +170,12 @@ struct SchedDims {
     unsigned cap;      // entries per XCD list
     unsigned bound;    // upper bound of the number of items (= entries of the overflow list)
     int nsplit;        // K ranges per Q tile (1 = none); each range is an item of its own
+    int pair;          // 1: the first two Q tiles of a long sequence may become one item
 };
 
-static SchedDims sched_dims(const hstu_fwd_params& p) {
+static SchedDims sched_dims(const hstu_fwd_params& p, bool whole_tiles = false) {
     SchedDims d;
+    d.pair = 1;
     d.ntiles_attr = (p.max_seq_len_q + BM - 1) / BM;
     // sum over sequences of min(ceil(lq / BM), ntiles_attr) <= min(total_q / BM + batch, batch * ntiles_attr)
     const int64_t by_rows = p.total_q / BM + p.batch, by_attr = (int64_t)p.batch * d.ntiles_attr;
@@ -183,7 +185,7 @@ static SchedDims sched_dims(const hstu_fwd_params& p) {
     // they simply add up) go through the workspace and a small reduction kernel.
     d.nsplit = 1;
     const int ktiles = (p.max_seq_len_k + BN - 1) / BN;
-    if (d.bound < 384 && ktiles >= 16) {
+    if (!whole_tiles && d.bound < 384 && ktiles >= 16) {
         int s = 768 / (int)(d.bound ? d.bound : 1);
         if (s > 4) s = 4;
         if (s > ktiles / 4) s = ktiles / 4;
@@ -205,6 +207,17 @@ uint64_t mfma_workspace_bytes(const KArgs& a) {
     if (d.nsplit > 1) b += (uint64_t)d.nsplit * a.p.total_q * a.p.heads_q * a.p.dim_v * sizeof(float);   // partial sums
     return b;
 }
+
+// The work list for kernels other than the forward (the backward's): every Q tile is one item (no K ranges; the
+// first two tiles of a long sequence become one item only if `pair`).
+WorkList work_list_shape(const hstu_fwd_params& p) {
+    const SchedDims d = sched_dims(p, true);
+    WorkList w;
+    w.grid = 8 * d.cap;
+    w.bytes = list_bytes(d);
+    return w;
+}
+
 
 __device__ __forceinline__ int xcd_of_group(unsigned r) { return (r & 8) ? 7 - (int)(r & 7) : (int)(r & 7); }
 
@@ -246,7 +259,7 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
         // The two first Q tiles of a long sequence see few K columns; as items of their own they mostly pay the start and
         // end of a workgroup.  They become one item when together they stay under 70 % of the sequence's last tile.
         bool pair = false;
-        if (d.nsplit == 1 && t == nt && nt >= 3) {
+        if (d.pair && d.nsplit == 1 && t == nt && nt >= 3) {
             const int c0 = (k_extent(a, s, 0, BM) + 63) / 64, c1 = (k_extent(a, s, BM, min(2 * BM, s.lq)) + 63) / 64;
             const int ctop = (k_extent(a, s, (nt - 1) * BM, s.lq) + 63) / 64;
             pair = 10 * (c0 + c1) <= 7 * ctop;
@@ -971,6 +984,15 @@ bool mfma_supported(const KArgs& a, const char** name) {
     if (p.dim_qk == 128) *name = bf ? "mfma_bf16_d128" : "mfma_f16_d128";
     else *name = bf ? "mfma_bf16_d64" : "mfma_f16_d64";
     return true;
+}
+
+hipError_t launch_work_list(const KArgs& a, unsigned* ws, bool pair, hipStream_t stream) {
+    SchedDims d = sched_dims(a.p, true);
+    d.pair = pair ? 1 : 0;
+    const int groups = a.p.batch * a.p.heads_q;
+    const int sched_threads = groups <= 128 ? 256 : (groups <= 512 ? 512 : SCHED_NT);
+    hipLaunchKernelGGL(hstu_schedule_kernel, dim3(1), dim3(sched_threads), 0, stream, a, d, ws);
+    return hipGetLastError();
 }
 
 template <typename T, int D>

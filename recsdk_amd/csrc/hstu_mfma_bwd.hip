@@ -50,7 +50,7 @@ constexpr int WBN = 64;    // rows of the other side per step
 
 template <typename T, int D, int MODE>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
-void hstu_bwd_mfma_kernel(const BArgs a, const int ntiles_grid) {
+void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
     typedef typename BMM<T>::v8 v8;
     const hstu_fwd_params& p = a.f.p;
     // row strides of the LDS tiles in elements: +16 bytes keeps the 16-byte row-wise reads of 16 rows on distinct banks,
@@ -68,16 +68,15 @@ void hstu_bwd_mfma_kernel(const BArgs a, const int ntiles_grid) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int g = lane >> 5, l32 = lane & 31;
-    // Workgroup -> (sequence, head, tile).  Workgroup i runs on XCD i % 8: the (sequence, head) groups are dealt to the
-    // XCDs round robin and all tiles of a group follow each other on one XCD, so that the tiles that stream the same
-    // rows share an L2 and no XCD collects the heavy tiles of every group.
-    const int heads_own = MODE == MODE_DQ ? p.heads_q : p.heads_k;
-    const int ngroups = p.batch * heads_own;
-    const int slot = blockIdx.x >> 3;
-    const int gi = 8 * (slot / ntiles_grid) + (blockIdx.x & 7);
-    const int tl0 = slot % ntiles_grid;
-    const bool idle = gi >= ngroups;
-    const int b = idle ? 0 : gi / heads_own, ho = idle ? 0 : gi % heads_own;
+    // Workgroup -> item of the work list (built on the device from the sequence lengths: tiles of the sequences sorted
+    // by length, (sequence, head) groups dealt to the XCDs, a group's tiles next to each other, no empty workgroups
+    // ahead of real work).  The K-side kernels use a list built with the roles of Q and K swapped: its "Q tiles" are
+    // their K tiles and its heads the K/V heads; only the indices of a record are used, the geometry is read again.
+    const unsigned item = ws[WORK_HEADER_WORDS + WORK_RECORD_WORDS * (size_t)blockIdx.x];
+    const bool idle = item == WORK_ITEM_EMPTY;
+    const int b = idle ? 0 : (int)(item & 0xfff), ho = idle ? 0 : (int)((item >> 12) & 0xf);
+    const int tl0 = idle ? 0 : (int)((item >> 16) & 0xff);
+    const int tl_last = idle ? -1 : (((item >> 24) & 1) ? 0x7fffff : tl0 + (int)((item >> 25) & 7));
     const Seq s = load_seq(a.f, b);
     const int ratio = a.f.head_ratio;
     const bool tril = p.mask_type == HSTU_MASK_TRIL;
@@ -89,10 +88,11 @@ void hstu_bwd_mfma_kernel(const BArgs a, const int ntiles_grid) {
 
     const int own_len = MODE == MODE_DQ ? s.lq : s.lk;
     // tiles beyond the grid (sequences longer than the max_seq_len attribute) are taken by the same workgroups
-    for (int tl = tl0; !idle && tl * WBM < own_len; tl += ntiles_grid) {
-        // heavy tiles first: the last Q tile sees the most K columns, the first K tile is seen by the most Q rows
+    for (int tl = tl0; tl <= tl_last && tl * WBM < own_len; tl++) {
+        // the list starts a group with its last tile, which is the heavy one for Q tiles (it sees the most K columns);
+        // the heavy K tile is the first (the most Q rows see it), so the K-side kernels count from the other end
         const int ntl = (own_len + WBM - 1) / WBM;
-        const int tile = MODE == MODE_DQ ? ntl - 1 - tl : tl;
+        const int tile = MODE == MODE_DQ ? tl : ntl - 1 - tl;
         const int o0 = tile * WBM;
         const int r0 = o0 + 32 * w, orow = r0 + l32;
         const bool ovalid = orow < own_len;
@@ -306,26 +306,51 @@ bool mfma_backward_supported(const BArgs& a) {
     return true;
 }
 
+// two lists: Q tiles (dQ kernel) and K tiles (dK, dV kernels: the roles of Q and K swapped)
+static KArgs swapped_roles(const KArgs& f) {
+    KArgs k = f;
+    k.p.seq_offset_q = f.p.seq_offset_k;
+    k.p.seq_offset_k = f.p.seq_offset_q;
+    k.p.total_q = f.p.total_k;
+    k.p.total_k = f.p.total_q;
+    k.p.heads_q = f.p.heads_k;
+    k.p.max_seq_len_q = f.p.max_seq_len_k;
+    k.p.max_seq_len_k = f.p.max_seq_len_q;
+    k.p.num_context = nullptr;   // the list only orders the tiles; the kernels read the true geometry themselves
+    k.p.num_target = nullptr;
+    k.head_ratio = 1;
+    return k;
+}
+
+uint64_t mfma_backward_workspace_bytes(const BArgs& a) {
+    return work_list_shape(a.f.p).bytes + work_list_shape(swapped_roles(a.f).p).bytes;
+}
+
 template <typename T, int D>
-static hipError_t launch_bwd_td(const BArgs& a, hipStream_t stream) {
-    const hstu_fwd_params& p = a.f.p;
-    // sequences longer than the max_seq_len attributes are covered as well: tiles over the larger of attribute and rows
-    const int qt = (int)((p.max_seq_len_q + WBM - 1) / WBM), kt = (int)((p.max_seq_len_k + WBM - 1) / WBM);
-    const unsigned gq = 8u * (unsigned)((p.batch * p.heads_q + 7) / 8) * qt, gk = 8u * (unsigned)((p.batch * p.heads_k + 7) / 8) * kt;
-    hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DQ>), dim3(gq), dim3(256), 0, stream, a, qt);
-    hipError_t e = hipGetLastError();
+static hipError_t launch_bwd_td(const BArgs& a, unsigned* ws, hipStream_t stream) {
+    const KArgs kside = swapped_roles(a.f);
+    const WorkList lq = work_list_shape(a.f.p), lk = work_list_shape(kside.p);
+    unsigned* wsq = ws;
+    unsigned* wsk = ws + lq.bytes / sizeof(unsigned);
+    hipError_t e = launch_work_list(a.f, wsq, true, stream);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DK>), dim3(gk), dim3(256), 0, stream, a, kt);
+    e = launch_work_list(kside, wsk, false, stream);   // the first K tiles are the heavy ones: never paired
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DQ>), dim3(lq.grid), dim3(256), 0, stream, a, wsq);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DV>), dim3(gk), dim3(256), 0, stream, a, kt);
+    hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DK>), dim3(lk.grid), dim3(256), 0, stream, a, wsk);
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DV>), dim3(lk.grid), dim3(256), 0, stream, a, wsk);
     return hipGetLastError();
 }
 
-hipError_t launch_backward_mfma(const BArgs& a, hipStream_t stream) {
+hipError_t launch_backward_mfma(const BArgs& a, void* workspace, hipStream_t stream) {
     const hstu_fwd_params& p = a.f.p;
-    if (p.dtype == HSTU_BF16) return p.dim_qk == 128 ? launch_bwd_td<__bf16, 128>(a, stream) : launch_bwd_td<__bf16, 64>(a, stream);
-    return p.dim_qk == 128 ? launch_bwd_td<_Float16, 128>(a, stream) : launch_bwd_td<_Float16, 64>(a, stream);
+    unsigned* ws = reinterpret_cast<unsigned*>(workspace);
+    if (p.dtype == HSTU_BF16) return p.dim_qk == 128 ? launch_bwd_td<__bf16, 128>(a, ws, stream) : launch_bwd_td<__bf16, 64>(a, ws, stream);
+    return p.dim_qk == 128 ? launch_bwd_td<_Float16, 128>(a, ws, stream) : launch_bwd_td<_Float16, 64>(a, ws, stream);
 }
 
 }  // namespace hstu
