@@ -322,20 +322,30 @@ static KArgs swapped_roles(const KArgs& f) {
     return k;
 }
 
+// Self-attention without GQA (the .equal overload): K tile n-1-t has the work of Q tile t, so the Q list, read from
+// the other end of each sequence, serves the K-side kernels as well (and pairs their two light tiles).
+static bool one_list(const hstu_fwd_params& p) {
+    return p.seq_offset_q == p.seq_offset_k && p.heads_q == p.heads_k && p.max_seq_len_q == p.max_seq_len_k;
+}
+
 uint64_t mfma_backward_workspace_bytes(const BArgs& a) {
-    return work_list_shape(a.f.p).bytes + work_list_shape(swapped_roles(a.f).p).bytes;
+    const uint64_t q = work_list_shape(a.f.p).bytes;
+    return one_list(a.f.p) ? q : q + work_list_shape(swapped_roles(a.f).p).bytes;
 }
 
 template <typename T, int D>
 static hipError_t launch_bwd_td(const BArgs& a, unsigned* ws, hipStream_t stream) {
     const KArgs kside = swapped_roles(a.f);
-    const WorkList lq = work_list_shape(a.f.p), lk = work_list_shape(kside.p);
+    const bool shared = one_list(a.f.p);
+    const WorkList lq = work_list_shape(a.f.p), lk = shared ? lq : work_list_shape(kside.p);
     unsigned* wsq = ws;
-    unsigned* wsk = ws + lq.bytes / sizeof(unsigned);
+    unsigned* wsk = shared ? ws : ws + lq.bytes / sizeof(unsigned);
     hipError_t e = launch_work_list(a.f, wsq, true, stream);
     if (e != hipSuccess) return e;
-    e = launch_work_list(kside, wsk, false, stream);   // the first K tiles are the heavy ones: never paired
-    if (e != hipSuccess) return e;
+    if (!shared) {
+        e = launch_work_list(kside, wsk, false, stream);   // tile costs are only roughly those of the K tiles: no pairs
+        if (e != hipSuccess) return e;
+    }
     hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DQ>), dim3(lq.grid), dim3(256), 0, stream, a, wsq);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
