@@ -22,7 +22,7 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
 # HBM-side bytes per launch from rocprofv3 FETCH_SIZE/WRITE_SIZE, each scaled by what the same counter reads for the
 # plain 256 MiB copy of `--workload copy` (factors 2.000 and 1.000); see profiles/hstu_mfma_kernel_configs2-5.md
-MEASURED_TRAFFIC_BYTES = {"config2": 171.5e6}
+MEASURED_TRAFFIC_BYTES = {"config2": 184.3e6}
 
 
 def build_workload(name, torch, W):
