@@ -237,3 +237,53 @@ int main(int argc, char** argv) {
     env = dict(os.environ, LD_LIBRARY_PATH=os.path.join(os.path.dirname(torch.__file__), "lib") + ":/opt/rocm/lib:" + os.environ.get("LD_LIBRARY_PATH", ""))
     out = subprocess.run([str(exe), _build.hip_lib_path()], check=True, capture_output=True, text=True, env=env).stdout.split(None, 3)
     assert out[0] == "1" and int(out[1]) == C.sizeof(_capi.HstuFwdParams) and out[2] == "-1" and "size mismatch" in out[3]
+
+
+def _bwd_params(**over):
+    f = _params()
+    f.out = None                       # the backward does not read the forward's output
+    b = _capi.HstuBwdParams()
+    b.struct_size = C.sizeof(_capi.HstuBwdParams)
+    b.fwd = f
+    for name in ("grad_out", "grad_q", "grad_k", "grad_v"):
+        setattr(b, name, 0x1000)       # never dereferenced on the host
+    for k, v in over.items():
+        if hasattr(b, k):
+            setattr(b, k, v)
+        else:
+            setattr(b.fwd, k, v)
+    return b
+
+
+def _bwd_ws(b):
+    n = C.c_uint64(123)
+    rc = _capi.lib().hstu_hip_jagged_backward_get_workspace_size(C.byref(b), C.byref(n))
+    return rc, n.value, _capi.lib().hstu_hip_last_error().decode()
+
+
+def test_backward_validation_and_workspace():
+    rc, n, msg = _bwd_ws(_bwd_params())
+    # bf16, d=128, built-in mask, no bias: the MFMA kernels; self-attention without GQA -> one work list (as the forward's)
+    assert rc == 0 and n == 1024, msg
+    rc, n, msg = _bwd_ws(_bwd_params(heads_k=2))            # GQA: a second list for the K-side kernels (2 K/V heads:
+    assert rc == 0 and n == 1024 + 768, msg                 # 4 tiles -> 4 * (16 + 8 * (8 * 2 + 4)) = 704 -> 768 bytes)
+    rc, n, msg = _bwd_ws(_bwd_params(dtype=_capi.HSTU_F32))  # plain kernels: nothing to stage
+    assert rc == 0 and n == 0, msg
+    rc, n, msg = _bwd_ws(_bwd_params(attn_bias=0x1000, grad_bias=0x1000))
+    assert rc == 0 and n == 0, msg                           # dense bias -> plain kernels
+    rc, _, msg = _bwd_ws(_bwd_params(attn_bias=0x1000))
+    assert rc == -1 and "grad_bias must be given exactly when attn_bias is" in msg
+    rc, _, msg = _bwd_ws(_bwd_params(grad_bias=0x1000))
+    assert rc == -1 and "grad_bias" in msg
+    rc, _, msg = _bwd_ws(_bwd_params(grad_k=None))
+    assert rc == -1 and "must not be NULL" in msg
+    rc, _, msg = _bwd_ws(_bwd_params(pos_table=0x1000))
+    assert rc == -2 and "dense attn_bias only" in msg
+    rc, _, msg = _bwd_ws(_bwd_params(struct_size=8))
+    assert rc == -1 and "size mismatch" in msg
+    rc, _, msg = _bwd_ws(_bwd_params(batch=0))               # the forward's checks apply
+    assert rc == -1 and "batchSize" in msg
+    # a call without the workspace is refused before anything is launched
+    b = _bwd_params()
+    rc = _capi.lib().hstu_hip_jagged_backward(C.byref(b), None, 0, None)
+    assert rc == -3 and "workspace" in _capi.lib().hstu_hip_last_error().decode()
