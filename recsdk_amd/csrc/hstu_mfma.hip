@@ -1,7 +1,8 @@
 // HSTU forward on the gfx950 matrix cores (bf16 / fp16 I/O, head dim 64 or 128).
 //
 // One workgroup (4 waves) owns a 128-row Q tile of one (sequence, head); wave w owns rows 32w..32w+31.
-// K and V tiles of 64 columns stream through LDS, double buffered, one barrier per tile.
+// K and V tiles of 64 columns (32 in the plain head-dim-128 variant, see Shape) stream through LDS, double buffered,
+// one barrier per tile.
 // Per tile and wave:
 //     S^T = K Q^T           v_mfma_f32_32x32x16 with A = K fragment (ds_read_b128), B = Q fragment (registers)
 //     P   = s*sigmoid(a*s)  in registers (v_exp_f32 + v_rcp_f32), mask/bias fused, packed to 16 bit
