@@ -1,5 +1,6 @@
-// torch op registration for the HSTU forward family under the reference's names and schemas:
+// torch op registration for the HSTU attention family under the reference's names and schemas:
 //   mxrec::hstu_jagged.equal / .delta   (cust_op/framework/torch_plugin/torch_library/hstu/hstu_jagged.cpp:186-231)
+//   mxrec::hstu_jagged_backward.equal / .delta and the autograd formula of hstu_jagged (hstu_jagged.cpp:69-138,202-356)
 //   mxrec::hstu_paged                    (hstu_paged.cpp:73-95)
 //   mxrec::hstu_dense                    (hstu_dense.cpp:155-164)
 // plus two ops the reference has no counterpart for (fused bias tables, fp8 paged cache).
@@ -10,6 +11,7 @@
 #include <ATen/ATen.h>
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <torch/csrc/autograd/custom_function.h>
 #include <torch/library.h>
 
 #include <cmath>
@@ -327,6 +329,67 @@ GradTuple hstu_jagged_backward_delta(const at::Tensor& grad, const at::Tensor& q
     jagged_forward_impl(q, k, v, mask, attn_bias, mask_type, max_seq_len, max_seq_len_k, silu_scale, seq_offset, seq_offset_k,
                         num_context, num_target, target_group_size, alpha, false, nullptr, "hstu_jagged_backward", &grad, &g);
     return g;
+}
+
+// Autograd wiring of hstu_jagged.equal / .delta, as the reference's HstuJaggedNpuFusion (hstu_jagged.cpp:258-345): the
+// forward saves its inputs, the backward calls the backward op and returns gradients for q, k, v and attn_bias.
+class HstuJaggedFunction : public torch::autograd::Function<HstuJaggedFunction> {
+public:
+    static at::Tensor forward(torch::autograd::AutogradContext* ctx, const at::Tensor& q, const at::Tensor& k, const at::Tensor& v,
+                              const c10::optional<at::Tensor>& mask, const c10::optional<at::Tensor>& attn_bias, int64_t mask_type,
+                              int64_t max_seq_len_q, int64_t max_seq_len_k, double silu_scale, const at::Tensor& seq_offset_q,
+                              const at::Tensor& seq_offset_k, const c10::optional<at::Tensor>& num_context,
+                              const c10::optional<at::Tensor>& num_target, c10::optional<int64_t> target_group_size,
+                              c10::optional<double> alpha, bool deterministic) {
+        at::AutoDispatchBelowADInplaceOrView guard;
+        ctx->save_for_backward({q, k, v, mask.value_or(at::Tensor()), attn_bias.value_or(at::Tensor()),
+                                num_context.value_or(at::Tensor()), num_target.value_or(at::Tensor()), seq_offset_q, seq_offset_k});
+        ctx->saved_data["mask_type"] = mask_type;
+        ctx->saved_data["max_seq_len_q"] = max_seq_len_q;
+        ctx->saved_data["max_seq_len_k"] = max_seq_len_k;
+        ctx->saved_data["silu_scale"] = silu_scale;
+        ctx->saved_data["target_group_size"] = target_group_size.value_or(0);
+        ctx->saved_data["alpha"] = alpha.value_or(1.0);
+        return jagged_forward_impl(q, k, v, mask, attn_bias, mask_type, max_seq_len_q, max_seq_len_k, silu_scale, seq_offset_q,
+                                   seq_offset_k, num_context, num_target, target_group_size, alpha, deterministic, nullptr, "hstu_jagged");
+    }
+
+    static torch::autograd::tensor_list backward(torch::autograd::AutogradContext* ctx, torch::autograd::tensor_list grad_outputs) {
+        const auto saved = ctx->get_saved_variables();
+        auto opt = [](const at::Tensor& t) { return t.defined() ? c10::optional<at::Tensor>(t) : c10::nullopt; };
+        GradTuple g;
+        jagged_forward_impl(saved[0], saved[1], saved[2], opt(saved[3]), opt(saved[4]), ctx->saved_data["mask_type"].toInt(),
+                            ctx->saved_data["max_seq_len_q"].toInt(), ctx->saved_data["max_seq_len_k"].toInt(),
+                            ctx->saved_data["silu_scale"].toDouble(), saved[7], saved[8], opt(saved[5]), opt(saved[6]),
+                            ctx->saved_data["target_group_size"].toInt(), ctx->saved_data["alpha"].toDouble(), false, nullptr,
+                            "hstu_jagged_backward", &grad_outputs[0], &g);
+        // one entry per forward argument: q, k, v, mask, attn_bias, then the eleven attributes and index tensors
+        torch::autograd::tensor_list out(16);
+        out[0] = std::get<0>(g);
+        out[1] = std::get<1>(g);
+        out[2] = std::get<2>(g);
+        out[4] = std::get<3>(g);
+        return out;
+    }
+};
+
+at::Tensor hstu_jagged_equal_autograd(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v,
+                                      const c10::optional<at::Tensor>& mask, const c10::optional<at::Tensor>& attn_bias,
+                                      int64_t mask_type, int64_t max_seq_len, double silu_scale, const at::Tensor& seq_offset,
+                                      const c10::optional<at::Tensor>& num_context, const c10::optional<at::Tensor>& num_target,
+                                      c10::optional<int64_t> target_group_size, c10::optional<double> alpha, bool deterministic) {
+    return HstuJaggedFunction::apply(q, k, v, mask, attn_bias, mask_type, max_seq_len, max_seq_len, silu_scale, seq_offset, seq_offset,
+                                     num_context, num_target, target_group_size, alpha, deterministic);
+}
+
+at::Tensor hstu_jagged_delta_autograd(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v,
+                                      const c10::optional<at::Tensor>& mask, const c10::optional<at::Tensor>& attn_bias,
+                                      int64_t mask_type, int64_t max_seq_len, int64_t max_seq_len_k, double silu_scale,
+                                      const at::Tensor& seq_offset, const at::Tensor& seq_offset_k,
+                                      const c10::optional<at::Tensor>& num_context, const c10::optional<at::Tensor>& num_target,
+                                      c10::optional<int64_t> target_group_size, c10::optional<double> alpha, bool deterministic) {
+    return HstuJaggedFunction::apply(q, k, v, mask, attn_bias, mask_type, max_seq_len, max_seq_len_k, silu_scale, seq_offset, seq_offset_k,
+                                     num_context, num_target, target_group_size, alpha, deterministic);
 }
 
 at::Tensor hstu_jagged_table_bias(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v,
@@ -665,5 +728,10 @@ TORCH_LIBRARY_FRAGMENT(mxrec, m) {
 // reports that there is no CPU implementation.
 TORCH_LIBRARY_IMPL(mxrec, CUDA, m) { HSTU_IMPLS(m) }
 TORCH_LIBRARY_IMPL(mxrec, CPU, m) { HSTU_IMPLS(m) }
+// differentiable entry of the jagged op (reference: TORCH_LIBRARY_IMPL(mxrec, AutogradPrivateUse1, ...), hstu_jagged.cpp:352-356)
+TORCH_LIBRARY_IMPL(mxrec, AutogradCUDA, m) {
+    m.impl("hstu_jagged.equal", TORCH_FN(hstu_jagged_equal_autograd));
+    m.impl("hstu_jagged.delta", TORCH_FN(hstu_jagged_delta_autograd));
+}
 
 }  // namespace mxrec_hstu

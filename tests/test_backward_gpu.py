@@ -168,3 +168,33 @@ def test_backward_mfma_sequences_longer_than_the_attribute():
     want = _oracle(cfg, grad)
     for name, g, w in zip(("dq", "dk", "dv"), got, want):
         T.assert_parity(g, w, torch.bfloat16, what=f"long {name}")
+
+
+def test_hstu_jagged_is_differentiable_like_the_reference_op():
+    """out.backward() through torch.ops.mxrec.hstu_jagged (.equal and .delta) gives the backward op's gradients."""
+    say("autograd through the torch op")
+    import recsdk_amd  # noqa: F401
+    dev = lambda t: None if t is None else t.cuda()
+    for lens_k, bias in (([60, 35], True), ([90, 35], False)):
+        c, grad = _case(9, [60, 35], 2, 2, 64, 64, torch.bfloat16, lens_k=lens_k, bias=bias)
+        want = T.run_capi_backward(c, grad)
+        q, k, v = (dev(c[n]).requires_grad_(True) for n in ("q", "k", "v"))
+        b = dev(c.get("attn_bias"))
+        if b is not None:
+            b.requires_grad_(True)
+        if lens_k == [60, 35]:
+            out = torch.ops.mxrec.hstu_jagged(q, k, v, None, b, 0, c["max_seq_len"], c["silu_scale"], dev(c["seq_offset"]), None, None, 0,
+                                              c["alpha"])
+        else:
+            out = torch.ops.mxrec.hstu_jagged(q, k, v, None, b, 0, c["max_seq_len"], c["max_seq_len_k"], c["silu_scale"],
+                                              dev(c["seq_offset"]), dev(c["seq_offset_k"]), None, None, 0, c["alpha"])
+        out.backward(dev(grad))
+        assert torch.equal(q.grad.cpu(), want[0]) and torch.equal(k.grad.cpu(), want[1]) and torch.equal(v.grad.cpu(), want[2])
+        if b is not None:
+            assert torch.equal(b.grad.cpu(), want[3])
+    # no gradient requested: the plain forward
+    with torch.no_grad():
+        c, _ = _case(10, [20], 1, 1, 64, 64, torch.bfloat16)
+        out = torch.ops.mxrec.hstu_jagged(dev(c["q"]), dev(c["k"]), dev(c["v"]), None, None, 0, 20, c["silu_scale"], dev(c["seq_offset"]),
+                                          None, None, 0, c["alpha"])
+        assert not out.requires_grad
