@@ -179,6 +179,12 @@ typedef struct hstu_bwd_params {
 int hstu_hip_jagged_backward_get_workspace_size(const hstu_bwd_params* p, uint64_t* workspace_bytes);
 int hstu_hip_jagged_backward(const hstu_bwd_params* p, void* workspace, uint64_t workspace_bytes, void* stream);
 
+/* Backward of the dense op: replaces aclnnHstuDenseBackwardGetWorkspaceSize / aclnnHstuDenseBackward
+ * (hstu_dense.cpp:43-153).  Same argument block; fwd as for hstu_hip_dense_forward (seq_offset_* NULL, q/k/v and the
+ * gradients [batch, max_seq_len_q, heads, dim]). */
+int hstu_hip_dense_backward_get_workspace_size(const hstu_bwd_params* p, uint64_t* workspace_bytes);
+int hstu_hip_dense_backward(const hstu_bwd_params* p, void* workspace, uint64_t workspace_bytes, void* stream);
+
 /* replaces aclGetRecentErrMsg() (pytorch_npu_helper.hpp:510-543): message of the last failing call on this thread */
 const char* hstu_hip_last_error(void);
 

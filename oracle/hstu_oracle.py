@@ -350,6 +350,20 @@ def hstu_dense_forward(q, k, v, *, max_seq_len: int, mask_type: int = MASK_TRIL,
     return o.reshape(b, s, n, -1)
 
 
+def hstu_dense_backward(grad, q, k, v, *, max_seq_len: int, mask_type: int = MASK_TRIL, mask=None, attn_bias=None,
+                        silu_scale: float = 0.0):
+    """Backward of the ``[B, S, N, D]`` layout (hstu_dense.cpp:43-153: the jagged backward's kernel with layout
+    "normal", alpha fixed at 1).  Returns ``(dq, dk, dv, dbias)`` shaped like q, k, v, attn_bias.
+    PINNED by autograd through hstu_dense_forward (tests/test_oracle_backward.py)."""
+    b, s, n, d = q.shape
+    off = torch.arange(b + 1, dtype=torch.int64) * s
+    dq, dk, dv, db = hstu_jagged_backward(grad.reshape(b * s, n, -1), q.reshape(b * s, n, d), k.reshape(b * s, n, d),
+                                          v.reshape(b * s, n, -1), off, off, max_seq_len_q=max_seq_len,
+                                          max_seq_len_k=max_seq_len, mask_type=mask_type, mask=mask, attn_bias=attn_bias,
+                                          silu_scale=silu_scale, alpha=1.0)
+    return dq.reshape(q.shape), dk.reshape(k.shape), dv.reshape(v.shape), db
+
+
 # --------------------------------------------------------------------------
 # paged KV cache
 # --------------------------------------------------------------------------

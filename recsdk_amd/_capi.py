@@ -25,6 +25,7 @@ EXPORTS = [
     "hstu_hip_paged_forward_get_workspace_size", "hstu_hip_paged_forward",
     "hstu_hip_dense_forward_get_workspace_size", "hstu_hip_dense_forward",
     "hstu_hip_jagged_backward_get_workspace_size", "hstu_hip_jagged_backward",
+    "hstu_hip_dense_backward_get_workspace_size", "hstu_hip_dense_backward",
     "hstu_hip_last_error", "hstu_hip_describe_kernel", "hstu_hip_abi_version",
 ]
 
@@ -75,8 +76,9 @@ def lib() -> C.CDLL:
         for n in ("jagged", "paged", "dense"):
             getattr(_lib, f"hstu_hip_{n}_forward").argtypes = [C.POINTER(HstuFwdParams), C.c_void_p, C.c_uint64, C.c_void_p]
             getattr(_lib, f"hstu_hip_{n}_forward_get_workspace_size").argtypes = [C.POINTER(HstuFwdParams), C.POINTER(C.c_uint64)]
-        _lib.hstu_hip_jagged_backward.argtypes = [C.POINTER(HstuBwdParams), C.c_void_p, C.c_uint64, C.c_void_p]
-        _lib.hstu_hip_jagged_backward_get_workspace_size.argtypes = [C.POINTER(HstuBwdParams), C.POINTER(C.c_uint64)]
+        for n in ("jagged", "dense"):
+            getattr(_lib, f"hstu_hip_{n}_backward").argtypes = [C.POINTER(HstuBwdParams), C.c_void_p, C.c_uint64, C.c_void_p]
+            getattr(_lib, f"hstu_hip_{n}_backward_get_workspace_size").argtypes = [C.POINTER(HstuBwdParams), C.POINTER(C.c_uint64)]
         _lib.hstu_hip_describe_kernel.argtypes = [C.POINTER(HstuFwdParams), C.c_char_p, C.c_size_t]
     return _lib
 
@@ -174,13 +176,13 @@ def make_backward_params(fwd: HstuFwdParams, grad_out, grad_q, grad_k, grad_v, g
     return p
 
 
-def run_backward(params: HstuBwdParams, stream=None):
-    """Two-phase call of the jagged backward."""
+def run_backward(params: HstuBwdParams, stream=None, op: str = "jagged"):
+    """Two-phase call of the jagged (or dense) backward."""
     L = lib()
     n = C.c_uint64(0)
-    _check(L.hstu_hip_jagged_backward_get_workspace_size(C.byref(params), C.byref(n)))
+    _check(getattr(L, f"hstu_hip_{op}_backward_get_workspace_size")(C.byref(params), C.byref(n)))
     ws = torch.empty(n.value, dtype=torch.uint8, device="cuda") if n.value else None
-    _check(L.hstu_hip_jagged_backward(C.byref(params), _ptr(ws), n.value, stream if stream is not None else _stream()))
+    _check(getattr(L, f"hstu_hip_{op}_backward")(C.byref(params), _ptr(ws), n.value, stream if stream is not None else _stream()))
     return ws
 
 

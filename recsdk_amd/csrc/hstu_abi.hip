@@ -136,12 +136,12 @@ static int ws_size(const hstu_fwd_params* p, int op, uint64_t* bytes) {
 }
 
 // the jagged backward: the forward's checks plus what the reference's backward does not take
-static int validate_backward(const hstu_bwd_params* p, BArgs* out) {
+static int validate_backward(const hstu_bwd_params* p, int op, BArgs* out) {
     if (!p) return fail(HSTU_ERR_INVALID_ARGUMENT, "params is NULL");
     if (p->struct_size != sizeof(hstu_bwd_params))
         return fail(HSTU_ERR_INVALID_ARGUMENT, "hstu_bwd_params size mismatch: caller %u, library %zu (ABI version %d)",
                     p->struct_size, sizeof(hstu_bwd_params), HSTU_HIP_ABI_VERSION);
-    int rc = validate(&p->fwd, OP_JAGGED, &out->f, false);
+    int rc = validate(&p->fwd, op, &out->f, false);
     if (rc != HSTU_OK) return rc;
     if (p->fwd.pos_table || p->fwd.ts_table)
         return fail(HSTU_ERR_UNSUPPORTED, "the backward takes a dense attn_bias only (no bias tables)");
@@ -170,20 +170,20 @@ int hstu_hip_paged_forward(const hstu_fwd_params* p, void* ws, uint64_t n, void*
 int hstu_hip_dense_forward_get_workspace_size(const hstu_fwd_params* p, uint64_t* b) { return ws_size(p, OP_DENSE, b); }
 int hstu_hip_dense_forward(const hstu_fwd_params* p, void* ws, uint64_t n, void* s) { return run(p, OP_DENSE, ws, n, s); }
 
-int hstu_hip_jagged_backward_get_workspace_size(const hstu_bwd_params* p, uint64_t* bytes) {
+static int backward_ws_size(const hstu_bwd_params* p, int op, uint64_t* bytes) {
     if (!bytes) return fail(HSTU_ERR_INVALID_ARGUMENT, "workspace_bytes is NULL");
     BArgs a;
-    int rc = validate_backward(p, &a);
+    int rc = validate_backward(p, op, &a);
     if (rc != HSTU_OK) return rc;
-    // every gradient element has one producing workgroup: no partial sums; the MFMA kernels keep their two work lists here
+    // every gradient element has one producing workgroup: no partial sums; the MFMA kernels keep their work lists here
     const bool mfma = !(p->fwd.flags & HSTU_FLAG_FORCE_GENERIC) && mfma_backward_supported(a);
     *bytes = mfma ? mfma_backward_workspace_bytes(a) : 0;
     return HSTU_OK;
 }
 
-int hstu_hip_jagged_backward(const hstu_bwd_params* p, void* workspace, uint64_t workspace_bytes, void* stream) {
+static int backward_run(const hstu_bwd_params* p, int op, void* workspace, uint64_t workspace_bytes, void* stream) {
     BArgs a;
-    int rc = validate_backward(p, &a);
+    int rc = validate_backward(p, op, &a);
     if (rc != HSTU_OK) return rc;
     if (p->fwd.total_q == 0 && p->fwd.total_k == 0) return HSTU_OK;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
@@ -198,6 +198,11 @@ int hstu_hip_jagged_backward(const hstu_bwd_params* p, void* workspace, uint64_t
     if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString(e));
     return HSTU_OK;
 }
+
+int hstu_hip_jagged_backward_get_workspace_size(const hstu_bwd_params* p, uint64_t* b) { return backward_ws_size(p, OP_JAGGED, b); }
+int hstu_hip_jagged_backward(const hstu_bwd_params* p, void* ws, uint64_t n, void* s) { return backward_run(p, OP_JAGGED, ws, n, s); }
+int hstu_hip_dense_backward_get_workspace_size(const hstu_bwd_params* p, uint64_t* b) { return backward_ws_size(p, OP_DENSE, b); }
+int hstu_hip_dense_backward(const hstu_bwd_params* p, void* ws, uint64_t n, void* s) { return backward_run(p, OP_DENSE, ws, n, s); }
 
 const char* hstu_hip_last_error(void) { return g_last_error.c_str(); }
 

@@ -170,7 +170,7 @@ __global__ __launch_bounds__(256) void hstu_bwd_dq_kernel(const BArgs a) {
 
     // rows past the last offset carry no gradient
     const int is64 = p.index_type == HSTU_I64;
-    const int64_t tail = ld_idx(p.seq_offset_q, p.batch, is64);
+    const int64_t tail = p.seq_offset_q ? ld_idx(p.seq_offset_q, p.batch, is64) : p.total_q;
     if (tail < p.total_q) {
         const int64_t n = (p.total_q - tail) * p.heads_q * (int64_t)p.dim_qk;
         const int64_t nblk = (int64_t)gridDim.x * gridDim.y * gridDim.z;
@@ -303,7 +303,7 @@ __global__ __launch_bounds__(256) void hstu_bwd_dkv_kernel(const BArgs a) {
 
     // rows past the last offset carry no gradient
     const int is64 = p.index_type == HSTU_I64;
-    const int64_t tail = ld_idx(p.seq_offset_k, p.batch, is64);
+    const int64_t tail = p.seq_offset_k ? ld_idx(p.seq_offset_k, p.batch, is64) : p.total_k;
     if (tail < p.total_k) {
         const int64_t nblk = (int64_t)gridDim.x * gridDim.y * gridDim.z;
         const int64_t blk = ((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;

@@ -289,7 +289,8 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
         const int is64 = p.index_type == HSTU_I64;
         const int64_t total = MODE == MODE_DQ ? p.total_q : p.total_k;
         const int heads = MODE == MODE_DQ ? p.heads_q : p.heads_k;
-        const int64_t tail = ld_idx(MODE == MODE_DQ ? p.seq_offset_q : p.seq_offset_k, p.batch, is64);
+        const void* offs = MODE == MODE_DQ ? p.seq_offset_q : p.seq_offset_k;
+        const int64_t tail = offs ? ld_idx(offs, p.batch, is64) : total;
         if (tail < total) {
             T* o = reinterpret_cast<T*>(MODE == MODE_DQ ? a.grad_q : (MODE == MODE_DK ? a.grad_k : a.grad_v)) + tail * heads * (int64_t)D;
             const int64_t n = (total - tail) * heads * (int64_t)D;

@@ -2,7 +2,7 @@
 //   mxrec::hstu_jagged.equal / .delta   (cust_op/framework/torch_plugin/torch_library/hstu/hstu_jagged.cpp:186-231)
 //   mxrec::hstu_jagged_backward.equal / .delta and the autograd formula of hstu_jagged (hstu_jagged.cpp:69-138,202-356)
 //   mxrec::hstu_paged                    (hstu_paged.cpp:73-95)
-//   mxrec::hstu_dense                    (hstu_dense.cpp:155-164)
+//   mxrec::hstu_dense, hstu_dense_backward and the autograd formula of hstu_dense (hstu_dense.cpp:13-248)
 // plus two ops the reference has no counterpart for (fused bias tables, fp8 paged cache).
 // The host logic mirrors hstu_deltaq_forward_impl_npu (hstu_jagged.cpp:22-67): same checks and
 // messages, same defaults, output allocated here; the device work is one call into the C ABI of
@@ -562,8 +562,9 @@ at::Tensor hstu_paged_fp8(const at::Tensor& q, const at::Tensor& k, const at::Te
 // ---------------------------------------------------------------------------------------------
 // dense
 // ---------------------------------------------------------------------------------------------
-at::Tensor hstu_dense(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, const c10::optional<at::Tensor>& mask,
-                      const c10::optional<at::Tensor>& attn_bias, int64_t mask_type, int64_t max_seq_len, double silu_scale) {
+static at::Tensor dense_impl(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, const c10::optional<at::Tensor>& mask,
+                             const c10::optional<at::Tensor>& attn_bias, int64_t mask_type, int64_t max_seq_len, double silu_scale,
+                             const char* op, const at::Tensor* grad = nullptr, GradTuple* grads = nullptr) {
     TORCH_CHECK(q.dim() == 4, "The q should be 4D in dense layout");
     Holder h;
     auto dq = h.same(q), dk = h.same(k), dv = h.same(v);
@@ -600,15 +601,100 @@ at::Tensor hstu_dense(const at::Tensor& q, const at::Tensor& k, const at::Tensor
         TORCH_CHECK(dbias.scalar_type() == dq.scalar_type(), "attn_bias dtype must equal the q dtype");
         TORCH_CHECK(dbias.sizes() == at::IntArrayRef(full), "attn_bias shape expect [batch, heads, seq, seq], but get ", dbias.sizes());
     }
-    auto out = at::empty_like(dq);
     p.q = dq.const_data_ptr();
     p.k = dk.const_data_ptr();
     p.v = dv.const_data_ptr();
-    p.out = out.data_ptr();
     p.mask = ptr_or_null(dmask);
     p.attn_bias = ptr_or_null(dbias);
-    run_abi(hstu_hip_dense_forward_get_workspace_size, hstu_hip_dense_forward, p, dq, "hstu_dense");
+    if (grad) {
+        // reference: hstu_dense_backward_impl_npu (hstu_dense.cpp:43-153).  Gradients shaped like q, k, v; the fourth
+        // output is the bias gradient, or without a bias the reference's zero tensor with the sequence dimension
+        // rounded up to a multiple of 256
+        auto dgrad = h.same(*grad);
+        TORCH_CHECK(dgrad.dim() == 4, "The grad should be 4D in normal layout");
+        TORCH_CHECK(dgrad.sizes() == dq.sizes(), "Q and grad batch size check failed");
+        TORCH_CHECK(dgrad.scalar_type() == dq.scalar_type() && dgrad.device() == dq.device(),
+                    "grad dtype should be the same as q dtype, but got grad: ", dgrad.scalar_type(), " and q: ", dq.scalar_type());
+        hstu_bwd_params b;
+        std::memset(&b, 0, sizeof(b));
+        b.struct_size = sizeof(b);
+        b.fwd = p;
+        auto gq = at::empty_like(dq), gk = at::empty_like(dk), gv = at::empty_like(dv);
+        at::Tensor gb;
+        if (dbias.defined()) gb = at::empty_like(dbias);
+        b.grad_out = dgrad.const_data_ptr();
+        b.grad_q = gq.data_ptr();
+        b.grad_k = gk.data_ptr();
+        b.grad_v = gv.data_ptr();
+        b.grad_bias = gb.defined() ? gb.data_ptr() : nullptr;
+        uint64_t ws_bytes = 0;
+        int rc = hstu_hip_dense_backward_get_workspace_size(&b, &ws_bytes);
+        TORCH_CHECK(rc == HSTU_OK, "mxrec::", op, ": ", hstu_hip_last_error());
+        require_gpu(dq, op);
+        at::Tensor ws;
+        if (ws_bytes) ws = at::empty({(int64_t)ws_bytes}, dq.options().dtype(at::kByte));
+        c10::hip::OptionalHIPGuardMasqueradingAsCUDA guard(dq.device());
+        auto stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA();
+        rc = hstu_hip_dense_backward(&b, ws_bytes ? ws.data_ptr() : nullptr, ws_bytes, (void*)stream.stream());
+        TORCH_CHECK(rc == HSTU_OK, "mxrec::", op, ": ", hstu_hip_last_error());
+        if (!gb.defined()) {
+            const int64_t padded = (max_seq_len + 255) / 256 * 256;
+            gb = at::zeros({dq.size(0), dq.size(2), padded, padded}, dq.options());
+        }
+        *grads = std::make_tuple(gq, gk, gv, gb);
+        return at::Tensor();
+    }
+    auto out = at::empty_like(dq);
+    p.out = out.data_ptr();
+    run_abi(hstu_hip_dense_forward_get_workspace_size, hstu_hip_dense_forward, p, dq, op);
     return out;
+}
+
+at::Tensor hstu_dense(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, const c10::optional<at::Tensor>& mask,
+                      const c10::optional<at::Tensor>& attn_bias, int64_t mask_type, int64_t max_seq_len, double silu_scale) {
+    return dense_impl(q, k, v, mask, attn_bias, mask_type, max_seq_len, silu_scale, "hstu_dense");
+}
+
+GradTuple hstu_dense_backward(const at::Tensor& grad, const at::Tensor& q, const at::Tensor& k, const at::Tensor& v,
+                              const c10::optional<at::Tensor>& mask, const c10::optional<at::Tensor>& attn_bias,
+                              int64_t mask_type, int64_t max_seq_len, double silu_scale) {
+    GradTuple g;
+    dense_impl(q, k, v, mask, attn_bias, mask_type, max_seq_len, silu_scale, "hstu_dense_backward", &grad, &g);
+    return g;
+}
+
+// Autograd wiring of hstu_dense, as the reference's HstuDenseNpuFusion (hstu_dense.cpp:177-235): gradients for q, k, v
+// and, when given, attn_bias.
+class HstuDenseFunction : public torch::autograd::Function<HstuDenseFunction> {
+public:
+    static at::Tensor forward(torch::autograd::AutogradContext* ctx, const at::Tensor& q, const at::Tensor& k, const at::Tensor& v,
+                              const c10::optional<at::Tensor>& mask, const c10::optional<at::Tensor>& attn_bias,
+                              int64_t mask_type, int64_t max_seq_len, double silu_scale) {
+        at::AutoDispatchBelowADInplaceOrView guard;
+        ctx->save_for_backward({q, k, v, mask.value_or(at::Tensor()), attn_bias.value_or(at::Tensor())});
+        ctx->saved_data["mask_type"] = mask_type;
+        ctx->saved_data["max_seq_len"] = max_seq_len;
+        ctx->saved_data["silu_scale"] = silu_scale;
+        return hstu_dense(q, k, v, mask, attn_bias, mask_type, max_seq_len, silu_scale);
+    }
+    static torch::autograd::tensor_list backward(torch::autograd::AutogradContext* ctx, torch::autograd::tensor_list grad_outputs) {
+        auto saved = ctx->get_saved_variables();
+        auto opt = [](const at::Tensor& t) { return t.defined() ? c10::optional<at::Tensor>(t) : c10::nullopt; };
+        GradTuple g = hstu_dense_backward(grad_outputs[0], saved[0], saved[1], saved[2], opt(saved[3]), opt(saved[4]),
+                                          ctx->saved_data["mask_type"].toInt(), ctx->saved_data["max_seq_len"].toInt(),
+                                          ctx->saved_data["silu_scale"].toDouble());
+        torch::autograd::tensor_list out(8);
+        out[0] = std::get<0>(g);
+        out[1] = std::get<1>(g);
+        out[2] = std::get<2>(g);
+        if (saved[4].defined()) out[4] = std::get<3>(g);
+        return out;
+    }
+};
+
+at::Tensor hstu_dense_autograd(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, const c10::optional<at::Tensor>& mask,
+                               const c10::optional<at::Tensor>& attn_bias, int64_t mask_type, int64_t max_seq_len, double silu_scale) {
+    return HstuDenseFunction::apply(q, k, v, mask, attn_bias, mask_type, max_seq_len, silu_scale);
 }
 
 TORCH_LIBRARY_FRAGMENT(mxrec, m) {
@@ -701,6 +787,15 @@ TORCH_LIBRARY_FRAGMENT(mxrec, m) {
           "           int mask_type=0, "
           "           int max_seq_len=0, "
           "           float silu_scale=0.0) -> Tensor");
+    m.def("hstu_dense_backward(Tensor grad, "
+          "                    Tensor q, "
+          "                    Tensor k, "
+          "                    Tensor v, "
+          "                    Tensor? mask, "
+          "                    Tensor? attn_bias, "
+          "                    int mask_type=0, "
+          "                    int max_seq_len=0, "
+          "                    float silu_scale=0.0) -> (Tensor, Tensor, Tensor, Tensor)");
     // no counterpart in the reference:
     m.def("hstu_jagged_table_bias(Tensor q, Tensor k, Tensor v, Tensor? pos_table=None, Tensor? ts_table=None, "
           "Tensor? timestamps=None, Tensor? attn_bias=None, int mask_type=0, int max_seq_len=0, int max_seq_len_k=0, "
@@ -721,6 +816,7 @@ TORCH_LIBRARY_FRAGMENT(mxrec, m) {
     m.impl("hstu_jagged_backward.delta", TORCH_FN(hstu_jagged_backward_delta)); \
     m.impl("hstu_paged", TORCH_FN(hstu_paged));                               \
     m.impl("hstu_dense", TORCH_FN(hstu_dense));                               \
+    m.impl("hstu_dense_backward", TORCH_FN(hstu_dense_backward));             \
     m.impl("hstu_jagged_table_bias", TORCH_FN(hstu_jagged_table_bias));       \
     m.impl("hstu_paged_fp8", TORCH_FN(hstu_paged_fp8));
 
@@ -732,6 +828,7 @@ TORCH_LIBRARY_IMPL(mxrec, CPU, m) { HSTU_IMPLS(m) }
 TORCH_LIBRARY_IMPL(mxrec, AutogradCUDA, m) {
     m.impl("hstu_jagged.equal", TORCH_FN(hstu_jagged_equal_autograd));
     m.impl("hstu_jagged.delta", TORCH_FN(hstu_jagged_delta_autograd));
+    m.impl("hstu_dense", TORCH_FN(hstu_dense_autograd));
 }
 
 }  // namespace mxrec_hstu

@@ -57,8 +57,8 @@ def run_capi(cfg, *, op="jagged", flags=0, reuse_from=None, **over):
     return out.cpu(), name
 
 
-def run_capi_backward(cfg, grad, flags=0, **over):
-    """Call hstu_hip_jagged_backward through ctypes.  Returns (dq, dk, dv, dbias or None) on the CPU."""
+def run_capi_backward(cfg, grad, flags=0, op="jagged", **over):
+    """Call hstu_hip_<op>_backward (jagged or dense) through ctypes.  Returns (dq, dk, dv, dbias or None) on the CPU."""
     from recsdk_amd import _capi
     c = dict(cfg)
     c.update(over)
@@ -67,15 +67,16 @@ def run_capi_backward(cfg, grad, flags=0, **over):
     kw = dict(max_seq_len_q=c["max_seq_len"], max_seq_len_k=c.get("max_seq_len_k"), mask_type=c.get("mask_type", 0),
               mask=_dev(c.get("mask")), attn_bias=bias, silu_scale=c.get("silu_scale", 0.0), alpha=c.get("alpha", 1.0),
               num_context=_dev(c.get("num_context")), num_target=_dev(c.get("num_target")),
-              target_group_size=c.get("target_group_size", 0), seq_offset_q=_dev(c["seq_offset"]),
-              seq_offset_k=_dev(c.get("seq_offset_k")), flags=flags)
+              target_group_size=c.get("target_group_size", 0), flags=flags, dense=op == "dense")
+    if op != "dense":
+        kw.update(seq_offset_q=_dev(c["seq_offset"]), seq_offset_k=_dev(c.get("seq_offset_k")))
     fwd, keep = _capi.make_params(q, k, v, q, **kw)     # the forward's `out` is not read by the backward
     fwd.out = None
     nan = float("nan")
     dq, dk, dv = torch.full_like(q, nan), torch.full_like(k, nan), torch.full_like(v, nan)
     db = None if bias is None else torch.full_like(bias, nan)
     p = _capi.make_backward_params(fwd, g, dq, dk, dv, db)
-    _capi.run_backward(p)
+    _capi.run_backward(p, op=op)
     torch.cuda.synchronize()
     return dq.cpu(), dk.cpu(), dv.cpu(), None if db is None else db.cpu()
 

@@ -198,3 +198,73 @@ def test_hstu_jagged_is_differentiable_like_the_reference_op():
         out = torch.ops.mxrec.hstu_jagged(dev(c["q"]), dev(c["k"]), dev(c["v"]), None, None, 0, 20, c["silu_scale"], dev(c["seq_offset"]),
                                           None, None, 0, c["alpha"])
         assert not out.requires_grad
+
+
+def _dense_case(seed, b, s, n, d, dtype, bias=False, mask=None):
+    rng = np.random.default_rng(seed)
+    mk = lambda shape, std=0.5: torch.from_numpy(rng.normal(0, std, shape).astype(np.float32)).to(dtype)
+    sd = d ** -0.25   # the dense op has no alpha: scores of unit variance
+    c = dict(q=mk((b, s, n, d), sd), k=mk((b, s, n, d), sd), v=mk((b, s, n, d)), max_seq_len=s, mask_type=0, silu_scale=1.0 / 8)
+    if bias:
+        c["attn_bias"] = mk((b, n, s, s), 0.3)
+    if mask == "custom":
+        c["mask_type"] = 3
+        c["mask"] = (torch.from_numpy(rng.random((b, n, s, s))) < 0.6).to(dtype)
+    return c, mk((b, s, n, d), 1.0)
+
+
+@pytest.mark.parametrize("kind", ["mfma_bf16", "mfma_f16_d64", "bias_f32", "custom_mask_bf16"])
+def test_dense_backward(kind):
+    """hstu_hip_dense_backward ([B, S, N, D] layout, no offsets) against the oracle, for the MFMA and the plain kernels."""
+    say("dense backward", kind)
+    c, grad = {"mfma_bf16": lambda: _dense_case(21, 3, 200, 2, 128, torch.bfloat16),
+               "mfma_f16_d64": lambda: _dense_case(22, 2, 130, 3, 64, torch.float16),
+               "bias_f32": lambda: _dense_case(23, 2, 45, 2, 32, torch.float32, bias=True),
+               "custom_mask_bf16": lambda: _dense_case(24, 2, 70, 2, 64, torch.bfloat16, bias=True, mask="custom")}[kind]()
+    dtype = c["q"].dtype
+    got = T.run_capi_backward(c, grad, op="dense")
+    want = O.hstu_dense_backward(grad, c["q"], c["k"], c["v"], max_seq_len=c["max_seq_len"], mask_type=c["mask_type"],
+                                 mask=c.get("mask"), attn_bias=c.get("attn_bias"), silu_scale=c["silu_scale"])
+    for name, g, w in zip(("dq", "dk", "dv", "dbias"), got, want):
+        if w is None:
+            assert g is None
+            continue
+        T.assert_parity(g, w, dtype, what=f"dense backward {kind} {name}")
+    if kind.startswith("mfma"):
+        gen = T.run_capi_backward(c, grad, op="dense", flags=2)
+        for name, g, x in zip(("dq", "dk", "dv"), got, gen):
+            T.assert_parity(g, x.double(), dtype, what=f"dense mfma vs plain kernels {name}")
+        # the same rows as a jagged batch of equal lengths give the same bits
+        b, s, n, d = c["q"].shape
+        j = dict(c, q=c["q"].reshape(b * s, n, d), k=c["k"].reshape(b * s, n, d), v=c["v"].reshape(b * s, n, d),
+                 seq_offset=W.offsets([s] * b, torch.int64), seq_offset_k=None, max_seq_len_k=s)
+        jag = T.run_capi_backward(j, grad.reshape(b * s, n, d))
+        for g, x in zip(got[:3], jag[:3]):
+            assert torch.equal(g.reshape(b * s, n, d), x)
+
+
+def test_hstu_dense_backward_op_and_autograd():
+    """torch.ops.mxrec.hstu_dense_backward with the reference's schema, and out.backward() through hstu_dense."""
+    say("dense backward torch op + autograd")
+    import recsdk_amd  # noqa: F401
+    dev = lambda t: None if t is None else t.cuda()
+    for bias in (True, False):
+        c, grad = _dense_case(25, 2, 96, 2, 64, torch.bfloat16, bias=bias)
+        want = T.run_capi_backward(c, grad, op="dense")
+        got = torch.ops.mxrec.hstu_dense_backward(dev(grad), dev(c["q"]), dev(c["k"]), dev(c["v"]), None, dev(c.get("attn_bias")), 0,
+                                                  c["max_seq_len"], c["silu_scale"])
+        for g, w in zip(got[:3], want[:3]):
+            assert torch.equal(g.cpu(), w)
+        if bias:
+            assert torch.equal(got[3].cpu(), want[3])
+        else:   # the reference returns zeros with the sequence dimension rounded up to 256 (hstu_dense.cpp:131-136)
+            assert tuple(got[3].shape) == (2, 2, 256, 256) and float(got[3].abs().max()) == 0.0
+        q, k, v = (dev(c[n]).requires_grad_(True) for n in ("q", "k", "v"))
+        b = dev(c.get("attn_bias"))
+        if b is not None:
+            b.requires_grad_(True)
+        out = torch.ops.mxrec.hstu_dense(q, k, v, None, b, 0, c["max_seq_len"], c["silu_scale"])
+        out.backward(dev(grad))
+        assert torch.equal(q.grad.cpu(), want[0]) and torch.equal(k.grad.cpu(), want[1]) and torch.equal(v.grad.cpu(), want[2])
+        if b is not None:
+            assert torch.equal(b.grad.cpu(), want[3])

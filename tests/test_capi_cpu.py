@@ -255,9 +255,9 @@ def _bwd_params(**over):
     return b
 
 
-def _bwd_ws(b):
+def _bwd_ws(b, op="jagged"):
     n = C.c_uint64(123)
-    rc = _capi.lib().hstu_hip_jagged_backward_get_workspace_size(C.byref(b), C.byref(n))
+    rc = getattr(_capi.lib(), f"hstu_hip_{op}_backward_get_workspace_size")(C.byref(b), C.byref(n))
     return rc, n.value, _capi.lib().hstu_hip_last_error().decode()
 
 
@@ -286,4 +286,14 @@ def test_backward_validation_and_workspace():
     # a call without the workspace is refused before anything is launched
     b = _bwd_params()
     rc = _capi.lib().hstu_hip_jagged_backward(C.byref(b), None, 0, None)
+    assert rc == -3 and "workspace" in _capi.lib().hstu_hip_last_error().decode()
+
+
+def test_dense_backward_validation():
+    rc, _, msg = _bwd_ws(_bwd_params(), op="dense")
+    assert rc == -1 and "no sequence offsets" in msg
+    d = _bwd_params(seq_offset_q=None, seq_offset_k=None, total_q=128, total_k=128)
+    rc, n, msg = _bwd_ws(d, op="dense")
+    assert rc == 0 and n > 0 and n % 256 == 0, msg           # bf16 d=128: the MFMA kernels with one work list
+    rc = _capi.lib().hstu_hip_dense_backward(C.byref(d), None, 0, None)
     assert rc == -3 and "workspace" in _capi.lib().hstu_hip_last_error().decode()

@@ -90,3 +90,17 @@ def test_bias_gradient_is_zero_outside_the_sequences():
     assert float(db[1].abs().max()) > 0.0
     # masked (non-causal) entries carry no gradient either
     assert float(torch.triu(db[1, 0], diagonal=1).abs().max()) == 0.0
+
+
+def test_dense_backward_matches_autograd_of_the_dense_forward():
+    g = torch.Generator().manual_seed(5)
+    b, s_, n, d = 2, 7, 2, 16
+    q, k, v, grad = (torch.randn(b, s_, n, d, generator=g, dtype=torch.float64) * 0.6 for _ in range(4))
+    bias = torch.randn(b, n, s_, s_, generator=g, dtype=torch.float64) * 0.3
+    leaves = [t.clone().requires_grad_(True) for t in (q, k, v, bias)]
+    out = O.hstu_dense_forward(leaves[0], leaves[1], leaves[2], max_seq_len=s_, attn_bias=leaves[3], mode="exact",
+                               compute_dtype=torch.float64)
+    auto = torch.autograd.grad(out, leaves, grad_outputs=grad)
+    got = O.hstu_dense_backward(grad, q, k, v, max_seq_len=s_, attn_bias=bias)
+    for name, a, w in zip(("dq", "dk", "dv", "dbias"), got, auto):
+        assert a.shape == w.shape and torch.allclose(a, w, rtol=1e-10, atol=1e-12), name
