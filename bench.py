@@ -57,7 +57,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=1000)
-    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "config2_bwd", "copy"],
+    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "config2_bwd", "kv_append", "copy"],
                     help="'copy' runs a plain 256 MiB device copy: the known-size kernel the FETCH_SIZE/WRITE_SIZE counters are scaled by")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
@@ -73,6 +73,8 @@ def main():
         return copy_calibration(args, torch)
     if args.workload == "config2_bwd":
         return backward_bench(args, torch, W, _capi)
+    if args.workload == "kv_append":
+        return kv_append_bench(args, torch, W)
     cfg, op, flops, alg_bytes, desc = build_workload(args.workload, torch, W)
     dev = W.to_device(cfg)
     q, k, v = dev["q"], dev["k"], dev["v"]
@@ -208,6 +210,59 @@ def backward_bench(args, torch, W, _capi):
                      "frac": round(flops / (kern_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4), "traffic": None,
                      "kernel_us": round(kern_ms * 1e3, 2)},
     }), flush=True)
+
+
+def kv_append_bench(args, torch, W):
+    """The write side of the paged cache at the shape of config 5's history: 32 users, 1024-4096 new tokens each, 4 heads
+    x 128, bf16, 64-token pages in shuffled order.  Every K and V row is read once and written once."""
+    from recsdk_amd import kvcache
+    cfg = W.kv_append_config(0, users=32, heads=4, dim=128, prev_lo=0, prev_hi=0, new_lo=1024, new_hi=4096, page_size=64)
+    dev = W.to_device(cfg)
+    n = cfg["nnz"]
+    bi = torch.empty(n, dtype=torch.int32, device="cuda")
+    pos = torch.empty_like(bi)
+    kc, vc = dev["kv_cache"].unbind(1)
+
+    def step():
+        kvcache.get_paged_batch_indices_positions(dev["append_indptr"], dev["seq_lens"], bi, pos)
+        kvcache.append_kvcache(dev["append_key"], dev["append_value"], bi, pos, dev["offsets"], dev["nnz_dev"], n, kc, vc,
+                               dev["kv_indices"], dev["kv_indptr"], dev["kv_last_page_len"], 0)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    kern_ms = e0.elapsed_time(e1) / args.steps
+    row_bytes = 4 * 128 * 2
+    alg_bytes = n * row_bytes * 4 + n * 4 * 4      # K, V rows read and written; batch_indices / positions written and read
+    out = {
+        "metric": "paged_kv_append_gbps", "value": round(alg_bytes / (ms * 1e-3) / 1e9, 1), "unit": "GB/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "u16", "data": "synthetic", "us_per_call": round(ms * 1e3, 2),
+        "config": {"workload": f"append of {n} new tokens (32 users x U[1024,4096]) x 4 heads x 128, bf16, 64-token pages, seed 0",
+                   "algorithmic_bytes_per_call": alg_bytes, "entry": "hstu_hip_kv_token_positions + hstu_hip_kv_append (C ABI)"},
+        "roofline": {"bound": "hbm", "achieved": round(alg_bytes / (kern_ms * 1e-3) / 1e9, 1), "peak": 8000.0, "unit": "GB/s",
+                     "frac": round(alg_bytes / (kern_ms * 1e-3) / 1e9 / 8000.0, 4), "traffic": None, "kernel_us": round(kern_ms * 1e3, 2)},
+    }
+    if not args.no_cpu_baseline:
+        from oracle import kvcache_oracle as KO
+        t = cfg["kv_cache"].view(torch.int16).numpy()
+        k16, v16 = cfg["append_key"].view(torch.int16).numpy(), cfg["append_value"].view(torch.int16).numpy()
+        t0 = time.perf_counter()
+        b_, p_ = KO.paged_batch_indices_positions(cfg["append_indptr"].numpy(), cfg["seq_lens"].numpy())
+        KO.append_paged_kvcache(t[:, 0], t[:, 1], k16, v16, b_, p_, cfg["offsets"].numpy(), n, cfg["kv_indices"].numpy(),
+                                cfg["kv_indptr"].numpy())
+        dt = time.perf_counter() - t0
+        out["cpu_baseline"] = {"value": round(alg_bytes / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+                               "sample": f"the whole append once, token loop in numpy, {dt:.2f} s"}
+    print(json.dumps(out), flush=True)
 
 
 def copy_calibration(args, torch):

@@ -13,7 +13,7 @@ namespace hstu {
 
 static thread_local std::string g_last_error;
 
-static int fail(int code, const char* fmt, ...) {
+int fail(int code, const char* fmt, ...) {
     char buf[512];
     va_list ap;
     va_start(ap, fmt);

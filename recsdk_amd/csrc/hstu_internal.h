@@ -7,6 +7,9 @@
 
 namespace hstu {
 
+// records the message hstu_hip_last_error() returns to the calling thread; returns `code`
+int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+
 enum OpKind : int32_t { OP_JAGGED = 0, OP_PAGED = 1, OP_DENSE = 2 };
 
 // Kernel argument block: the caller's parameters plus what the host derives from them.

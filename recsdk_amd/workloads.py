@@ -150,5 +150,34 @@ def config5(seed=0, users=32):
     return c
 
 
+def kv_append_config(seed, users, heads, dim, prev_lo, prev_hi, new_lo, new_hi, page_size, dtype=torch.bfloat16,
+                     shuffle=True) -> Dict:
+    """One append into a paged K/V table: user u already holds ``prev[u]`` tokens (their rows are in the table) and
+    gets ``new[u]`` more.  Pages are allocated per user, in shuffled order; metadata as the reference's cache manager
+    hands it to ``append_kvcache`` (kvcache_metadata.py:97-125)."""
+    rng = np.random.default_rng(seed)
+    prev = [int(x) for x in rng.integers(prev_lo, prev_hi + 1, users)]
+    new = [int(x) for x in rng.integers(new_lo, new_hi + 1, users)]
+    total = [a + b for a, b in zip(prev, new)]
+    npages = [(t + page_size - 1) // page_size for t in total]
+    order = rng.permutation(sum(npages)) if shuffle else np.arange(sum(npages))
+    i32 = torch.int32
+    cache = torch.zeros(sum(npages), 2, page_size, heads, dim, dtype=dtype)
+    indptr = offsets(npages, i32)
+    ids = torch.from_numpy(order.astype(np.int32))
+    history = []
+    for u in range(users):                      # rows already cached
+        kv = _normal(rng, (2, prev[u], heads, dim), dtype)
+        history.append(kv)
+        for t in range(prev[u]):
+            cache[int(ids[int(indptr[u]) + t // page_size]), :, t % page_size] = kv[:, t]
+    nnz = sum(new)
+    return dict(kv_cache=cache, append_key=_normal(rng, (nnz, heads, dim), dtype), append_value=_normal(rng, (nnz, heads, dim), dtype),
+                append_indptr=offsets(new, i32), seq_lens=torch.tensor(total, dtype=i32), kv_indices=ids, kv_indptr=indptr,
+                kv_last_page_len=torch.tensor([t % page_size or page_size for t in total], dtype=i32),
+                offsets=torch.zeros(users, dtype=i32), nnz=nnz, nnz_dev=torch.tensor([nnz], dtype=i32), prev=prev, new=new,
+                history=history, page_size=page_size)
+
+
 def to_device(cfg: Dict, device="cuda") -> Dict:
     return {k: (v.to(device) if isinstance(v, torch.Tensor) else v) for k, v in cfg.items()}

@@ -1,0 +1,140 @@
+"""GPU parity of the paged K/V append (through the C ABI, via the host mirror of the reference's binding) against the
+oracle: bit-exact, like every byte-moving path; plus the round trip append -> hstu_paged."""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import kvcache_oracle as KO
+from recsdk_amd import kvcache, workloads as W
+from tests import hstu_testlib as T
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print("[case]", *a, flush=True)
+    sys.stdout.flush()
+
+
+def _positions(c):
+    bi = torch.full((c["nnz"] + 3,), -7, dtype=torch.int32, device="cuda")   # slack entries must stay untouched
+    pos = torch.full_like(bi, -7)
+    kvcache.get_paged_batch_indices_positions(c["append_indptr"].cuda(), c["seq_lens"].cuda(), bi, pos)
+    return bi, pos
+
+
+def _append(c, bi, pos, table, layout=0, offsets=None, key=None, value=None, nnz=None):
+    kc, vc = table.unbind(1)
+    kvcache.append_kvcache(c["append_key"].cuda() if key is None else key, c["append_value"].cuda() if value is None else value, bi, pos,
+                           (c["offsets"] if offsets is None else offsets).cuda(), c["nnz_dev"].cuda(), c["nnz"] if nnz is None else nnz,
+                           kc, vc, c["kv_indices"].cuda(), c["kv_indptr"].cuda(), c["kv_last_page_len"].cuda(), layout)
+    torch.cuda.synchronize()
+
+
+def _oracle(c, layout=0, offsets=None, key=None, value=None):
+    t = c["kv_cache"].view(torch.int16).numpy().copy()
+    if layout == 1:
+        t = np.ascontiguousarray(t.transpose(0, 1, 3, 2, 4))
+    bi, pos = KO.paged_batch_indices_positions(c["append_indptr"].numpy(), c["seq_lens"].numpy())
+    k = (c["append_key"] if key is None else key).view(torch.int16).numpy()
+    v = (c["append_value"] if value is None else value).view(torch.int16).numpy()
+    KO.append_paged_kvcache(t[:, 0], t[:, 1], k, v, bi, pos, (c["offsets"] if offsets is None else offsets).numpy(), c["nnz"],
+                            c["kv_indices"].numpy(), c["kv_indptr"].numpy(), kv_layout=layout)
+    return bi, pos, t
+
+
+@pytest.mark.parametrize("dim,heads,page,dtype", [(64, 2, 32, torch.bfloat16), (128, 4, 64, torch.float16), (256, 1, 16, torch.bfloat16),
+                                                  (512, 3, 8, torch.bfloat16)])
+def test_append_matches_oracle_bit_for_bit(dim, heads, page, dtype):
+    say("kv append", dim, heads, page, dtype)
+    c = W.kv_append_config(40, users=7, heads=heads, dim=dim, prev_lo=0, prev_hi=100, new_lo=0, new_hi=150, page_size=page, dtype=dtype)
+    wbi, wpos, want = _oracle(c)
+    bi, pos = _positions(c)
+    assert np.array_equal(bi[:c["nnz"]].cpu().numpy(), wbi) and np.array_equal(pos[:c["nnz"]].cpu().numpy(), wpos)
+    assert bool((bi[c["nnz"]:] == -7).all()) and bool((pos[c["nnz"]:] == -7).all())
+    table = c["kv_cache"].cuda()
+    _append(c, bi, pos, table)
+    assert np.array_equal(table.cpu().view(torch.int16).numpy(), want)
+
+
+def test_append_hnd_layout_source_offsets_and_strided_source():
+    """kv_layout 1 ([pages, heads, page_size, dim] views), per-user source offsets, append_key as a slice of a wider tensor."""
+    say("kv append hnd/offsets/strides")
+    c = W.kv_append_config(41, users=4, heads=2, dim=64, prev_lo=0, prev_hi=50, new_lo=1, new_hi=60, page_size=16)
+    off = torch.tensor([0, 2, 5, 9], dtype=torch.int32)
+    bi_np, _ = KO.paged_batch_indices_positions(c["append_indptr"].numpy(), c["seq_lens"].numpy())
+    rows = torch.arange(c["nnz"]) + off[torch.from_numpy(bi_np).long()]
+    wide = torch.zeros(c["nnz"] + 9, 2, 2, 64, dtype=torch.bfloat16)            # [rows, k|v, heads, dim]: row stride 2*heads*dim
+    wide[rows, 0], wide[rows, 1] = c["append_key"], c["append_value"]
+    _, _, want = _oracle(c, layout=1, offsets=off, key=wide[:, 0].contiguous(), value=wide[:, 1].contiguous())
+    bi, pos = _positions(c)
+    table = c["kv_cache"].transpose(2, 3).contiguous().cuda()                    # [pages, 2, heads, page_size, dim]
+    wd = wide.cuda()
+    _append(c, bi, pos, table, layout=1, offsets=off, key=wd[:, 0], value=wd[:, 1])
+    assert np.array_equal(table.cpu().view(torch.int16).numpy(), want)
+
+
+def test_append_skips_what_points_outside_and_honours_the_device_count():
+    """nnz on the device smaller than the host bound: the tail is not written; a page id outside the table, a negative
+    position or a user id outside the batch skip that token (no fault, nothing else disturbed)."""
+    say("kv append guards")
+    c = W.kv_append_config(42, users=3, heads=2, dim=64, prev_lo=0, prev_hi=0, new_lo=20, new_hi=40, page_size=16)
+    bi, pos = _positions(c)
+    n = c["nnz"]
+    short = dict(c, nnz_dev=torch.tensor([n - 5], dtype=torch.int32))
+    _, _, want = _oracle(dict(short, nnz=n - 5))
+    table = c["kv_cache"].cuda()
+    _append(short, bi, pos, table)
+    assert np.array_equal(table.cpu().view(torch.int16).numpy(), want)
+    # corrupt three tokens of a fresh append
+    bad = dict(c, kv_indices=c["kv_indices"].clone())
+    first_page_u0 = int(bad["kv_indices"][0])
+    bad["kv_indices"][0] = 10 ** 6                   # user 0's first page: its first 16 tokens are skipped
+    bi2, pos2 = bi.clone(), pos.clone()
+    bi2[n - 1] = 99
+    pos2[n - 2] = -3
+    table = c["kv_cache"].cuda()
+    _append(bad, bi2, pos2, table)
+    _, _, want = _oracle(c)
+    want[first_page_u0] = 0
+    wbi, wpos = KO.paged_batch_indices_positions(c["append_indptr"].numpy(), c["seq_lens"].numpy())
+    for t in (n - 1, n - 2):
+        u, p = int(wbi[t]), int(wpos[t])
+        want[int(c["kv_indices"][int(c["kv_indptr"][u]) + p // 16]), :, p % 16] = 0
+    assert np.array_equal(table.cpu().view(torch.int16).numpy(), want)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16])
+def test_roundtrip_append_then_hstu_paged(dtype):
+    """The write side feeds the read side: a table filled by two appends (history, then its extension) gives the paged
+    forward the bits it gets from the table the workload builder filled on the host."""
+    say("kv append -> hstu_paged", dtype)
+    cfg = W.paged_config(43, 5, 2, 128, 60, 400, 40, 64, dtype)
+    users, ps = 5, 64
+    hist = cfg["hist"]
+    ref_table = cfg["kv_cache"]
+    po, ids = cfg["page_offsets"], cfg["page_ids"]
+    rows = [torch.cat([ref_table[int(ids[p])] for p in range(int(po[u]), int(po[u + 1]))], dim=1)[:, :hist[u]] for u in range(users)]
+    table = torch.zeros_like(ref_table).cuda()
+    done = [0] * users
+    for frac in (0.4, 1.0):
+        upto = [max(int(h * frac), 1) if frac < 1 else h for h in hist]
+        new = [a - b for a, b in zip(upto, done)]
+        k = torch.cat([rows[u][0, done[u]:upto[u]] for u in range(users)]).cuda()
+        v = torch.cat([rows[u][1, done[u]:upto[u]] for u in range(users)]).cuda()
+        n = sum(new)
+        bi = torch.empty(n, dtype=torch.int32, device="cuda")
+        pos = torch.empty_like(bi)
+        kvcache.get_paged_batch_indices_positions(W.offsets(new, torch.int32).cuda(), torch.tensor(upto, dtype=torch.int32).cuda(), bi, pos)
+        kc, vc = table.unbind(1)
+        kvcache.append_kvcache(k, v, bi, pos, torch.zeros(users, dtype=torch.int32, device="cuda"), torch.tensor([n], dtype=torch.int32).cuda(), n,
+                               kc, vc, ids.cuda(), po.cuda(), cfg["last_page_len"].cuda(), 0)
+        done = upto
+    torch.cuda.synchronize()
+    assert torch.equal(table.cpu(), ref_table)
+    out_ref, _ = T.run_capi(cfg, op="paged")
+    out, _ = T.run_capi(dict(cfg, kv_cache=table.cpu()), op="paged")
+    assert torch.equal(out, out_ref)
+    T.assert_parity(out, T.oracle_paged(cfg), dtype, what="paged forward over the appended table")
