@@ -22,7 +22,7 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
 # HBM-side bytes per launch from rocprofv3 FETCH_SIZE/WRITE_SIZE, each scaled by what the same counter reads for the
 # plain 256 MiB copy of `--workload copy` (factors 2.000 and 1.000); see profiles/hstu_mfma_kernel_configs2-5.md
-MEASURED_TRAFFIC_BYTES = {"config2": 184.3e6}
+MEASURED_TRAFFIC_BYTES = {"config2": 184.3e6, "kv_append": 351.9e6}
 
 
 def build_workload(name, torch, W):
@@ -228,28 +228,38 @@ def kv_append_bench(args, torch, W):
         kvcache.append_kvcache(dev["append_key"], dev["append_value"], bi, pos, dev["offsets"], dev["nnz_dev"], n, kc, vc,
                                dev["kv_indices"], dev["kv_indptr"], dev["kv_last_page_len"], 0)
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record()
-    for _ in range(args.steps):
-        step()
-    e1.record()
-    torch.cuda.synchronize()
-    ms = (time.perf_counter() - t0) * 1e3 / args.steps
-    kern_ms = e0.elapsed_time(e1) / args.steps
+    def append_only():
+        kvcache.append_kvcache(dev["append_key"], dev["append_value"], bi, pos, dev["offsets"], dev["nnz_dev"], n, kc, vc,
+                               dev["kv_indices"], dev["kv_indptr"], dev["kv_last_page_len"], 0)
+
+    def timed(fn):
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()
+        for _ in range(args.steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / args.steps, e0.elapsed_time(e1) / args.steps
+
+    ms, _ = timed(step)                 # the whole job: positions + append
+    _, kern_ms = timed(append_only)     # the dominant kernel alone, for the roofline
     row_bytes = 4 * 128 * 2
     alg_bytes = n * row_bytes * 4 + n * 4 * 4      # K, V rows read and written; batch_indices / positions written and read
+    kern_bytes = n * row_bytes * 4 + n * 2 * 4     # the append kernel: rows, and its two index arrays read
     out = {
         "metric": "paged_kv_append_gbps", "value": round(alg_bytes / (ms * 1e-3) / 1e9, 1), "unit": "GB/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "u16", "data": "synthetic", "us_per_call": round(ms * 1e3, 2),
         "config": {"workload": f"append of {n} new tokens (32 users x U[1024,4096]) x 4 heads x 128, bf16, 64-token pages, seed 0",
                    "algorithmic_bytes_per_call": alg_bytes, "entry": "hstu_hip_kv_token_positions + hstu_hip_kv_append (C ABI)"},
-        "roofline": {"bound": "hbm", "achieved": round(alg_bytes / (kern_ms * 1e-3) / 1e9, 1), "peak": 8000.0, "unit": "GB/s",
-                     "frac": round(alg_bytes / (kern_ms * 1e-3) / 1e9 / 8000.0, 4), "traffic": None, "kernel_us": round(kern_ms * 1e3, 2)},
+        "roofline": {"bound": "hbm", "kernel": "hstu_kv_append_kernel", "achieved": round(kern_bytes / (kern_ms * 1e-3) / 1e9, 1),
+                     "peak": 8000.0, "unit": "GB/s", "frac": round(kern_bytes / (kern_ms * 1e-3) / 1e9 / 8000.0, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES["kv_append"], "kernel_us": round(kern_ms * 1e3, 2),
+                     "algorithmic_bytes_per_launch": kern_bytes},
     }
     if not args.no_cpu_baseline:
         from oracle import kvcache_oracle as KO
