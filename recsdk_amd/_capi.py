@@ -1,4 +1,4 @@
-"""ctypes binding of the C ABI declared in ``include/hstu_hip.h`` and ``include/hstu_kvcache.h``.
+"""ctypes binding of the C ABI declared in ``include/hstu_hip.h``, ``include/hstu_kvcache.h`` and ``include/hstu_bias.h``.
 
 This is the thinnest possible host binding: raw device pointers and sizes in, status code out.
 It exists so that callers (and the parity tests) can drive the library without the torch op
@@ -28,6 +28,7 @@ EXPORTS = [
     "hstu_hip_dense_backward_get_workspace_size", "hstu_hip_dense_backward",
     "hstu_hip_last_error", "hstu_hip_describe_kernel", "hstu_hip_abi_version",
     "hstu_hip_kv_append", "hstu_hip_kv_token_positions",
+    "hstu_hip_rab_time", "hstu_hip_rab_time_backward", "hstu_hip_rab_pos",
 ]
 
 
@@ -72,6 +73,23 @@ class HstuKvAppendParams(C.Structure):
     ]
 
 
+class HstuRabTimeParams(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32), ("dtype", C.c_int32), ("index_type", C.c_int32), ("num_layers", C.c_int32),
+        ("batch", C.c_int32), ("seq_len", C.c_int32), ("weight_cols", C.c_int32), ("reserved", C.c_int32),
+        ("timestamps", C.c_void_p), ("weights", C.c_void_p), ("bucket_bounds", C.c_void_p),
+        ("rab_time_out", C.c_void_p), ("bucket_ts_out", C.c_void_p),
+    ]
+
+
+class HstuRabTimeBwdParams(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32), ("dtype", C.c_int32), ("index_type", C.c_int32), ("num_layers", C.c_int32),
+        ("batch", C.c_int32), ("seq_len", C.c_int32), ("num_buckets", C.c_int32), ("reserved", C.c_int32),
+        ("grad", C.c_void_p), ("bucket_ts", C.c_void_p), ("grad_weights", C.c_void_p),
+    ]
+
+
 _lib: Optional[C.CDLL] = None
 
 
@@ -96,6 +114,9 @@ def lib() -> C.CDLL:
             getattr(_lib, f"hstu_hip_{n}_backward_get_workspace_size").argtypes = [C.POINTER(HstuBwdParams), C.POINTER(C.c_uint64)]
         _lib.hstu_hip_describe_kernel.argtypes = [C.POINTER(HstuFwdParams), C.c_char_p, C.c_size_t]
         _lib.hstu_hip_kv_append.argtypes = [C.POINTER(HstuKvAppendParams), C.c_void_p]
+        _lib.hstu_hip_rab_time.argtypes = [C.POINTER(HstuRabTimeParams), C.c_void_p]
+        _lib.hstu_hip_rab_time_backward.argtypes = [C.POINTER(HstuRabTimeBwdParams), C.c_void_p]
+        _lib.hstu_hip_rab_pos.argtypes = [C.c_int32, C.c_int32, C.c_void_p, C.c_void_p, C.POINTER(C.c_int64), C.c_int32, C.c_void_p, C.c_void_p]
         _lib.hstu_hip_kv_token_positions.argtypes = [C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]
     return _lib
 

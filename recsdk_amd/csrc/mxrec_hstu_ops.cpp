@@ -19,6 +19,7 @@
 #include <mutex>
 
 #include "hstu_hip.h"
+#include "hstu_bias.h"
 
 namespace mxrec_hstu {
 
@@ -697,6 +698,144 @@ at::Tensor hstu_dense_autograd(const at::Tensor& q, const at::Tensor& k, const a
     return HstuDenseFunction::apply(q, k, v, mask, attn_bias, mask_type, max_seq_len, silu_scale);
 }
 
+// ---------------------------------------------------------------------------------------------
+// standalone bias producers (cust_op/framework/torch_plugin/torch_library/relative_attn_bias/)
+// ---------------------------------------------------------------------------------------------
+static void check_tensor_non_empty(const at::Tensor& t, const char* name) {   // common_utils.h:30-35
+    TORCH_CHECK(t.defined(), name, " tensor must be defined");
+    TORCH_CHECK(t.numel() > 0, name, " tensor must be non-empty");
+    TORCH_CHECK(t.dim() > 0, name, " tensor must have non-zero dimensions");
+}
+
+static int32_t index_dtype(const at::Tensor& t, const char* name) {
+    TORCH_CHECK(t.scalar_type() == at::kInt || t.scalar_type() == at::kLong, name, " dtype expect int32 or int64, but get ", t.scalar_type());
+    return t.scalar_type() == at::kLong ? HSTU_I64 : HSTU_I32;
+}
+
+// relative_attn_bias_time_impl (relative_attn_bias_time.cpp:29-62); the repeat of the reference's wrapper is part of the kernel
+static std::tuple<at::Tensor, at::Tensor> rab_time_impl(const at::Tensor& timestamps, const at::Tensor& weights, double bucket_divisor,
+                                                        const char* op) {
+    check_tensor_non_empty(timestamps, "timestampsConti");
+    check_tensor_non_empty(weights, "timestampsWeightsConti");
+    TORCH_CHECK(weights.dim() == 2, "timestampsWeightsConti must be 2D");
+    TORCH_CHECK(timestamps.dim() == 2, "timestampsConti must be 2D");
+    TORCH_CHECK(timestamps.device() == weights.device(), "timestamps and timestampsWeights must be on the same device");
+    TORCH_CHECK(bucket_divisor > 0, "bucket_divisor must be positive");
+    Holder h;
+    auto ts = h.same(timestamps), w = h.same(weights);
+    const int64_t n = w.size(0), cols = w.size(1), bs = ts.size(0), s = ts.size(1);
+    TORCH_CHECK(s > 0 && s <= HSTU_RAB_MAX_SEQ_LEN, "timestamps size must be between 1 and ", HSTU_RAB_MAX_SEQ_LEN);
+    hstu_rab_time_params p;
+    std::memset(&p, 0, sizeof(p));
+    p.struct_size = sizeof(p);
+    p.dtype = io_dtype(w, "timestamps_weights");
+    p.index_type = index_dtype(ts, "timestamps");
+    p.num_layers = (int32_t)n;
+    p.batch = (int32_t)bs;
+    p.seq_len = (int32_t)s;
+    p.weight_cols = (int32_t)cols;
+    require_gpu(w, op);
+    at::Tensor bounds = cols > 1 ? cached_bounds(cols - 1, bucket_divisor, w.device())
+                                 : at::tensor({0.0f, std::numeric_limits<float>::infinity()}).to(w.device());
+    auto out = at::empty({n, bs, 2 * s, 2 * s}, w.options());
+    auto ids = at::empty({bs, s, s}, ts.options());
+    p.timestamps = ts.const_data_ptr();
+    p.weights = w.const_data_ptr();
+    p.bucket_bounds = bounds.const_data_ptr<float>();
+    p.rab_time_out = out.data_ptr();
+    p.bucket_ts_out = ids.data_ptr();
+    c10::hip::OptionalHIPGuardMasqueradingAsCUDA guard(w.device());
+    auto stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA();
+    const int rc = hstu_hip_rab_time(&p, (void*)stream.stream());
+    TORCH_CHECK(rc == HSTU_OK, "mxrec::", op, ": ", hstu_hip_last_error());
+    return {out, ids};
+}
+
+// relative_attn_bias_time_backward_impl (relative_attn_bias_time.cpp:64-85)
+at::Tensor relative_attn_bias_time_backward(const at::Tensor& rab_time_grad, const at::Tensor& bucket_timestamps, int64_t num_buckets) {
+    check_tensor_non_empty(rab_time_grad, "rabTimeGrad");
+    check_tensor_non_empty(bucket_timestamps, "bucketTimestamps");
+    TORCH_CHECK(rab_time_grad.dim() == 4, "rabTimeGrad must be 4D");
+    Holder h;
+    auto g = h.same(rab_time_grad), ids = h.same(bucket_timestamps);
+    const int64_t n = g.size(0), bs = g.size(1), sx2 = g.size(2), s = sx2 / 2;
+    TORCH_CHECK(g.size(3) == sx2 && sx2 % 2 == 0 && ids.numel() == bs * s * s,
+                "Sequence len mismatch between grad(_, _, ", sx2, ", ", g.size(3), ") and bucket_timestamps of ", ids.numel(), " elements");
+    hstu_rab_time_bwd_params p;
+    std::memset(&p, 0, sizeof(p));
+    p.struct_size = sizeof(p);
+    p.dtype = io_dtype(g, "rab_time_grad");
+    p.index_type = index_dtype(ids, "bucket_timestamps");
+    p.num_layers = (int32_t)n;
+    p.batch = (int32_t)bs;
+    p.seq_len = (int32_t)s;
+    p.num_buckets = (int32_t)num_buckets;
+    require_gpu(g, "relative_attn_bias_time_backward");
+    auto out = at::empty({n, num_buckets > 0 ? num_buckets : 0}, g.options().dtype(at::kFloat));
+    p.grad = g.const_data_ptr();
+    p.bucket_ts = ids.const_data_ptr();
+    p.grad_weights = out.data_ptr<float>();
+    c10::hip::OptionalHIPGuardMasqueradingAsCUDA guard(g.device());
+    auto stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA();
+    const int rc = hstu_hip_rab_time_backward(&p, (void*)stream.stream());
+    TORCH_CHECK(rc == HSTU_OK, "mxrec::relative_attn_bias_time_backward: ", hstu_hip_last_error());
+    return g.scalar_type() == at::kFloat ? out : out.to(g.scalar_type());
+}
+
+at::Tensor relative_attn_bias_time(const at::Tensor& timestamps, const at::Tensor& weights, double bucket_divisor) {
+    return std::get<0>(rab_time_impl(timestamps, weights, bucket_divisor, "relative_attn_bias_time"));
+}
+
+std::vector<at::Tensor> relative_attn_bias_time_with_index(const at::Tensor& timestamps, const at::Tensor& weights, double bucket_divisor) {
+    auto r = rab_time_impl(timestamps, weights, bucket_divisor, "relative_attn_bias_time_with_index");
+    return {std::get<0>(r), std::get<1>(r)};
+}
+
+// autograd of relative_attn_bias_time, as the reference's RelativeAttnBiasTime (relative_attn_bias_time.cpp:101-131)
+class RabTimeFunction : public torch::autograd::Function<RabTimeFunction> {
+public:
+    static at::Tensor forward(torch::autograd::AutogradContext* ctx, const at::Tensor& timestamps, const at::Tensor& weights, double bucket_divisor) {
+        at::AutoDispatchBelowADInplaceOrView guard;
+        auto r = rab_time_impl(timestamps, weights, bucket_divisor, "relative_attn_bias_time");
+        ctx->save_for_backward({std::get<1>(r)});
+        ctx->saved_data["num_buckets"] = weights.size(1);
+        return std::get<0>(r);
+    }
+    static torch::autograd::tensor_list backward(torch::autograd::AutogradContext* ctx, torch::autograd::tensor_list grad_outputs) {
+        auto ids = ctx->get_saved_variables()[0];
+        auto gw = relative_attn_bias_time_backward(grad_outputs[0], ids, ctx->saved_data["num_buckets"].toInt());
+        return {at::Tensor(), gw, at::Tensor()};
+    }
+};
+
+at::Tensor relative_attn_bias_time_autograd(const at::Tensor& timestamps, const at::Tensor& weights, double bucket_divisor) {
+    return RabTimeFunction::apply(timestamps, weights, bucket_divisor);
+}
+
+// relative_attn_bias_pos_forward (relative_attn_bias_pos.cpp:22-43)
+at::Tensor relative_attn_bias_pos(const at::Tensor& rel_pos_bias, const at::Tensor& identity, at::IntArrayRef past_valid_lens) {
+    check_tensor_non_empty(rel_pos_bias, "relPosBias");
+    check_tensor_non_empty(identity, "identity");
+    TORCH_CHECK(rel_pos_bias.dim() == 2, "Invalid rel_pos_bias shape.");
+    TORCH_CHECK(identity.dim() == 2, "Invalid identity shape.");
+    TORCH_CHECK(rel_pos_bias.device() == identity.device(), "relPosBias and identity must be on the same device");
+    TORCH_CHECK(identity.scalar_type() == rel_pos_bias.scalar_type(), "Mismatch data type of identity and rel_pos_bias.");
+    Holder h;
+    auto rel = h.same(rel_pos_bias), ident = h.same(identity);
+    const int64_t sx2 = rel.size(0), bs = (int64_t)past_valid_lens.size();
+    TORCH_CHECK(rel.size(1) == sx2 && ident.size(0) == sx2 && ident.size(1) == sx2, "Mismatch sequence len of rel_pos_bias and identity.");
+    const int32_t dt = io_dtype(rel, "rel_pos_bias");
+    require_gpu(rel, "relative_attn_bias_pos");
+    auto out = at::empty({bs, sx2, sx2}, rel.options());
+    std::vector<int64_t> lens(past_valid_lens.begin(), past_valid_lens.end());
+    c10::hip::OptionalHIPGuardMasqueradingAsCUDA guard(rel.device());
+    auto stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA();
+    const int rc = hstu_hip_rab_pos(dt, (int32_t)sx2, rel.const_data_ptr(), ident.const_data_ptr(), lens.data(), (int32_t)bs, out.data_ptr(),
+                                    (void*)stream.stream());
+    TORCH_CHECK(rc == HSTU_OK, "mxrec::relative_attn_bias_pos: ", hstu_hip_last_error());
+    return out;
+}
+
 TORCH_LIBRARY_FRAGMENT(mxrec, m) {
     m.def("hstu_jagged.equal(Tensor q, "
           "                  Tensor k, "
@@ -796,6 +935,22 @@ TORCH_LIBRARY_FRAGMENT(mxrec, m) {
           "                    int mask_type=0, "
           "                    int max_seq_len=0, "
           "                    float silu_scale=0.0) -> (Tensor, Tensor, Tensor, Tensor)");
+    m.def("relative_attn_bias_pos(Tensor rel_pos_bias, "
+          "                       Tensor identity, "
+          "                       int[] past_valid_lens"
+          "                       ) -> Tensor");
+    m.def("relative_attn_bias_time(Tensor timestamps, "
+          "                        Tensor timestamps_weights, "
+          "                        float bucket_divisor"
+          "                        ) -> Tensor");
+    m.def("relative_attn_bias_time_backward(Tensor rab_time_grad, "
+          "                                 Tensor bucket_timestamps, "
+          "                                 int num_buckets"
+          "                                 ) -> Tensor");
+    m.def("relative_attn_bias_time_with_index(Tensor timestamps, "
+          "                                   Tensor timestamps_weights, "
+          "                                   float bucket_divisor"
+          "                                   ) -> Tensor[]");
     // no counterpart in the reference:
     m.def("hstu_jagged_table_bias(Tensor q, Tensor k, Tensor v, Tensor? pos_table=None, Tensor? ts_table=None, "
           "Tensor? timestamps=None, Tensor? attn_bias=None, int mask_type=0, int max_seq_len=0, int max_seq_len_k=0, "
@@ -818,7 +973,11 @@ TORCH_LIBRARY_FRAGMENT(mxrec, m) {
     m.impl("hstu_dense", TORCH_FN(hstu_dense));                               \
     m.impl("hstu_dense_backward", TORCH_FN(hstu_dense_backward));             \
     m.impl("hstu_jagged_table_bias", TORCH_FN(hstu_jagged_table_bias));       \
-    m.impl("hstu_paged_fp8", TORCH_FN(hstu_paged_fp8));
+    m.impl("hstu_paged_fp8", TORCH_FN(hstu_paged_fp8));                       \
+    m.impl("relative_attn_bias_pos", TORCH_FN(relative_attn_bias_pos));       \
+    m.impl("relative_attn_bias_time", TORCH_FN(relative_attn_bias_time));     \
+    m.impl("relative_attn_bias_time_backward", TORCH_FN(relative_attn_bias_time_backward)); \
+    m.impl("relative_attn_bias_time_with_index", TORCH_FN(relative_attn_bias_time_with_index));
 
 // ROCm tensors dispatch on the CUDA key.  The CPU key runs the same host checks and then
 // reports that there is no CPU implementation.
@@ -829,6 +988,7 @@ TORCH_LIBRARY_IMPL(mxrec, AutogradCUDA, m) {
     m.impl("hstu_jagged.equal", TORCH_FN(hstu_jagged_equal_autograd));
     m.impl("hstu_jagged.delta", TORCH_FN(hstu_jagged_delta_autograd));
     m.impl("hstu_dense", TORCH_FN(hstu_dense_autograd));
+    m.impl("relative_attn_bias_time", TORCH_FN(relative_attn_bias_time_autograd));   // relative_attn_bias_time.cpp:143-146
 }
 
 }  // namespace mxrec_hstu
