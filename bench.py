@@ -21,8 +21,8 @@ sys.path.insert(0, ROOT)
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
 # HBM-side bytes per launch from rocprofv3 FETCH_SIZE/WRITE_SIZE, each scaled by what the same counter reads for the
-# plain 256 MiB copy of `--workload copy` (factors 2.000 and 1.000); see profiles/hstu_mfma_kernel_configs2-5.md
-MEASURED_TRAFFIC_BYTES = {"config2": 184.3e6, "kv_append": 351.9e6}
+# plain 256 MiB copy of `--workload copy` (factors 2.000 and 1.000); see profiles/*.md
+MEASURED_TRAFFIC_BYTES = {"config2": 184.3e6, "kv_append": 351.9e6, "rab_time": 1479.8e6, "rab_time_bwd": 2242.4e6, "rab_pos": 305.2e6}
 
 
 def build_workload(name, torch, W):
@@ -57,7 +57,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=1000)
-    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "config2_bwd", "kv_append", "copy"],
+    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "config2_bwd", "kv_append", "rab_time", "rab_time_bwd", "rab_pos", "copy"],
                     help="'copy' runs a plain 256 MiB device copy: the known-size kernel the FETCH_SIZE/WRITE_SIZE counters are scaled by")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
@@ -75,6 +75,8 @@ def main():
         return backward_bench(args, torch, W, _capi)
     if args.workload == "kv_append":
         return kv_append_bench(args, torch, W)
+    if args.workload in ("rab_time", "rab_time_bwd", "rab_pos"):
+        return bias_bench(args, torch)
     cfg, op, flops, alg_bytes, desc = build_workload(args.workload, torch, W)
     dev = W.to_device(cfg)
     q, k, v = dev["q"], dev["k"], dev["v"]
@@ -272,6 +274,87 @@ def kv_append_bench(args, torch, W):
         dt = time.perf_counter() - t0
         out["cpu_baseline"] = {"value": round(alg_bytes / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
                                "sample": f"the whole append once, token loop in numpy, {dt:.2f} s"}
+    print(json.dumps(out), flush=True)
+
+
+def bias_bench(args, torch):
+    """The standalone bias producers at the reference's evaluation shape (test_relative_attn_bias.py:106-113): 8 layers,
+    train_len 2000 + 600 candidates -> s = 2300, 4 users, fp16 tables, int32 timestamps.  HBM-bound: the (2s)^2 outputs
+    (the gradient input for the backward) dominate the bytes."""
+    import torch.nn.functional as F  # noqa: F401
+    from oracle import bias_oracle as BO
+    n, bs, train, cand = 8, 4, 2000, 600
+    s = train + cand // 2
+    g = torch.Generator().manual_seed(0)
+    lens = torch.randint(0, train, (bs,), generator=g).tolist()
+    ts = torch.zeros(bs, s)
+    for i, v in enumerate(lens):
+        ts[i, :v] = torch.arange(1, v + 1)
+    ts[:, -(cand // 2):] = train + 1
+    ts = ts.to(torch.int32)
+    w = (torch.arange(129, dtype=torch.float32).repeat(n).reshape(n, 129) + torch.randn(n, 129, generator=g)).half()
+    m = torch.ops.mxrec
+    esz = 2
+    if args.workload == "rab_time":
+        tsd, wd = ts.cuda(), w.cuda()
+        fn = lambda: m.relative_attn_bias_time_with_index(tsd, wd, 0.301)
+        alg = n * bs * 4 * s * s * esz + bs * s * s * 4 + bs * s * 4
+        kernel, desc = "hstu_rab_time_kernel", "rab_time_out [8,4,4600,4600] fp16 + bucket ids [4,2300,2300] int32 written"
+        cpu = lambda: BO.rab_time(ts, w, 0.301)
+        cpu_bytes = alg
+        sample = "the whole call once (oracle in torch)"
+    elif args.workload == "rab_time_bwd":
+        grad = (torch.randn(n, bs, 2 * s, 2 * s, generator=g, dtype=torch.float16) * 1e-2).cuda()
+        ids = BO.time_buckets(ts).to(torch.int32)
+        idd = ids.cuda()
+        fn = lambda: m.relative_attn_bias_time_backward(grad, idd, 129)
+        alg = n * bs * 4 * s * s * esz + bs * s * s * 4
+        kernel, desc = "hstu_rab_time_bwd_kernel", "grad [8,4,4600,4600] fp16 and ids [4,2300,2300] int32 read (algorithmic: once each)"
+        gc = grad[:, :1].cpu()
+        cpu = lambda: BO.rab_time_backward(gc, ids[:1], 129)
+        cpu_bytes = alg // bs
+        sample = "one of the four users once (oracle in torch, fp64 sums)"
+    else:
+        s2 = 2 * s
+        rel = torch.randn(s2, s2, generator=g).half()
+        idx = torch.arange(s).repeat(s).view(s, s).unsqueeze(-1).repeat(1, 2, 2).reshape(s2, s2)
+        ident = (idx.t() == idx).half().contiguous()
+        reld, identd = rel.cuda(), ident.cuda()
+        fn = lambda: m.relative_attn_bias_pos(reld, identd, lens)
+        alg = bs * s2 * s2 * esz + 2 * s2 * s2 * esz
+        kernel, desc = "hstu_rab_pos_kernel", "out [4,4600,4600] fp16 written, the two [4600,4600] tables read"
+        cpu = lambda: [BO.rab_pos(rel, ident, lens) for _ in range(20)]
+        cpu_bytes = 20 * alg
+        sample = "the whole call 20 times (oracle in torch)"
+
+    for _ in range(args.warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    kern_ms = e0.elapsed_time(e1) / args.steps
+    out = {
+        "metric": f"{args.workload}_gbps", "value": round(alg / (ms * 1e-3) / 1e9, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic", "us_per_call": round(ms * 1e3, 2),
+        "config": {"workload": f"{args.workload}: 8 layers, 4 users, s = 2300 (train 2000 + 600 candidates), fp16, seed 0; {desc}",
+                   "algorithmic_bytes_per_call": alg, "entry": f"torch.ops.mxrec.* -> {kernel} (C ABI in include/hstu_bias.h)"},
+        "roofline": {"bound": "hbm", "kernel": kernel, "achieved": round(alg / (kern_ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(alg / (kern_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                     "kernel_us": round(kern_ms * 1e3, 2)},
+    }
+    if not args.no_cpu_baseline:
+        t0 = time.perf_counter()
+        cpu()
+        dt = time.perf_counter() - t0
+        out["cpu_baseline"] = {"value": round(cpu_bytes / dt / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"{sample}, {dt:.2f} s"}
     print(json.dumps(out), flush=True)
 
 

@@ -34,7 +34,8 @@ typedef struct hstu_rab_time_params {
     int32_t batch;
     int32_t seq_len;            /* s */
     int32_t weight_cols;        /* W */
-    int32_t reserved;
+    float bucket_divisor;       /* the divisor the bounds were made for: a first guess only, the ids are decided by
+                                   bucket_bounds; <= 0: not known */
     const void* timestamps;     /* [batch, s] */
     const void* weights;        /* [num_layers, W] */
     const float* bucket_bounds; /* [W + 1] */

@@ -76,7 +76,7 @@ class HstuKvAppendParams(C.Structure):
 class HstuRabTimeParams(C.Structure):
     _fields_ = [
         ("struct_size", C.c_uint32), ("dtype", C.c_int32), ("index_type", C.c_int32), ("num_layers", C.c_int32),
-        ("batch", C.c_int32), ("seq_len", C.c_int32), ("weight_cols", C.c_int32), ("reserved", C.c_int32),
+        ("batch", C.c_int32), ("seq_len", C.c_int32), ("weight_cols", C.c_int32), ("bucket_divisor", C.c_float),
         ("timestamps", C.c_void_p), ("weights", C.c_void_p), ("bucket_bounds", C.c_void_p),
         ("rab_time_out", C.c_void_p), ("bucket_ts_out", C.c_void_p),
     ]

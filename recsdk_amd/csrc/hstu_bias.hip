@@ -24,23 +24,45 @@ __device__ __forceinline__ float abs_diff_f32(I a, I b) {
     return (float)d;
 }
 
-// grid: x = column groups of RAB_NT * RAB_JPT, y = b * s + i
+// Bucket of x from the bounds table: a first guess from the hardware log2 (within one of the answer), settled by
+// comparisons with the table, so the id is the table's whatever the guess was.  inv = ln 2 / divisor, or 0: search only.
+__device__ __forceinline__ int bucket_of(const float* bounds, int nb, float x, float inv) {
+    if (inv > 0.f) {
+        int e = min((int)(__log2f(fmaxf(x, 1.0f)) * inv), nb);
+        if (x < bounds[e]) e--;
+        else if (x >= bounds[e + 1]) e++;
+        if (e >= 0 && e <= nb && x >= bounds[e] && x < bounds[e + 1]) return e;
+    }
+    return ts_bucket(bounds, nb, x);
+}
+
+// grid: x = (b * s + i) * column groups + column group of RAB_NT * RAB_JPT.  The table sits in LDS transposed,
+// [bucket][layer], so that one bucket's values for all layers are one or a few 16-byte reads.
 template <typename T, typename I>
 __global__ __launch_bounds__(RAB_NT) void hstu_rab_time_kernel(const hstu_rab_time_params p) {
+    constexpr int LPV = 16 / sizeof(T);   // layers per 16-byte read
+    constexpr int MAXL = (HSTU_RAB_MAX_LAYERS + LPV - 1) / LPV * LPV;
+    typedef __attribute__((ext_vector_type(4))) unsigned int u4;
     __shared__ float bounds[HSTU_RAB_MAX_BUCKETS + 1];
-    const int W = p.weight_cols, s = p.seq_len;
+    __shared__ __attribute__((aligned(16))) T wtab[HSTU_RAB_MAX_BUCKETS * MAXL];
+    const int W = p.weight_cols, s = p.seq_len, nl = p.num_layers;
+    const int lpad = (nl + LPV - 1) / LPV * LPV;
     for (int k = threadIdx.x; k <= W; k += RAB_NT) bounds[k] = p.bucket_bounds[k];
+    for (int k = threadIdx.x; k < nl * W; k += RAB_NT) wtab[(k % W) * lpad + k / W] = reinterpret_cast<const T*>(p.weights)[k];
     __syncthreads();
-    const int b = blockIdx.y / s, i = blockIdx.y % s;
-    const int j0 = (blockIdx.x * RAB_NT + threadIdx.x) * RAB_JPT;
+    const unsigned groups = (unsigned)(s + RAB_NT * RAB_JPT - 1) / (RAB_NT * RAB_JPT);
+    const unsigned row = blockIdx.x / groups;
+    const int b = row / s, i = row % s;
+    const int j0 = ((blockIdx.x % groups) * RAB_NT + threadIdx.x) * RAB_JPT;
     if (j0 >= s) return;
+    const float inv = p.bucket_divisor > 0.f ? 0.69314718f / p.bucket_divisor : 0.f;
     const I* ts = reinterpret_cast<const I*>(p.timestamps) + (int64_t)b * s;
     const I ti = ts[i];
     int bucket[RAB_JPT];
 #pragma unroll
     for (int k = 0; k < RAB_JPT; k++) {
         const int j = min(j0 + k, s - 1);
-        bucket[k] = ts_bucket(bounds, W - 1, abs_diff_f32<I>(ti, ts[j]));
+        bucket[k] = bucket_of(bounds, W - 1, abs_diff_f32<I>(ti, ts[j]), inv);
     }
     if (p.bucket_ts_out) {
         I* bo = reinterpret_cast<I*>(p.bucket_ts_out) + ((int64_t)b * s + i) * s;
@@ -48,39 +70,55 @@ __global__ __launch_bounds__(RAB_NT) void hstu_rab_time_kernel(const hstu_rab_ti
         for (int k = 0; k < RAB_JPT; k++)
             if (j0 + k < s) bo[j0 + k] = (I)bucket[k];
     }
-    const T* w = reinterpret_cast<const T*>(p.weights);
     T* out = reinterpret_cast<T*>(p.rab_time_out);
     const int64_t s2 = 2 * (int64_t)s;
     const bool wide = j0 + RAB_JPT <= s && (s2 * sizeof(T)) % 16 == 0;   // whole group, rows start on 16-byte boundaries
-    for (int n = 0; n < p.num_layers; n++) {
-        T v[RAB_JPT];
+    for (int n0 = 0; n0 < nl; n0 += LPV) {
+        T v[RAB_JPT][LPV];
 #pragma unroll
-        for (int k = 0; k < RAB_JPT; k++) v[k] = w[n * W + bucket[k]];
-        T* row = out + (((int64_t)n * p.batch + b) * s2 + 2 * i) * s2 + 2 * j0;
-        if (wide) {
-            T pk[2 * RAB_JPT];
+        for (int k = 0; k < RAB_JPT; k++) *reinterpret_cast<u4*>(v[k]) = *reinterpret_cast<const u4*>(wtab + bucket[k] * lpad + n0);
 #pragma unroll
-            for (int k = 0; k < RAB_JPT; k++) pk[2 * k] = pk[2 * k + 1] = v[k];
-            typedef __attribute__((ext_vector_type(4))) unsigned int u4;
-            constexpr int NV = 2 * RAB_JPT * sizeof(T) / 16;
-            const u4* src = reinterpret_cast<const u4*>(pk);
+        for (int l = 0; l < LPV; l++) {
+            const int n = n0 + l;
+            if (n >= nl) break;
+            T* orow = out + (((int64_t)n * p.batch + b) * s2 + 2 * i) * s2 + 2 * j0;
+            if (wide) {
+                T pk[2 * RAB_JPT];
 #pragma unroll
-            for (int q = 0; q < NV; q++) {
-                reinterpret_cast<u4*>(row)[q] = src[q];
-                reinterpret_cast<u4*>(row + s2)[q] = src[q];
-            }
-        } else {
+                for (int k = 0; k < RAB_JPT; k++) pk[2 * k] = pk[2 * k + 1] = v[k][l];
+                constexpr int NV = 2 * RAB_JPT * sizeof(T) / 16;
+                const u4* src = reinterpret_cast<const u4*>(pk);
 #pragma unroll
-            for (int k = 0; k < RAB_JPT; k++) {
-                if (j0 + k >= s) break;
-                row[2 * k] = row[2 * k + 1] = v[k];
-                row[s2 + 2 * k] = row[s2 + 2 * k + 1] = v[k];
+                for (int q = 0; q < NV; q++) {
+                    __builtin_nontemporal_store(src[q], reinterpret_cast<u4*>(orow) + q);
+                    __builtin_nontemporal_store(src[q], reinterpret_cast<u4*>(orow + s2) + q);
+                }
+            } else {
+#pragma unroll
+                for (int k = 0; k < RAB_JPT; k++) {
+                    if (j0 + k >= s) break;
+                    orow[2 * k] = orow[2 * k + 1] = v[k][l];
+                    orow[s2 + 2 * k] = orow[s2 + 2 * k + 1] = v[k][l];
+                }
             }
         }
     }
 }
 
-// grid: x = column groups, y = row groups of RAB_ROWS rows i, z = n * batch + b
+// sum of x over the 64 lanes
+__device__ __forceinline__ float wave_sum(float x) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o, 64);
+    return x;
+}
+
+// grid: x = column groups of 64 * RAB_JPT, y = row groups of RAB_ROWS rows i, z = n * batch + b; wave w takes rows
+// w, w + 4, ...  Neighbouring columns mostly share a bucket, so equal neighbours are first merged inside a lane and the
+// lanes of a wave that hold one id are then summed across the wave (one LDS atomic per distinct id and wave instead of
+// 64 colliding ones).  A workgroup per layer re-reads the ids for every layer (a third of the gradient's bytes again
+// at fp16) but measured fastest at 8 layers: 480 us, against 620-720 us with 4 layers per workgroup and 630-940 us
+// with all of them -- the reduction leaves a wave's loads idle, and more workgroups hide that better than fewer
+// bytes do.
 constexpr int RAB_ROWS = 16;
 template <typename T, typename I>
 __global__ __launch_bounds__(RAB_NT) void hstu_rab_time_bwd_kernel(const hstu_rab_time_bwd_params p) {
@@ -89,15 +127,20 @@ __global__ __launch_bounds__(RAB_NT) void hstu_rab_time_bwd_kernel(const hstu_ra
     for (int k = threadIdx.x; k < nb; k += RAB_NT) hist[k] = 0.f;
     __syncthreads();
     const int n = blockIdx.z / p.batch, b = blockIdx.z % p.batch;
-    const int j0 = (blockIdx.x * RAB_NT + threadIdx.x) * RAB_JPT;
+    const int lane = threadIdx.x & 63;
+    const int j0 = (blockIdx.x * 64 + lane) * RAB_JPT;
     const int64_t s2 = 2 * (int64_t)s;
     const T* g = reinterpret_cast<const T*>(p.grad) + ((int64_t)n * p.batch + b) * s2 * s2;
     const I* bt = reinterpret_cast<const I*>(p.bucket_ts) + (int64_t)b * s * s;
     const bool wide = j0 + RAB_JPT <= s && (s2 * sizeof(T)) % 16 == 0;
-    if (j0 < s) {
-        for (int i = blockIdx.y * RAB_ROWS; i < min((int)(blockIdx.y + 1) * RAB_ROWS, s); i++) {
+    const int i_end = min((int)(blockIdx.y + 1) * RAB_ROWS, s);
+    for (int i = blockIdx.y * RAB_ROWS + (threadIdx.x >> 6); i < i_end; i += RAB_NT / 64) {   // wave-uniform
+        float sum[RAB_JPT];
+        int id[RAB_JPT];
+#pragma unroll
+        for (int k = 0; k < RAB_JPT; k++) { sum[k] = 0.f; id[k] = -1; }
+        if (j0 < s) {
             const T* row = g + (2 * (int64_t)i) * s2 + 2 * j0;
-            float sum[RAB_JPT];
             if (wide) {
                 typedef __attribute__((ext_vector_type(4))) unsigned int u4;
                 constexpr int NV = 2 * RAB_JPT * sizeof(T) / 16;
@@ -112,17 +155,33 @@ __global__ __launch_bounds__(RAB_NT) void hstu_rab_time_bwd_kernel(const hstu_ra
                     sum[k] = (to_float(r0[2 * k]) + to_float(r0[2 * k + 1])) + (to_float(r1[2 * k]) + to_float(r1[2 * k + 1]));
             } else {
 #pragma unroll
-                for (int k = 0; k < RAB_JPT; k++) {
-                    sum[k] = 0.f;
+                for (int k = 0; k < RAB_JPT; k++)
                     if (j0 + k < s)
                         sum[k] = (to_float(row[2 * k]) + to_float(row[2 * k + 1])) + (to_float(row[s2 + 2 * k]) + to_float(row[s2 + 2 * k + 1]));
-                }
             }
 #pragma unroll
             for (int k = 0; k < RAB_JPT; k++) {
                 if (j0 + k >= s) break;
-                const int64_t id = (int64_t)bt[(int64_t)i * s + j0 + k];
-                if (id >= 0 && id < nb) atomicAdd(&hist[id], sum[k]);
+                const int64_t v = (int64_t)bt[(int64_t)i * s + j0 + k];
+                id[k] = (v >= 0 && v < nb) ? (int)v : -1;
+            }
+            // equal neighbours inside the lane first
+#pragma unroll
+            for (int k = RAB_JPT - 1; k > 0; k--)
+                if (id[k] == id[k - 1] && id[k] >= 0) { sum[k - 1] += sum[k]; id[k] = -1; }
+        }
+#pragma unroll
+        for (int k = 0; k < RAB_JPT; k++) {
+            bool todo = id[k] >= 0;
+            unsigned long long m = __ballot(todo);
+            while (m) {   // wave-uniform loop: one pass per distinct id still pending
+                const int leader = __ffsll((long long)m) - 1;
+                const int lid = __shfl(id[k], leader, 64);
+                const bool mine = todo && id[k] == lid;
+                const float tot = wave_sum(mine ? sum[k] : 0.f);
+                if (lane == leader) atomicAdd(&hist[lid], tot);
+                todo = todo && !mine;
+                m = __ballot(todo);
             }
         }
     }
@@ -144,37 +203,67 @@ struct RabPosLens {
 template <typename T> __device__ __forceinline__ float rnd(float x) { return to_float(from_float<T>(x)); }
 template <> __device__ __forceinline__ float rnd<float>(float x) { return x; }
 
-// grid: x = column groups of RAB_NT * 8, y = row, z = user within this launch
+// grid: x = column groups of RAB_NT * 8, y = row; the users of this launch one after the other, so that the identity
+// row and rel row i (what every user with past_valid_len >= i takes) are read once.  A lane takes 8 consecutive columns
+// with 16-byte (fp32: two) accesses when the rows start on 16-byte boundaries, else the 8 columns lane + 256 * k.
 template <typename T>
-__global__ __launch_bounds__(RAB_NT) void hstu_rab_pos_kernel(const T* rel, const T* identity, T* out, int seq2, RabPosLens lens) {
-    const int i = blockIdx.y, u = blockIdx.z;
-    const int src_row = min(i, lens.v[u]);
+__global__ __launch_bounds__(RAB_NT) void hstu_rab_pos_kernel(const T* rel, const T* identity, T* out, int seq2, int users, RabPosLens lens) {
+    const int i = blockIdx.y;
     const float r00 = to_float(rel[0]);
-    const T* rrow = rel + (int64_t)src_row * seq2;
     const T* irow = identity + (int64_t)i * seq2;
-    T* orow = out + ((int64_t)u * seq2 + i) * seq2;
-    const int j0 = (blockIdx.x * RAB_NT + threadIdx.x) * 8;
-#pragma unroll
-    for (int k = 0; k < 8; k++) {
-        const int j = j0 + k;
-        if (j >= seq2) break;
-        const float id = to_float(irow[j]), r = to_float(rrow[j]);
+    auto blend = [&](T r_, T id_) __attribute__((always_inline)) -> T {
+        const float id = to_float(id_), r = to_float(r_);
         // the golden's tensor expression, one rounding per operation (exact for a 0/1 identity)
         const float keep = rnd<T>(__fmul_rn(r, rnd<T>(__fsub_rn(1.0f, id))));
         const float fill = rnd<T>(__fmul_rn(id, r00));
-        orow[j] = from_float<T>(__fadd_rn(keep, fill));
+        return from_float<T>(__fadd_rn(keep, fill));
+    };
+    const int base = blockIdx.x * RAB_NT * 8;
+    const int j0 = base + threadIdx.x * 8;
+    if (seq2 % 8 == 0) {
+        if (j0 >= seq2) return;
+        typedef __attribute__((ext_vector_type(4))) unsigned int u4;
+        constexpr int NV = 8 * sizeof(T) / 16;
+        T own[8], d[8];
+#pragma unroll
+        for (int q = 0; q < NV; q++) {
+            reinterpret_cast<u4*>(own)[q] = reinterpret_cast<const u4*>(rel + (int64_t)i * seq2 + j0)[q];
+            reinterpret_cast<u4*>(d)[q] = reinterpret_cast<const u4*>(irow + j0)[q];
+        }
+        for (int u = 0; u < users; u++) {
+            T r[8], o[8];
+            const int v = lens.v[u];
+#pragma unroll
+            for (int q = 0; q < NV; q++)
+                reinterpret_cast<u4*>(r)[q] = i <= v ? reinterpret_cast<const u4*>(own)[q] : reinterpret_cast<const u4*>(rel + (int64_t)v * seq2 + j0)[q];
+#pragma unroll
+            for (int k = 0; k < 8; k++) o[k] = blend(r[k], d[k]);
+            T* orow = out + ((int64_t)u * seq2 + i) * seq2;
+#pragma unroll
+            for (int q = 0; q < NV; q++) __builtin_nontemporal_store(reinterpret_cast<const u4*>(o)[q], reinterpret_cast<u4*>(orow + j0) + q);
+        }
+    } else {
+        for (int u = 0; u < users; u++) {
+            const T* rrow = rel + (int64_t)min(i, lens.v[u]) * seq2;
+            T* orow = out + ((int64_t)u * seq2 + i) * seq2;
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                const int j = base + threadIdx.x + RAB_NT * k;
+                if (j < seq2) orow[j] = blend(rrow[j], irow[j]);
+            }
+        }
     }
 }
 
 template <typename T, typename I>
 static void launch_rab_time(const hstu_rab_time_params& p, hipStream_t st) {
     const unsigned gx = (unsigned)((p.seq_len + RAB_NT * RAB_JPT - 1) / (RAB_NT * RAB_JPT));
-    hipLaunchKernelGGL((hstu_rab_time_kernel<T, I>), dim3(gx, (unsigned)(p.batch * p.seq_len)), dim3(RAB_NT), 0, st, p);
+    hipLaunchKernelGGL((hstu_rab_time_kernel<T, I>), dim3(gx * (unsigned)(p.batch * p.seq_len)), dim3(RAB_NT), 0, st, p);
 }
 
 template <typename T, typename I>
 static void launch_rab_time_bwd(const hstu_rab_time_bwd_params& p, hipStream_t st) {
-    const unsigned gx = (unsigned)((p.seq_len + RAB_NT * RAB_JPT - 1) / (RAB_NT * RAB_JPT));
+    const unsigned gx = (unsigned)((p.seq_len + 64 * RAB_JPT - 1) / (64 * RAB_JPT));
     const unsigned gy = (unsigned)((p.seq_len + RAB_ROWS - 1) / RAB_ROWS);
     hipLaunchKernelGGL((hstu_rab_time_bwd_kernel<T, I>), dim3(gx, gy, (unsigned)(p.num_layers * p.batch)), dim3(RAB_NT), 0, st, p);
 }
@@ -186,8 +275,8 @@ static void launch_rab_pos(int seq2, const void* rel, const void* identity, cons
         RabPosLens l;
         const int nu = batch - u0 < RAB_POS_USERS ? batch - u0 : RAB_POS_USERS;
         for (int u = 0; u < RAB_POS_USERS; u++) l.v[u] = u < nu ? (int)lens[u0 + u] : 0;
-        hipLaunchKernelGGL((hstu_rab_pos_kernel<T>), dim3(gx, (unsigned)seq2, (unsigned)nu), dim3(RAB_NT), 0, st, reinterpret_cast<const T*>(rel),
-                           reinterpret_cast<const T*>(identity), reinterpret_cast<T*>(out) + (int64_t)u0 * seq2 * seq2, seq2, l);
+        hipLaunchKernelGGL((hstu_rab_pos_kernel<T>), dim3(gx, (unsigned)seq2), dim3(RAB_NT), 0, st, reinterpret_cast<const T*>(rel),
+                           reinterpret_cast<const T*>(identity), reinterpret_cast<T*>(out) + (int64_t)u0 * seq2 * seq2, seq2, nu, l);
     }
 }
 
@@ -228,7 +317,6 @@ extern "C" int hstu_hip_rab_time(const hstu_rab_time_params* p, void* stream) {
     if (!p->timestamps || !p->weights || !p->bucket_bounds || !p->rab_time_out)
         return fail(HSTU_ERR_INVALID_ARGUMENT, "timestamps, weights, bucket_bounds and rab_time_out must not be NULL");
     if (reinterpret_cast<uintptr_t>(p->rab_time_out) & 15) return fail(HSTU_ERR_UNSUPPORTED, "rab_time_out must be 16-byte aligned");
-    if ((int64_t)p->batch * p->seq_len > 65535 * 32768LL) return fail(HSTU_ERR_UNSUPPORTED, "batch * s too large for one launch");
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     RAB_DISPATCH(p->dtype, p->index_type, launch_rab_time, *p, st);
     return launched();
@@ -245,8 +333,8 @@ extern "C" int hstu_hip_rab_time_backward(const hstu_rab_time_bwd_params* p, voi
         return fail(HSTU_ERR_INVALID_ARGUMENT, "num_buckets expects a value in the range [1, %d], but the actual value is %d.", HSTU_RAB_MAX_BUCKETS, p->num_buckets);
     if (p->seq_len <= 0 || p->seq_len > HSTU_RAB_MAX_SEQ_LEN)
         return fail(HSTU_ERR_INVALID_ARGUMENT, "Sequence len expects a value in the range [1, %d], but the actual value is %d.", 2 * HSTU_RAB_MAX_SEQ_LEN, 2 * p->seq_len);
-    if (p->batch <= 0 || (int64_t)p->batch * p->num_layers > 65535)
-        return fail(HSTU_ERR_INVALID_ARGUMENT, "Batchsize expects a positive value with num_layer * batchsize <= 65535, but the actual value is %d.", p->batch);
+    if (p->batch <= 0 || p->batch > 65535 / HSTU_RAB_MAX_LAYERS)
+        return fail(HSTU_ERR_INVALID_ARGUMENT, "Batchsize expects a value in the range [1, %d], but the actual value is %d.", 65535 / HSTU_RAB_MAX_LAYERS, p->batch);
     if (!p->grad || !p->bucket_ts || !p->grad_weights) return fail(HSTU_ERR_INVALID_ARGUMENT, "grad, bucket_ts and grad_weights must not be NULL");
     if (reinterpret_cast<uintptr_t>(p->grad) & 15) return fail(HSTU_ERR_UNSUPPORTED, "grad must be 16-byte aligned");
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);

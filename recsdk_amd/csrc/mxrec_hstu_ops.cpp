@@ -734,6 +734,7 @@ static std::tuple<at::Tensor, at::Tensor> rab_time_impl(const at::Tensor& timest
     p.batch = (int32_t)bs;
     p.seq_len = (int32_t)s;
     p.weight_cols = (int32_t)cols;
+    p.bucket_divisor = (float)bucket_divisor;
     require_gpu(w, op);
     at::Tensor bounds = cols > 1 ? cached_bounds(cols - 1, bucket_divisor, w.device())
                                  : at::tensor({0.0f, std::numeric_limits<float>::infinity()}).to(w.device());
