@@ -1,0 +1,84 @@
+/*
+ * hstu_layer.h -- C ABI of the step after the attention in an HSTU layer: LayerNorm(x) * u with dropout, forward and
+ * backward (mxrec::norm_multiply_dropout).
+ *
+ * Same conventions as hstu_hip.h: device pointers, asynchronous on `stream`, nothing read on the host, 0 or a negative
+ * hstu_status with the message in hstu_hip_last_error().  dtype: HSTU_F32 / HSTU_F16 / HSTU_BF16 for x, u, weight,
+ * bias and the outputs shaped like them.
+ *
+ *   x_hat = (x - mean) / sqrt(var + eps)              mean, var over the columns of a row (var biased), fp32
+ *   y     = dropout((x_hat * weight + bias) * u, p)   dropout: kept elements scaled by 1 / (1 - p)
+ * (cust_op/ascendc_op/ai_core_op/norm_multiply_dropout/v220/README.md:41-60).
+ *
+ * Dropout mask: bit (e % 8) of byte (e / 8) is 1 where flat element e = row * cols + col is kept; the buffer holds
+ * ceil(rows * cols / 128) * 16 bytes like the reference's (norm_multiply_dropout.cpp:38-45).  The forward fills it
+ * from (seed, element index) with a counter-based generator of this library; which elements are dropped therefore
+ * differs from the reference's generator (aclnnDropoutGenMaskV2), as it differs between any two seeds.
+ */
+#ifndef HSTU_LAYER_H
+#define HSTU_LAYER_H
+
+#include "hstu_hip.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HSTU_NMD_MAX_ROWS 1000000 /* norm_multiply_dropout.cpp:28-31: rows in [1, 1e6], cols 512 or 1024 */
+
+/* Replaces aclnnNormMultiplyDropout (norm_multiply_dropout.cpp:69-94). */
+typedef struct hstu_nmd_params {
+    uint32_t struct_size;
+    int32_t dtype;
+    int64_t rows;
+    int32_t cols;
+    float eps;             /* [1e-10, 1e-4] */
+    float dropout_ratio;   /* [0, 1]; <= 1e-10: no dropout, drop_mask is neither written nor read */
+    uint32_t reserved;
+    uint64_t seed;
+    const void* x;         /* [rows, cols] */
+    const void* u;         /* [rows, cols] */
+    const void* weight;    /* [cols] */
+    const void* bias;      /* [cols] */
+    void* out;             /* [rows, cols] */
+    float* mean;           /* [rows] */
+    float* var;            /* [rows] */
+    uint8_t* drop_mask;    /* see above; may be NULL without dropout */
+} hstu_nmd_params;
+int hstu_hip_norm_multiply_dropout(const hstu_nmd_params* p, void* stream);
+
+/* Replaces aclnnNormMultiplyDropoutBackward (norm_multiply_dropout.cpp:97-111; formulas of the golden
+ * cust_op/test/norm_multiply_dropout/torch/test_norm_multiply_dropout.py:220-243):
+ *   g = dropout'(d_out) * u          d_weight = sum over rows of x_hat * g        d_bias = sum over rows of g
+ *   a = g * weight                   d_x = (a - (sum_c a + x_hat * sum_c a * x_hat) / cols) / sqrt(var + eps)
+ *   d_u = dropout'(d_out) * (weight * x_hat + bias)
+ * The column sums are formed in a fixed order (per-workgroup partial sums in the workspace, then one pass over them):
+ * results are reproducible. */
+typedef struct hstu_nmd_bwd_params {
+    uint32_t struct_size;
+    int32_t dtype;
+    int64_t rows;
+    int32_t cols;
+    float eps;
+    float dropout_ratio;
+    uint32_t reserved;
+    const void* d_out;
+    const void* x;
+    const void* u;
+    const void* weight;
+    const void* bias;
+    const float* mean;         /* from the forward */
+    const float* var;
+    const uint8_t* drop_mask;  /* from the forward; may be NULL without dropout */
+    void* d_x;
+    void* d_u;
+    float* d_weight;           /* [cols] fp32, overwritten */
+    float* d_bias;             /* [cols] fp32, overwritten */
+} hstu_nmd_bwd_params;
+int hstu_hip_norm_multiply_dropout_backward_get_workspace_size(const hstu_nmd_bwd_params* p, uint64_t* workspace_bytes);
+int hstu_hip_norm_multiply_dropout_backward(const hstu_nmd_bwd_params* p, void* workspace, uint64_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HSTU_LAYER_H */

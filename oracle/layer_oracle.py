@@ -1,0 +1,60 @@
+"""CPU oracle for ``mxrec::norm_multiply_dropout``.  TEST INFRASTRUCTURE ONLY.
+
+Restates the reference's goldens; used by ``tests/`` and by the ``cpu_baseline`` leg of ``bench.py``.  Nothing in the
+shipped package imports it.
+
+Definition followed (reference file:line):
+
+* forward: cust_op/ascendc_op/ai_core_op/norm_multiply_dropout/v220/README.md:41-60 -- LayerNorm over the last axis
+  (biased variance, affine), times u, dropout (kept elements scaled by 1/(1-p)), computed in a wider type and rounded
+  once to the I/O dtype; mean and var as the explicit golden returns them
+  (cust_op/test/norm_multiply_dropout/torch/test_norm_multiply_dropout.py:137-156).
+* backward: test_norm_multiply_dropout.py:220-243 (``ln_mul_bwd``), with the upstream gradient passed through the
+  dropout mask first.
+* mask layout: bit (e % 8) of byte (e / 8) = element e kept.  WHICH elements a seed keeps is this build's own choice
+  (the reference draws its mask from aclnnDropoutGenMaskV2 and its tests only check that the call runs,
+  test_norm_multiply_dropout.py:336-342): parity with the reference's random stream is neither possible nor claimed;
+  the tests check the op against this oracle under the mask the op itself returned, and the keep rate.
+
+Everything here is fp64 so that it can serve as the exact value for every I/O dtype.
+
+Pinning status (tests/test_oracle_layer.py): forward against ``torch.nn.functional.layer_norm`` (a library routine
+that shares no code with the explicit mean / var formula here) and ``F.dropout`` semantics under a given mask; backward
+against autograd through that library forward, including the mask.  PINNED
+"""
+from __future__ import annotations
+
+import torch
+
+
+def unpack_mask(mask_bytes: torch.Tensor, numel: int) -> torch.Tensor:
+    """uint8 ``[ceil(numel/128)*16]`` -> bool ``[numel]`` (bit e % 8 of byte e / 8)."""
+    bits = (mask_bytes.to(torch.int32)[:, None] >> torch.arange(8, dtype=torch.int32)[None, :]) & 1
+    return bits.reshape(-1)[:numel].bool()
+
+
+def nmd_forward(x, u, weight, bias, eps: float, dropout_ratio: float = 0.0, keep=None):
+    """Returns (y, mean, var) in fp64; ``keep``: bool ``[rows, cols]`` when ``dropout_ratio`` > 1e-10."""
+    x, u, weight, bias = (t.double() for t in (x, u, weight, bias))
+    mean = x.mean(dim=1, keepdim=True)
+    var = ((x - mean) ** 2).mean(dim=1, keepdim=True)
+    y = ((x - mean) / torch.sqrt(var + eps) * weight + bias) * u
+    if dropout_ratio > 1e-10:
+        y = torch.where(keep, y / (1.0 - dropout_ratio), torch.zeros_like(y)) if dropout_ratio < 1 else torch.zeros_like(y)
+    return y, mean[:, 0], var[:, 0]
+
+
+def nmd_backward(d_out, x, u, weight, bias, mean, var, eps: float, dropout_ratio: float = 0.0, keep=None):
+    """Returns (d_x, d_u, d_weight, d_bias) in fp64."""
+    dy, x, u, weight, bias = (t.double() for t in (d_out, x, u, weight, bias))
+    mean, var = mean.double()[:, None], var.double()[:, None]
+    if dropout_ratio > 1e-10:
+        dy = torch.where(keep, dy / (1.0 - dropout_ratio), torch.zeros_like(dy)) if dropout_ratio < 1 else torch.zeros_like(dy)
+    rstd = 1.0 / torch.sqrt(var + eps)
+    xh = (x - mean) * rstd
+    g = dy * u
+    a = g * weight
+    c = x.shape[1]
+    dx = (a - (a.sum(dim=1, keepdim=True) + xh * (a * xh).sum(dim=1, keepdim=True)) / c) * rstd
+    du = dy * (weight * xh + bias)
+    return dx, du, (xh * g).sum(dim=0), g.sum(dim=0)

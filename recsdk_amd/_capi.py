@@ -1,4 +1,4 @@
-"""ctypes binding of the C ABI declared in ``include/hstu_hip.h``, ``include/hstu_kvcache.h`` and ``include/hstu_bias.h``.
+"""ctypes binding of the C ABI declared in ``include/*.h``.
 
 This is the thinnest possible host binding: raw device pointers and sizes in, status code out.
 It exists so that callers (and the parity tests) can drive the library without the torch op
@@ -29,6 +29,8 @@ EXPORTS = [
     "hstu_hip_last_error", "hstu_hip_describe_kernel", "hstu_hip_abi_version",
     "hstu_hip_kv_append", "hstu_hip_kv_token_positions",
     "hstu_hip_rab_time", "hstu_hip_rab_time_backward", "hstu_hip_rab_pos",
+    "hstu_hip_norm_multiply_dropout", "hstu_hip_norm_multiply_dropout_backward",
+    "hstu_hip_norm_multiply_dropout_backward_get_workspace_size",
 ]
 
 
@@ -90,6 +92,25 @@ class HstuRabTimeBwdParams(C.Structure):
     ]
 
 
+class HstuNmdParams(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32), ("dtype", C.c_int32), ("rows", C.c_int64), ("cols", C.c_int32), ("eps", C.c_float),
+        ("dropout_ratio", C.c_float), ("reserved", C.c_uint32), ("seed", C.c_uint64),
+        ("x", C.c_void_p), ("u", C.c_void_p), ("weight", C.c_void_p), ("bias", C.c_void_p), ("out", C.c_void_p),
+        ("mean", C.c_void_p), ("var", C.c_void_p), ("drop_mask", C.c_void_p),
+    ]
+
+
+class HstuNmdBwdParams(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32), ("dtype", C.c_int32), ("rows", C.c_int64), ("cols", C.c_int32), ("eps", C.c_float),
+        ("dropout_ratio", C.c_float), ("reserved", C.c_uint32),
+        ("d_out", C.c_void_p), ("x", C.c_void_p), ("u", C.c_void_p), ("weight", C.c_void_p), ("bias", C.c_void_p),
+        ("mean", C.c_void_p), ("var", C.c_void_p), ("drop_mask", C.c_void_p), ("d_x", C.c_void_p), ("d_u", C.c_void_p),
+        ("d_weight", C.c_void_p), ("d_bias", C.c_void_p),
+    ]
+
+
 _lib: Optional[C.CDLL] = None
 
 
@@ -115,6 +136,9 @@ def lib() -> C.CDLL:
         _lib.hstu_hip_describe_kernel.argtypes = [C.POINTER(HstuFwdParams), C.c_char_p, C.c_size_t]
         _lib.hstu_hip_kv_append.argtypes = [C.POINTER(HstuKvAppendParams), C.c_void_p]
         _lib.hstu_hip_rab_time.argtypes = [C.POINTER(HstuRabTimeParams), C.c_void_p]
+        _lib.hstu_hip_norm_multiply_dropout.argtypes = [C.POINTER(HstuNmdParams), C.c_void_p]
+        _lib.hstu_hip_norm_multiply_dropout_backward.argtypes = [C.POINTER(HstuNmdBwdParams), C.c_void_p, C.c_uint64, C.c_void_p]
+        _lib.hstu_hip_norm_multiply_dropout_backward_get_workspace_size.argtypes = [C.POINTER(HstuNmdBwdParams), C.POINTER(C.c_uint64)]
         _lib.hstu_hip_rab_time_backward.argtypes = [C.POINTER(HstuRabTimeBwdParams), C.c_void_p]
         _lib.hstu_hip_rab_pos.argtypes = [C.c_int32, C.c_int32, C.c_void_p, C.c_void_p, C.POINTER(C.c_int64), C.c_int32, C.c_void_p, C.c_void_p]
         _lib.hstu_hip_kv_token_positions.argtypes = [C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]

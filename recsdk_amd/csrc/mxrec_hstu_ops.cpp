@@ -9,6 +9,7 @@
 // libhstu_hip.so on the current stream.  There is no CPU implementation: CPU tensors get the same
 // argument checks and then a clear error.
 #include <ATen/ATen.h>
+#include <ATen/CPUGeneratorImpl.h>
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <torch/csrc/autograd/custom_function.h>
@@ -20,6 +21,7 @@
 
 #include "hstu_hip.h"
 #include "hstu_bias.h"
+#include "hstu_layer.h"
 
 namespace mxrec_hstu {
 
@@ -837,6 +839,151 @@ at::Tensor relative_attn_bias_pos(const at::Tensor& rel_pos_bias, const at::Tens
     return out;
 }
 
+// ---------------------------------------------------------------------------------------------
+// norm_multiply_dropout (cust_op/framework/torch_plugin/torch_library/norm_multiply_dropout/norm_multiply_dropout.cpp)
+// ---------------------------------------------------------------------------------------------
+static void nmd_check_params(const at::Tensor& x, const at::Tensor& u, const at::Tensor& weight, const at::Tensor& bias, double eps,
+                             double dropout_ratio) {   // check_params, norm_multiply_dropout.cpp:150-171
+    TORCH_CHECK(x.dim() == 2, "norm_multiply_dropout input x must be 2D");
+    TORCH_CHECK(u.dim() == 2, "norm_multiply_dropout input u must be 2D");
+    TORCH_CHECK(weight.dim() == 1, "norm_multiply_dropout input weight must be 1D");
+    TORCH_CHECK(bias.dim() == 1, "norm_multiply_dropout input bias must be 1D");
+    const auto d0 = x.size(0), d1 = x.size(1);
+    TORCH_CHECK(d0 == u.size(0), "param input x dim0: ", d0, " is not equal to u dim0: ", u.size(0));
+    TORCH_CHECK(d1 == u.size(1), "param input x dim1: ", d1, " is not equal to u dim1: ", u.size(1));
+    TORCH_CHECK(d1 == weight.size(0) && weight.size(0) == bias.size(0), "param input x dim1: ", d1, ", weight dim0: ", weight.size(0),
+                ", bias dim0:", bias.size(0), " must be same but not equal.");
+    TORCH_CHECK(d0 >= 1 && d0 <= HSTU_NMD_MAX_ROWS, "x dim0 must in range:[1,", HSTU_NMD_MAX_ROWS, "].");
+    TORCH_CHECK(d1 == 512 || d1 == 1024, "x dim1 must equal with ", 512, " or ", 1024);
+    TORCH_CHECK(eps >= 1e-10 && eps <= 1e-4, "eps must in range:[", 1e-10, ",", 1e-4, "].");
+    TORCH_CHECK(dropout_ratio >= 0.0 && dropout_ratio <= 1.0, "dropout_ratio must in range:[", 0.0, ",", 1.0, "].");
+    TORCH_CHECK(u.scalar_type() == x.scalar_type() && weight.scalar_type() == x.scalar_type() && bias.scalar_type() == x.scalar_type(),
+                "u, weight and bias must have the dtype of x");
+}
+
+// norm_multiply_dropout_impl_npu (norm_multiply_dropout.cpp:69-94): {result, mean, var, drop_mask}
+static std::vector<at::Tensor> nmd_forward_impl(const at::Tensor& x, const at::Tensor& u, const at::Tensor& weight, const at::Tensor& bias,
+                                                double eps, double dropout_ratio) {
+    Holder h;
+    auto dx = h.same(x), du = h.same(u), dw = h.same(weight), db = h.same(bias);
+    hstu_nmd_params p;
+    std::memset(&p, 0, sizeof(p));
+    p.struct_size = sizeof(p);
+    p.dtype = io_dtype(dx, "x");
+    p.rows = dx.size(0);
+    p.cols = (int32_t)dx.size(1);
+    p.eps = (float)eps;
+    p.dropout_ratio = (float)dropout_ratio;
+    require_gpu(dx, "norm_multiply_dropout");
+    const bool drop = std::fabs(dropout_ratio) > 1e-10;
+    auto out = at::empty_like(dx);
+    auto mean = at::empty({dx.size(0)}, dx.options().dtype(at::kFloat));
+    auto var = at::empty({dx.size(0)}, dx.options().dtype(at::kFloat));
+    at::Tensor mask;
+    if (drop) {
+        mask = at::empty({(dx.numel() + 127) / 128 * 16}, dx.options().dtype(at::kByte));
+        auto gen = at::detail::getDefaultCPUGenerator();
+        std::lock_guard<std::mutex> lock(gen.mutex());
+        p.seed = at::check_generator<at::CPUGeneratorImpl>(gen)->random64();
+    } else {
+        mask = at::empty({1}, dx.options().dtype(at::kByte));
+    }
+    p.x = dx.const_data_ptr();
+    p.u = du.const_data_ptr();
+    p.weight = dw.const_data_ptr();
+    p.bias = db.const_data_ptr();
+    p.out = out.data_ptr();
+    p.mean = mean.data_ptr<float>();
+    p.var = var.data_ptr<float>();
+    p.drop_mask = mask.data_ptr<uint8_t>();
+    c10::hip::OptionalHIPGuardMasqueradingAsCUDA guard(dx.device());
+    auto stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA();
+    const int rc = hstu_hip_norm_multiply_dropout(&p, (void*)stream.stream());
+    TORCH_CHECK(rc == HSTU_OK, "mxrec::norm_multiply_dropout: ", hstu_hip_last_error());
+    return {out, mean, var, mask};
+}
+
+// norm_multiply_dropout_backward_impl_npu (norm_multiply_dropout.cpp:97-111): {d_x, d_u, d_weight, d_bias}
+static std::vector<at::Tensor> nmd_backward_impl(const at::Tensor& d_out, const at::Tensor& x, const at::Tensor& u, const at::Tensor& weight,
+                                                 const at::Tensor& bias, const at::Tensor& mean, const at::Tensor& var, const at::Tensor& mask,
+                                                 double eps, double dropout_ratio) {
+    Holder h;
+    auto dy = h.same(d_out), dx = h.same(x), du = h.same(u), dw = h.same(weight), db = h.same(bias), dm = h.same(mean), dv = h.same(var), dk = h.same(mask);
+    TORCH_CHECK(dy.sizes() == dx.sizes() && dy.scalar_type() == dx.scalar_type(), "d_out must have the shape and dtype of x");
+    hstu_nmd_bwd_params p;
+    std::memset(&p, 0, sizeof(p));
+    p.struct_size = sizeof(p);
+    p.dtype = io_dtype(dx, "x");
+    p.rows = dx.size(0);
+    p.cols = (int32_t)dx.size(1);
+    p.eps = (float)eps;
+    p.dropout_ratio = (float)dropout_ratio;
+    require_gpu(dx, "norm_multiply_dropout");
+    auto gx = at::empty_like(dx), gu = at::empty_like(dx);
+    auto gw = at::empty({dx.size(1)}, dx.options().dtype(at::kFloat)), gb = at::empty({dx.size(1)}, dx.options().dtype(at::kFloat));
+    p.d_out = dy.const_data_ptr();
+    p.x = dx.const_data_ptr();
+    p.u = du.const_data_ptr();
+    p.weight = dw.const_data_ptr();
+    p.bias = db.const_data_ptr();
+    p.mean = dm.const_data_ptr<float>();
+    p.var = dv.const_data_ptr<float>();
+    p.drop_mask = dk.const_data_ptr<uint8_t>();
+    p.d_x = gx.data_ptr();
+    p.d_u = gu.data_ptr();
+    p.d_weight = gw.data_ptr<float>();
+    p.d_bias = gb.data_ptr<float>();
+    uint64_t ws_bytes = 0;
+    int rc = hstu_hip_norm_multiply_dropout_backward_get_workspace_size(&p, &ws_bytes);
+    TORCH_CHECK(rc == HSTU_OK, "mxrec::norm_multiply_dropout: ", hstu_hip_last_error());
+    auto ws = at::empty({(int64_t)ws_bytes}, dx.options().dtype(at::kByte));
+    c10::hip::OptionalHIPGuardMasqueradingAsCUDA guard(dx.device());
+    auto stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA();
+    rc = hstu_hip_norm_multiply_dropout_backward(&p, ws.data_ptr(), ws_bytes, (void*)stream.stream());
+    TORCH_CHECK(rc == HSTU_OK, "mxrec::norm_multiply_dropout: ", hstu_hip_last_error());
+    return {gx, gu, gw, gb};
+}
+
+// NormMultiplyDropout (norm_multiply_dropout.cpp:114-148)
+class NmdFunction : public torch::autograd::Function<NmdFunction> {
+public:
+    static torch::autograd::tensor_list forward(torch::autograd::AutogradContext* ctx, const at::Tensor& x, const at::Tensor& u,
+                                                const at::Tensor& weight, const at::Tensor& bias, double eps, double dropout_ratio) {
+        at::AutoDispatchBelowADInplaceOrView guard;
+        auto outs = nmd_forward_impl(x, u, weight, bias, eps, dropout_ratio);
+        ctx->save_for_backward({x, u, weight, bias, outs[1], outs[2], outs[3]});
+        ctx->saved_data["eps"] = eps;
+        ctx->saved_data["dropout_ratio"] = dropout_ratio;
+        return {outs[0]};
+    }
+    static torch::autograd::tensor_list backward(torch::autograd::AutogradContext* ctx, torch::autograd::tensor_list grad_outputs) {
+        auto s = ctx->get_saved_variables();
+        auto g = nmd_backward_impl(grad_outputs[0], s[0], s[1], s[2], s[3], s[4], s[5], s[6], ctx->saved_data["eps"].toDouble(),
+                                   ctx->saved_data["dropout_ratio"].toDouble());
+        // the parameter gradients are accumulated in fp32 and handed over in the parameters' dtype
+        return {g[0], g[1], g[2].to(s[2].scalar_type()), g[3].to(s[3].scalar_type()), at::Tensor(), at::Tensor()};
+    }
+};
+
+std::vector<at::Tensor> norm_multiply_dropout(const at::Tensor& x, const at::Tensor& u, const at::Tensor& weight, const at::Tensor& bias, double eps,
+                                              double dropout_ratio) {
+    nmd_check_params(x, u, weight, bias, eps, dropout_ratio);
+    return NmdFunction::apply(x, u, weight, bias, eps, dropout_ratio);
+}
+
+// the two halves as plain ops (no counterpart in the reference's registrations, which expose the pair only through autograd)
+std::vector<at::Tensor> norm_multiply_dropout_forward(const at::Tensor& x, const at::Tensor& u, const at::Tensor& weight, const at::Tensor& bias,
+                                                      double eps, double dropout_ratio) {
+    nmd_check_params(x, u, weight, bias, eps, dropout_ratio);
+    return nmd_forward_impl(x, u, weight, bias, eps, dropout_ratio);
+}
+std::vector<at::Tensor> norm_multiply_dropout_backward(const at::Tensor& d_out, const at::Tensor& x, const at::Tensor& u, const at::Tensor& weight,
+                                                       const at::Tensor& bias, const at::Tensor& mean, const at::Tensor& var, const at::Tensor& mask,
+                                                       double eps, double dropout_ratio) {
+    nmd_check_params(x, u, weight, bias, eps, dropout_ratio);
+    return nmd_backward_impl(d_out, x, u, weight, bias, mean, var, mask, eps, dropout_ratio);
+}
+
 TORCH_LIBRARY_FRAGMENT(mxrec, m) {
     m.def("hstu_jagged.equal(Tensor q, "
           "                  Tensor k, "
@@ -952,7 +1099,12 @@ TORCH_LIBRARY_FRAGMENT(mxrec, m) {
           "                                   Tensor timestamps_weights, "
           "                                   float bucket_divisor"
           "                                   ) -> Tensor[]");
+    m.def("norm_multiply_dropout(Tensor x, Tensor u, Tensor weight, Tensor bias, float eps, float dropout_ratio) -> "
+          "Tensor[]");
     // no counterpart in the reference:
+    m.def("norm_multiply_dropout_forward(Tensor x, Tensor u, Tensor weight, Tensor bias, float eps, float dropout_ratio) -> Tensor[]");
+    m.def("norm_multiply_dropout_backward(Tensor d_out, Tensor x, Tensor u, Tensor weight, Tensor bias, Tensor mean, Tensor var, Tensor mask, "
+          "float eps, float dropout_ratio) -> Tensor[]");
     m.def("hstu_jagged_table_bias(Tensor q, Tensor k, Tensor v, Tensor? pos_table=None, Tensor? ts_table=None, "
           "Tensor? timestamps=None, Tensor? attn_bias=None, int mask_type=0, int max_seq_len=0, int max_seq_len_k=0, "
           "float silu_scale=0.0, Tensor seq_offset=None, Tensor seq_offset_k=None, Tensor? num_context=None, "
@@ -978,7 +1130,9 @@ TORCH_LIBRARY_FRAGMENT(mxrec, m) {
     m.impl("relative_attn_bias_pos", TORCH_FN(relative_attn_bias_pos));       \
     m.impl("relative_attn_bias_time", TORCH_FN(relative_attn_bias_time));     \
     m.impl("relative_attn_bias_time_backward", TORCH_FN(relative_attn_bias_time_backward)); \
-    m.impl("relative_attn_bias_time_with_index", TORCH_FN(relative_attn_bias_time_with_index));
+    m.impl("relative_attn_bias_time_with_index", TORCH_FN(relative_attn_bias_time_with_index)); \
+    m.impl("norm_multiply_dropout_forward", TORCH_FN(norm_multiply_dropout_forward));           \
+    m.impl("norm_multiply_dropout_backward", TORCH_FN(norm_multiply_dropout_backward));
 
 // ROCm tensors dispatch on the CUDA key.  The CPU key runs the same host checks and then
 // reports that there is no CPU implementation.
@@ -991,5 +1145,10 @@ TORCH_LIBRARY_IMPL(mxrec, AutogradCUDA, m) {
     m.impl("hstu_dense", TORCH_FN(hstu_dense_autograd));
     m.impl("relative_attn_bias_time", TORCH_FN(relative_attn_bias_time_autograd));   // relative_attn_bias_time.cpp:143-146
 }
+// norm_multiply_dropout is registered under the device key and the Autograd key with one function, like the reference
+// (norm_multiply_dropout.cpp:185-192): the checks, then the autograd Function
+TORCH_LIBRARY_IMPL(mxrec, CUDA, m) { m.impl("norm_multiply_dropout", TORCH_FN(norm_multiply_dropout)); }
+TORCH_LIBRARY_IMPL(mxrec, CPU, m) { m.impl("norm_multiply_dropout", TORCH_FN(norm_multiply_dropout)); }
+TORCH_LIBRARY_IMPL(mxrec, Autograd, m) { m.impl("norm_multiply_dropout", TORCH_FN(norm_multiply_dropout)); }
 
 }  // namespace mxrec_hstu

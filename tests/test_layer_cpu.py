@@ -1,0 +1,58 @@
+"""Host-side checks of norm_multiply_dropout (no GPU needed): the C ABI's validation and the torch op's schema, checks
+and messages (the reference's own exception tests, test_norm_multiply_dropout.py:365-470, run on the CPU key here)."""
+import ctypes as C
+
+import pytest
+import torch
+
+import recsdk_amd  # noqa: F401
+from recsdk_amd import _capi
+
+
+def _params(cls=_capi.HstuNmdParams, **over):
+    p = cls()
+    p.struct_size = C.sizeof(cls)
+    p.dtype, p.rows, p.cols, p.eps, p.dropout_ratio = _capi.HSTU_BF16, 100, 512, 1e-5, 0.0
+    for name, _ in cls._fields_:
+        if name in ("x", "u", "weight", "bias", "out", "mean", "var", "d_out", "d_x", "d_u", "d_weight", "d_bias"):
+            setattr(p, name, 0x1000)
+    for k, v in over.items():
+        setattr(p, k, v)
+    return p
+
+
+def test_c_abi_validation():
+    L = _capi.lib()
+    err = lambda: L.hstu_hip_last_error().decode()
+    for over, text in ((dict(struct_size=3), "size mismatch"), (dict(rows=0), "x dim0 must in range:[1,1000000]"),
+                       (dict(rows=1000001), "x dim0 must in range"), (dict(cols=768), "x dim1 must equal with 512 or 1024"),
+                       (dict(eps=1e-3), "eps must in range"), (dict(eps=1e-11), "eps must in range"), (dict(dropout_ratio=1.5), "dropout_ratio must in range"),
+                       (dict(dropout_ratio=-0.1), "dropout_ratio must in range"), (dict(dtype=9), "dtype expect"), (dict(u=None), "must not be NULL"),
+                       (dict(dropout_ratio=0.3), "drop_mask with dropout")):
+        assert L.hstu_hip_norm_multiply_dropout(C.byref(_params(**over)), None) == -1 and text in err(), (over, err())
+    assert L.hstu_hip_norm_multiply_dropout(C.byref(_params(x=0x1004)), None) == -2 and "16-byte aligned" in err()
+    b = _params(_capi.HstuNmdBwdParams)
+    n = C.c_uint64(0)
+    assert L.hstu_hip_norm_multiply_dropout_backward_get_workspace_size(C.byref(b), C.byref(n)) == 0
+    assert n.value == 25 * 2 * 512 * 4           # 100 rows -> 25 workgroups of 4 rows, one [2, cols] fp32 partial each
+    big = _params(_capi.HstuNmdBwdParams, rows=1000000, cols=1024)
+    assert L.hstu_hip_norm_multiply_dropout_backward_get_workspace_size(C.byref(big), C.byref(n)) == 0 and n.value == 1024 * 2 * 1024 * 4
+    assert L.hstu_hip_norm_multiply_dropout_backward(C.byref(b), None, 0, None) == -3 and "workspace" in err()
+    assert L.hstu_hip_norm_multiply_dropout_backward(C.byref(_params(_capi.HstuNmdBwdParams, d_x=None)), 0x1000, 1 << 20, None) == -1
+
+
+def test_torch_op_schema_and_checks():
+    m = torch.ops.mxrec
+    assert str(m.norm_multiply_dropout.default._schema) == \
+        "mxrec::norm_multiply_dropout(Tensor x, Tensor u, Tensor weight, Tensor bias, float eps, float dropout_ratio) -> Tensor[]"
+    x, w = torch.zeros(8, 512, dtype=torch.float16), torch.zeros(512, dtype=torch.float16)
+    run = lambda x_=x, u_=x, w_=w, b_=w, eps=1e-5, r=0.1: m.norm_multiply_dropout(x_, u_, w_, b_, eps, r)
+    for kw, text in ((dict(x_=x[None]), "norm_multiply_dropout input x must be 2D"), (dict(u_=x[None]), "norm_multiply_dropout input u must be 2D"),
+                     (dict(w_=w[None]), "norm_multiply_dropout input weight must be 1D"), (dict(b_=w[None]), "norm_multiply_dropout input bias must be 1D"),
+                     (dict(u_=x[:4]), "is not equal to u dim0"), (dict(u_=torch.zeros(8, 1024, dtype=torch.float16)), "is not equal to u dim1"),
+                     (dict(b_=w[:256]), "must be same but not equal"), (dict(x_=torch.zeros(8, 768, dtype=torch.float16), u_=torch.zeros(8, 768, dtype=torch.float16),
+                                                                        w_=torch.zeros(768, dtype=torch.float16), b_=torch.zeros(768, dtype=torch.float16)), "x dim1 must equal with"),
+                     (dict(eps=1e-11), "eps must in range"), (dict(eps=1e-3), "eps must in range"), (dict(r=-0.1), "dropout_ratio must in range"),
+                     (dict(r=1.1), "dropout_ratio must in range"), (dict(), "no CPU implementation")):
+        with pytest.raises(RuntimeError, match=text):
+            run(**kw)

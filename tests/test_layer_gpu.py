@@ -1,0 +1,102 @@
+"""GPU parity of norm_multiply_dropout (forward and backward, through the torch op and its autograd formula, which call
+the C ABI) against the fp64 oracle on the reference's test inputs (uniform [-1, 1), seed 321;
+test_norm_multiply_dropout.py:105-118).  Floating point: the tolerances of this build (fp32 1e-5 relative to the
+tensor's scale, bf16 / fp16 rtol = atol = 2e-2); the column sums d_weight / d_bias are fp32 sums over all rows, compared
+relative to their scale."""
+import sys
+
+import pytest
+import torch
+
+import recsdk_amd  # noqa: F401
+from oracle import layer_oracle as LO
+from tests import hstu_testlib as T
+
+pytestmark = pytest.mark.gpu
+EPS = 1e-5
+
+
+def say(*a):
+    print("[case]", *a, flush=True)
+    sys.stdout.flush()
+
+
+def _inputs(dim0, dim1, dtype):
+    g = torch.Generator().manual_seed(321)
+    mk = lambda *s: (torch.rand(*s, generator=g) * 2 - 1).to(dtype)
+    return mk(dim0, dim1), mk(dim0, dim1), mk(dim1), mk(dim1), mk(dim0, dim1)
+
+
+def _close(got, want, dtype, what, colsum=False):
+    got, want = got.double().cpu(), want.double()
+    if dtype == torch.float32 or colsum:
+        tol = 1e-5 if dtype == torch.float32 else 4e-3
+        scale = float(want.abs().max()) or 1.0
+        assert float((got - want).abs().max()) <= tol * scale, f"{what}: {float((got - want).abs().max()):.3e} vs scale {scale:.3e}"
+    else:
+        assert torch.allclose(got, want, rtol=2e-2, atol=2e-2), what
+
+
+@pytest.mark.parametrize("dim0", [1, 1000, 2345, 16384])
+@pytest.mark.parametrize("dim1", [512, 1024])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_forward_and_backward_without_dropout(dim0, dim1, dtype):
+    say("nmd", dim0, dim1, dtype)
+    x, u, w, b, dy = _inputs(dim0, dim1, dtype)
+    y_want, mean_want, var_want = LO.nmd_forward(x, u, w, b, EPS)
+    leaves = [t.cuda().requires_grad_(True) for t in (x, u, w, b)]
+    outs = torch.ops.mxrec.norm_multiply_dropout(*leaves, EPS, 0.0)
+    assert len(outs) == 1 and outs[0].dtype == dtype
+    _close(outs[0].detach(), y_want, dtype, "y")
+    outs[0].backward(dy.cuda())
+    want = LO.nmd_backward(dy, x, u, w, b, mean_want, var_want, EPS)
+    _close(leaves[0].grad, want[0], dtype, "d_x")
+    _close(leaves[1].grad, want[1], dtype, "d_u")
+    assert leaves[2].grad.dtype == dtype
+    # the fp32 column sums before the cast to the parameter dtype
+    raw = torch.ops.mxrec.norm_multiply_dropout_forward(x.cuda(), u.cuda(), w.cuda(), b.cuda(), EPS, 0.0)
+    assert torch.allclose(raw[1].cpu().double(), mean_want, rtol=0, atol=2e-6) and torch.allclose(raw[2].cpu().double(), var_want, rtol=1e-5, atol=1e-6)
+    g = torch.ops.mxrec.norm_multiply_dropout_backward(dy.cuda(), x.cuda(), u.cuda(), w.cuda(), b.cuda(), raw[1], raw[2], raw[3], EPS, 0.0)
+    assert g[2].dtype == torch.float32 and g[3].dtype == torch.float32
+    _close(g[2], want[2], dtype, "d_weight", colsum=True)
+    _close(g[3], want[3], dtype, "d_bias", colsum=True)
+    # reproducible: the column sums are formed in a fixed order
+    g2 = torch.ops.mxrec.norm_multiply_dropout_backward(dy.cuda(), x.cuda(), u.cuda(), w.cuda(), b.cuda(), raw[1], raw[2], raw[3], EPS, 0.0)
+    assert all(torch.equal(a, c) for a, c in zip(g, g2))
+
+
+@pytest.mark.parametrize("dim1,dtype,ratio", [(512, torch.bfloat16, 0.3), (1024, torch.float32, 0.3), (512, torch.float16, 0.75)])
+def test_dropout_under_the_mask_the_op_returns(dim1, dtype, ratio):
+    say("nmd dropout", dim1, dtype, ratio)
+    dim0 = 3000
+    x, u, w, b, dy = _inputs(dim0, dim1, dtype)
+    torch.manual_seed(5)
+    y, mean, var, mask = torch.ops.mxrec.norm_multiply_dropout_forward(x.cuda(), u.cuda(), w.cuda(), b.cuda(), EPS, ratio)
+    assert mask.dtype == torch.uint8 and mask.numel() == (dim0 * dim1 + 127) // 128 * 16
+    keep = LO.unpack_mask(mask.cpu(), dim0 * dim1).reshape(dim0, dim1)
+    rate = float(keep.double().mean())
+    assert abs(rate - (1 - ratio)) < 4 * (ratio * (1 - ratio) / keep.numel()) ** 0.5 + 2e-5, rate     # 16-bit threshold: 1.5e-5 resolution
+    # rows and columns are not correlated with the mask
+    assert abs(float(keep[:, ::7].double().mean()) - rate) < 5e-3 and abs(float(keep[::5].double().mean()) - rate) < 5e-3
+    y_want, mean_want, var_want = LO.nmd_forward(x, u, w, b, EPS, ratio, keep)
+    _close(y, y_want, dtype, "y with dropout")
+    assert torch.equal(y.cpu() == 0, ~keep | (y.cpu() == 0))
+    g = torch.ops.mxrec.norm_multiply_dropout_backward(dy.cuda(), x.cuda(), u.cuda(), w.cuda(), b.cuda(), mean, var, mask, EPS, ratio)
+    want = LO.nmd_backward(dy, x, u, w, b, mean_want, var_want, EPS, ratio, keep)
+    _close(g[0], want[0], dtype, "d_x with dropout")
+    _close(g[1], want[1], dtype, "d_u with dropout")
+    _close(g[2], want[2], dtype, "d_weight with dropout", colsum=True)
+    _close(g[3], want[3], dtype, "d_bias with dropout", colsum=True)
+    # same seed, same mask; another seed, another mask
+    torch.manual_seed(5)
+    again = torch.ops.mxrec.norm_multiply_dropout_forward(x.cuda(), u.cuda(), w.cuda(), b.cuda(), EPS, ratio)[3]
+    other = torch.ops.mxrec.norm_multiply_dropout_forward(x.cuda(), u.cuda(), w.cuda(), b.cuda(), EPS, ratio)[3]
+    assert torch.equal(again, mask) and not torch.equal(other, mask)
+    # through autograd (the reference's only route, test_norm_multiply_dropout.py:336-342)
+    leaves = [t.cuda().requires_grad_(True) for t in (x, u, w, b)]
+    out = torch.ops.mxrec.norm_multiply_dropout(*leaves, EPS, ratio)[0]
+    out.backward(dy.cuda())
+    assert all(l.grad is not None and bool(torch.isfinite(l.grad).all()) for l in leaves)
+    # everything dropped
+    y1 = torch.ops.mxrec.norm_multiply_dropout_forward(x.cuda(), u.cuda(), w.cuda(), b.cuda(), EPS, 1.0)[0]
+    assert not bool(y1.any())

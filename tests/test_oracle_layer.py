@@ -1,0 +1,50 @@
+"""Pins of the norm_multiply_dropout oracle against library routines and autograd."""
+import torch
+import torch.nn.functional as F
+
+from oracle import layer_oracle as LO
+
+
+def _inputs(seed, rows=7, cols=512):
+    g = torch.Generator().manual_seed(seed)
+    mk = lambda *s: torch.rand(*s, generator=g, dtype=torch.float64) * 2 - 1
+    return mk(rows, cols), mk(rows, cols), mk(cols), mk(cols), mk(rows, cols)
+
+
+def test_forward_is_layer_norm_times_u():
+    x, u, w, b, _ = _inputs(0)
+    y, mean, var = LO.nmd_forward(x, u, w, b, 1e-5)
+    assert torch.allclose(y, F.layer_norm(x, [512], w, b, 1e-5) * u, rtol=1e-12, atol=1e-12)
+    assert torch.allclose(mean, x.mean(1)) and torch.allclose(var, x.var(1, unbiased=False))
+
+
+def test_dropout_follows_the_mask_with_the_usual_scale():
+    x, u, w, b, _ = _inputs(1)
+    keep = torch.rand(x.shape, generator=torch.Generator().manual_seed(2)) >= 0.3
+    y0 = LO.nmd_forward(x, u, w, b, 1e-5)[0]
+    y = LO.nmd_forward(x, u, w, b, 1e-5, 0.3, keep)[0]
+    assert torch.equal(y == 0, ~keep | (y0 == 0)) and torch.allclose(y[keep], y0[keep] / 0.7)
+    assert not LO.nmd_forward(x, u, w, b, 1e-5, 1.0, keep)[0].any()
+    # mask bytes: bit e % 8 of byte e / 8
+    packed = torch.zeros(((keep.numel() + 127) // 128) * 16, dtype=torch.uint8)
+    flat = keep.reshape(-1)
+    for e in range(0, flat.numel(), 97):
+        if flat[e]:
+            packed[e // 8] |= 1 << (e % 8)
+    got = LO.unpack_mask(packed, flat.numel())
+    assert torch.equal(got[::97], flat[::97])
+
+
+def test_backward_matches_autograd_through_the_library_forward():
+    for ratio in (0.0, 0.25):
+        x, u, w, b, dy = _inputs(3, rows=5, cols=1024)
+        keep = torch.rand(x.shape, generator=torch.Generator().manual_seed(4)) >= ratio
+        leaves = [t.clone().requires_grad_(True) for t in (x, u, w, b)]
+        y = F.layer_norm(leaves[0], [1024], leaves[2], leaves[3], 1e-5) * leaves[1]
+        if ratio:
+            y = y * keep / (1 - ratio)
+        auto = torch.autograd.grad(y, leaves, grad_outputs=dy)
+        _, mean, var = LO.nmd_forward(x, u, w, b, 1e-5)
+        got = LO.nmd_backward(dy, x, u, w, b, mean, var, 1e-5, ratio, keep)
+        for name, a, wnt in zip(("dx", "du", "dw", "db"), got, auto):
+            assert torch.allclose(a, wnt, rtol=1e-9, atol=1e-11), (ratio, name)
