@@ -22,7 +22,8 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
 # HBM-side bytes per launch from rocprofv3 FETCH_SIZE/WRITE_SIZE, each scaled by what the same counter reads for the
 # plain 256 MiB copy of `--workload copy` (factors 2.000 and 1.000); see profiles/*.md
-MEASURED_TRAFFIC_BYTES = {"config2": 184.3e6, "kv_append": 351.9e6, "rab_time": 1479.8e6, "rab_time_bwd": 2242.4e6, "rab_pos": 305.2e6}
+MEASURED_TRAFFIC_BYTES = {"config2": 184.3e6, "kv_append": 351.9e6, "rab_time": 1479.8e6, "rab_time_bwd": 2242.4e6, "rab_pos": 305.2e6,
+                          "nmd_fwd": 827.4e6, "nmd_bwd": 1382.0e6}
 
 
 def build_workload(name, torch, W):
@@ -57,7 +58,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=1000)
-    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "config2_bwd", "kv_append", "rab_time", "rab_time_bwd", "rab_pos", "copy"],
+    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "config2_bwd", "kv_append", "rab_time", "rab_time_bwd", "rab_pos", "nmd_fwd", "nmd_bwd", "copy"],
                     help="'copy' runs a plain 256 MiB device copy: the known-size kernel the FETCH_SIZE/WRITE_SIZE counters are scaled by")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
@@ -77,6 +78,8 @@ def main():
         return kv_append_bench(args, torch, W)
     if args.workload in ("rab_time", "rab_time_bwd", "rab_pos"):
         return bias_bench(args, torch)
+    if args.workload in ("nmd_fwd", "nmd_bwd"):
+        return nmd_bench(args, torch)
     cfg, op, flops, alg_bytes, desc = build_workload(args.workload, torch, W)
     dev = W.to_device(cfg)
     q, k, v = dev["q"], dev["k"], dev["v"]
@@ -355,6 +358,65 @@ def bias_bench(args, torch):
         dt = time.perf_counter() - t0
         out["cpu_baseline"] = {"value": round(cpu_bytes / dt / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
                                "sample": f"{sample}, {dt:.2f} s"}
+    print(json.dumps(out), flush=True)
+
+
+def nmd_bench(args, torch):
+    """norm_multiply_dropout at the shape of the reference's sample (README of the op: 262144 x 512, bf16, eps 1e-5), with
+    dropout 0.3 so that the mask is written and read.  HBM-bound: forward reads x, u and writes y (+ mask, mean, var);
+    backward reads d_out, x, u (+ mask, mean, var) and writes d_x, d_u."""
+    from oracle import layer_oracle as LO
+    rows, cols, ratio, eps = 262144, 512, 0.3, 1e-5
+    g = torch.Generator().manual_seed(321)
+    mk = lambda *s: (torch.rand(*s, generator=g) * 2 - 1).to(torch.bfloat16)
+    x, u, w, b, dy = mk(rows, cols), mk(rows, cols), mk(cols), mk(cols), mk(rows, cols)
+    xd, ud, wd, bd, dyd = (t.cuda() for t in (x, u, w, b, dy))
+    m = torch.ops.mxrec
+    small = rows * 8 + rows * cols // 8      # mean, var (fp32) and the mask bits
+    if args.workload == "nmd_fwd":
+        fn = lambda: m.norm_multiply_dropout_forward(xd, ud, wd, bd, eps, ratio)
+        alg = 3 * rows * cols * 2 + small
+        kernel = "hstu_nmd_fwd_kernel"
+        n_cpu = rows
+        cpu = lambda: LO.nmd_forward(x[:n_cpu], u[:n_cpu], w, b, eps, ratio, torch.ones(n_cpu, cols, dtype=torch.bool))
+        cpu_bytes = alg * n_cpu // rows
+    else:
+        _, mean, var, mask = m.norm_multiply_dropout_forward(xd, ud, wd, bd, eps, ratio)
+        fn = lambda: m.norm_multiply_dropout_backward(dyd, xd, ud, wd, bd, mean, var, mask, eps, ratio)
+        alg = 5 * rows * cols * 2 + small
+        kernel = "hstu_nmd_bwd_kernel"
+        n_cpu = rows // 2
+        mc, vc = mean[:n_cpu].cpu(), var[:n_cpu].cpu()
+        cpu = lambda: LO.nmd_backward(dy[:n_cpu], x[:n_cpu], u[:n_cpu], w, b, mc, vc, eps, ratio, torch.ones(n_cpu, cols, dtype=torch.bool))
+        cpu_bytes = alg * n_cpu // rows
+    for _ in range(args.warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    kern_ms = e0.elapsed_time(e1) / args.steps
+    out = {
+        "metric": f"norm_multiply_dropout_{args.workload[4:]}_gbps", "value": round(alg / (ms * 1e-3) / 1e9, 1), "unit": "GB/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic", "us_per_call": round(ms * 1e3, 2),
+        "config": {"workload": f"{args.workload}: x, u [262144, 512] bf16, eps 1e-5, dropout 0.3, seed 321", "algorithmic_bytes_per_call": alg,
+                   "entry": f"torch.ops.mxrec.norm_multiply_dropout_{'forward' if args.workload == 'nmd_fwd' else 'backward'} -> {kernel} (C ABI in include/hstu_layer.h)"},
+        "roofline": {"bound": "hbm", "kernel": kernel, "achieved": round(alg / (kern_ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(alg / (kern_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                     "kernel_us": round(kern_ms * 1e3, 2)},
+    }
+    if not args.no_cpu_baseline:
+        t0 = time.perf_counter()
+        cpu()
+        dt = time.perf_counter() - t0
+        out["cpu_baseline"] = {"value": round(cpu_bytes / dt / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"the first {n_cpu} rows once (oracle in torch, fp64), {dt:.2f} s"}
     print(json.dumps(out), flush=True)
 
 

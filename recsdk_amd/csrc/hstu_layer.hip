@@ -193,14 +193,24 @@ __global__ __launch_bounds__(NMD_NT) void hstu_nmd_bwd_kernel(const hstu_nmd_bwd
     }
 }
 
-// d_weight / d_bias = partial sums of the workgroups, added in workgroup order
+// d_weight / d_bias = partial sums of the workgroups, added in a fixed order: 32 columns x 8 row slots per workgroup,
+// slot r adds the rows r, r + 8, ... of the partial table, then the slots are added 0..7
 __global__ __launch_bounds__(256) void hstu_nmd_colsum_kernel(const float* partial, int wgs, int cols, float* d_weight, float* d_bias) {
-    const int c = blockIdx.x * blockDim.x + threadIdx.x;
-    if (c >= 2 * cols) return;
+    __shared__ float part[8][32];
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+    const int c = blockIdx.x * 32 + tx;            // column of the [2 * cols] row: d_weight then d_bias
     const int which = c / cols, col = c % cols;
     float s = 0.f;
-    for (int g = 0; g < wgs; g++) s += partial[((int64_t)g * 2 + which) * cols + col];
-    (which ? d_bias : d_weight)[col] = s;
+#pragma unroll 8
+    for (int g = ty; g < wgs; g += 8) s += partial[((int64_t)g * 2 + which) * cols + col];
+    part[ty][tx] = s;
+    __syncthreads();
+    if (ty == 0) {
+        float t = 0.f;
+#pragma unroll
+        for (int r = 0; r < 8; r++) t += part[r][tx];
+        (which ? d_bias : d_weight)[col] = t;
+    }
 }
 
 static unsigned nmd_grid(int64_t rows) {
@@ -288,7 +298,7 @@ extern "C" int hstu_hip_norm_multiply_dropout_backward(const hstu_nmd_bwd_params
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     float* partial = reinterpret_cast<float*>(workspace);
     NMD_DISPATCH(p->dtype, p->cols, hstu_nmd_bwd_kernel, dim3(grid), st, *p, nmd_keep_scale(p->dropout_ratio), partial);
-    hipLaunchKernelGGL(hstu_nmd_colsum_kernel, dim3((unsigned)((2 * p->cols + 255) / 256)), dim3(256), 0, st, partial, (int)grid, p->cols, p->d_weight,
+    hipLaunchKernelGGL(hstu_nmd_colsum_kernel, dim3((unsigned)(2 * p->cols / 32)), dim3(256), 0, st, partial, (int)grid, p->cols, p->d_weight,
                        p->d_bias);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString(e));
