@@ -1,6 +1,7 @@
 /*
- * hstu_layer.h -- C ABI of the step after the attention in an HSTU layer: LayerNorm(x) * u with dropout, forward and
- * backward (mxrec::norm_multiply_dropout).
+ * hstu_layer.h -- C ABI of the steps either side of the attention in an HSTU layer: the input projection
+ * SiLU(x W^T + b) split into U, V, Q, K before it (mxrec::distance_in_linear_silu, forward), and LayerNorm(x) * u with
+ * dropout after it, forward and backward (mxrec::norm_multiply_dropout).
  *
  * Same conventions as hstu_hip.h: device pointers, asynchronous on `stream`, nothing read on the host, 0 or a negative
  * hstu_status with the message in hstu_hip_last_error().  dtype: HSTU_F32 / HSTU_F16 / HSTU_BF16 for x, u, weight,
@@ -77,6 +78,28 @@ typedef struct hstu_nmd_bwd_params {
 } hstu_nmd_bwd_params;
 int hstu_hip_norm_multiply_dropout_backward_get_workspace_size(const hstu_nmd_bwd_params* p, uint64_t* workspace_bytes);
 int hstu_hip_norm_multiply_dropout_backward(const hstu_nmd_bwd_params* p, void* workspace, uint64_t workspace_bytes, void* stream);
+
+/* Input projection.  Replaces aclnnInLinearSilu (cust_op/framework/torch_plugin/torch_library/in_linear_silu/
+ * in_linear_silu.cpp:96-117; golden cust_op/test/in_linear_silu_test/test_in_linear_silu.py:31-45):
+ *   linear_output = round(x W^T + bias)               [m, n], fp32 accumulation, rounded to the I/O dtype
+ *   (user | value | query | key) = round(silu(linear_output)) split along n into widths split[0..3]
+ * dtype: HSTU_F16 / HSTU_BF16 for x, weight and the outputs; bias is fp32 and may be NULL (no bias).
+ * Limits of the reference's checks (in_linear_silu.cpp:34-66): k in [16, 8192], n in [64, 32768], every split width in
+ * [16, 8192], all multiples of 16; sum(split) == n; n a multiple of 4 k. */
+typedef struct hstu_in_linear_silu_params {
+    uint32_t struct_size;
+    int32_t dtype;
+    int64_t m;
+    int32_t k;
+    int32_t n;
+    int32_t split[4];         /* widths of user, value, query, key */
+    const void* x;            /* [m, k] */
+    const void* weight;       /* [n, k] */
+    const float* bias;        /* [n] or NULL */
+    void* out[4];             /* user [m, split[0]], value [m, split[1]], query [m, split[2]], key [m, split[3]] */
+    void* linear_output;      /* [m, n] */
+} hstu_in_linear_silu_params;
+int hstu_hip_in_linear_silu(const hstu_in_linear_silu_params* p, void* stream);
 
 #ifdef __cplusplus
 }

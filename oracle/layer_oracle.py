@@ -1,4 +1,4 @@
-"""CPU oracle for ``mxrec::norm_multiply_dropout``.  TEST INFRASTRUCTURE ONLY.
+"""CPU oracle for ``mxrec::norm_multiply_dropout`` and ``mxrec::distance_in_linear_silu``.  TEST INFRASTRUCTURE ONLY.
 
 Restates the reference's goldens; used by ``tests/`` and by the ``cpu_baseline`` leg of ``bench.py``.  Nothing in the
 shipped package imports it.
@@ -16,11 +16,16 @@ Definition followed (reference file:line):
   test_norm_multiply_dropout.py:336-342): parity with the reference's random stream is neither possible nor claimed;
   the tests check the op against this oracle under the mask the op itself returned, and the keep rate.
 
-Everything here is fp64 so that it can serve as the exact value for every I/O dtype.
+* in_linear_silu: cust_op/test/in_linear_silu_test/test_in_linear_silu.py:31-45 -- ``addmm(bias, x, W^T)`` rounded to the
+  I/O dtype (= linear_output), SiLU of that rounded tensor, rounded again, split along the last axis.
+
+Everything here is fp64 so that it can serve as the exact value for every I/O dtype (``in_linear_silu`` applies the
+golden's two roundings to the I/O dtype on top of fp64 arithmetic).
 
 Pinning status (tests/test_oracle_layer.py): forward against ``torch.nn.functional.layer_norm`` (a library routine
 that shares no code with the explicit mean / var formula here) and ``F.dropout`` semantics under a given mask; backward
-against autograd through that library forward, including the mask.  PINNED
+against autograd through that library forward, including the mask.  ``in_linear_silu`` against ``torch.addmm``,
+``F.silu`` and ``torch.split`` evaluated in fp32 on values where fp32 is exact.  PINNED
 """
 from __future__ import annotations
 
@@ -58,3 +63,14 @@ def nmd_backward(d_out, x, u, weight, bias, mean, var, eps: float, dropout_ratio
     dx = (a - (a.sum(dim=1, keepdim=True) + xh * (a * xh).sum(dim=1, keepdim=True)) / c) * rstd
     du = dy * (weight * xh + bias)
     return dx, du, (xh * g).sum(dim=0), g.sum(dim=0)
+
+
+def in_linear_silu(x, weight, bias, split):
+    """Returns (user, value, query, key, linear_output) in the dtype of x."""
+    lin = x.double() @ weight.double().t()
+    if bias is not None:
+        lin = lin + bias.double()
+    lin = lin.to(x.dtype)
+    act = (lin.double() * torch.sigmoid(lin.double())).to(x.dtype)
+    u, v, q, k = torch.split(act, list(split), dim=-1)
+    return u.contiguous(), v.contiguous(), q.contiguous(), k.contiguous(), lin

@@ -30,7 +30,7 @@ EXPORTS = [
     "hstu_hip_kv_append", "hstu_hip_kv_token_positions",
     "hstu_hip_rab_time", "hstu_hip_rab_time_backward", "hstu_hip_rab_pos",
     "hstu_hip_norm_multiply_dropout", "hstu_hip_norm_multiply_dropout_backward",
-    "hstu_hip_norm_multiply_dropout_backward_get_workspace_size",
+    "hstu_hip_norm_multiply_dropout_backward_get_workspace_size", "hstu_hip_in_linear_silu",
 ]
 
 
@@ -111,6 +111,14 @@ class HstuNmdBwdParams(C.Structure):
     ]
 
 
+class HstuInLinearSiluParams(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32), ("dtype", C.c_int32), ("m", C.c_int64), ("k", C.c_int32), ("n", C.c_int32),
+        ("split", C.c_int32 * 4), ("x", C.c_void_p), ("weight", C.c_void_p), ("bias", C.c_void_p),
+        ("out", C.c_void_p * 4), ("linear_output", C.c_void_p),
+    ]
+
+
 _lib: Optional[C.CDLL] = None
 
 
@@ -137,6 +145,7 @@ def lib() -> C.CDLL:
         _lib.hstu_hip_kv_append.argtypes = [C.POINTER(HstuKvAppendParams), C.c_void_p]
         _lib.hstu_hip_rab_time.argtypes = [C.POINTER(HstuRabTimeParams), C.c_void_p]
         _lib.hstu_hip_norm_multiply_dropout.argtypes = [C.POINTER(HstuNmdParams), C.c_void_p]
+        _lib.hstu_hip_in_linear_silu.argtypes = [C.POINTER(HstuInLinearSiluParams), C.c_void_p]
         _lib.hstu_hip_norm_multiply_dropout_backward.argtypes = [C.POINTER(HstuNmdBwdParams), C.c_void_p, C.c_uint64, C.c_void_p]
         _lib.hstu_hip_norm_multiply_dropout_backward_get_workspace_size.argtypes = [C.POINTER(HstuNmdBwdParams), C.POINTER(C.c_uint64)]
         _lib.hstu_hip_rab_time_backward.argtypes = [C.POINTER(HstuRabTimeBwdParams), C.c_void_p]

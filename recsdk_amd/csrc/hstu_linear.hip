@@ -1,0 +1,185 @@
+// Input projection of an HSTU layer: linear_output = x W^T + b, (U | V | Q | K) = silu(linear_output) split along n
+// (mxrec::distance_in_linear_silu).  k is an embedding width (tens to a few hundred) and n four times a hidden width
+// (thousands), so at 2 * k FLOPs per output element against 4 bytes written the op is bounded by the HBM writes of
+// its two [m, n] results, not by the matrix cores: the kernel is an MFMA GEMM without any pipelining of the k loop,
+// built around its stores.
+//   workgroup = 128 rows m x 128 columns n; wave w = rows 32 w .. 32 w + 31, all 128 columns (four 32 x 32 blocks)
+//   out^T block = W x^T: v_mfma_f32_32x32x16 with A = W fragment, B = x fragment, both straight from global memory
+//   (each lane reads 16 contiguous bytes of a row: x and W are k-contiguous, which is what both operands want)
+//   epilogue: + bias, round -> linear_output; silu of the rounded value, round -> the four outputs; both leave through
+//   a per-wave LDS tile so that a lane stores 16 bytes of one output row and a wave instruction covers four 256-byte runs
+// Definition: cust_op/test/in_linear_silu_test/test_in_linear_silu.py:31-45.
+#include "hstu_device.h"
+#include "../../include/hstu_layer.h"
+
+namespace hstu {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 ils_bf16x8;
+typedef __attribute__((ext_vector_type(8))) _Float16 ils_f16x8;
+typedef __attribute__((ext_vector_type(2))) __bf16 ils_bf16x2;
+typedef __attribute__((ext_vector_type(2))) _Float16 ils_f16x2;
+typedef __attribute__((ext_vector_type(16))) float ils_f32x16;
+typedef __attribute__((ext_vector_type(4))) float ils_f32x4;
+typedef __attribute__((ext_vector_type(4))) unsigned int ils_u4;
+typedef __attribute__((ext_vector_type(2))) unsigned int ils_u2;
+
+template <typename T> struct IlsMM;
+template <> struct IlsMM<__bf16> {
+    typedef ils_bf16x8 v8;
+    static __device__ __forceinline__ ils_f32x16 mfma(v8 a, v8 b, ils_f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+    static __device__ __forceinline__ unsigned pack2(__bf16 x, __bf16 y) { ils_bf16x2 r; r[0] = x; r[1] = y; return __builtin_bit_cast(unsigned, r); }
+};
+template <> struct IlsMM<_Float16> {
+    typedef ils_f16x8 v8;
+    static __device__ __forceinline__ ils_f32x16 mfma(v8 a, v8 b, ils_f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+    static __device__ __forceinline__ unsigned pack2(_Float16 x, _Float16 y) { ils_f16x2 r; r[0] = x; r[1] = y; return __builtin_bit_cast(unsigned, r); }
+};
+
+constexpr int ILS_BM = 128, ILS_BN = 128, ILS_NT = 256;
+constexpr int ILS_ROW = ILS_BN * 2 + 16;   // bytes of one parked row: + 16 keeps the 8-byte column writes of 32 rows off one bank
+
+struct IlsArgs {
+    hstu_in_linear_silu_params p;
+    int base[5];   // first column of user, value, query, key, and n
+};
+
+template <typename T>
+__global__ __launch_bounds__(ILS_NT) void hstu_in_linear_silu_kernel(const IlsArgs a) {
+    typedef typename IlsMM<T>::v8 v8;
+    __shared__ __attribute__((aligned(16))) char park_all[(ILS_NT / 64) * 32 * ILS_ROW];
+    const hstu_in_linear_silu_params& p = a.p;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int g = lane >> 5, l32 = lane & 31;
+    const int K = p.k, N = p.n;
+    const int n0 = blockIdx.x * ILS_BN;
+    const int64_t m0 = (int64_t)blockIdx.y * ILS_BM + 32 * w;
+    if (m0 >= p.m) return;   // whole wave; nothing below synchronises across waves
+    const T* x = reinterpret_cast<const T*>(p.x);
+    const T* wt = reinterpret_cast<const T*>(p.weight);
+    // operand rows of this lane, clamped into the tensors (what is read for rows past the end is never stored)
+    const T* xrow = x + (m0 + l32 < p.m ? m0 + l32 : p.m - 1) * K + 8 * g;
+    const T* wrow[4];
+#pragma unroll
+    for (int nb = 0; nb < 4; nb++) wrow[nb] = wt + (int64_t)min(n0 + 32 * nb + l32, N - 1) * K + 8 * g;
+    ils_f32x16 acc[4];
+#pragma unroll
+    for (int nb = 0; nb < 4; nb++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[nb][r] = 0.f;
+    auto step = [&](int k0) __attribute__((always_inline)) {
+        const v8 xf = *reinterpret_cast<const v8*>(xrow + k0);
+        v8 wf[4];
+#pragma unroll
+        for (int nb = 0; nb < 4; nb++) wf[nb] = *reinterpret_cast<const v8*>(wrow[nb] + k0);
+#pragma unroll
+        for (int nb = 0; nb < 4; nb++) acc[nb] = IlsMM<T>::mfma(wf[nb], xf, acc[nb]);
+    };
+    int k0 = 0;
+    for (; k0 + 64 <= K; k0 += 64) {   // four steps' loads in flight together
+        step(k0);
+        step(k0 + 16);
+        step(k0 + 32);
+        step(k0 + 48);
+    }
+    for (; k0 < K; k0 += 16) step(k0);
+    // accumulator register r of block nb holds column n0 + 32 nb + 8 (r / 4) + 4 g + r % 4 of row m0 + l32
+    char* park = park_all + w * (32 * ILS_ROW);
+    T lin[4][16];
+#pragma unroll
+    for (int nb = 0; nb < 4; nb++) {
+#pragma unroll
+        for (int rr = 0; rr < 4; rr++) {
+            ils_f32x4 b = {0.f, 0.f, 0.f, 0.f};
+            const int col = n0 + 32 * nb + 8 * rr + 4 * g;
+            if (p.bias && col < N) b = *reinterpret_cast<const ils_f32x4*>(p.bias + col);
+#pragma unroll
+            for (int e = 0; e < 4; e++) lin[nb][4 * rr + e] = from_float<T>(acc[nb][4 * rr + e] + b[e]);
+        }
+    }
+    const int orow = lane >> 4, ochunk = lane & 15;   // store phase: 16 lanes per row, 8 columns each
+    const int col = n0 + 8 * ochunk;
+    int which = 0;
+#pragma unroll
+    for (int sidx = 1; sidx < 4; sidx++) which += col >= a.base[sidx] ? 1 : 0;
+#pragma unroll
+    for (int phase = 0; phase < 2; phase++) {
+#pragma unroll
+        for (int nb = 0; nb < 4; nb++) {
+#pragma unroll
+            for (int rr = 0; rr < 4; rr++) {
+                T v[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const T l = lin[nb][4 * rr + e];
+                    if (phase == 0) v[e] = l;
+                    else {
+                        const float f = to_float(l);
+                        v[e] = from_float<T>(f / (1.0f + __expf(-f)));
+                    }
+                }
+                ils_u2 o = {IlsMM<T>::pack2(v[0], v[1]), IlsMM<T>::pack2(v[2], v[3])};
+                *reinterpret_cast<ils_u2*>(park + l32 * ILS_ROW + (32 * nb + 8 * rr + 4 * g) * 2) = o;
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+        if (col < N) {
+            T* dst;
+            int64_t stride;
+            if (phase == 0) { dst = reinterpret_cast<T*>(p.linear_output) + col; stride = N; }
+            else {
+                void* o = p.out[0];
+                int first = a.base[0], width = p.split[0];
+#pragma unroll
+                for (int sidx = 1; sidx < 4; sidx++)
+                    if (which == sidx) { o = p.out[sidx]; first = a.base[sidx]; width = p.split[sidx]; }
+                dst = reinterpret_cast<T*>(o) + (col - first);
+                stride = width;
+            }
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const int row = 4 * i + orow;
+                const ils_u4 v = *reinterpret_cast<const ils_u4*>(park + row * ILS_ROW + ochunk * 16);
+                if (m0 + row < p.m) __builtin_nontemporal_store(v, reinterpret_cast<ils_u4*>(dst + (m0 + row) * stride));
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
+}  // namespace hstu
+
+using namespace hstu;
+
+extern "C" int hstu_hip_in_linear_silu(const hstu_in_linear_silu_params* p, void* stream) {
+    if (!p) return fail(HSTU_ERR_INVALID_ARGUMENT, "params is NULL");
+    if (p->struct_size != sizeof(hstu_in_linear_silu_params))
+        return fail(HSTU_ERR_INVALID_ARGUMENT, "hstu_in_linear_silu_params size mismatch: caller %u, library %zu", p->struct_size,
+                    sizeof(hstu_in_linear_silu_params));
+    if (p->dtype != HSTU_F16 && p->dtype != HSTU_BF16) return fail(HSTU_ERR_INVALID_ARGUMENT, "dtype expect float16 or bfloat16, but value is %d", p->dtype);
+    if (p->m < 1 || p->m > 65535LL * ILS_BM) return fail(HSTU_ERR_INVALID_ARGUMENT, "x dim[0] must in range[1, %lld], but got %lld", 65535LL * ILS_BM, (long long)p->m);
+    IlsArgs a;
+    a.p = *p;
+    int total = 0;
+    for (int i = 0; i < 4; i++) {
+        if (p->split[i] < 16 || p->split[i] > 8192 || p->split[i] % 16) return fail(HSTU_ERR_INVALID_ARGUMENT, "uvqk dim must in range[16, 8192] and multiples of 16.");
+        a.base[i] = total;
+        total += p->split[i];
+    }
+    a.base[4] = total;
+    if (p->k < 16 || p->k > 8192 || p->k % 16) return fail(HSTU_ERR_INVALID_ARGUMENT, "x dim[1] must in range[16, 8192] and multiples of 16.");
+    if (p->n < 64 || p->n > 32768 || p->n % 16) return fail(HSTU_ERR_INVALID_ARGUMENT, "weight dim[0] must in range[64, 32768] and multiples of 16.");
+    if (total != p->n) return fail(HSTU_ERR_INVALID_ARGUMENT, "weight_dim[0] must equal to sum(splitList).");
+    if (p->n % (4 * p->k)) return fail(HSTU_ERR_INVALID_ARGUMENT, "weight dim[0] must be a multiple of 4 x dim[1]");
+    if (!p->x || !p->weight || !p->linear_output || !p->out[0] || !p->out[1] || !p->out[2] || !p->out[3])
+        return fail(HSTU_ERR_INVALID_ARGUMENT, "x, weight, the four outputs and linear_output must not be NULL");
+    const void* ptrs[] = {p->x, p->weight, p->bias, p->linear_output, p->out[0], p->out[1], p->out[2], p->out[3]};
+    for (const void* q : ptrs)
+        if (reinterpret_cast<uintptr_t>(q) & 15) return fail(HSTU_ERR_UNSUPPORTED, "x, weight, bias and the outputs must be 16-byte aligned");
+    const dim3 grid((unsigned)((p->n + ILS_BN - 1) / ILS_BN), (unsigned)((p->m + ILS_BM - 1) / ILS_BM));
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (p->dtype == HSTU_BF16) hipLaunchKernelGGL(hstu_in_linear_silu_kernel<__bf16>, grid, dim3(ILS_NT), 0, st, a);
+    else hipLaunchKernelGGL(hstu_in_linear_silu_kernel<_Float16>, grid, dim3(ILS_NT), 0, st, a);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString(e));
+    return HSTU_OK;
+}

@@ -984,6 +984,64 @@ std::vector<at::Tensor> norm_multiply_dropout_backward(const at::Tensor& d_out, 
     return nmd_backward_impl(d_out, x, u, weight, bias, mean, var, mask, eps, dropout_ratio);
 }
 
+// ---------------------------------------------------------------------------------------------
+// in_linear_silu, forward (cust_op/framework/torch_plugin/torch_library/in_linear_silu/in_linear_silu.cpp:34-117)
+// ---------------------------------------------------------------------------------------------
+std::vector<at::Tensor> distance_in_linear_silu(const at::Tensor& x, const at::Tensor& weight, const at::Tensor& bias, at::IntArrayRef split_list) {
+    // IsValidShape, in_linear_silu.cpp:34-66
+    check_tensor_non_empty(x, "x");
+    check_tensor_non_empty(weight, "weight");
+    TORCH_CHECK(x.dim() == 2, "x must be 2D");
+    TORCH_CHECK(weight.dim() == 2, "weight must be 2D");
+    TORCH_CHECK(split_list.size() == 4, "splitList must have 4 elements.");
+    int64_t total = 0;
+    for (int i = 0; i < 4; i++) {
+        TORCH_CHECK(split_list[i] >= 16 && split_list[i] <= 8192 && split_list[i] % 16 == 0, "uvqk dim must in range[16, 8192] and multiples of 16.");
+        total += split_list[i];
+    }
+    const auto k = x.size(1), n = weight.size(0), m = x.size(0);
+    TORCH_CHECK(k >= 16 && k <= 8192 && k % 16 == 0, "x dim[1] must in range[16, 8192] and multiples of 16.");
+    TORCH_CHECK(n >= 64 && n <= 32768 && n % 16 == 0, "weight dim[0] must in range[64, 32768] and multiples of 16.");
+    TORCH_CHECK(total == n, "weight_dim[0] must equal to sum(splitList).");
+    TORCH_CHECK(weight.size(1) == k, "weight dim[1] must equal to x dim[1].");
+    TORCH_CHECK(n % (4 * k) == 0, "weight dim[0] must be a multiple of 4 x dim[1]");
+    if (bias.defined()) {
+        check_tensor_non_empty(bias, "bias");
+        TORCH_CHECK(bias.dim() == 1, "bias must be 1D");
+        TORCH_CHECK(bias.size(0) == n, "bias dim[0] must equal to weight dim[0].");
+    }
+    TORCH_CHECK(x.scalar_type() == at::kHalf || x.scalar_type() == at::kBFloat16, "x dtype expect float16 or bfloat16, but get ", x.scalar_type());
+    TORCH_CHECK(weight.scalar_type() == x.scalar_type(), "weight must have the dtype of x");
+    Holder h;
+    auto dx = h.same(x), dw = h.same(weight);
+    at::Tensor db;
+    if (bias.defined()) db = h.same(bias.to(at::kFloat));
+    hstu_in_linear_silu_params p;
+    std::memset(&p, 0, sizeof(p));
+    p.struct_size = sizeof(p);
+    p.dtype = io_dtype(dx, "x");
+    p.m = m;
+    p.k = (int32_t)k;
+    p.n = (int32_t)n;
+    require_gpu(dx, "distance_in_linear_silu");
+    std::vector<at::Tensor> outs;
+    for (int i = 0; i < 4; i++) {
+        p.split[i] = (int32_t)split_list[i];
+        outs.push_back(at::empty({m, split_list[i]}, dx.options()));
+        p.out[i] = outs.back().data_ptr();
+    }
+    outs.push_back(at::empty({m, n}, dx.options()));
+    p.linear_output = outs.back().data_ptr();
+    p.x = dx.const_data_ptr();
+    p.weight = dw.const_data_ptr();
+    p.bias = db.defined() ? db.const_data_ptr<float>() : nullptr;
+    c10::hip::OptionalHIPGuardMasqueradingAsCUDA guard(dx.device());
+    auto stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA();
+    const int rc = hstu_hip_in_linear_silu(&p, (void*)stream.stream());
+    TORCH_CHECK(rc == HSTU_OK, "mxrec::distance_in_linear_silu: ", hstu_hip_last_error());
+    return outs;
+}
+
 TORCH_LIBRARY_FRAGMENT(mxrec, m) {
     m.def("hstu_jagged.equal(Tensor q, "
           "                  Tensor k, "
@@ -1099,6 +1157,7 @@ TORCH_LIBRARY_FRAGMENT(mxrec, m) {
           "                                   Tensor timestamps_weights, "
           "                                   float bucket_divisor"
           "                                   ) -> Tensor[]");
+    m.def("distance_in_linear_silu(Tensor x, Tensor weight, Tensor bias, int[] attr_dict) -> Tensor[]");
     m.def("norm_multiply_dropout(Tensor x, Tensor u, Tensor weight, Tensor bias, float eps, float dropout_ratio) -> "
           "Tensor[]");
     // no counterpart in the reference:
@@ -1132,6 +1191,7 @@ TORCH_LIBRARY_FRAGMENT(mxrec, m) {
     m.impl("relative_attn_bias_time_backward", TORCH_FN(relative_attn_bias_time_backward)); \
     m.impl("relative_attn_bias_time_with_index", TORCH_FN(relative_attn_bias_time_with_index)); \
     m.impl("norm_multiply_dropout_forward", TORCH_FN(norm_multiply_dropout_forward));           \
+    m.impl("distance_in_linear_silu", TORCH_FN(distance_in_linear_silu));                       \
     m.impl("norm_multiply_dropout_backward", TORCH_FN(norm_multiply_dropout_backward));
 
 // ROCm tensors dispatch on the CUDA key.  The CPU key runs the same host checks and then

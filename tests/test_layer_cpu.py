@@ -56,3 +56,41 @@ def test_torch_op_schema_and_checks():
                      (dict(r=1.1), "dropout_ratio must in range"), (dict(), "no CPU implementation")):
         with pytest.raises(RuntimeError, match=text):
             run(**kw)
+
+
+def test_in_linear_silu_validation():
+    """C ABI and torch op reject what the reference rejects (in_linear_silu.cpp:34-66; its tests
+    test_in_linear_silu.py:133-161), before any launch."""
+    L = _capi.lib()
+    def call(**over):
+        p = _capi.HstuInLinearSiluParams()
+        p.struct_size = C.sizeof(_capi.HstuInLinearSiluParams)
+        p.dtype, p.m, p.k, p.n = _capi.HSTU_F16, 100, 16, 64
+        for i in range(4):
+            p.split[i] = 16
+            p.out[i] = 0x1000
+        p.x = p.weight = p.bias = p.linear_output = 0x1000
+        for k, v in over.items():
+            if k == "split":
+                for i, s_ in enumerate(v):
+                    p.split[i] = s_
+            else:
+                setattr(p, k, v)
+        return L.hstu_hip_in_linear_silu(C.byref(p), None), L.hstu_hip_last_error().decode()
+    for over, text in ((dict(split=[16, 17, 15, 16]), "uvqk dim must in range[16, 8192] and multiples of 16"),
+                       (dict(split=[16, 16, 32, 32]), "weight_dim[0] must equal to sum(splitList)"), (dict(k=24), "x dim[1] must in range[16, 8192] and multiples of 16"),
+                       (dict(n=48, split=[16, 16, 16, 0]), "uvqk dim"), (dict(k=32), "weight dim[0] must be a multiple of 4 x dim[1]"),
+                       (dict(dtype=_capi.HSTU_F32), "dtype expect float16 or bfloat16"), (dict(m=0), "x dim[0] must in range"), (dict(x=None), "must not be NULL")):
+        rc, msg = call(**over)
+        assert rc == -1 and text in msg, (over, msg)
+    rc, msg = call(bias=0x1004)
+    assert rc == -2 and "16-byte aligned" in msg
+    m = torch.ops.mxrec
+    assert str(m.distance_in_linear_silu.default._schema) == "mxrec::distance_in_linear_silu(Tensor x, Tensor weight, Tensor bias, int[] attr_dict) -> Tensor[]"
+    x, w, b = torch.zeros(100, 16, dtype=torch.float16), torch.zeros(64, 16, dtype=torch.float16), torch.ones(64)
+    for args, text in (((x, w, b, [16, 17, 15, 16]), "uvqk dim must in range"), ((x, w, b, [16, 16, 32, 32]), "must equal to sum"),
+                       ((x, w, b, [16, 16, 32]), "splitList must have 4 elements"), ((x, w, x.clone(), [16] * 4), "bias must be 1D"),
+                       ((x, w[None], b, [16] * 4), "weight must be 2D"), ((x, w[:, :8], b, [16] * 4), "weight dim\\[1\\] must equal to x dim\\[1\\]"),
+                       ((x, w, b, [16] * 4), "no CPU implementation")):
+        with pytest.raises(RuntimeError, match=text):
+            m.distance_in_linear_silu(*args)

@@ -100,3 +100,48 @@ def test_dropout_under_the_mask_the_op_returns(dim1, dtype, ratio):
     # everything dropped
     y1 = torch.ops.mxrec.norm_multiply_dropout_forward(x.cuda(), u.cuda(), w.cuda(), b.cuda(), EPS, 1.0)[0]
     assert not bool(y1.any())
+
+
+@pytest.mark.parametrize("m,n,k,split,dtype", [
+    (2789, 9216, 64, None, torch.bfloat16), (256, 1024, 16, None, torch.float16), (2561, 1024, 128, "diff", torch.bfloat16),
+    (512, 4096, 32, None, torch.float16), (1000, 9216, 48, "diff", torch.float16), (100, 64, 16, None, torch.bfloat16),
+    (129, 2048, 256, "diff", torch.bfloat16), (33, 192, 48, None, torch.float16)])
+def test_in_linear_silu_forward(m, n, k, split, dtype):
+    """The reference's generators (test_in_linear_silu.py:70-99): integer x in [-100, 100], Xavier-uniform W, bias of ones;
+    equal splits or (s - 16, s - 16, s + 16, s + 16).  Against the oracle's exactly rounded values the fp32 accumulation
+    order can move a result by one unit in the last place of the I/O dtype; nothing more is allowed."""
+    say("in_linear_silu", m, n, k, split, dtype)
+    g = torch.Generator().manual_seed(13)
+    x = torch.randint(-100, 101, (m, k), generator=g).to(dtype)
+    bound = (6.0 / (n + k)) ** 0.5
+    w = ((torch.rand(n, k, generator=g) * 2 - 1) * bound).to(dtype)
+    bias = torch.ones(n)
+    s = n // 4
+    sp = [s, s, s, s] if split is None else [s - 16, s - 16, s + 16, s + 16]
+    want = LO.in_linear_silu(x, w, bias, sp)
+    got = torch.ops.mxrec.distance_in_linear_silu(x.cuda(), w.cuda(), bias.cuda(), sp)
+    assert len(got) == 5
+    ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
+
+    # fp32 accumulation of k products against the oracle's fp64: absolute error up to about 2^-20 of the largest sum of
+    # absolute products, which matters where the result itself cancels to almost nothing
+    acc_err = 2.0 ** -20 * float((x.double().abs() @ w.double().abs().t()).max())
+
+    def within_one_ulp(a, wnt, name, extra=0.0):
+        assert a.shape == wnt.shape and a.dtype == dtype, name
+        d = (a.cpu().double() - wnt.double()).abs()
+        lim = ulp * wnt.double().abs().clamp(min=2.0 ** -14) * 1.001 + extra
+        assert bool((d <= lim).all()), f"{name}: more than one unit in the last place, max {float((d / lim).max()):.2f}"
+        assert float((d > 0).double().mean()) < 0.02, f"{name}: {float((d > 0).double().mean()):.4f} of the elements differ"
+
+    within_one_ulp(got[4], want[4], "linear_output", acc_err)
+    # the four outputs are SiLU of the *rounded* linear output (a last-place difference there is magnified by up to
+    # |1 + x (1 - sigmoid x)| in SiLU): checked against the oracle's SiLU of the linear output the kernel produced
+    lin = got[4].cpu()
+    act = (lin.double() * torch.sigmoid(lin.double())).to(dtype)
+    for name, a, wnt in zip(("user", "value", "query", "key"), got[:4], torch.split(act, sp, dim=-1)):
+        within_one_ulp(a, wnt, name)
+    # no bias
+    got0 = torch.ops.mxrec.distance_in_linear_silu(x.cuda(), w.cuda(), torch.zeros(n).cuda(), sp)
+    want0 = LO.in_linear_silu(x, w, None, sp)
+    within_one_ulp(got0[4], want0[4], "linear_output without bias", acc_err)

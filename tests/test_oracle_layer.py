@@ -48,3 +48,20 @@ def test_backward_matches_autograd_through_the_library_forward():
         got = LO.nmd_backward(dy, x, u, w, b, mean, var, 1e-5, ratio, keep)
         for name, a, wnt in zip(("dx", "du", "dw", "db"), got, auto):
             assert torch.allclose(a, wnt, rtol=1e-9, atol=1e-11), (ratio, name)
+
+
+def test_in_linear_silu_is_addmm_silu_split():
+    """Small integers and dyadic weights: every product and sum is exact in fp32, so the library routines in fp32 and the
+    oracle's fp64 agree to the last bit before and after the roundings."""
+    g = torch.Generator().manual_seed(6)
+    x = torch.randint(-8, 9, (37, 32), generator=g).to(torch.bfloat16)
+    w = (torch.randint(-4, 5, (128, 32), generator=g).float() / 8).to(torch.bfloat16)
+    b = torch.randint(-3, 4, (128,), generator=g).float()
+    split = [16, 48, 32, 32]
+    lin = torch.addmm(b, x.float(), w.float().t()).to(torch.bfloat16)
+    want = list(torch.split(F.silu(lin.float()).to(torch.bfloat16), split, dim=-1)) + [lin]
+    got = LO.in_linear_silu(x, w, b, split)
+    for a, wnt in zip(got, want):
+        assert a.dtype == torch.bfloat16 and torch.equal(a, wnt)
+    assert [t.shape[1] for t in got] == split + [128]
+    assert torch.equal(LO.in_linear_silu(x, w, None, split)[4], (x.float() @ w.float().t()).to(torch.bfloat16))
