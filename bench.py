@@ -23,7 +23,7 @@ PEAK_HBM_GBS = 8000.0
 # HBM-side bytes per launch from rocprofv3 FETCH_SIZE/WRITE_SIZE, each scaled by what the same counter reads for the
 # plain 256 MiB copy of `--workload copy` (factors 2.000 and 1.000); see profiles/*.md
 MEASURED_TRAFFIC_BYTES = {"config2": 184.3e6, "kv_append": 351.9e6, "rab_time": 1479.8e6, "rab_time_bwd": 2242.4e6, "rab_pos": 305.2e6,
-                          "nmd_fwd": 827.4e6, "nmd_bwd": 1382.0e6}
+                          "nmd_fwd": 827.4e6, "nmd_bwd": 1382.0e6, "in_linear_silu": 1092.9e6}
 
 
 def build_workload(name, torch, W):
@@ -58,7 +58,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=1000)
-    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "config2_bwd", "kv_append", "rab_time", "rab_time_bwd", "rab_pos", "nmd_fwd", "nmd_bwd", "copy"],
+    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "config2_bwd", "kv_append", "rab_time", "rab_time_bwd", "rab_pos", "nmd_fwd", "nmd_bwd", "in_linear_silu", "copy"],
                     help="'copy' runs a plain 256 MiB device copy: the known-size kernel the FETCH_SIZE/WRITE_SIZE counters are scaled by")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
@@ -80,6 +80,8 @@ def main():
         return bias_bench(args, torch)
     if args.workload in ("nmd_fwd", "nmd_bwd"):
         return nmd_bench(args, torch)
+    if args.workload == "in_linear_silu":
+        return in_linear_silu_bench(args, torch)
     cfg, op, flops, alg_bytes, desc = build_workload(args.workload, torch, W)
     dev = W.to_device(cfg)
     q, k, v = dev["q"], dev["k"], dev["v"]
@@ -417,6 +419,54 @@ def nmd_bench(args, torch):
         dt = time.perf_counter() - t0
         out["cpu_baseline"] = {"value": round(cpu_bytes / dt / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
                                "sample": f"the first {n_cpu} rows once (oracle in torch, fp64), {dt:.2f} s"}
+    print(json.dumps(out), flush=True)
+
+
+def in_linear_silu_bench(args, torch):
+    """The input projection at the largest shape of the reference's tests (test_in_linear_silu.py:101-109): m = 16384,
+    n = 16384, k = 64, bf16, equal splits.  4 bytes written per output element against 2 k = 128 FLOPs: bounded by the HBM
+    writes of linear_output and the four split outputs."""
+    from oracle import layer_oracle as LO
+    m_, n, k = 16384, 16384, 64
+    g = torch.Generator().manual_seed(13)
+    x = torch.randint(-100, 101, (m_, k), generator=g).to(torch.bfloat16)
+    w = ((torch.rand(n, k, generator=g) * 2 - 1) * (6.0 / (n + k)) ** 0.5).to(torch.bfloat16)
+    bias = torch.ones(n)
+    sp = [n // 4] * 4
+    xd, wd, bd = x.cuda(), w.cuda(), bias.cuda()
+    fn = lambda: torch.ops.mxrec.distance_in_linear_silu(xd, wd, bd, sp)
+    for _ in range(args.warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    kern_ms = e0.elapsed_time(e1) / args.steps
+    alg = 2 * m_ * n * 2 + m_ * k * 2 + n * k * 2 + n * 4
+    flops = 2.0 * m_ * n * k
+    out = {
+        "metric": "in_linear_silu_gbps", "value": round(alg / (ms * 1e-3) / 1e9, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic", "us_per_call": round(ms * 1e3, 2), "tflops": round(flops / (ms * 1e-3) / 1e12, 1),
+        "config": {"workload": "in_linear_silu: x [16384, 64], W [16384, 64] bf16, bias fp32, splits 4 x 4096, seed 13",
+                   "algorithmic_bytes_per_call": alg, "flops_per_call": flops,
+                   "entry": "torch.ops.mxrec.distance_in_linear_silu -> hstu_in_linear_silu_kernel (C ABI in include/hstu_layer.h)"},
+        "roofline": {"bound": "hbm", "kernel": "hstu_in_linear_silu_kernel", "achieved": round(alg / (kern_ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS,
+                     "unit": "GB/s", "frac": round(alg / (kern_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                     "kernel_us": round(kern_ms * 1e3, 2)},
+    }
+    if not args.no_cpu_baseline:
+        rows = 4096
+        t0 = time.perf_counter()
+        LO.in_linear_silu(x[:rows], w, bias, sp)
+        dt = time.perf_counter() - t0
+        out["cpu_baseline"] = {"value": round(alg * rows / m_ / dt / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"the first {rows} rows once (oracle in torch, fp64), {dt:.2f} s"}
     print(json.dumps(out), flush=True)
 
 

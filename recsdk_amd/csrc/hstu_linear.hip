@@ -51,8 +51,21 @@ __global__ __launch_bounds__(ILS_NT) void hstu_in_linear_silu_kernel(const IlsAr
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int g = lane >> 5, l32 = lane & 31;
     const int K = p.k, N = p.n;
-    const int n0 = blockIdx.x * ILS_BN;
-    const int64_t m0 = (int64_t)blockIdx.y * ILS_BM + 32 * w;
+    // Workgroup i of the 1-D grid runs on XCD i % 8 (each with its own L2).  Tiles are numbered so that one XCD sweeps
+    // a contiguous eighth of the n range for a block of rows: what its L2 writes back to HBM is then runs of 16 tiles
+    // (4 KiB) per row instead of 256-byte pieces interleaved with the other XCDs' at other times.
+    const unsigned nt = (unsigned)(N + ILS_BN - 1) / ILS_BN;
+    unsigned tn, tm;
+    if (nt % 8 == 0) {
+        const unsigned xcd = blockIdx.x & 7, j = blockIdx.x >> 3, per = nt / 8;
+        tn = xcd * per + j % per;
+        tm = j / per;
+    } else {
+        tn = blockIdx.x % nt;
+        tm = blockIdx.x / nt;
+    }
+    const int n0 = tn * ILS_BN;
+    const int64_t m0 = (int64_t)tm * ILS_BM + 32 * w;
     if (m0 >= p.m) return;   // whole wave; nothing below synchronises across waves
     const T* x = reinterpret_cast<const T*>(p.x);
     const T* wt = reinterpret_cast<const T*>(p.weight);
@@ -114,7 +127,7 @@ __global__ __launch_bounds__(ILS_NT) void hstu_in_linear_silu_kernel(const IlsAr
                     if (phase == 0) v[e] = l;
                     else {
                         const float f = to_float(l);
-                        v[e] = from_float<T>(f / (1.0f + __expf(-f)));
+                        v[e] = from_float<T>(f * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504f * f)));
                     }
                 }
                 ils_u2 o = {IlsMM<T>::pack2(v[0], v[1]), IlsMM<T>::pack2(v[2], v[3])};
@@ -156,7 +169,8 @@ extern "C" int hstu_hip_in_linear_silu(const hstu_in_linear_silu_params* p, void
         return fail(HSTU_ERR_INVALID_ARGUMENT, "hstu_in_linear_silu_params size mismatch: caller %u, library %zu", p->struct_size,
                     sizeof(hstu_in_linear_silu_params));
     if (p->dtype != HSTU_F16 && p->dtype != HSTU_BF16) return fail(HSTU_ERR_INVALID_ARGUMENT, "dtype expect float16 or bfloat16, but value is %d", p->dtype);
-    if (p->m < 1 || p->m > 65535LL * ILS_BM) return fail(HSTU_ERR_INVALID_ARGUMENT, "x dim[0] must in range[1, %lld], but got %lld", 65535LL * ILS_BM, (long long)p->m);
+    if (p->m < 1 || p->m > (1LL << 30)) return fail(HSTU_ERR_INVALID_ARGUMENT, "x dim[0] must in range[1, %lld], but got %lld", 1LL << 30, (long long)p->m);
+    if (((p->n + ILS_BN - 1) / ILS_BN) * ((p->m + ILS_BM - 1) / ILS_BM) > 0x7fffffffLL) return fail(HSTU_ERR_UNSUPPORTED, "m * n too large for one launch");
     IlsArgs a;
     a.p = *p;
     int total = 0;
@@ -175,7 +189,7 @@ extern "C" int hstu_hip_in_linear_silu(const hstu_in_linear_silu_params* p, void
     const void* ptrs[] = {p->x, p->weight, p->bias, p->linear_output, p->out[0], p->out[1], p->out[2], p->out[3]};
     for (const void* q : ptrs)
         if (reinterpret_cast<uintptr_t>(q) & 15) return fail(HSTU_ERR_UNSUPPORTED, "x, weight, bias and the outputs must be 16-byte aligned");
-    const dim3 grid((unsigned)((p->n + ILS_BN - 1) / ILS_BN), (unsigned)((p->m + ILS_BM - 1) / ILS_BM));
+    const dim3 grid((unsigned)((p->n + ILS_BN - 1) / ILS_BN) * (unsigned)((p->m + ILS_BM - 1) / ILS_BM));
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     if (p->dtype == HSTU_BF16) hipLaunchKernelGGL(hstu_in_linear_silu_kernel<__bf16>, grid, dim3(ILS_NT), 0, st, a);
     else hipLaunchKernelGGL(hstu_in_linear_silu_kernel<_Float16>, grid, dim3(ILS_NT), 0, st, a);
