@@ -1,6 +1,6 @@
 /*
  * hstu_layer.h -- C ABI of the steps either side of the attention in an HSTU layer: the input projection
- * SiLU(x W^T + b) split into U, V, Q, K before it (mxrec::distance_in_linear_silu, forward), and LayerNorm(x) * u with
+ * SiLU(x W^T + b) split into U, V, Q, K before it (mxrec::in_linear_silu, forward and backward), and LayerNorm(x) * u with
  * dropout after it, forward and backward (mxrec::norm_multiply_dropout).
  *
  * Same conventions as hstu_hip.h: device pointers, asynchronous on `stream`, nothing read on the host, 0 or a negative
@@ -100,6 +100,35 @@ typedef struct hstu_in_linear_silu_params {
     void* linear_output;      /* [m, n] */
 } hstu_in_linear_silu_params;
 int hstu_hip_in_linear_silu(const hstu_in_linear_silu_params* p, void* stream);
+
+/* Backward of the input projection.  Replaces aclnnInLinearSiluBackward (in_linear_silu.cpp:121-163; golden
+ * cust_op/test/in_linear_silu_test_backward/test_in_linear_silu_backward.py:37-66):
+ *   dlin = round(grad * silu'(linear_output))   grad = (grad[0] | grad[1] | grad[2] | grad[3]) along n,
+ *                                               silu'(z) = s (1 + z (1 - s)), s = sigmoid(z)
+ *   x_grad = dlin W  [m, k]     weight_grad = dlin^T x  [n, k]     bias_grad = column sums of the unrounded dlin  [n]
+ * The four gradients are read where they are (the reference concatenates them first when the widths differ, :143-146).
+ * x_grad and weight_grad are written in grad_dtype: HSTU_F32 (what the reference's kernel produces, :139-140) or the
+ * dtype of x (what its wrapper hands back after a cast, :158); nothing needs zeroing.  Sums over m are formed in a fixed
+ * order: results are reproducible.  The workspace needs no initialisation and must be 16-byte aligned. */
+typedef struct hstu_in_linear_silu_bwd_params {
+    uint32_t struct_size;
+    int32_t dtype;            /* HSTU_F16 / HSTU_BF16: x, weight, grad[], linear_output */
+    int64_t m;
+    int32_t k;
+    int32_t n;
+    int32_t split[4];
+    int32_t grad_dtype;       /* HSTU_F32 or dtype */
+    int32_t reserved;
+    const void* x;            /* [m, k] */
+    const void* weight;       /* [n, k] */
+    const void* grad[4];      /* user_grad [m, split[0]], value_grad, query_grad, key_grad */
+    const void* linear_output;/* [m, n], from the forward */
+    void* x_grad;             /* [m, k] */
+    void* weight_grad;        /* [n, k] */
+    float* bias_grad;         /* [n] fp32, or NULL */
+} hstu_in_linear_silu_bwd_params;
+int hstu_hip_in_linear_silu_backward_get_workspace_size(const hstu_in_linear_silu_bwd_params* p, uint64_t* workspace_bytes);
+int hstu_hip_in_linear_silu_backward(const hstu_in_linear_silu_bwd_params* p, void* workspace, uint64_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus
 }

@@ -19,13 +19,21 @@ Definition followed (reference file:line):
 * in_linear_silu: cust_op/test/in_linear_silu_test/test_in_linear_silu.py:31-45 -- ``addmm(bias, x, W^T)`` rounded to the
   I/O dtype (= linear_output), SiLU of that rounded tensor, rounded again, split along the last axis.
 
+* in_linear_silu_backward: cust_op/test/in_linear_silu_test_backward/test_in_linear_silu_backward.py:37-88 --
+  ``dlin = grad * sigmoid(lin) * (1 + lin * (1 - sigmoid(lin)))`` with grad the four gradients side by side,
+  ``bias_grad = dlin.sum(0)`` from the unrounded dlin, ``x_grad = dlin @ W``, ``weight_grad = dlin^T @ x``; the
+  device-side golden (:37-66) rounds dlin to the I/O dtype before the two products, the CPU golden (:69-88) does not:
+  ``round_dlin`` selects.
+
 Everything here is fp64 so that it can serve as the exact value for every I/O dtype (``in_linear_silu`` applies the
 golden's two roundings to the I/O dtype on top of fp64 arithmetic).
 
 Pinning status (tests/test_oracle_layer.py): forward against ``torch.nn.functional.layer_norm`` (a library routine
 that shares no code with the explicit mean / var formula here) and ``F.dropout`` semantics under a given mask; backward
 against autograd through that library forward, including the mask.  ``in_linear_silu`` against ``torch.addmm``,
-``F.silu`` and ``torch.split`` evaluated in fp32 on values where fp32 is exact.  PINNED
+``F.silu`` and ``torch.split`` evaluated in fp32 on values where fp32 is exact; ``in_linear_silu_backward`` against
+autograd through ``F.linear`` / ``F.silu`` in fp64 (which knows nothing of the closed-form derivative used here) and
+against central differences.  PINNED
 """
 from __future__ import annotations
 
@@ -74,3 +82,15 @@ def in_linear_silu(x, weight, bias, split):
     act = (lin.double() * torch.sigmoid(lin.double())).to(x.dtype)
     u, v, q, k = torch.split(act, list(split), dim=-1)
     return u.contiguous(), v.contiguous(), q.contiguous(), k.contiguous(), lin
+
+
+def in_linear_silu_backward(grads, x, weight, linear_output, with_bias=True, round_dlin=True):
+    """Returns (x_grad, weight_grad, bias_grad or None) in fp64."""
+    grad = torch.cat([g.double() for g in grads], dim=-1)
+    lin = linear_output.double()
+    sg = torch.sigmoid(lin)
+    dlin = grad * (sg * (1 + lin * (1 - sg)))
+    bias_grad = dlin.sum(dim=0) if with_bias else None
+    if round_dlin:
+        dlin = dlin.to(x.dtype).double()
+    return dlin @ weight.double(), dlin.t() @ x.double(), bias_grad

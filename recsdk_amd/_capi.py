@@ -31,6 +31,7 @@ EXPORTS = [
     "hstu_hip_rab_time", "hstu_hip_rab_time_backward", "hstu_hip_rab_pos",
     "hstu_hip_norm_multiply_dropout", "hstu_hip_norm_multiply_dropout_backward",
     "hstu_hip_norm_multiply_dropout_backward_get_workspace_size", "hstu_hip_in_linear_silu",
+    "hstu_hip_in_linear_silu_backward", "hstu_hip_in_linear_silu_backward_get_workspace_size",
 ]
 
 
@@ -119,6 +120,15 @@ class HstuInLinearSiluParams(C.Structure):
     ]
 
 
+class HstuInLinearSiluBwdParams(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32), ("dtype", C.c_int32), ("m", C.c_int64), ("k", C.c_int32), ("n", C.c_int32),
+        ("split", C.c_int32 * 4), ("grad_dtype", C.c_int32), ("reserved", C.c_int32),
+        ("x", C.c_void_p), ("weight", C.c_void_p), ("grad", C.c_void_p * 4), ("linear_output", C.c_void_p),
+        ("x_grad", C.c_void_p), ("weight_grad", C.c_void_p), ("bias_grad", C.c_void_p),
+    ]
+
+
 _lib: Optional[C.CDLL] = None
 
 
@@ -146,6 +156,8 @@ def lib() -> C.CDLL:
         _lib.hstu_hip_rab_time.argtypes = [C.POINTER(HstuRabTimeParams), C.c_void_p]
         _lib.hstu_hip_norm_multiply_dropout.argtypes = [C.POINTER(HstuNmdParams), C.c_void_p]
         _lib.hstu_hip_in_linear_silu.argtypes = [C.POINTER(HstuInLinearSiluParams), C.c_void_p]
+        _lib.hstu_hip_in_linear_silu_backward.argtypes = [C.POINTER(HstuInLinearSiluBwdParams), C.c_void_p, C.c_uint64, C.c_void_p]
+        _lib.hstu_hip_in_linear_silu_backward_get_workspace_size.argtypes = [C.POINTER(HstuInLinearSiluBwdParams), C.POINTER(C.c_uint64)]
         _lib.hstu_hip_norm_multiply_dropout_backward.argtypes = [C.POINTER(HstuNmdBwdParams), C.c_void_p, C.c_uint64, C.c_void_p]
         _lib.hstu_hip_norm_multiply_dropout_backward_get_workspace_size.argtypes = [C.POINTER(HstuNmdBwdParams), C.POINTER(C.c_uint64)]
         _lib.hstu_hip_rab_time_backward.argtypes = [C.POINTER(HstuRabTimeBwdParams), C.c_void_p]

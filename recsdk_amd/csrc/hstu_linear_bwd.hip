@@ -1,0 +1,440 @@
+// Backward of the input projection of an HSTU layer (mxrec::in_linear_silu_backward):
+//   dlin        = round(grad * silu'(linear_output))      grad = (user_grad | value_grad | query_grad | key_grad) along n
+//   x_grad      = dlin W            [m, k]   sum over n
+//   weight_grad = dlin^T x          [n, k]   sum over m
+//   bias_grad   = column sums of the unrounded dlin       [n], fp32
+// (golden cust_op/test/in_linear_silu_test_backward/test_in_linear_silu_backward.py:37-66; the reference kernel also
+// rounds dlin to the I/O dtype before its two matrix products and sums the bias gradient in fp32:
+// cust_op/ascendc_op/ai_core_op/in_linear_silu_backward/v220/op_kernel/in_linear_silu_backward.h:267-332).
+//
+// n is at least 4 k, so both products are skinny: every element of dlin meets only k multiply-adds per product and the
+// op is bounded by reading grad and linear_output from HBM.  dlin is therefore never written to memory: each of the two
+// product kernels streams grad and linear_output once and rebuilds dlin in registers.
+//   * hstu_ilb_xgrad_kernel: a workgroup owns 32 rows m; its four waves take every fourth 64-column piece of n, build
+//     dlin straight in the layout of an MFMA operand (a lane = one row, 8 consecutive n) and multiply by rows of W^T;
+//     the four partial results meet in LDS.
+//   * hstu_ilb_wgrad_kernel: a wave owns 64 columns n and walks down m in tiles of 32 rows; dlin is built in the layout
+//     the loads arrive in (a lane = 8 consecutive n of one row), parked in LDS and read back transposed (a lane = one
+//     column n, 8 consecutive m) against rows of x^T.  m is cut into S ranges to fill the chip; the S partial results
+//     are added in a fixed order by hstu_ilb_reduce_kernel, so the result is reproducible.
+// Both products want their small operand with the summed index contiguous: W^T [k, n] and x^T [k, m] are written to the
+// workspace first (hstu_ilb_transpose_kernel; together at most half of what grad alone takes, usually a few percent).
+#include "hstu_device.h"
+#include "../../include/hstu_layer.h"
+
+namespace hstu {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 ilb_bf16x8;
+typedef __attribute__((ext_vector_type(8))) _Float16 ilb_f16x8;
+typedef __attribute__((ext_vector_type(16))) float ilb_f32x16;
+typedef __attribute__((ext_vector_type(4))) float ilb_f32x4;
+
+template <typename T> struct IlbMM;
+template <> struct IlbMM<__bf16> {
+    typedef ilb_bf16x8 v8;
+    static __device__ __forceinline__ ilb_f32x16 mfma(v8 a, v8 b, ilb_f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+};
+template <> struct IlbMM<_Float16> {
+    typedef ilb_f16x8 v8;
+    static __device__ __forceinline__ ilb_f32x16 mfma(v8 a, v8 b, ilb_f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+};
+
+constexpr int ILB_NT = 256;
+constexpr int ILB_PARK = 64 * 2 + 16;   // bytes of one parked row of 64 columns: 8 rows further down is 32 banks away
+
+struct IlbArgs {
+    hstu_in_linear_silu_bwd_params p;
+    int base[5];          // first column of user, value, query, key, and n
+    const void* xt;       // [k, mpad]  x^T, zero for m <= column < mpad
+    const void* wt;       // [k, n]     W^T
+    float* wpart;         // [S, n, k]
+    float* bpart;         // [S, n]
+    int64_t mpad;         // m rounded up to 32
+    int64_t rows_per_part;
+    int parts;            // S
+};
+
+// grad * silu'(lin), unrounded
+template <typename T>
+__device__ __forceinline__ void ilb_dlin8(const typename IlbMM<T>::v8& g, const typename IlbMM<T>::v8& l, float* out) {
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        const float x = to_float(l[e]);
+        const float s = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504f * x));
+        out[e] = to_float(g[e]) * (s * (1.0f + x * (1.0f - s)));
+    }
+}
+
+// out[c][r] = in[r][c] for r < rows, c < cols; out has row stride rpad >= rows, zero for rows <= r < rpad
+__global__ __launch_bounds__(256) void hstu_ilb_transpose_kernel(const uint16_t* in, int64_t rows, int cols, uint16_t* out, int64_t rpad) {
+    __shared__ uint16_t tile[32][33];
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+    const int64_t r0 = (int64_t)blockIdx.x * 32;
+    const int c0 = blockIdx.y * 32;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int64_t r = r0 + ty + 8 * i;
+        const int c = c0 + tx;
+        tile[ty + 8 * i][tx] = (r < rows && c < cols) ? in[r * cols + c] : (uint16_t)0;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int c = c0 + ty + 8 * i;
+        if (c < cols && r0 + tx < rpad) out[(int64_t)c * rpad + r0 + tx] = tile[tx][ty + 8 * i];
+    }
+}
+
+// pointer to 8 consecutive gradient columns starting at column n (a multiple of 8) of row `row`
+template <typename T>
+__device__ __forceinline__ const T* ilb_grad_ptr(const IlbArgs& a, int n, int64_t row) {
+    int sel = 0;
+#pragma unroll
+    for (int i = 1; i < 4; i++) sel += n >= a.base[i] ? 1 : 0;
+    const void* g = a.p.grad[0];
+    int first = a.base[0], width = a.p.split[0];
+#pragma unroll
+    for (int i = 1; i < 4; i++)
+        if (sel == i) { g = a.p.grad[i]; first = a.base[i]; width = a.p.split[i]; }
+    return reinterpret_cast<const T*>(g) + row * width + (n - first);
+}
+
+template <typename T> __device__ __forceinline__ void ilb_store(void* out, int64_t idx, float v, int as_f32) {
+    if (as_f32) reinterpret_cast<float*>(out)[idx] = v;
+    else reinterpret_cast<T*>(out)[idx] = from_float<T>(v);
+}
+
+// x_grad.  grid = (ceil(m / 32), ceil(k / KC)), 4 waves.
+template <typename T, int KC>
+__global__ __launch_bounds__(ILB_NT) void hstu_ilb_xgrad_kernel(const IlbArgs a) {
+    typedef typename IlbMM<T>::v8 v8;
+    constexpr int KB = KC / 32;
+    __shared__ float red[3][32][KC + 1];
+    const hstu_in_linear_silu_bwd_params& p = a.p;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int g = lane >> 5, l32 = lane & 31;
+    const int N = p.n, K = p.k;
+    const int64_t m0 = (int64_t)blockIdx.x * 32;
+    const int k0 = blockIdx.y * KC;
+    const int64_t row = m0 + l32 < p.m ? m0 + l32 : p.m - 1;   // rows past the end repeat the last one and are not stored
+    const T* lin = reinterpret_cast<const T*>(p.linear_output) + row * N + 8 * g;
+    const T* wrow[KB];
+#pragma unroll
+    for (int kb = 0; kb < KB; kb++) wrow[kb] = reinterpret_cast<const T*>(a.wt) + (int64_t)min(k0 + 32 * kb + l32, K - 1) * N + 8 * g;
+    ilb_f32x16 acc[KB];
+#pragma unroll
+    for (int kb = 0; kb < KB; kb++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[kb][r] = 0.f;
+    auto step = [&](int n0) __attribute__((always_inline)) {   // 16 columns of n, inside one of the four gradients
+        const v8 gf = *reinterpret_cast<const v8*>(ilb_grad_ptr<T>(a, n0, row) + 8 * g);
+        const v8 lf = *reinterpret_cast<const v8*>(lin + n0);
+        v8 wf[KB];
+#pragma unroll
+        for (int kb = 0; kb < KB; kb++) wf[kb] = *reinterpret_cast<const v8*>(wrow[kb] + n0);
+        float d[8];
+        ilb_dlin8<T>(gf, lf, d);
+        v8 df;
+#pragma unroll
+        for (int e = 0; e < 8; e++) df[e] = from_float<T>(d[e]);
+#pragma unroll
+        for (int kb = 0; kb < KB; kb++) acc[kb] = IlbMM<T>::mfma(wf[kb], df, acc[kb]);
+    };
+    for (int c = 64 * w; c < N; c += 256) {
+        if (c + 64 <= N) {
+            step(c);
+            step(c + 16);
+            step(c + 32);
+            step(c + 48);
+        } else {
+            for (int n0 = c; n0 < N; n0 += 16) step(n0);
+        }
+    }
+    // accumulator register r of block kb: column k0 + 32 kb + 8 (r / 4) + 4 g + r % 4 of row m0 + l32.
+    // Waves 1..3 park their sums, wave 0 adds them to its own in that order and parks the total in the first slot.
+    if (w > 0) {
+#pragma unroll
+        for (int kb = 0; kb < KB; kb++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) red[w - 1][l32][32 * kb + 8 * (r / 4) + 4 * g + (r % 4)] = acc[kb][r];
+    }
+    __syncthreads();
+    if (w == 0) {
+#pragma unroll
+        for (int kb = 0; kb < KB; kb++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int c = 32 * kb + 8 * (r / 4) + 4 * g + (r % 4);
+                red[0][l32][c] = ((acc[kb][r] + red[0][l32][c]) + red[1][l32][c]) + red[2][l32][c];
+            }
+    }
+    __syncthreads();
+    const int as_f32 = p.grad_dtype == HSTU_F32;
+    for (int i = threadIdx.x; i < 32 * KC; i += ILB_NT) {
+        const int r = i / KC, c = i % KC;
+        if (m0 + r < p.m && k0 + c < K) ilb_store<T>(p.x_grad, (m0 + r) * K + k0 + c, red[0][r][c], as_f32);
+    }
+}
+
+// weight_grad and bias_grad partial sums.  grid = (ceil(n / 256), ceil(k / KC), S), 4 waves of 64 columns n each.
+template <typename T, int KC>
+__global__ __launch_bounds__(ILB_NT) void hstu_ilb_wgrad_kernel(const IlbArgs a) {
+    typedef typename IlbMM<T>::v8 v8;
+    constexpr int KB = KC / 32;
+    __shared__ __attribute__((aligned(16))) char park_all[(ILB_NT / 64) * 32 * ILB_PARK];
+    const hstu_in_linear_silu_bwd_params& p = a.p;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int g = lane >> 5, l32 = lane & 31;
+    const int N = p.n, K = p.k;
+    const int nw = blockIdx.x * 256 + 64 * w;     // first column of this wave
+    if (nw >= N) return;                          // whole wave; nothing below synchronises across waves
+    const int k0 = blockIdx.y * KC;
+    const int64_t mbeg = (int64_t)blockIdx.z * a.rows_per_part;
+    const int64_t mend = mbeg + a.rows_per_part < p.m ? mbeg + a.rows_per_part : p.m;
+    // load phase: lane = 8 consecutive columns (chunk) of the rows lrow, lrow + 8, lrow + 16, lrow + 24 of a tile
+    const int chunk = lane & 7, lrow = lane >> 3;
+    const int ncol = nw + 8 * chunk;
+    const bool live = ncol < N;
+    const int ncl = live ? ncol : 0;
+    int sel = 0;
+#pragma unroll
+    for (int i = 1; i < 4; i++) sel += ncl >= a.base[i] ? 1 : 0;
+    const void* gbase = p.grad[0];
+    int gfirst = a.base[0], gwidth = p.split[0];
+#pragma unroll
+    for (int i = 1; i < 4; i++)
+        if (sel == i) { gbase = p.grad[i]; gfirst = a.base[i]; gwidth = p.split[i]; }
+    const T* gptr = reinterpret_cast<const T*>(gbase) + (ncl - gfirst);
+    const T* lptr = reinterpret_cast<const T*>(p.linear_output) + ncl;
+    const T* xrow[KB];
+#pragma unroll
+    for (int kb = 0; kb < KB; kb++) xrow[kb] = reinterpret_cast<const T*>(a.xt) + (int64_t)min(k0 + 32 * kb + l32, K - 1) * a.mpad + 8 * g;
+    char* park = park_all + w * (32 * ILB_PARK);
+    ilb_f32x16 acc[2][KB];
+#pragma unroll
+    for (int nb = 0; nb < 2; nb++)
+#pragma unroll
+        for (int kb = 0; kb < KB; kb++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[nb][kb][r] = 0.f;
+    float bsum[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) bsum[e] = 0.f;
+    for (int64_t m0 = mbeg; m0 < mend; m0 += 32) {
+        v8 gf[4], lf[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int64_t r = m0 + lrow + 8 * i;
+            const int64_t rc = r < mend ? r : mend - 1;
+            gf[i] = *reinterpret_cast<const v8*>(gptr + rc * gwidth);
+            lf[i] = *reinterpret_cast<const v8*>(lptr + rc * N);
+        }
+        v8 xf[2][KB];   // rows of x^T: columns m0 + 16 ks + 8 g .. + 7 (zero past m)
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+            for (int kb = 0; kb < KB; kb++) xf[ks][kb] = *reinterpret_cast<const v8*>(xrow[kb] + m0 + 16 * ks);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            float d[8];
+            ilb_dlin8<T>(gf[i], lf[i], d);
+            const bool in = live && m0 + lrow + 8 * i < mend;
+            v8 df;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const float v = in ? d[e] : 0.f;
+                bsum[e] += v;
+                df[e] = from_float<T>(v);
+            }
+            *reinterpret_cast<v8*>(park + (lrow + 8 * i) * ILB_PARK + chunk * 16) = df;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++) {
+#pragma unroll
+            for (int nb = 0; nb < 2; nb++) {
+                v8 af;   // column nw + 32 nb + l32 of dlin, rows m0 + 16 ks + 8 g .. + 7
+#pragma unroll
+                for (int j = 0; j < 8; j++) af[j] = *reinterpret_cast<const T*>(park + (16 * ks + 8 * g + j) * ILB_PARK + (32 * nb + l32) * 2);
+#pragma unroll
+                for (int kb = 0; kb < KB; kb++) acc[nb][kb] = IlbMM<T>::mfma(af, xf[ks][kb], acc[nb][kb]);
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+    // accumulator register r of block (nb, kb): row nw + 32 nb + 8 (r / 4) + 4 g + r % 4, column k0 + 32 kb + l32
+    float* wp = a.wpart + (int64_t)blockIdx.z * N * K;
+#pragma unroll
+    for (int nb = 0; nb < 2; nb++)
+#pragma unroll
+        for (int kb = 0; kb < KB; kb++) {
+            const int kc = k0 + 32 * kb + l32;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int nr = nw + 32 * nb + 8 * (r / 4) + 4 * g + (r % 4);
+                if (nr < N && kc < K) wp[(int64_t)nr * K + kc] = acc[nb][kb][r];
+            }
+        }
+    if (blockIdx.y == 0) {
+        // the eight lanes of one chunk (one per row group) hold the sums of the same 8 columns
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            float s = bsum[e];
+            s += __shfl_xor(s, 8);
+            s += __shfl_xor(s, 16);
+            s += __shfl_xor(s, 32);
+            bsum[e] = s;
+        }
+        if (lrow == 0 && live) {
+            float* bp = a.bpart + (int64_t)blockIdx.z * N + ncol;
+            *reinterpret_cast<ilb_f32x4*>(bp) = ilb_f32x4{bsum[0], bsum[1], bsum[2], bsum[3]};
+            *reinterpret_cast<ilb_f32x4*>(bp + 4) = ilb_f32x4{bsum[4], bsum[5], bsum[6], bsum[7]};
+        }
+    }
+}
+
+// out[i] = part[0][i] + part[1][i] + ... in that order, four elements per thread (count is a multiple of 4)
+template <typename T>
+__global__ __launch_bounds__(256) void hstu_ilb_reduce_kernel(const float* part, int parts, int64_t count, void* out, int as_f32) {
+    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= count) return;
+    ilb_f32x4 s = *reinterpret_cast<const ilb_f32x4*>(part + i);
+    for (int z = 1; z < parts; z++) {
+        const ilb_f32x4 v = *reinterpret_cast<const ilb_f32x4*>(part + (int64_t)z * count + i);
+#pragma unroll
+        for (int e = 0; e < 4; e++) s[e] += v[e];
+    }
+#pragma unroll
+    for (int e = 0; e < 4; e++) ilb_store<T>(out, i + e, s[e], as_f32);
+}
+
+struct IlbPlan {
+    int kc;               // k columns per workgroup: 64 or 128
+    int parts;
+    int64_t rows_per_part, mpad;
+    uint64_t off_xt, off_wt, off_wpart, off_bpart, total;
+};
+
+static uint64_t ilb_align(uint64_t v) { return (v + 255) & ~(uint64_t)255; }
+
+static IlbPlan ilb_plan(const hstu_in_linear_silu_bwd_params* p) {
+    IlbPlan pl;
+    pl.kc = p->k > 64 ? 128 : 64;
+    const int64_t tiles = (p->m + 31) / 32;
+    const int64_t blocks = (int64_t)((p->n + 255) / 256) * ((p->k + pl.kc - 1) / pl.kc);
+    int64_t parts = (1024 + blocks - 1) / blocks;
+    if (parts > tiles) parts = tiles;
+    if (parts < 1) parts = 1;
+    pl.rows_per_part = ((tiles + parts - 1) / parts) * 32;
+    pl.parts = (int)((p->m + pl.rows_per_part - 1) / pl.rows_per_part);
+    pl.mpad = tiles * 32;
+    uint64_t o = 0;
+    pl.off_xt = o;
+    o = ilb_align(o + (uint64_t)p->k * pl.mpad * 2);
+    pl.off_wt = o;
+    o = ilb_align(o + (uint64_t)p->k * p->n * 2);
+    pl.off_wpart = o;
+    o = ilb_align(o + (uint64_t)pl.parts * p->n * p->k * 4);
+    pl.off_bpart = o;
+    o = ilb_align(o + (uint64_t)pl.parts * p->n * 4);
+    pl.total = o;
+    return pl;
+}
+
+static int ilb_check(const hstu_in_linear_silu_bwd_params* p) {
+    if (!p) return fail(HSTU_ERR_INVALID_ARGUMENT, "params is NULL");
+    if (p->struct_size != sizeof(hstu_in_linear_silu_bwd_params))
+        return fail(HSTU_ERR_INVALID_ARGUMENT, "hstu_in_linear_silu_bwd_params size mismatch: caller %u, library %zu", p->struct_size,
+                    sizeof(hstu_in_linear_silu_bwd_params));
+    if (p->dtype != HSTU_F16 && p->dtype != HSTU_BF16) return fail(HSTU_ERR_INVALID_ARGUMENT, "dtype expect float16 or bfloat16, but value is %d", p->dtype);
+    if (p->grad_dtype != HSTU_F32 && p->grad_dtype != p->dtype)
+        return fail(HSTU_ERR_INVALID_ARGUMENT, "grad_dtype expect float32 or the dtype of x, but value is %d", p->grad_dtype);
+    if (p->m < 1 || p->m > (1LL << 30)) return fail(HSTU_ERR_INVALID_ARGUMENT, "x dim[0] must in range[1, %lld], but got %lld", 1LL << 30, (long long)p->m);
+    int total = 0;
+    for (int i = 0; i < 4; i++) {
+        if (p->split[i] < 16 || p->split[i] > 8192 || p->split[i] % 16) return fail(HSTU_ERR_INVALID_ARGUMENT, "uvqk dim must in range[16, 8192] and multiples of 16.");
+        total += p->split[i];
+    }
+    if (p->k < 16 || p->k > 8192 || p->k % 16) return fail(HSTU_ERR_INVALID_ARGUMENT, "x dim[1] must in range[16, 8192] and multiples of 16.");
+    if (p->n < 64 || p->n > 32768 || p->n % 16) return fail(HSTU_ERR_INVALID_ARGUMENT, "weight dim[0] must in range[64, 32768] and multiples of 16.");
+    if (total != p->n) return fail(HSTU_ERR_INVALID_ARGUMENT, "weight_dim[0] must equal to sum(splitList).");
+    if (p->n % (4 * p->k)) return fail(HSTU_ERR_INVALID_ARGUMENT, "weight dim[0] must be a multiple of 4 x dim[1]");
+    return HSTU_OK;
+}
+
+}  // namespace hstu
+
+using namespace hstu;
+
+extern "C" int hstu_hip_in_linear_silu_backward_get_workspace_size(const hstu_in_linear_silu_bwd_params* p, uint64_t* workspace_bytes) {
+    const int rc = ilb_check(p);
+    if (rc != HSTU_OK) return rc;
+    if (!workspace_bytes) return fail(HSTU_ERR_INVALID_ARGUMENT, "workspace_bytes is NULL");
+    *workspace_bytes = ilb_plan(p).total;
+    return HSTU_OK;
+}
+
+template <typename T>
+static void ilb_launch(const IlbArgs& a, const IlbPlan& pl, hipStream_t st) {
+    const hstu_in_linear_silu_bwd_params& p = a.p;
+    // W [n, k] -> W^T [k, n];  x [m, k] -> x^T [k, mpad]
+    hipLaunchKernelGGL(hstu_ilb_transpose_kernel, dim3((unsigned)((p.n + 31) / 32), (unsigned)((p.k + 31) / 32)), dim3(256), 0, st,
+                       reinterpret_cast<const uint16_t*>(p.weight), (int64_t)p.n, p.k, reinterpret_cast<uint16_t*>(const_cast<void*>(a.wt)), (int64_t)p.n);
+    hipLaunchKernelGGL(hstu_ilb_transpose_kernel, dim3((unsigned)(pl.mpad / 32), (unsigned)((p.k + 31) / 32)), dim3(256), 0, st,
+                       reinterpret_cast<const uint16_t*>(p.x), p.m, p.k, reinterpret_cast<uint16_t*>(const_cast<void*>(a.xt)), pl.mpad);
+    const unsigned kchunks = (unsigned)((p.k + pl.kc - 1) / pl.kc);
+    const dim3 gx((unsigned)(pl.mpad / 32), kchunks), gw((unsigned)((p.n + 255) / 256), kchunks, (unsigned)pl.parts);
+    if (pl.kc == 64) {
+        hipLaunchKernelGGL((hstu_ilb_xgrad_kernel<T, 64>), gx, dim3(ILB_NT), 0, st, a);
+        hipLaunchKernelGGL((hstu_ilb_wgrad_kernel<T, 64>), gw, dim3(ILB_NT), 0, st, a);
+    } else {
+        hipLaunchKernelGGL((hstu_ilb_xgrad_kernel<T, 128>), gx, dim3(ILB_NT), 0, st, a);
+        hipLaunchKernelGGL((hstu_ilb_wgrad_kernel<T, 128>), gw, dim3(ILB_NT), 0, st, a);
+    }
+    const int64_t cw = (int64_t)p.n * p.k;
+    hipLaunchKernelGGL(hstu_ilb_reduce_kernel<T>, dim3((unsigned)((cw / 4 + 255) / 256)), dim3(256), 0, st, a.wpart, pl.parts, cw, p.weight_grad,
+                       (int)(p.grad_dtype == HSTU_F32));
+    if (p.bias_grad)
+        hipLaunchKernelGGL(hstu_ilb_reduce_kernel<T>, dim3((unsigned)((p.n / 4 + 255) / 256)), dim3(256), 0, st, a.bpart, pl.parts, (int64_t)p.n,
+                           (void*)p.bias_grad, 1);
+}
+
+extern "C" int hstu_hip_in_linear_silu_backward(const hstu_in_linear_silu_bwd_params* p, void* workspace, uint64_t workspace_bytes, void* stream) {
+    const int rc = ilb_check(p);
+    if (rc != HSTU_OK) return rc;
+    if (!p->x || !p->weight || !p->linear_output || !p->grad[0] || !p->grad[1] || !p->grad[2] || !p->grad[3] || !p->x_grad || !p->weight_grad)
+        return fail(HSTU_ERR_INVALID_ARGUMENT, "x, weight, the four gradients, linear_output, x_grad and weight_grad must not be NULL");
+    const void* ptrs[] = {p->x, p->weight, p->linear_output, p->grad[0], p->grad[1], p->grad[2], p->grad[3], p->x_grad, p->weight_grad, p->bias_grad, workspace};
+    for (const void* q : ptrs)
+        if (reinterpret_cast<uintptr_t>(q) & 15) return fail(HSTU_ERR_UNSUPPORTED, "every tensor and the workspace must be 16-byte aligned");
+    const IlbPlan pl = ilb_plan(p);
+    if (!workspace || workspace_bytes < pl.total)
+        return fail(HSTU_ERR_WORKSPACE, "workspace of %llu bytes needed, %llu given", (unsigned long long)pl.total, (unsigned long long)workspace_bytes);
+    if (pl.mpad / 32 > 0x7fffffffLL || pl.parts > 65535) return fail(HSTU_ERR_UNSUPPORTED, "m too large for one launch");
+    IlbArgs a;
+    a.p = *p;
+    int total = 0;
+    for (int i = 0; i < 4; i++) {
+        a.base[i] = total;
+        total += p->split[i];
+    }
+    a.base[4] = total;
+    char* ws = reinterpret_cast<char*>(workspace);
+    a.xt = ws + pl.off_xt;
+    a.wt = ws + pl.off_wt;
+    a.wpart = reinterpret_cast<float*>(ws + pl.off_wpart);
+    a.bpart = reinterpret_cast<float*>(ws + pl.off_bpart);
+    a.mpad = pl.mpad;
+    a.rows_per_part = pl.rows_per_part;
+    a.parts = pl.parts;
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (p->dtype == HSTU_BF16) ilb_launch<__bf16>(a, pl, st);
+    else ilb_launch<_Float16>(a, pl, st);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString(e));
+    return HSTU_OK;
+}

@@ -1042,6 +1042,117 @@ std::vector<at::Tensor> distance_in_linear_silu(const at::Tensor& x, const at::T
     return outs;
 }
 
+// in_linear_silu_backward (in_linear_silu.cpp:68-95 IsValidShapeBackward, :121-163 RunInLinearSiluBackward)
+static void in_linear_silu_check(const at::Tensor& x, const at::Tensor& weight, const at::Tensor& bias, at::IntArrayRef split_list) {
+    // IsValidShape, in_linear_silu.cpp:34-66
+    check_tensor_non_empty(x, "x");
+    check_tensor_non_empty(weight, "weight");
+    TORCH_CHECK(x.dim() == 2, "x must be 2D");
+    TORCH_CHECK(weight.dim() == 2, "weight must be 2D");
+    TORCH_CHECK(split_list.size() == 4, "splitList must have 4 elements.");
+    int64_t total = 0;
+    for (int i = 0; i < 4; i++) {
+        TORCH_CHECK(split_list[i] >= 16 && split_list[i] <= 8192 && split_list[i] % 16 == 0, "uvqk dim must in range[16, 8192] and multiples of 16.");
+        total += split_list[i];
+    }
+    const auto k = x.size(1), n = weight.size(0);
+    TORCH_CHECK(k >= 16 && k <= 8192 && k % 16 == 0, "x dim[1] must in range[16, 8192] and multiples of 16.");
+    TORCH_CHECK(n >= 64 && n <= 32768 && n % 16 == 0, "weight dim[0] must in range[64, 32768] and multiples of 16.");
+    TORCH_CHECK(total == n, "weight_dim[0] must equal to sum(splitList).");
+    TORCH_CHECK(weight.size(1) == k, "weight dim[1] must equal to x dim[1].");
+    TORCH_CHECK(n % (4 * k) == 0, "weight dim[0] must be a multiple of 4 x dim[1]");
+    if (bias.defined()) {
+        check_tensor_non_empty(bias, "bias");
+        TORCH_CHECK(bias.dim() == 1, "bias must be 1D");
+        TORCH_CHECK(bias.size(0) == n, "bias dim[0] must equal to weight dim[0].");
+    }
+    TORCH_CHECK(x.scalar_type() == at::kHalf || x.scalar_type() == at::kBFloat16, "x dtype expect float16 or bfloat16, but get ", x.scalar_type());
+    TORCH_CHECK(weight.scalar_type() == x.scalar_type(), "weight must have the dtype of x");
+}
+
+std::vector<at::Tensor> in_linear_silu_backward(const at::Tensor& x, const at::Tensor& weight, const c10::optional<at::Tensor>& bias,
+                                                const at::Tensor& user_grad, const at::Tensor& value_grad, const at::Tensor& query_grad,
+                                                const at::Tensor& key_grad, const at::Tensor& linear_output, at::IntArrayRef split_list) {
+    const at::Tensor b = bias.has_value() ? bias.value() : at::Tensor();
+    in_linear_silu_check(x, weight, b, split_list);
+    const at::Tensor* grads[4] = {&user_grad, &value_grad, &query_grad, &key_grad};
+    const char* names[4] = {"user_grad", "value_grad", "query_grad", "key_grad"};
+    const auto m = x.size(0), k = x.size(1), n = weight.size(0);
+    for (int i = 0; i < 4; i++) {
+        check_tensor_non_empty(*grads[i], names[i]);
+        TORCH_CHECK(grads[i]->dim() == 2, names[i], " must be 2D");
+        TORCH_CHECK(grads[i]->size(1) == split_list[i], "user_grad, value_grad, query_grad, key_grad dim[1] must be equal to splitList.");
+        TORCH_CHECK(grads[i]->size(0) == m, "user_grad, value_grad, query_grad, key_grad linear_output dim[0] must equal to x dim[0].");
+        TORCH_CHECK(grads[i]->scalar_type() == x.scalar_type(), names[i], " must have the dtype of x");
+    }
+    check_tensor_non_empty(linear_output, "linear_output");
+    TORCH_CHECK(linear_output.dim() == 2, "linear_output must be 2D");
+    TORCH_CHECK(linear_output.size(0) == m, "user_grad, value_grad, query_grad, key_grad linear_output dim[0] must equal to x dim[0].");
+    TORCH_CHECK(linear_output.size(1) == n, "linear_output dim[1] must equal to weight dim[0].");
+    TORCH_CHECK(linear_output.scalar_type() == x.scalar_type(), "linear_output must have the dtype of x");
+    Holder h;
+    auto dx = h.same(x), dw = h.same(weight), dl = h.same(linear_output);
+    require_gpu(dx, "in_linear_silu_backward");
+    hstu_in_linear_silu_bwd_params p;
+    std::memset(&p, 0, sizeof(p));
+    p.struct_size = sizeof(p);
+    p.dtype = io_dtype(dx, "x");
+    p.grad_dtype = p.dtype;   // the reference's wrapper hands x_grad and weight_grad back in the dtype of x and weight (:158)
+    p.m = m;
+    p.k = (int32_t)k;
+    p.n = (int32_t)n;
+    for (int i = 0; i < 4; i++) {
+        p.split[i] = (int32_t)split_list[i];
+        p.grad[i] = h.same(*grads[i]).const_data_ptr();
+    }
+    p.x = dx.const_data_ptr();
+    p.weight = dw.const_data_ptr();
+    p.linear_output = dl.const_data_ptr();
+    auto x_grad = at::empty_like(dx), weight_grad = at::empty_like(dw);
+    at::Tensor bias_grad32;
+    if (b.defined()) bias_grad32 = at::empty({n}, dx.options().dtype(at::kFloat));
+    p.x_grad = x_grad.data_ptr();
+    p.weight_grad = weight_grad.data_ptr();
+    p.bias_grad = bias_grad32.defined() ? bias_grad32.data_ptr<float>() : nullptr;
+    uint64_t ws_bytes = 0;
+    int rc = hstu_hip_in_linear_silu_backward_get_workspace_size(&p, &ws_bytes);
+    TORCH_CHECK(rc == HSTU_OK, "mxrec::in_linear_silu_backward: ", hstu_hip_last_error());
+    c10::hip::OptionalHIPGuardMasqueradingAsCUDA guard(dx.device());
+    auto ws = at::empty({(int64_t)ws_bytes}, dx.options().dtype(at::kByte));
+    auto stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA();
+    rc = hstu_hip_in_linear_silu_backward(&p, ws.data_ptr(), ws_bytes, (void*)stream.stream());
+    TORCH_CHECK(rc == HSTU_OK, "mxrec::in_linear_silu_backward: ", hstu_hip_last_error());
+    at::Tensor bias_grad;
+    if (b.defined()) bias_grad = bias_grad32.to(b.scalar_type());
+    return {x_grad, weight_grad, bias_grad, at::Tensor()};
+}
+
+// in_linear_silu: the forward with the backward attached (RunInLinearSiluFunction, in_linear_silu.cpp:165-197)
+class InLinearSiluFunction : public torch::autograd::Function<InLinearSiluFunction> {
+public:
+    static torch::autograd::tensor_list forward(torch::autograd::AutogradContext* ctx, const at::Tensor& x, const at::Tensor& weight,
+                                                const at::Tensor& bias, at::IntArrayRef split_list) {
+        at::AutoDispatchBelowADInplaceOrView guard;
+        auto outs = distance_in_linear_silu(x, weight, bias, split_list);
+        ctx->save_for_backward({x, weight, bias, outs[4]});
+        ctx->saved_data["splitList"] = c10::List<int64_t>(split_list);
+        return outs;
+    }
+    static torch::autograd::tensor_list backward(torch::autograd::AutogradContext* ctx, torch::autograd::tensor_list grad_outputs) {
+        auto s = ctx->get_saved_variables();
+        auto split = ctx->saved_data["splitList"].toIntVector();
+        // an output that took no part in the loss arrives undefined: its gradient is zero
+        for (int i = 0; i < 4; i++)
+            if (!grad_outputs[i].defined()) grad_outputs[i] = at::zeros({s[0].size(0), split[i]}, s[0].options());
+        return in_linear_silu_backward(s[0], s[1], s[2].defined() ? c10::optional<at::Tensor>(s[2]) : c10::nullopt, grad_outputs[0],
+                                       grad_outputs[1], grad_outputs[2], grad_outputs[3], s[3], split);
+    }
+};
+
+std::vector<at::Tensor> in_linear_silu(const at::Tensor& x, const at::Tensor& weight, const at::Tensor& bias, at::IntArrayRef split_list) {
+    return InLinearSiluFunction::apply(x, weight, bias, split_list);
+}
+
 TORCH_LIBRARY_FRAGMENT(mxrec, m) {
     m.def("hstu_jagged.equal(Tensor q, "
           "                  Tensor k, "
@@ -1157,7 +1268,14 @@ TORCH_LIBRARY_FRAGMENT(mxrec, m) {
           "                                   Tensor timestamps_weights, "
           "                                   float bucket_divisor"
           "                                   ) -> Tensor[]");
+    // schemas of in_linear_silu.cpp:202-210
     m.def("distance_in_linear_silu(Tensor x, Tensor weight, Tensor bias, int[] attr_dict) -> Tensor[]");
+    m.def("in_linear_silu(Tensor x, Tensor weight, Tensor bias, int[] attr_dict) -> Tensor[]");
+    m.def("in_linear_silu_backward("
+          "Tensor x, Tensor weight, Tensor ? bias,"
+          "Tensor user_grad, Tensor value_grad, Tensor query_grad, Tensor key_grad,"
+          "Tensor linear_output,"
+          "int[] attr_dict) -> Tensor[]");
     m.def("norm_multiply_dropout(Tensor x, Tensor u, Tensor weight, Tensor bias, float eps, float dropout_ratio) -> "
           "Tensor[]");
     // no counterpart in the reference:
@@ -1192,6 +1310,7 @@ TORCH_LIBRARY_FRAGMENT(mxrec, m) {
     m.impl("relative_attn_bias_time_with_index", TORCH_FN(relative_attn_bias_time_with_index)); \
     m.impl("norm_multiply_dropout_forward", TORCH_FN(norm_multiply_dropout_forward));           \
     m.impl("distance_in_linear_silu", TORCH_FN(distance_in_linear_silu));                       \
+    m.impl("in_linear_silu_backward", TORCH_FN(in_linear_silu_backward));                       \
     m.impl("norm_multiply_dropout_backward", TORCH_FN(norm_multiply_dropout_backward));
 
 // ROCm tensors dispatch on the CUDA key.  The CPU key runs the same host checks and then
@@ -1210,5 +1329,9 @@ TORCH_LIBRARY_IMPL(mxrec, AutogradCUDA, m) {
 TORCH_LIBRARY_IMPL(mxrec, CUDA, m) { m.impl("norm_multiply_dropout", TORCH_FN(norm_multiply_dropout)); }
 TORCH_LIBRARY_IMPL(mxrec, CPU, m) { m.impl("norm_multiply_dropout", TORCH_FN(norm_multiply_dropout)); }
 TORCH_LIBRARY_IMPL(mxrec, Autograd, m) { m.impl("norm_multiply_dropout", TORCH_FN(norm_multiply_dropout)); }
+// in_linear_silu exists only as the differentiable entry (in_linear_silu.cpp:218-227); without autograd it is the forward
+TORCH_LIBRARY_IMPL(mxrec, CUDA, m) { m.impl("in_linear_silu", TORCH_FN(distance_in_linear_silu)); }
+TORCH_LIBRARY_IMPL(mxrec, CPU, m) { m.impl("in_linear_silu", TORCH_FN(distance_in_linear_silu)); }
+TORCH_LIBRARY_IMPL(mxrec, AutogradCUDA, m) { m.impl("in_linear_silu", TORCH_FN(in_linear_silu)); }
 
 }  // namespace mxrec_hstu

@@ -94,3 +94,62 @@ def test_in_linear_silu_validation():
                        ((x, w, b, [16] * 4), "no CPU implementation")):
         with pytest.raises(RuntimeError, match=text):
             m.distance_in_linear_silu(*args)
+
+
+def test_in_linear_silu_backward_validation_and_workspace():
+    """The backward's C ABI rejects what the reference's checks reject (in_linear_silu.cpp:34-66), sizes its workspace
+    without a GPU, and the torch ops carry the reference's schemas (in_linear_silu.cpp:202-210)."""
+    L = _capi.lib()
+    def mk(**over):
+        p = _capi.HstuInLinearSiluBwdParams()
+        p.struct_size = C.sizeof(_capi.HstuInLinearSiluBwdParams)
+        p.dtype, p.grad_dtype, p.m, p.k, p.n = _capi.HSTU_BF16, _capi.HSTU_BF16, 100, 16, 64
+        for i in range(4):
+            p.split[i] = 16
+            p.grad[i] = 0x1000
+        p.x = p.weight = p.linear_output = p.x_grad = p.weight_grad = p.bias_grad = 0x1000
+        for k, v in over.items():
+            if k == "split":
+                for i, s_ in enumerate(v):
+                    p.split[i] = s_
+            else:
+                setattr(p, k, v)
+        return p
+    def call(**over):
+        p = mk(**over)
+        return L.hstu_hip_in_linear_silu_backward(C.byref(p), 0x1000, 1 << 40, None), L.hstu_hip_last_error().decode()
+    for over, text in ((dict(split=[16, 17, 15, 16]), "uvqk dim must in range[16, 8192] and multiples of 16"),
+                       (dict(split=[16, 16, 32, 32]), "weight_dim[0] must equal to sum(splitList)"), (dict(k=24), "x dim[1] must in range"),
+                       (dict(k=32), "weight dim[0] must be a multiple of 4 x dim[1]"), (dict(dtype=_capi.HSTU_F32), "dtype expect float16 or bfloat16"),
+                       (dict(grad_dtype=_capi.HSTU_F16), "grad_dtype expect float32 or the dtype of x"), (dict(m=0), "x dim[0] must in range"),
+                       (dict(x_grad=None), "must not be NULL")):
+        rc, msg = call(**over)
+        assert rc == -1 and text in msg, (over, msg)
+    rc, msg = call(bias_grad=0x1004)
+    assert rc == -2 and "16-byte aligned" in msg
+    p = mk()
+    rc = L.hstu_hip_in_linear_silu_backward(C.byref(p), 0x1000, 16, None)
+    assert rc == -3 and "workspace" in L.hstu_hip_last_error().decode()
+    need = C.c_uint64(0)
+    # m = 100 -> x^T padded to 128 columns; one range of rows per 32-row tile at most
+    assert L.hstu_hip_in_linear_silu_backward_get_workspace_size(C.byref(p), C.byref(need)) == 0
+    parts = 4
+    al = lambda v: (v + 255) // 256 * 256
+    assert need.value == al(16 * 128 * 2) + al(16 * 64 * 2) + al(parts * 64 * 16 * 4) + al(parts * 64 * 4)
+    big = mk(m=16384, k=64, n=16384, split=[4096] * 4)
+    assert L.hstu_hip_in_linear_silu_backward_get_workspace_size(C.byref(big), C.byref(need)) == 0
+    assert need.value == al(64 * 16384 * 2) * 2 + al(16 * 16384 * 64 * 4) + al(16 * 16384 * 4)
+    m = torch.ops.mxrec
+    assert str(m.in_linear_silu.default._schema) == "mxrec::in_linear_silu(Tensor x, Tensor weight, Tensor bias, int[] attr_dict) -> Tensor[]"
+    assert str(m.in_linear_silu_backward.default._schema) == ("mxrec::in_linear_silu_backward(Tensor x, Tensor weight, Tensor? bias, Tensor user_grad, "
+        "Tensor value_grad, Tensor query_grad, Tensor key_grad, Tensor linear_output, int[] attr_dict) -> Tensor[]")
+    x, w = torch.zeros(100, 16, dtype=torch.float16), torch.zeros(64, 16, dtype=torch.float16)
+    gs = [torch.zeros(100, 16, dtype=torch.float16) for _ in range(4)]
+    lin = torch.zeros(100, 64, dtype=torch.float16)
+    for args, text in (((x, w, None, *gs, lin, [16, 17, 15, 16]), "uvqk dim must in range"),
+                       ((x, w, None, gs[0][:, :8], *gs[1:], lin, [16] * 4), "must be equal to splitList"),
+                       ((x, w, None, gs[0][:50], *gs[1:], lin, [16] * 4), "dim\\[0\\] must equal to x dim\\[0\\]"),
+                       ((x, w, None, *gs, lin[:, :32], [16] * 4), "linear_output dim\\[1\\] must equal to weight dim\\[0\\]"),
+                       ((x, w, None, *gs, lin, [16] * 4), "no CPU implementation")):
+        with pytest.raises(RuntimeError, match=text):
+            m.in_linear_silu_backward(*args)

@@ -145,3 +145,105 @@ def test_in_linear_silu_forward(m, n, k, split, dtype):
     got0 = torch.ops.mxrec.distance_in_linear_silu(x.cuda(), w.cuda(), torch.zeros(n).cuda(), sp)
     want0 = LO.in_linear_silu(x, w, None, sp)
     within_one_ulp(got0[4], want0[4], "linear_output without bias", acc_err)
+
+
+def _ilb_inputs(m, k, n, dtype, diff):
+    """The reference's generators (test_in_linear_silu_backward.py:100-125): gradients uniform [0, 1), x, W and
+    linear_output uniform [-1, 1); equal widths or (h - 32, h - 16, h + 16, h + 32)."""
+    g = torch.Generator().manual_seed(0)
+    h = n // 4
+    sp = [h - 32, h - 16, h + 16, h + 32] if diff else [h] * 4
+    grads = [torch.rand(m, s_, generator=g).to(dtype) for s_ in sp]
+    u = lambda *s: (torch.rand(*s, generator=g) * 2 - 1).to(dtype)
+    return grads, u(m, k), u(n, k), u(m, n), (torch.rand(n, generator=g) * 2 - 1), sp
+
+
+def _ilb_close(got, want, dtype, what, f32=False):
+    """fp32 sums of up to 32768 rounded products against the fp64 oracle, then (for the dtype outputs) one rounding to
+    the I/O dtype: half a unit in the last place of the value plus the accumulation error relative to the tensor's scale."""
+    got, want = got.double().cpu(), want.double()
+    scale = float(want.abs().max()) or 1.0
+    ulp = 0.0 if f32 else (2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11)
+    lim = ulp * want.abs() * 1.001 + 1e-4 * scale
+    d = (got - want).abs()
+    assert bool((d <= lim).all()), f"{what}: worst {float((d / lim).max()):.2f} x the limit, scale {scale:.3e}"
+
+
+@pytest.mark.parametrize("m", [1, 1123, 2048, 7687])
+@pytest.mark.parametrize("kn", [(16, 128), (64, 512), (240, 960), (128, 2048), (768, 3072)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_in_linear_silu_backward(m, kn, dtype):
+    """Shapes of the reference's test (test_in_linear_silu_backward.py:158-166), with and without bias, equal and unequal
+    widths, against the oracle (dlin rounded to the I/O dtype before the products, as the reference's kernel does)."""
+    k, n = kn
+    for diff, with_bias in ((False, True), (True, False)):
+        if diff and k <= 32:
+            continue
+        say("in_linear_silu_backward", m, k, n, dtype, "unequal" if diff else "equal", "bias" if with_bias else "no bias")
+        grads, x, w, lin, bias, sp = _ilb_inputs(m, k, n, dtype, diff)
+        want = LO.in_linear_silu_backward(grads, x, w, lin, with_bias=with_bias)
+        got = torch.ops.mxrec.in_linear_silu_backward(x.cuda(), w.cuda(), bias.cuda() if with_bias else None, *[t.cuda() for t in grads], lin.cuda(), sp)
+        assert len(got) == 4 and got[0].dtype == dtype and got[1].dtype == dtype and got[0].shape == x.shape and got[1].shape == w.shape
+        _ilb_close(got[0], want[0], dtype, "x_grad")
+        _ilb_close(got[1], want[1], dtype, "weight_grad")
+        if with_bias:
+            assert got[2].dtype == torch.float32
+            _ilb_close(got[2], want[2], dtype, "bias_grad", f32=True)
+        else:
+            assert got[2] is None or got[2].numel() == 0
+
+
+def test_in_linear_silu_backward_fp32_outputs_reproducible_and_large():
+    """The C ABI's fp32 outputs (what the reference's kernel writes before its wrapper casts) on a shape whose k needs
+    several column chunks (k = 512, n = 6144: test_in_linear_silu_backward.py:169-176); two runs give the same bits."""
+    import ctypes as C
+    from recsdk_amd import _capi
+    m, k, n, dtype = 511, 512, 6144, torch.bfloat16
+    say("in_linear_silu_backward C ABI fp32", m, k, n)
+    grads, x, w, lin, bias, sp = _ilb_inputs(m, k, n, dtype, False)
+    dev = [t.cuda() for t in grads]
+    xd, wd, ld = x.cuda(), w.cuda(), lin.cuda()
+    L = _capi.lib()
+    outs = []
+    for _ in range(2):
+        xg = torch.full((m, k), float("nan"), device="cuda")
+        wg = torch.full((n, k), float("nan"), device="cuda")
+        bg = torch.full((n,), float("nan"), device="cuda")
+        p = _capi.HstuInLinearSiluBwdParams()
+        p.struct_size = C.sizeof(p)
+        p.dtype, p.grad_dtype, p.m, p.k, p.n = _capi.HSTU_BF16, _capi.HSTU_F32, m, k, n
+        for i in range(4):
+            p.split[i] = sp[i]
+            p.grad[i] = dev[i].data_ptr()
+        p.x, p.weight, p.linear_output = xd.data_ptr(), wd.data_ptr(), ld.data_ptr()
+        p.x_grad, p.weight_grad, p.bias_grad = xg.data_ptr(), wg.data_ptr(), bg.data_ptr()
+        need = C.c_uint64(0)
+        assert L.hstu_hip_in_linear_silu_backward_get_workspace_size(C.byref(p), C.byref(need)) == 0
+        ws = torch.empty(need.value, dtype=torch.uint8, device="cuda")
+        rc = L.hstu_hip_in_linear_silu_backward(C.byref(p), ws.data_ptr(), need.value, torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, L.hstu_hip_last_error().decode()
+        torch.cuda.synchronize()
+        outs.append((xg.cpu(), wg.cpu(), bg.cpu()))
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+    want = LO.in_linear_silu_backward(grads, x, w, lin)
+    for name, a, wnt in zip(("x_grad", "weight_grad", "bias_grad"), outs[0], want):
+        _ilb_close(a, wnt, dtype, name, f32=True)
+
+
+def test_in_linear_silu_autograd():
+    """mxrec::in_linear_silu differentiates like the reference's (test_in_linear_silu_autograd.py): the gradients that
+    reach x, W and the bias equal the backward op applied to the forward's own linear_output."""
+    m, k, n, dtype = 777, 64, 512, torch.bfloat16
+    say("in_linear_silu autograd", m, k, n)
+    grads, x, w, _, bias, sp = _ilb_inputs(m, k, n, dtype, True)
+    leaves = [t.cuda().requires_grad_(True) for t in (x, w, bias)]
+    outs = torch.ops.mxrec.in_linear_silu(*leaves, sp)
+    assert len(outs) == 5
+    sum((o * g_.cuda()).sum() for o, g_ in zip(outs[:4], grads)).backward()
+    direct = torch.ops.mxrec.in_linear_silu_backward(x.cuda(), w.cuda(), bias.cuda(), *[t.cuda() for t in grads], outs[4].detach(), sp)
+    for leaf, d in zip(leaves, direct[:3]):
+        assert leaf.grad is not None and leaf.grad.dtype == leaf.dtype and torch.equal(leaf.grad, d.to(leaf.dtype))
+    want = LO.in_linear_silu_backward(grads, x, w, outs[4].detach().cpu())
+    _ilb_close(leaves[0].grad, want[0], dtype, "x.grad")
+    _ilb_close(leaves[1].grad, want[1], dtype, "weight.grad")

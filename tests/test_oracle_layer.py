@@ -65,3 +65,44 @@ def test_in_linear_silu_is_addmm_silu_split():
         assert a.dtype == torch.bfloat16 and torch.equal(a, wnt)
     assert [t.shape[1] for t in got] == split + [128]
     assert torch.equal(LO.in_linear_silu(x, w, None, split)[4], (x.float() @ w.float().t()).to(torch.bfloat16))
+
+
+def test_in_linear_silu_backward_is_autograd_of_linear_silu():
+    """fp64 autograd through F.linear and F.silu: an independent derivation of all three gradients (no closed-form
+    silu' anywhere in it), unequal splits; and central differences of the loss for a few coordinates."""
+    g = torch.Generator().manual_seed(8)
+    m, k, split = 23, 16, [16, 32, 48, 32]
+    n = sum(split)
+    x = torch.randn(m, k, generator=g, dtype=torch.float64)
+    w = torch.randn(n, k, generator=g, dtype=torch.float64) * 0.3
+    b = torch.randn(n, generator=g, dtype=torch.float64)
+    grads = [torch.randn(m, s_, generator=g, dtype=torch.float64) for s_ in split]
+    xa, wa, ba = (t.clone().requires_grad_() for t in (x, w, b))
+    lin = F.linear(xa, wa, ba)
+    outs = torch.split(F.silu(lin), split, dim=-1)
+    loss = sum((o * g_).sum() for o, g_ in zip(outs, grads))
+    loss.backward()
+    gx, gw, gb = LO.in_linear_silu_backward(grads, x, w, lin.detach(), with_bias=True, round_dlin=False)
+    for a, wnt in ((gx, xa.grad), (gw, wa.grad), (gb, ba.grad)):
+        assert torch.allclose(a, wnt, rtol=1e-11, atol=1e-12)
+    assert LO.in_linear_silu_backward(grads, x, w, lin.detach(), with_bias=False)[2] is None
+
+    def f(x_, w_, b_):
+        o = F.silu(F.linear(x_, w_, b_))
+        return float((o * torch.cat(grads, dim=-1)).sum())
+    h = 1e-6
+    for (i, j) in ((0, 0), (5, 7), (22, 15)):
+        d = torch.zeros_like(x); d[i, j] = h
+        assert abs((f(x + d, w, b) - f(x - d, w, b)) / (2 * h) - float(gx[i, j])) < 1e-6
+    for (i, j) in ((0, 0), (100, 3), (127, 15)):
+        d = torch.zeros_like(w); d[i, j] = h
+        assert abs((f(x, w + d, b) - f(x, w - d, b)) / (2 * h) - float(gw[i, j])) < 1e-6
+    # rounding dlin to the I/O dtype only moves the products by that rounding
+    xb, wb = x.to(torch.bfloat16), w.to(torch.bfloat16)
+    lb = lin.detach().to(torch.bfloat16)
+    gb16 = [t.to(torch.bfloat16) for t in grads]
+    r0 = LO.in_linear_silu_backward(gb16, xb, wb, lb, round_dlin=False)
+    r1 = LO.in_linear_silu_backward(gb16, xb, wb, lb, round_dlin=True)
+    assert torch.equal(r0[2], r1[2])
+    for a, c in zip(r0[:2], r1[:2]):
+        assert 0 < float((a - c).abs().max()) < 2.0 ** -7 * float(a.abs().max())
