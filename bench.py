@@ -58,7 +58,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=1000)
-    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "config2_bwd", "kv_append", "rab_time", "rab_time_bwd", "rab_pos", "nmd_fwd", "nmd_bwd", "in_linear_silu", "copy"],
+    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "config2_bwd", "kv_append", "rab_time", "rab_time_bwd", "rab_pos", "nmd_fwd", "nmd_bwd", "in_linear_silu", "in_linear_silu_bwd", "copy"],
                     help="'copy' runs a plain 256 MiB device copy: the known-size kernel the FETCH_SIZE/WRITE_SIZE counters are scaled by")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
@@ -82,6 +82,8 @@ def main():
         return nmd_bench(args, torch)
     if args.workload == "in_linear_silu":
         return in_linear_silu_bench(args, torch)
+    if args.workload == "in_linear_silu_bwd":
+        return in_linear_silu_bwd_bench(args, torch)
     cfg, op, flops, alg_bytes, desc = build_workload(args.workload, torch, W)
     dev = W.to_device(cfg)
     q, k, v = dev["q"], dev["k"], dev["v"]
@@ -464,6 +466,76 @@ def in_linear_silu_bench(args, torch):
         rows = 4096
         t0 = time.perf_counter()
         LO.in_linear_silu(x[:rows], w, bias, sp)
+        dt = time.perf_counter() - t0
+        out["cpu_baseline"] = {"value": round(alg * rows / m_ / dt / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"the first {rows} rows once (oracle in torch, fp64), {dt:.2f} s"}
+    print(json.dumps(out), flush=True)
+
+
+def in_linear_silu_bwd_bench(args, torch):
+    """Backward of the input projection at the forward workload's shape: m = n = 16384, k = 64, bf16, equal widths, with
+    bias.  Through the C ABI with the workspace allocated once.  Algorithmic bytes: the four gradients and linear_output
+    read once (2 m n esize), x and W read, x_grad, weight_grad and bias_grad written."""
+    import ctypes as C
+    from recsdk_amd import _capi
+    from oracle import layer_oracle as LO
+    m_, n, k = 16384, 16384, 64
+    g = torch.Generator().manual_seed(13)
+    sp = [n // 4] * 4
+    grads = [torch.rand(m_, s_, generator=g).to(torch.bfloat16) for s_ in sp]
+    u = lambda *s: (torch.rand(*s, generator=g) * 2 - 1).to(torch.bfloat16)
+    x, w, lin = u(m_, k), u(n, k), u(m_, n)
+    dev = [t.cuda() for t in grads]
+    xd, wd, ld = x.cuda(), w.cuda(), lin.cuda()
+    xg, wg = torch.empty_like(xd), torch.empty_like(wd)
+    bg = torch.empty(n, device="cuda")
+    L = _capi.lib()
+    p = _capi.HstuInLinearSiluBwdParams()
+    p.struct_size = C.sizeof(p)
+    p.dtype, p.grad_dtype, p.m, p.k, p.n = _capi.HSTU_BF16, _capi.HSTU_BF16, m_, k, n
+    for i in range(4):
+        p.split[i] = sp[i]
+        p.grad[i] = dev[i].data_ptr()
+    p.x, p.weight, p.linear_output = xd.data_ptr(), wd.data_ptr(), ld.data_ptr()
+    p.x_grad, p.weight_grad, p.bias_grad = xg.data_ptr(), wg.data_ptr(), bg.data_ptr()
+    need = C.c_uint64(0)
+    assert L.hstu_hip_in_linear_silu_backward_get_workspace_size(C.byref(p), C.byref(need)) == 0
+    ws = torch.empty(need.value, dtype=torch.uint8, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def fn():
+        rc = L.hstu_hip_in_linear_silu_backward(C.byref(p), ws.data_ptr(), need.value, stream)
+        assert rc == 0, L.hstu_hip_last_error().decode()
+    for _ in range(args.warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    kern_ms = e0.elapsed_time(e1) / args.steps
+    alg = 2 * m_ * n * 2 + 2 * (m_ * k * 2 + n * k * 2) + n * 4
+    flops = 4.0 * m_ * n * k
+    out = {
+        "metric": "in_linear_silu_bwd_gbps", "value": round(alg / (ms * 1e-3) / 1e9, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic", "us_per_call": round(ms * 1e3, 2), "tflops": round(flops / (ms * 1e-3) / 1e12, 1),
+        "config": {"workload": "in_linear_silu_bwd: x [16384, 64], W [16384, 64], gradients 4 x [16384, 4096], linear_output [16384, 16384] bf16, seed 13",
+                   "algorithmic_bytes_per_call": alg, "flops_per_call": flops, "workspace_bytes": need.value,
+                   "entry": "hstu_hip_in_linear_silu_backward (include/hstu_layer.h): two transposes, hstu_ilb_xgrad_kernel, hstu_ilb_wgrad_kernel, two reductions"},
+        "roofline": {"bound": "hbm", "kernel": "hstu_ilb_xgrad_kernel + hstu_ilb_wgrad_kernel (+ 4 small kernels; all inside the events)",
+                     "achieved": round(alg / (kern_ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS,
+                     "unit": "GB/s", "frac": round(alg / (kern_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                     "kernel_us": round(kern_ms * 1e3, 2)},
+    }
+    if not args.no_cpu_baseline:
+        rows = 2048
+        t0 = time.perf_counter()
+        LO.in_linear_silu_backward([t[:rows] for t in grads], x[:rows], w, lin[:rows])
         dt = time.perf_counter() - t0
         out["cpu_baseline"] = {"value": round(alg * rows / m_ / dt / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
                                "sample": f"the first {rows} rows once (oracle in torch, fp64), {dt:.2f} s"}

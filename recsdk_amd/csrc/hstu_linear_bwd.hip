@@ -11,14 +11,17 @@
 // op is bounded by reading grad and linear_output from HBM.  dlin is therefore never written to memory: each of the two
 // product kernels streams grad and linear_output once and rebuilds dlin in registers.
 //   * hstu_ilb_xgrad_kernel: a workgroup owns 32 rows m; its four waves take every fourth 64-column piece of n, build
-//     dlin straight in the layout of an MFMA operand (a lane = one row, 8 consecutive n) and multiply by rows of W^T;
-//     the four partial results meet in LDS.
+//     dlin in the layout the loads arrive in (eight lanes = 128 contiguous bytes of one row), park it in LDS, read it
+//     back as an MFMA operand (a lane = one row, 8 consecutive n: one 16-byte read) and multiply by rows of W^T; the
+//     four partial results meet in LDS.
 //   * hstu_ilb_wgrad_kernel: a wave owns 64 columns n and walks down m in tiles of 32 rows; dlin is built in the layout
 //     the loads arrive in (a lane = 8 consecutive n of one row), parked in LDS and read back transposed (a lane = one
 //     column n, 8 consecutive m) against rows of x^T.  m is cut into S ranges to fill the chip; the S partial results
 //     are added in a fixed order by hstu_ilb_reduce_kernel, so the result is reproducible.
-// Both products want their small operand with the summed index contiguous: W^T [k, n] and x^T [k, m] are written to the
-// workspace first (hstu_ilb_transpose_kernel; together at most half of what grad alone takes, usually a few percent).
+// Both products want their small operand with the summed index contiguous per lane: W^T and x^T are written to the
+// workspace first, already cut into MFMA operand fragments (hstu_ilb_pack_kernel: one fragment = 32 columns k x 16
+// summed indices = 1 KiB that a wave loads with one fully contiguous instruction; together at most half of what grad
+// alone takes, usually a few percent).
 #include "hstu_device.h"
 #include "../../include/hstu_layer.h"
 
@@ -45,13 +48,17 @@ constexpr int ILB_PARK = 64 * 2 + 16;   // bytes of one parked row of 64 columns
 struct IlbArgs {
     hstu_in_linear_silu_bwd_params p;
     int base[5];          // first column of user, value, query, key, and n
-    const void* xt;       // [k, mpad]  x^T, zero for m <= column < mpad
-    const void* wt;       // [k, n]     W^T
+    const void* xt;       // [mpad / 16, kbt] fragments of x^T, zero for rows >= m and columns >= k
+    const void* wt;       // [n / 16, kbt]    fragments of W^T
+    int kbt;              // ceil(k / 32)
     float* wpart;         // [S, n, k]
     float* bpart;         // [S, n]
     int64_t mpad;         // m rounded up to 32
     int64_t rows_per_part;
     int parts;            // S
+    float* xpart;         // [ranges of n, m, k], only with more than one range
+    int nparts;           // ranges of n of the x_grad kernel
+    int cols_per_part;    // a multiple of 256
 };
 
 // grad * silu'(lin), unrounded
@@ -65,24 +72,22 @@ __device__ __forceinline__ void ilb_dlin8(const typename IlbMM<T>::v8& g, const 
     }
 }
 
-// out[c][r] = in[r][c] for r < rows, c < cols; out has row stride rpad >= rows, zero for rows <= r < rpad
-__global__ __launch_bounds__(256) void hstu_ilb_transpose_kernel(const uint16_t* in, int64_t rows, int cols, uint16_t* out, int64_t rpad) {
-    __shared__ uint16_t tile[32][33];
-    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
-    const int64_t r0 = (int64_t)blockIdx.x * 32;
-    const int c0 = blockIdx.y * 32;
+// Fragments of in^T for in [rows, cols]: fragment (step, kb) holds columns 32 kb .. + 31 of the rows 16 step .. + 15 in
+// the order an MFMA operand wants them: lane (l32, g) = column 32 kb + l32, rows 16 step + 8 g .. + 7 as 16 bytes at
+// ((step * kbt + kb) * 64 + lane) * 16.  Zero outside in.  One thread per 16 bytes.
+__global__ __launch_bounds__(256) void hstu_ilb_pack_kernel(const uint16_t* in, int64_t rows, int cols, int kbt, int64_t units, uint16_t* out) {
+    typedef __attribute__((ext_vector_type(8))) uint16_t u16x8;
+    const int64_t unit = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (unit >= units) return;
+    const int lane = (int)(unit & 63);
+    const int64_t blk = unit >> 6;
+    const int kb = (int)(blk % kbt);
+    const int64_t r0 = (blk / kbt) * 16 + 8 * (lane >> 5);
+    const int c = 32 * kb + (lane & 31);
+    u16x8 v;
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const int64_t r = r0 + ty + 8 * i;
-        const int c = c0 + tx;
-        tile[ty + 8 * i][tx] = (r < rows && c < cols) ? in[r * cols + c] : (uint16_t)0;
-    }
-    __syncthreads();
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const int c = c0 + ty + 8 * i;
-        if (c < cols && r0 + tx < rpad) out[(int64_t)c * rpad + r0 + tx] = tile[tx][ty + 8 * i];
-    }
+    for (int e = 0; e < 8; e++) v[e] = (r0 + e < rows && c < cols) ? in[(r0 + e) * cols + c] : (uint16_t)0;
+    *reinterpret_cast<u16x8*>(out + unit * 8) = v;
 }
 
 // pointer to 8 consecutive gradient columns starting at column n (a multiple of 8) of row `row`
@@ -104,52 +109,91 @@ template <typename T> __device__ __forceinline__ void ilb_store(void* out, int64
     else reinterpret_cast<T*>(out)[idx] = from_float<T>(v);
 }
 
-// x_grad.  grid = (ceil(m / 32), ceil(k / KC)), 4 waves.
+// x_grad.  grid = (ceil(m / 32), ceil(k / KC), ranges of n), 4 waves.
 template <typename T, int KC>
 __global__ __launch_bounds__(ILB_NT) void hstu_ilb_xgrad_kernel(const IlbArgs a) {
     typedef typename IlbMM<T>::v8 v8;
     constexpr int KB = KC / 32;
-    __shared__ float red[3][32][KC + 1];
+    constexpr int RED_BYTES = 3 * 32 * (KC + 1) * 4, PARK_BYTES = (ILB_NT / 64) * 32 * ILB_PARK;
+    // the parked tiles of the loop and the sums of the epilogue share one buffer
+    __shared__ __attribute__((aligned(16))) char lds[RED_BYTES > PARK_BYTES ? RED_BYTES : PARK_BYTES];
+    float (*red)[32][KC + 1] = reinterpret_cast<float (*)[32][KC + 1]>(lds);
     const hstu_in_linear_silu_bwd_params& p = a.p;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int g = lane >> 5, l32 = lane & 31;
     const int N = p.n, K = p.k;
     const int64_t m0 = (int64_t)blockIdx.x * 32;
     const int k0 = blockIdx.y * KC;
-    const int64_t row = m0 + l32 < p.m ? m0 + l32 : p.m - 1;   // rows past the end repeat the last one and are not stored
-    const T* lin = reinterpret_cast<const T*>(p.linear_output) + row * N + 8 * g;
-    const T* wrow[KB];
+    // load phase: lane = 8 consecutive columns (chunk) of the rows lrow, lrow + 8, lrow + 16, lrow + 24 of the tile, so that
+    // eight lanes read 128 contiguous bytes; rows past the end repeat the last one and are not stored
+    const int chunk = lane & 7, lrow = lane >> 3;
+    int64_t rows[4];
 #pragma unroll
-    for (int kb = 0; kb < KB; kb++) wrow[kb] = reinterpret_cast<const T*>(a.wt) + (int64_t)min(k0 + 32 * kb + l32, K - 1) * N + 8 * g;
+    for (int i = 0; i < 4; i++) rows[i] = m0 + lrow + 8 * i < p.m ? m0 + lrow + 8 * i : p.m - 1;
+    const T* lin = reinterpret_cast<const T*>(p.linear_output);
+    const T* wfrag[KB];   // fragment column of this block of k (past the last one: repeats it, never stored), this lane
+#pragma unroll
+    for (int kb = 0; kb < KB; kb++) wfrag[kb] = reinterpret_cast<const T*>(a.wt) + ((int64_t)min(k0 / 32 + kb, a.kbt - 1) * 64 + lane) * 8;
+    char* park = lds + w * (32 * ILB_PARK);
     ilb_f32x16 acc[KB];
 #pragma unroll
     for (int kb = 0; kb < KB; kb++)
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[kb][r] = 0.f;
-    auto step = [&](int n0) __attribute__((always_inline)) {   // 16 columns of n, inside one of the four gradients
-        const v8 gf = *reinterpret_cast<const v8*>(ilb_grad_ptr<T>(a, n0, row) + 8 * g);
-        const v8 lf = *reinterpret_cast<const v8*>(lin + n0);
-        v8 wf[KB];
+    const int cbeg = blockIdx.z * a.cols_per_part, cend = min(cbeg + a.cols_per_part, N);
+    auto fetch = [&](int c, v8* gf, v8* lf) __attribute__((always_inline)) {
+        const int ncol = c + 8 * chunk;
+        const int ncl = ncol < N ? ncol : c;   // the last piece may be narrower than 64 columns
+        const T* gp = ilb_grad_ptr<T>(a, ncl, 0);
+        int gwidth = a.p.split[0];
 #pragma unroll
-        for (int kb = 0; kb < KB; kb++) wf[kb] = *reinterpret_cast<const v8*>(wrow[kb] + n0);
-        float d[8];
-        ilb_dlin8<T>(gf, lf, d);
-        v8 df;
+        for (int i = 1; i < 4; i++)
+            if (ncl >= a.base[i]) gwidth = a.p.split[i];
 #pragma unroll
-        for (int e = 0; e < 8; e++) df[e] = from_float<T>(d[e]);
-#pragma unroll
-        for (int kb = 0; kb < KB; kb++) acc[kb] = IlbMM<T>::mfma(wf[kb], df, acc[kb]);
-    };
-    for (int c = 64 * w; c < N; c += 256) {
-        if (c + 64 <= N) {
-            step(c);
-            step(c + 16);
-            step(c + 32);
-            step(c + 48);
-        } else {
-            for (int n0 = c; n0 < N; n0 += 16) step(n0);
+        for (int i = 0; i < 4; i++) {
+            gf[i] = *reinterpret_cast<const v8*>(gp + rows[i] * gwidth);
+            lf[i] = *reinterpret_cast<const v8*>(lin + rows[i] * N + ncl);
         }
+    };
+    v8 gf[4], lf[4];
+    int c = cbeg + 64 * w;
+    if (c < cend) fetch(c, gf, lf);
+    for (; c < cend; c += 256) {
+        // the loads of the next piece are in flight while this one is worked on (the last piece asks for itself again)
+        v8 gn[4], ln[4];
+        fetch(c + 256 < cend ? c + 256 : c, gn, ln);
+        const bool live = c + 8 * chunk < N;
+        v8 wf[4][KB];   // W^T: columns c + 16 s + 8 g .. + 7 (a step past n re-reads the last one against zeros)
+#pragma unroll
+        for (int s = 0; s < 4; s++)
+#pragma unroll
+            for (int kb = 0; kb < KB; kb++) wf[s][kb] = *reinterpret_cast<const v8*>(wfrag[kb] + (int64_t)min(c / 16 + s, N / 16 - 1) * a.kbt * 512);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            float d[8];
+            ilb_dlin8<T>(gf[i], lf[i], d);
+            v8 df;
+#pragma unroll
+            for (int e = 0; e < 8; e++) df[e] = from_float<T>(live ? d[e] : 0.f);
+            *reinterpret_cast<v8*>(park + (lrow + 8 * i) * ILB_PARK + chunk * 16) = df;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+            // row m0 + l32 of dlin, columns c + 16 s + 8 g .. + 7
+            const v8 bf = *reinterpret_cast<const v8*>(park + l32 * ILB_PARK + (16 * s + 8 * g) * 2);
+#pragma unroll
+            for (int kb = 0; kb < KB; kb++) acc[kb] = IlbMM<T>::mfma(wf[s][kb], bf, acc[kb]);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int i = 0; i < 4; i++) { gf[i] = gn[i]; lf[i] = ln[i]; }
     }
+    __syncthreads();   // every wave is done with its parked tile before the sums overwrite the buffer
     // accumulator register r of block kb: column k0 + 32 kb + 8 (r / 4) + 4 g + r % 4 of row m0 + l32.
     // Waves 1..3 park their sums, wave 0 adds them to its own in that order and parks the total in the first slot.
     if (w > 0) {
@@ -169,10 +213,12 @@ __global__ __launch_bounds__(ILB_NT) void hstu_ilb_xgrad_kernel(const IlbArgs a)
             }
     }
     __syncthreads();
-    const int as_f32 = p.grad_dtype == HSTU_F32;
+    // one range of n: the result; several: fp32 partial sums for hstu_ilb_reduce_kernel
+    const int as_f32 = a.nparts > 1 || p.grad_dtype == HSTU_F32;
+    void* dst = a.nparts > 1 ? (void*)(a.xpart + (int64_t)blockIdx.z * p.m * K) : p.x_grad;
     for (int i = threadIdx.x; i < 32 * KC; i += ILB_NT) {
-        const int r = i / KC, c = i % KC;
-        if (m0 + r < p.m && k0 + c < K) ilb_store<T>(p.x_grad, (m0 + r) * K + k0 + c, red[0][r][c], as_f32);
+        const int r = i / KC, cc = i % KC;
+        if (m0 + r < p.m && k0 + cc < K) ilb_store<T>(dst, (m0 + r) * K + k0 + cc, red[0][r][cc], as_f32);
     }
 }
 
@@ -206,9 +252,9 @@ __global__ __launch_bounds__(ILB_NT) void hstu_ilb_wgrad_kernel(const IlbArgs a)
         if (sel == i) { gbase = p.grad[i]; gfirst = a.base[i]; gwidth = p.split[i]; }
     const T* gptr = reinterpret_cast<const T*>(gbase) + (ncl - gfirst);
     const T* lptr = reinterpret_cast<const T*>(p.linear_output) + ncl;
-    const T* xrow[KB];
+    const T* xfrag[KB];
 #pragma unroll
-    for (int kb = 0; kb < KB; kb++) xrow[kb] = reinterpret_cast<const T*>(a.xt) + (int64_t)min(k0 + 32 * kb + l32, K - 1) * a.mpad + 8 * g;
+    for (int kb = 0; kb < KB; kb++) xfrag[kb] = reinterpret_cast<const T*>(a.xt) + ((int64_t)min(k0 / 32 + kb, a.kbt - 1) * 64 + lane) * 8;
     char* park = park_all + w * (32 * ILB_PARK);
     ilb_f32x16 acc[2][KB];
 #pragma unroll
@@ -220,8 +266,7 @@ __global__ __launch_bounds__(ILB_NT) void hstu_ilb_wgrad_kernel(const IlbArgs a)
     float bsum[8];
 #pragma unroll
     for (int e = 0; e < 8; e++) bsum[e] = 0.f;
-    for (int64_t m0 = mbeg; m0 < mend; m0 += 32) {
-        v8 gf[4], lf[4];
+    auto fetch = [&](int64_t m0, v8* gf, v8* lf) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const int64_t r = m0 + lrow + 8 * i;
@@ -229,11 +274,18 @@ __global__ __launch_bounds__(ILB_NT) void hstu_ilb_wgrad_kernel(const IlbArgs a)
             gf[i] = *reinterpret_cast<const v8*>(gptr + rc * gwidth);
             lf[i] = *reinterpret_cast<const v8*>(lptr + rc * N);
         }
-        v8 xf[2][KB];   // rows of x^T: columns m0 + 16 ks + 8 g .. + 7 (zero past m)
+    };
+    v8 gf[4], lf[4];
+    fetch(mbeg, gf, lf);
+    for (int64_t m0 = mbeg; m0 < mend; m0 += 32) {
+        // the loads of the next tile are in flight while this one is worked on (the last tile asks for itself again)
+        v8 gn[4], ln[4];
+        fetch(m0 + 32 < mend ? m0 + 32 : m0, gn, ln);
+        v8 xf[2][KB];   // x^T: columns m0 + 16 ks + 8 g .. + 7 (zero past m)
 #pragma unroll
         for (int ks = 0; ks < 2; ks++)
 #pragma unroll
-            for (int kb = 0; kb < KB; kb++) xf[ks][kb] = *reinterpret_cast<const v8*>(xrow[kb] + m0 + 16 * ks);
+            for (int kb = 0; kb < KB; kb++) xf[ks][kb] = *reinterpret_cast<const v8*>(xfrag[kb] + (m0 / 16 + ks) * a.kbt * 512);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             float d[8];
@@ -265,6 +317,8 @@ __global__ __launch_bounds__(ILB_NT) void hstu_ilb_wgrad_kernel(const IlbArgs a)
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int i = 0; i < 4; i++) { gf[i] = gn[i]; lf[i] = ln[i]; }
     }
     // accumulator register r of block (nb, kb): row nw + 32 nb + 8 (r / 4) + 4 g + r % 4, column k0 + 32 kb + l32
     float* wp = a.wpart + (int64_t)blockIdx.z * N * K;
@@ -315,8 +369,9 @@ __global__ __launch_bounds__(256) void hstu_ilb_reduce_kernel(const float* part,
 struct IlbPlan {
     int kc;               // k columns per workgroup: 64 or 128
     int parts;
+    int kbt, nparts, cols_per_part;
     int64_t rows_per_part, mpad;
-    uint64_t off_xt, off_wt, off_wpart, off_bpart, total;
+    uint64_t off_xt, off_wt, off_wpart, off_bpart, off_xpart, total;
 };
 
 static uint64_t ilb_align(uint64_t v) { return (v + 255) & ~(uint64_t)255; }
@@ -332,15 +387,26 @@ static IlbPlan ilb_plan(const hstu_in_linear_silu_bwd_params* p) {
     pl.rows_per_part = ((tiles + parts - 1) / parts) * 32;
     pl.parts = (int)((p->m + pl.rows_per_part - 1) / pl.rows_per_part);
     pl.mpad = tiles * 32;
+    pl.kbt = (p->k + 31) / 32;
     uint64_t o = 0;
     pl.off_xt = o;
-    o = ilb_align(o + (uint64_t)p->k * pl.mpad * 2);
+    o = ilb_align(o + (uint64_t)(pl.mpad / 16) * pl.kbt * 1024);
     pl.off_wt = o;
-    o = ilb_align(o + (uint64_t)p->k * p->n * 2);
+    o = ilb_align(o + (uint64_t)(p->n / 16) * pl.kbt * 1024);
     pl.off_wpart = o;
     o = ilb_align(o + (uint64_t)pl.parts * p->n * p->k * 4);
     pl.off_bpart = o;
     o = ilb_align(o + (uint64_t)pl.parts * p->n * 4);
+    // x_grad: ranges of n (whole 256-column rounds of a workgroup) until about 1024 workgroups are there
+    const int64_t xwgs = tiles * ((p->k + pl.kc - 1) / pl.kc);
+    int64_t nparts = (1024 + xwgs / 2) / xwgs;
+    const int64_t rounds = (p->n + 255) / 256;
+    if (nparts > rounds / 4) nparts = rounds / 4;
+    if (nparts < 1) nparts = 1;
+    pl.cols_per_part = (int)((rounds + nparts - 1) / nparts) * 256;
+    pl.nparts = (p->n + pl.cols_per_part - 1) / pl.cols_per_part;
+    pl.off_xpart = o;
+    if (pl.nparts > 1) o = ilb_align(o + (uint64_t)pl.nparts * p->m * p->k * 4);
     pl.total = o;
     return pl;
 }
@@ -381,19 +447,24 @@ extern "C" int hstu_hip_in_linear_silu_backward_get_workspace_size(const hstu_in
 template <typename T>
 static void ilb_launch(const IlbArgs& a, const IlbPlan& pl, hipStream_t st) {
     const hstu_in_linear_silu_bwd_params& p = a.p;
-    // W [n, k] -> W^T [k, n];  x [m, k] -> x^T [k, mpad]
-    hipLaunchKernelGGL(hstu_ilb_transpose_kernel, dim3((unsigned)((p.n + 31) / 32), (unsigned)((p.k + 31) / 32)), dim3(256), 0, st,
-                       reinterpret_cast<const uint16_t*>(p.weight), (int64_t)p.n, p.k, reinterpret_cast<uint16_t*>(const_cast<void*>(a.wt)), (int64_t)p.n);
-    hipLaunchKernelGGL(hstu_ilb_transpose_kernel, dim3((unsigned)(pl.mpad / 32), (unsigned)((p.k + 31) / 32)), dim3(256), 0, st,
-                       reinterpret_cast<const uint16_t*>(p.x), p.m, p.k, reinterpret_cast<uint16_t*>(const_cast<void*>(a.xt)), pl.mpad);
+    const int64_t wunits = (int64_t)(p.n / 16) * pl.kbt * 64, xunits = (pl.mpad / 16) * pl.kbt * 64;
+    hipLaunchKernelGGL(hstu_ilb_pack_kernel, dim3((unsigned)((wunits + 255) / 256)), dim3(256), 0, st, reinterpret_cast<const uint16_t*>(p.weight),
+                       (int64_t)p.n, p.k, pl.kbt, wunits, reinterpret_cast<uint16_t*>(const_cast<void*>(a.wt)));
+    hipLaunchKernelGGL(hstu_ilb_pack_kernel, dim3((unsigned)((xunits + 255) / 256)), dim3(256), 0, st, reinterpret_cast<const uint16_t*>(p.x), p.m,
+                       p.k, pl.kbt, xunits, reinterpret_cast<uint16_t*>(const_cast<void*>(a.xt)));
     const unsigned kchunks = (unsigned)((p.k + pl.kc - 1) / pl.kc);
-    const dim3 gx((unsigned)(pl.mpad / 32), kchunks), gw((unsigned)((p.n + 255) / 256), kchunks, (unsigned)pl.parts);
+    const dim3 gx((unsigned)(pl.mpad / 32), kchunks, (unsigned)pl.nparts), gw((unsigned)((p.n + 255) / 256), kchunks, (unsigned)pl.parts);
     if (pl.kc == 64) {
         hipLaunchKernelGGL((hstu_ilb_xgrad_kernel<T, 64>), gx, dim3(ILB_NT), 0, st, a);
         hipLaunchKernelGGL((hstu_ilb_wgrad_kernel<T, 64>), gw, dim3(ILB_NT), 0, st, a);
     } else {
         hipLaunchKernelGGL((hstu_ilb_xgrad_kernel<T, 128>), gx, dim3(ILB_NT), 0, st, a);
         hipLaunchKernelGGL((hstu_ilb_wgrad_kernel<T, 128>), gw, dim3(ILB_NT), 0, st, a);
+    }
+    if (pl.nparts > 1) {
+        const int64_t cx = p.m * p.k;
+        hipLaunchKernelGGL(hstu_ilb_reduce_kernel<T>, dim3((unsigned)((cx / 4 + 255) / 256)), dim3(256), 0, st, a.xpart, pl.nparts, cx, p.x_grad,
+                           (int)(p.grad_dtype == HSTU_F32));
     }
     const int64_t cw = (int64_t)p.n * p.k;
     hipLaunchKernelGGL(hstu_ilb_reduce_kernel<T>, dim3((unsigned)((cw / 4 + 255) / 256)), dim3(256), 0, st, a.wpart, pl.parts, cw, p.weight_grad,
@@ -429,6 +500,10 @@ extern "C" int hstu_hip_in_linear_silu_backward(const hstu_in_linear_silu_bwd_pa
     a.wpart = reinterpret_cast<float*>(ws + pl.off_wpart);
     a.bpart = reinterpret_cast<float*>(ws + pl.off_bpart);
     a.mpad = pl.mpad;
+    a.kbt = pl.kbt;
+    a.xpart = reinterpret_cast<float*>(ws + pl.off_xpart);
+    a.nparts = pl.nparts;
+    a.cols_per_part = pl.cols_per_part;
     a.rows_per_part = pl.rows_per_part;
     a.parts = pl.parts;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);

@@ -131,14 +131,16 @@ def test_in_linear_silu_backward_validation_and_workspace():
     rc = L.hstu_hip_in_linear_silu_backward(C.byref(p), 0x1000, 16, None)
     assert rc == -3 and "workspace" in L.hstu_hip_last_error().decode()
     need = C.c_uint64(0)
-    # m = 100 -> x^T padded to 128 columns; one range of rows per 32-row tile at most
+    # m = 100 -> x^T padded to 128 rows; operand fragments of 1 KiB (32 columns k x 16 rows, k padded to 32); one range
+    # of rows per 32-row tile at most
     assert L.hstu_hip_in_linear_silu_backward_get_workspace_size(C.byref(p), C.byref(need)) == 0
     parts = 4
     al = lambda v: (v + 255) // 256 * 256
-    assert need.value == al(16 * 128 * 2) + al(16 * 64 * 2) + al(parts * 64 * 16 * 4) + al(parts * 64 * 4)
+    assert need.value == al(128 // 16 * 1024) + al(64 // 16 * 1024) + al(parts * 64 * 16 * 4) + al(parts * 64 * 4)
     big = mk(m=16384, k=64, n=16384, split=[4096] * 4)
     assert L.hstu_hip_in_linear_silu_backward_get_workspace_size(C.byref(big), C.byref(need)) == 0
-    assert need.value == al(64 * 16384 * 2) * 2 + al(16 * 16384 * 64 * 4) + al(16 * 16384 * 4)
+    # 16 ranges of m for weight_grad, 2 ranges of n for x_grad
+    assert need.value == al(64 * 16384 * 2) * 2 + al(16 * 16384 * 64 * 4) + al(16 * 16384 * 4) + al(2 * 16384 * 64 * 4)
     m = torch.ops.mxrec
     assert str(m.in_linear_silu.default._schema) == "mxrec::in_linear_silu(Tensor x, Tensor weight, Tensor bias, int[] attr_dict) -> Tensor[]"
     assert str(m.in_linear_silu_backward.default._schema) == ("mxrec::in_linear_silu_backward(Tensor x, Tensor weight, Tensor? bias, Tensor user_grad, "
