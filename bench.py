@@ -23,7 +23,7 @@ PEAK_HBM_GBS = 8000.0
 # HBM-side bytes per launch from rocprofv3 FETCH_SIZE/WRITE_SIZE, each scaled by what the same counter reads for the
 # plain 256 MiB copy of `--workload copy` (factors 2.000 and 1.000); see profiles/*.md
 MEASURED_TRAFFIC_BYTES = {"config2": 184.3e6, "kv_append": 351.9e6, "rab_time": 1479.8e6, "rab_time_bwd": 2242.4e6, "rab_pos": 305.2e6,
-                          "nmd_fwd": 827.4e6, "nmd_bwd": 1382.0e6, "in_linear_silu": 1092.9e6}
+                          "nmd_fwd": 827.4e6, "nmd_bwd": 1382.0e6, "in_linear_silu": 1092.9e6, "in_linear_silu_bwd": 2363.7e6}
 
 
 def build_workload(name, torch, W):
@@ -526,7 +526,7 @@ def in_linear_silu_bwd_bench(args, torch):
         "dtype": "bf16", "data": "synthetic", "us_per_call": round(ms * 1e3, 2), "tflops": round(flops / (ms * 1e-3) / 1e12, 1),
         "config": {"workload": "in_linear_silu_bwd: x [16384, 64], W [16384, 64], gradients 4 x [16384, 4096], linear_output [16384, 16384] bf16, seed 13",
                    "algorithmic_bytes_per_call": alg, "flops_per_call": flops, "workspace_bytes": need.value,
-                   "entry": "hstu_hip_in_linear_silu_backward (include/hstu_layer.h): two transposes, hstu_ilb_xgrad_kernel, hstu_ilb_wgrad_kernel, two reductions"},
+                   "entry": "hstu_hip_in_linear_silu_backward (include/hstu_layer.h): two operand packs, hstu_ilb_xgrad_kernel, hstu_ilb_wgrad_kernel, three reductions"},
         "roofline": {"bound": "hbm", "kernel": "hstu_ilb_xgrad_kernel + hstu_ilb_wgrad_kernel (+ 4 small kernels; all inside the events)",
                      "achieved": round(alg / (kern_ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS,
                      "unit": "GB/s", "frac": round(alg / (kern_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
