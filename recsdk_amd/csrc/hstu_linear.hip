@@ -3,11 +3,13 @@
 // (thousands), so at 2 * k FLOPs per output element against 4 bytes written the op is bounded by the HBM writes of
 // its two [m, n] results, not by the matrix cores: the kernel is an MFMA GEMM without any pipelining of the k loop,
 // built around its stores.
-//   workgroup = 128 rows m x 128 columns n; wave w = rows 32 w .. 32 w + 31, all 128 columns (four 32 x 32 blocks)
+//   workgroup = 128 rows m x 64 columns n; wave w = rows 32 w .. 32 w + 31, all 64 columns (two 32 x 32 blocks: at 73
+//   registers and 4.5 KiB of LDS per wave six waves share a SIMD, which is what keeps the stores flowing; four blocks
+//   per wave measured 9 % slower, one block 23 % slower)
 //   out^T block = W x^T: v_mfma_f32_32x32x16 with A = W fragment, B = x fragment, both straight from global memory
 //   (each lane reads 16 contiguous bytes of a row: x and W are k-contiguous, which is what both operands want)
 //   epilogue: + bias, round -> linear_output; silu of the rounded value, round -> the four outputs; both leave through
-//   a per-wave LDS tile so that a lane stores 16 bytes of one output row and a wave instruction covers four 256-byte runs
+//   a per-wave LDS tile so that a lane stores 16 bytes of one output row and a wave instruction covers eight 128-byte runs
 // Definition: cust_op/test/in_linear_silu_test/test_in_linear_silu.py:31-45.
 #include "hstu_device.h"
 #include "../../include/hstu_layer.h"
@@ -35,7 +37,9 @@ template <> struct IlsMM<_Float16> {
     static __device__ __forceinline__ unsigned pack2(_Float16 x, _Float16 y) { ils_f16x2 r; r[0] = x; r[1] = y; return __builtin_bit_cast(unsigned, r); }
 };
 
-constexpr int ILS_BM = 128, ILS_BN = 128, ILS_NT = 256;
+constexpr int ILS_NB = 2;                                   // 32 x 32 blocks side by side per wave
+constexpr int ILS_BM = 128, ILS_BN = 32 * ILS_NB, ILS_NT = 256;
+constexpr int ILS_LPR = ILS_BN / 8, ILS_RPI = 64 / ILS_LPR;   // store phase: lanes per row, rows per instruction
 constexpr int ILS_ROW = ILS_BN * 2 + 16;   // bytes of one parked row: + 16 keeps the 8-byte column writes of 32 rows off one bank
 
 struct IlsArgs {
@@ -52,7 +56,7 @@ __global__ __launch_bounds__(ILS_NT) void hstu_in_linear_silu_kernel(const IlsAr
     const int g = lane >> 5, l32 = lane & 31;
     const int K = p.k, N = p.n;
     // Workgroup i of the 1-D grid runs on XCD i % 8 (each with its own L2).  Tiles are numbered so that one XCD sweeps
-    // a contiguous eighth of the n range for a block of rows: what its L2 writes back to HBM is then runs of 16 tiles
+    // a contiguous eighth of the n range for a block of rows: what its L2 writes back to HBM is then runs of 32 tiles
     // (4 KiB) per row instead of 256-byte pieces interleaved with the other XCDs' at other times.
     const unsigned nt = (unsigned)(N + ILS_BN - 1) / ILS_BN;
     unsigned tn, tm;
@@ -71,21 +75,21 @@ __global__ __launch_bounds__(ILS_NT) void hstu_in_linear_silu_kernel(const IlsAr
     const T* wt = reinterpret_cast<const T*>(p.weight);
     // operand rows of this lane, clamped into the tensors (what is read for rows past the end is never stored)
     const T* xrow = x + (m0 + l32 < p.m ? m0 + l32 : p.m - 1) * K + 8 * g;
-    const T* wrow[4];
+    const T* wrow[ILS_NB];
 #pragma unroll
-    for (int nb = 0; nb < 4; nb++) wrow[nb] = wt + (int64_t)min(n0 + 32 * nb + l32, N - 1) * K + 8 * g;
-    ils_f32x16 acc[4];
+    for (int nb = 0; nb < ILS_NB; nb++) wrow[nb] = wt + (int64_t)min(n0 + 32 * nb + l32, N - 1) * K + 8 * g;
+    ils_f32x16 acc[ILS_NB];
 #pragma unroll
-    for (int nb = 0; nb < 4; nb++)
+    for (int nb = 0; nb < ILS_NB; nb++)
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[nb][r] = 0.f;
     auto step = [&](int k0) __attribute__((always_inline)) {
         const v8 xf = *reinterpret_cast<const v8*>(xrow + k0);
-        v8 wf[4];
+        v8 wf[ILS_NB];
 #pragma unroll
-        for (int nb = 0; nb < 4; nb++) wf[nb] = *reinterpret_cast<const v8*>(wrow[nb] + k0);
+        for (int nb = 0; nb < ILS_NB; nb++) wf[nb] = *reinterpret_cast<const v8*>(wrow[nb] + k0);
 #pragma unroll
-        for (int nb = 0; nb < 4; nb++) acc[nb] = IlsMM<T>::mfma(wf[nb], xf, acc[nb]);
+        for (int nb = 0; nb < ILS_NB; nb++) acc[nb] = IlsMM<T>::mfma(wf[nb], xf, acc[nb]);
     };
     int k0 = 0;
     for (; k0 + 64 <= K; k0 += 64) {   // four steps' loads in flight together
@@ -97,9 +101,9 @@ __global__ __launch_bounds__(ILS_NT) void hstu_in_linear_silu_kernel(const IlsAr
     for (; k0 < K; k0 += 16) step(k0);
     // accumulator register r of block nb holds column n0 + 32 nb + 8 (r / 4) + 4 g + r % 4 of row m0 + l32
     char* park = park_all + w * (32 * ILS_ROW);
-    T lin[4][16];
+    T lin[ILS_NB][16];
 #pragma unroll
-    for (int nb = 0; nb < 4; nb++) {
+    for (int nb = 0; nb < ILS_NB; nb++) {
 #pragma unroll
         for (int rr = 0; rr < 4; rr++) {
             ils_f32x4 b = {0.f, 0.f, 0.f, 0.f};
@@ -109,7 +113,7 @@ __global__ __launch_bounds__(ILS_NT) void hstu_in_linear_silu_kernel(const IlsAr
             for (int e = 0; e < 4; e++) lin[nb][4 * rr + e] = from_float<T>(acc[nb][4 * rr + e] + b[e]);
         }
     }
-    const int orow = lane >> 4, ochunk = lane & 15;   // store phase: 16 lanes per row, 8 columns each
+    const int orow = lane / ILS_LPR, ochunk = lane % ILS_LPR;   // store phase: a lane = 8 columns of a row
     const int col = n0 + 8 * ochunk;
     int which = 0;
 #pragma unroll
@@ -117,7 +121,7 @@ __global__ __launch_bounds__(ILS_NT) void hstu_in_linear_silu_kernel(const IlsAr
 #pragma unroll
     for (int phase = 0; phase < 2; phase++) {
 #pragma unroll
-        for (int nb = 0; nb < 4; nb++) {
+        for (int nb = 0; nb < ILS_NB; nb++) {
 #pragma unroll
             for (int rr = 0; rr < 4; rr++) {
                 T v[4];
@@ -149,8 +153,8 @@ __global__ __launch_bounds__(ILS_NT) void hstu_in_linear_silu_kernel(const IlsAr
                 stride = width;
             }
 #pragma unroll
-            for (int i = 0; i < 8; i++) {
-                const int row = 4 * i + orow;
+            for (int i = 0; i < 32 / ILS_RPI; i++) {
+                const int row = ILS_RPI * i + orow;
                 const ils_u4 v = *reinterpret_cast<const ils_u4*>(park + row * ILS_ROW + ochunk * 16);
                 if (m0 + row < p.m) __builtin_nontemporal_store(v, reinterpret_cast<ils_u4*>(dst + (m0 + row) * stride));
             }
