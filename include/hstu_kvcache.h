@@ -60,6 +60,42 @@ int hstu_hip_kv_append(const hstu_kv_append_params* p, void* stream);
 int hstu_hip_kv_token_positions(int32_t batch, const int32_t* append_indptr, const int32_t* seq_lens,
                                 int32_t* batch_indices, int32_t* positions, int32_t nnz_max, void* stream);
 
+/* Append to an fp8-e4m3 table with one fp32 scale per (page, K|V, head): the write side of what
+ * hstu_hip_paged_forward reads with cache_dtype = HSTU_FP8_E4M3 and kv_scales.  No counterpart in the reference (its
+ * cache manager stores 2-byte rows unscaled); for the callers that keep the history in fp8.  Tokens are routed like
+ * hstu_hip_kv_append.  After the call a touched (page, K|V, head) holds q = rne_e4m3(clamp(x / s, -448, 448)) with
+ *   s = max(s before, absmax(new rows) / 448)   if the page already held rows below its first new slot,
+ *   s = absmax(new rows) / 448 (1 if that is 0)  otherwise;
+ * rows already there are requantised from q * (s before) when s grew, and untouched when it did not.  Pages fill from
+ * slot 0 upwards (what the reference's manager does).  The workspace needs no initialisation. */
+typedef struct hstu_kv_append_fp8_params {
+    uint32_t struct_size;
+    int32_t src_dtype;        /* HSTU_F16 / HSTU_BF16: append_key, append_value */
+    uint8_t* kv_cache;        /* [num_pages, 2, page_size, num_heads, head_dim] e4m3 bytes, contiguous */
+    float* kv_scales;         /* [num_pages, 2, num_heads] */
+    int32_t num_pages;
+    int32_t page_size;
+    int32_t num_heads;
+    int32_t head_dim;         /* a power of two in [8, 512] */
+    const int32_t* kv_indices;
+    const int32_t* kv_indptr;
+    int32_t num_indices;
+    int32_t batch;
+    const void* append_key;   /* [append_rows, heads, dim] with the strides below (elements) */
+    const void* append_value;
+    int64_t append_k_stride_n, append_k_stride_h;
+    int64_t append_v_stride_n, append_v_stride_h;
+    int64_t append_rows;
+    const int32_t* batch_indices;
+    const int32_t* positions;
+    const int32_t* offsets;
+    const int32_t* nnz_dev;
+    int32_t nnz_max;
+    int32_t reserved;
+} hstu_kv_append_fp8_params;
+int hstu_hip_kv_append_fp8_get_workspace_size(const hstu_kv_append_fp8_params* p, uint64_t* workspace_bytes);
+int hstu_hip_kv_append_fp8(const hstu_kv_append_fp8_params* p, void* workspace, uint64_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

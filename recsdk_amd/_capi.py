@@ -27,7 +27,7 @@ EXPORTS = [
     "hstu_hip_jagged_backward_get_workspace_size", "hstu_hip_jagged_backward",
     "hstu_hip_dense_backward_get_workspace_size", "hstu_hip_dense_backward",
     "hstu_hip_last_error", "hstu_hip_describe_kernel", "hstu_hip_abi_version",
-    "hstu_hip_kv_append", "hstu_hip_kv_token_positions",
+    "hstu_hip_kv_append", "hstu_hip_kv_token_positions", "hstu_hip_kv_append_fp8", "hstu_hip_kv_append_fp8_get_workspace_size",
     "hstu_hip_rab_time", "hstu_hip_rab_time_backward", "hstu_hip_rab_pos",
     "hstu_hip_norm_multiply_dropout", "hstu_hip_norm_multiply_dropout_backward",
     "hstu_hip_norm_multiply_dropout_backward_get_workspace_size", "hstu_hip_in_linear_silu",
@@ -66,6 +66,19 @@ class HstuKvAppendParams(C.Structure):
     _fields_ = [
         ("struct_size", C.c_uint32), ("elem_bytes", C.c_int32), ("k_cache", C.c_void_p), ("v_cache", C.c_void_p),
         ("stride_page", C.c_int64), ("stride_n", C.c_int64), ("stride_h", C.c_int64),
+        ("num_pages", C.c_int32), ("page_size", C.c_int32), ("num_heads", C.c_int32), ("head_dim", C.c_int32),
+        ("kv_indices", C.c_void_p), ("kv_indptr", C.c_void_p), ("num_indices", C.c_int32), ("batch", C.c_int32),
+        ("append_key", C.c_void_p), ("append_value", C.c_void_p),
+        ("append_k_stride_n", C.c_int64), ("append_k_stride_h", C.c_int64),
+        ("append_v_stride_n", C.c_int64), ("append_v_stride_h", C.c_int64), ("append_rows", C.c_int64),
+        ("batch_indices", C.c_void_p), ("positions", C.c_void_p), ("offsets", C.c_void_p), ("nnz_dev", C.c_void_p),
+        ("nnz_max", C.c_int32), ("reserved", C.c_int32),
+    ]
+
+
+class HstuKvAppendFp8Params(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32), ("src_dtype", C.c_int32), ("kv_cache", C.c_void_p), ("kv_scales", C.c_void_p),
         ("num_pages", C.c_int32), ("page_size", C.c_int32), ("num_heads", C.c_int32), ("head_dim", C.c_int32),
         ("kv_indices", C.c_void_p), ("kv_indptr", C.c_void_p), ("num_indices", C.c_int32), ("batch", C.c_int32),
         ("append_key", C.c_void_p), ("append_value", C.c_void_p),
@@ -153,6 +166,8 @@ def lib() -> C.CDLL:
             getattr(_lib, f"hstu_hip_{n}_backward_get_workspace_size").argtypes = [C.POINTER(HstuBwdParams), C.POINTER(C.c_uint64)]
         _lib.hstu_hip_describe_kernel.argtypes = [C.POINTER(HstuFwdParams), C.c_char_p, C.c_size_t]
         _lib.hstu_hip_kv_append.argtypes = [C.POINTER(HstuKvAppendParams), C.c_void_p]
+        _lib.hstu_hip_kv_append_fp8.argtypes = [C.POINTER(HstuKvAppendFp8Params), C.c_void_p, C.c_uint64, C.c_void_p]
+        _lib.hstu_hip_kv_append_fp8_get_workspace_size.argtypes = [C.POINTER(HstuKvAppendFp8Params), C.POINTER(C.c_uint64)]
         _lib.hstu_hip_rab_time.argtypes = [C.POINTER(HstuRabTimeParams), C.c_void_p]
         _lib.hstu_hip_norm_multiply_dropout.argtypes = [C.POINTER(HstuNmdParams), C.c_void_p]
         _lib.hstu_hip_in_linear_silu.argtypes = [C.POINTER(HstuInLinearSiluParams), C.c_void_p]

@@ -102,6 +102,59 @@ def append_kvcache(append_key, append_value, batch_indices, positions, seqlen_of
         _capi._check(_capi.lib().hstu_hip_kv_append(C.byref(p), _capi._stream()))
 
 
+def append_kvcache_fp8(append_key, append_value, batch_indices, positions, seqlen_offsets, nnz_npu, nnz: int,
+                       kv_cache_fp8, kv_scales, kv_indices, kv_indptr, workspace=None):
+    """``append_kvcache`` for the fp8-e4m3 table that ``torch.ops.mxrec.hstu_paged_fp8`` reads (no counterpart in the
+    reference): ``kv_cache_fp8`` is ``[pages, 2, page_size, heads, dim]`` (uint8 or float8_e4m3fn, contiguous),
+    ``kv_scales`` ``[pages, 2, heads]`` fp32.  The new rows are quantised with one scale per (page, K|V, head); a page
+    that already holds rows keeps its scale unless the new rows need a larger one, in which case its old rows are
+    requantised.  ``workspace`` (uint8, at least ``pages * (2 * heads + 1) * 4`` bytes) is allocated when not given;
+    returns it for reuse."""
+    device = append_key.device
+    _check_kv_2byte(append_key, device, 3, "append_key")
+    _check_kv_2byte(append_value, device, 3, "append_value")
+    if append_key.shape != append_value.shape or append_key.dtype != append_value.dtype:
+        raise RuntimeError("append_key and append_value must have the same shape and dtype")
+    if append_key.dtype not in (torch.float16, torch.bfloat16):
+        raise RuntimeError("append_key must be float16 or bfloat16")
+    for t, name in ((batch_indices, "batch_indices"), (positions, "positions"), (seqlen_offsets, "seqlen_offsets"), (nnz_npu, "nnz_npu"),
+                    (kv_indices, "kv_indices"), (kv_indptr, "kv_indptr")):
+        _check_int32_1d(t, device, name)
+    if kv_cache_fp8.device != device or kv_cache_fp8.element_size() != 1 or kv_cache_fp8.dim() != 5 or kv_cache_fp8.size(1) != 2 \
+            or not kv_cache_fp8.is_contiguous():
+        raise RuntimeError("kv_cache_fp8 must be a contiguous 1-byte [pages, 2, page_size, heads, dim] tensor on the device of append_key")
+    pages, _, page_size, num_heads, head_dim = kv_cache_fp8.shape
+    if kv_scales.device != device or kv_scales.dtype != torch.float32 or tuple(kv_scales.shape) != (pages, 2, num_heads) or not kv_scales.is_contiguous():
+        raise RuntimeError(f"kv_scales must be a contiguous float32 [{pages}, 2, {num_heads}] tensor on the device of append_key")
+    if append_key.stride(2) != 1 or append_value.stride(2) != 1:
+        raise RuntimeError("the head_dim axis of append_key / append_value must be contiguous")
+    if tuple(append_key.shape[1:]) != (num_heads, head_dim):
+        raise RuntimeError(f"append_key shape {tuple(append_key.shape)} mismatch with cache heads {num_heads}, head_dim {head_dim}")
+    p = _capi.HstuKvAppendFp8Params()
+    p.struct_size = C.sizeof(_capi.HstuKvAppendFp8Params)
+    p.src_dtype = _capi.HSTU_BF16 if append_key.dtype == torch.bfloat16 else _capi.HSTU_F16
+    p.kv_cache, p.kv_scales = kv_cache_fp8.data_ptr(), kv_scales.data_ptr()
+    p.num_pages, p.page_size, p.num_heads, p.head_dim = pages, page_size, num_heads, head_dim
+    p.kv_indices, p.kv_indptr = kv_indices.data_ptr(), kv_indptr.data_ptr()
+    p.num_indices, p.batch = kv_indices.numel(), kv_indptr.numel() - 1
+    if seqlen_offsets.numel() < p.batch:
+        raise RuntimeError("seqlen_offsets must have one entry per user of kv_indptr")
+    p.append_key, p.append_value = append_key.data_ptr(), append_value.data_ptr()
+    p.append_k_stride_n, p.append_k_stride_h = append_key.stride(0), append_key.stride(1)
+    p.append_v_stride_n, p.append_v_stride_h = append_value.stride(0), append_value.stride(1)
+    p.append_rows = append_key.size(0)
+    p.batch_indices, p.positions, p.offsets = batch_indices.data_ptr(), positions.data_ptr(), seqlen_offsets.data_ptr()
+    p.nnz_dev, p.nnz_max = nnz_npu.data_ptr(), min(int(nnz), batch_indices.numel(), positions.numel())
+    need = C.c_uint64(0)
+    _capi._check(_capi.lib().hstu_hip_kv_append_fp8_get_workspace_size(C.byref(p), C.byref(need)))
+    _require_gpu(append_key, "append_kvcache_fp8")
+    with torch.cuda.device(device):
+        if workspace is None or workspace.numel() * workspace.element_size() < need.value:
+            workspace = torch.empty(need.value, dtype=torch.uint8, device=device)
+        _capi._check(_capi.lib().hstu_hip_kv_append_fp8(C.byref(p), workspace.data_ptr(), workspace.numel() * workspace.element_size(), _capi._stream()))
+    return workspace
+
+
 def get_paged_batch_indices_positions(append_indptr, seq_lens, batch_indices, positions) -> None:
     """Fill ``batch_indices`` / ``positions`` (int32, one entry per new token) from ``append_indptr`` (``[batch + 1]``
     offsets of the new tokens of every user) and ``seq_lens`` (``[batch]`` tokens of every user after the append)."""

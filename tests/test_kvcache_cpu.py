@@ -151,3 +151,76 @@ def test_host_mirror_checks_like_the_reference_binding():
         kvcache.append_kvcache(*args())
     with pytest.raises(RuntimeError, match="no CPU implementation"):
         kvcache.get_paged_batch_indices_positions(i32(2), i32(1), i32(4), i32(4))
+
+
+def test_fp8_append_oracle_is_whole_page_quantisation_and_bounded():
+    """The fp8 append has no reference counterpart; its oracle is pinned by what the definition implies: (1) pages filled
+    by one append equal quantising the whole 2-byte page at once (``quantize_kv_cache_fp8``, scale = absmax / 448);
+    (2) after a second append every stored value is within the e4m3 step (2^-4 relative to its own magnitude, or half the
+    smallest subnormal step of the page's scale) -- twice that for rows that were requantised; (3) a second append that
+    needs no larger scale leaves the old bytes alone."""
+    import torch
+    from oracle import hstu_oracle as O
+    g = torch.Generator().manual_seed(3)
+    page, heads, dim = 8, 2, 16
+    kv_indices, kv_indptr = np.array([2, 0, 3, 1], dtype=np.int32), np.array([0, 2, 4], dtype=np.int32)
+    cache = torch.zeros(5, 2, page, heads, dim, dtype=torch.uint8)
+    scales = torch.ones(5, 2, heads)
+    l1 = [11, 5]
+    k1 = torch.randn(sum(l1), heads, dim, generator=g).to(torch.bfloat16)
+    v1 = torch.randn(sum(l1), heads, dim, generator=g).to(torch.bfloat16)
+    bi, pos = KO.paged_batch_indices_positions([0, 11, 16], l1)
+    KO.append_paged_kvcache_fp8(cache, scales, k1, v1, bi, pos, [0, 0], 16, kv_indices, kv_indptr)
+    # the same rows in a 2-byte table, quantised page by page
+    table = torch.zeros(5, 2, page, heads, dim, dtype=torch.bfloat16)
+    t16 = table.view(torch.int16).numpy()
+    KO.append_paged_kvcache(t16[:, 0], t16[:, 1], k1.view(torch.int16).numpy(), v1.view(torch.int16).numpy(), bi, pos, [0, 0], 16, kv_indices, kv_indptr)
+    want8, want_s = O.quantize_kv_cache_fp8(table)
+    touched = [2, 0, 3]
+    assert torch.equal(cache[touched], want8[touched]) and torch.equal(scales[touched], want_s[touched])
+    assert torch.equal(scales[[1, 4]], torch.ones(2, 2, heads)) and int(cache[[1, 4]].abs().sum()) == 0
+    # second append: user 0 gets larger rows (scale of page 0 grows), user 1 smaller ones (scale of page 3 stays)
+    before = cache.clone()
+    s_before = scales.clone()
+    k2 = torch.cat([torch.randn(3, heads, dim, generator=g) * 8, torch.randn(2, heads, dim, generator=g) * 0.01]).to(torch.bfloat16)
+    v2 = (k2.float() * 0.5).to(torch.bfloat16)
+    bi2, pos2 = KO.paged_batch_indices_positions([0, 3, 5], [14, 7])
+    KO.append_paged_kvcache_fp8(cache, scales, k2, v2, bi2, pos2, [0, 0], 5, kv_indices, kv_indptr)
+    assert bool((scales[0] > s_before[0]).all()) and torch.equal(scales[3], s_before[3]) and torch.equal(scales[2], s_before[2])
+    assert torch.equal(cache[3, :, :5], before[3, :, :5]) and torch.equal(cache[2], before[2])
+    assert not torch.equal(cache[0, :, :3], before[0, :, :3])
+    deq = O.dequantize_kv_cache_fp8(cache, scales)
+    full_k = torch.cat([k1[:11], k2[:3]]).float()
+    got_k = torch.cat([deq[2, 0], deq[0, 0, :6]])
+    step = scales[[2] * 8 + [0] * 6, 0][:, :, None] * 2.0 ** -9          # half the subnormal spacing 2^-9 ... of e4m3 times the scale
+    lim = full_k.abs() * 2.0 ** -4 + step
+    lim[8:11] *= 2                                                         # requantised rows
+    assert bool(((got_k - full_k).abs() <= lim * 1.001).all())
+
+
+def test_fp8_append_abi_validation():
+    L = _capi.lib()
+    def call(ws=0x1000, ws_bytes=1 << 20, **over):
+        p = _capi.HstuKvAppendFp8Params()
+        p.struct_size = C.sizeof(_capi.HstuKvAppendFp8Params)
+        p.src_dtype, p.num_pages, p.page_size, p.num_heads, p.head_dim = _capi.HSTU_BF16, 10, 16, 2, 64
+        p.num_indices, p.batch, p.nnz_max, p.append_rows = 4, 2, 8, 8
+        p.append_k_stride_n = p.append_v_stride_n = 128
+        p.append_k_stride_h = p.append_v_stride_h = 64
+        for f in ("kv_cache", "kv_scales", "kv_indices", "kv_indptr", "append_key", "append_value", "batch_indices", "positions", "offsets", "nnz_dev"):
+            setattr(p, f, 0x1000)
+        for k, v in over.items():
+            setattr(p, k, v)
+        return L.hstu_hip_kv_append_fp8(C.byref(p), ws, ws_bytes, None), L.hstu_hip_last_error().decode(), p
+    for over, text in ((dict(src_dtype=_capi.HSTU_F32), "src_dtype expect float16 or bfloat16"), (dict(head_dim=96), "head_dim expect a power of two"),
+                       (dict(num_pages=0), "must be positive"), (dict(kv_scales=None), "must not be NULL")):
+        rc, msg, _ = call(**over)
+        assert rc == -1 and text in msg, (over, msg)
+    rc, msg, _ = call(append_k_stride_h=60)
+    assert rc == -2 and "multiples of 8" in msg
+    rc, msg, p = call(ws_bytes=16)
+    assert rc == -3 and "workspace" in msg
+    need = C.c_uint64(0)
+    assert L.hstu_hip_kv_append_fp8_get_workspace_size(C.byref(p), C.byref(need)) == 0 and need.value == 10 * (2 * 2 + 1) * 4
+    rc, _, _ = call(nnz_max=0)
+    assert rc == 0

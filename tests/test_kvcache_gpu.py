@@ -138,3 +138,77 @@ def test_roundtrip_append_then_hstu_paged(dtype):
     out, _ = T.run_capi(dict(cfg, kv_cache=table.cpu()), op="paged")
     assert torch.equal(out, out_ref)
     T.assert_parity(out, T.oracle_paged(cfg), dtype, what="paged forward over the appended table")
+
+
+def _fp8_scenario(seed, users, heads, dim, page, dtype):
+    """Two appends per user: a prefill of L1 rows, then A more rows whose amplitude is larger for some users (their
+    pages' scales grow and the old rows are requantised) and smaller for others (scales stay)."""
+    g = torch.Generator().manual_seed(seed)
+    l1 = torch.randint(0, 3 * page, (users,), generator=g)
+    add = torch.randint(0, 2 * page + 5, (users,), generator=g)
+    need = ((l1 + add + page - 1) // page).clamp(min=1)
+    pages = int(need.sum()) + 3
+    perm = torch.randperm(pages, generator=g)[: int(need.sum())].to(torch.int32)
+    indptr = torch.cat([torch.zeros(1, dtype=torch.int64), need.cumsum(0)]).to(torch.int32)
+    amp = torch.tensor([0.25, 1.0, 4.0])[torch.randint(0, 3, (users,), generator=g)]
+    steps = []
+    for n_new, seq, a in ((l1, l1, torch.ones(users)), (add, l1 + add, amp)):
+        ip = torch.cat([torch.zeros(1, dtype=torch.int64), n_new.cumsum(0)]).to(torch.int32)
+        rows = int(n_new.sum())
+        scale = torch.repeat_interleave(a, n_new)[:, None, None]
+        k = (torch.randn(rows, heads, dim, generator=g) * scale).to(dtype)
+        v = (torch.randn(rows, heads, dim, generator=g) * scale * 0.5).to(dtype)
+        steps.append(dict(append_indptr=ip, seq_lens=seq.to(torch.int32), key=k, value=v, nnz=rows))
+    return dict(pages=pages, kv_indices=perm, kv_indptr=indptr, steps=steps, users=users)
+
+
+@pytest.mark.parametrize("dim,heads,page,dtype", [(128, 4, 64, torch.bfloat16), (64, 2, 32, torch.float16), (256, 1, 16, torch.bfloat16),
+                                                  (8, 3, 8, torch.bfloat16)])
+def test_fp8_append_matches_oracle_bit_for_bit(dim, heads, page, dtype):
+    """Bytes and scales after a prefill and after an extension of partly filled pages, against the oracle's restatement
+    of this library's own definition (no reference counterpart: parity with the reference unpinned by construction)."""
+    say("kv append fp8", dim, heads, page, dtype)
+    s = _fp8_scenario(5, 9, heads, dim, page, dtype)
+    cache = torch.zeros(s["pages"], 2, page, heads, dim, dtype=torch.uint8)
+    scales = torch.ones(s["pages"], 2, heads)
+    dc, ds = cache.cuda(), scales.cuda()
+    ws = None
+    zeros = torch.zeros(s["users"], dtype=torch.int32)
+    for n, st in enumerate(s["steps"]):
+        bi, pos = KO.paged_batch_indices_positions(st["append_indptr"].numpy(), st["seq_lens"].numpy())
+        KO.append_paged_kvcache_fp8(cache, scales, st["key"], st["value"], bi, pos, zeros.numpy(), st["nnz"], s["kv_indices"].numpy(),
+                                    s["kv_indptr"].numpy())
+        dbi = torch.empty(max(st["nnz"], 1), dtype=torch.int32, device="cuda")
+        dpos = torch.empty_like(dbi)
+        kvcache.get_paged_batch_indices_positions(st["append_indptr"].cuda(), st["seq_lens"].cuda(), dbi, dpos)
+        ws = kvcache.append_kvcache_fp8(st["key"].cuda(), st["value"].cuda(), dbi, dpos, zeros.cuda(),
+                                        torch.tensor([st["nnz"]], dtype=torch.int32, device="cuda"), st["nnz"], dc, ds,
+                                        s["kv_indices"].cuda(), s["kv_indptr"].cuda(), workspace=ws)
+        torch.cuda.synchronize()
+        assert torch.equal(ds.cpu(), scales), f"scales after step {n}"
+        diff = (dc.cpu() != cache)
+        assert not bool(diff.any()), f"bytes after step {n}: {int(diff.sum())} differ"
+    assert int((cache != 0).sum()) > 0
+
+
+def test_fp8_prefill_equals_whole_page_quantisation_and_feeds_paged_fp8():
+    """One append into an empty table = quantising the 2-byte table (appended by the 2-byte kernel) page by page, which
+    is what the hstu_paged_fp8 tests feed the attention with."""
+    say("kv append fp8 prefill == quantize_pages_fp8")
+    c = W.kv_append_config(41, users=6, heads=4, dim=128, prev_lo=0, prev_hi=0, new_lo=1, new_hi=200, page_size=64, dtype=torch.bfloat16)
+    c["kv_cache"].zero_()
+    # users start empty: every page is filled by this append alone
+    assert int((c["seq_lens"] - (c["append_indptr"][1:] - c["append_indptr"][:-1])).abs().sum()) == 0
+    bi, pos = _positions(c)
+    table = c["kv_cache"].cuda()
+    _append(c, bi, pos, table)
+    want8, want_s = W.quantize_pages_fp8(table.cpu())
+    cache8 = torch.zeros(table.shape, dtype=torch.uint8, device="cuda")
+    sc = torch.ones(table.shape[0], 2, table.shape[3], device="cuda")
+    kvcache.append_kvcache_fp8(c["append_key"].cuda(), c["append_value"].cuda(), bi, pos, c["offsets"].cuda(), c["nnz_dev"].cuda(), c["nnz"],
+                               cache8, sc, c["kv_indices"].cuda(), c["kv_indptr"].cuda())
+    torch.cuda.synchronize()
+    touched = torch.zeros(table.shape[0], dtype=torch.bool)
+    touched[c["kv_indices"].long()] = True
+    assert torch.equal(sc.cpu()[touched], want_s[touched])
+    assert torch.equal(cache8.cpu()[touched], want8.view(torch.uint8)[touched])
