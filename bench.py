@@ -23,7 +23,7 @@ PEAK_HBM_GBS = 8000.0
 # HBM-side bytes per launch from rocprofv3 FETCH_SIZE/WRITE_SIZE, each scaled by what the same counter reads for the
 # plain 256 MiB copy of `--workload copy` (factors 2.000 and 1.000); see profiles/*.md
 MEASURED_TRAFFIC_BYTES = {"config2": 184.3e6, "kv_append": 351.9e6, "rab_time": 1479.8e6, "rab_time_bwd": 2242.4e6, "rab_pos": 305.2e6,
-                          "nmd_fwd": 827.4e6, "nmd_bwd": 1382.0e6, "in_linear_silu": 1092.8e6, "in_linear_silu_bwd": 2363.7e6}
+                          "nmd_fwd": 827.4e6, "nmd_bwd": 1382.0e6, "in_linear_silu": 1092.8e6, "in_linear_silu_bwd": 2363.7e6, "kv_append_fp8": 455.0e6}
 
 
 def build_workload(name, torch, W):
@@ -58,7 +58,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=1000)
-    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "config2_bwd", "kv_append", "rab_time", "rab_time_bwd", "rab_pos", "nmd_fwd", "nmd_bwd", "in_linear_silu", "in_linear_silu_bwd", "copy"],
+    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "config2_bwd", "kv_append", "kv_append_fp8", "rab_time", "rab_time_bwd", "rab_pos", "nmd_fwd", "nmd_bwd", "in_linear_silu", "in_linear_silu_bwd", "copy"],
                     help="'copy' runs a plain 256 MiB device copy: the known-size kernel the FETCH_SIZE/WRITE_SIZE counters are scaled by")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
@@ -76,6 +76,8 @@ def main():
         return backward_bench(args, torch, W, _capi)
     if args.workload == "kv_append":
         return kv_append_bench(args, torch, W)
+    if args.workload == "kv_append_fp8":
+        return kv_append_fp8_bench(args, torch, W)
     if args.workload in ("rab_time", "rab_time_bwd", "rab_pos"):
         return bias_bench(args, torch)
     if args.workload in ("nmd_fwd", "nmd_bwd"):
@@ -281,6 +283,65 @@ def kv_append_bench(args, torch, W):
         dt = time.perf_counter() - t0
         out["cpu_baseline"] = {"value": round(alg_bytes / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
                                "sample": f"the whole append once, token loop in numpy, {dt:.2f} s"}
+    print(json.dumps(out), flush=True)
+
+
+def kv_append_fp8_bench(args, torch, W):
+    """The fp8 write side at the kv_append workload's shape: the prefill of config 5's history (32 users, 1024-4096 tokens,
+    4 heads x 128, bf16 rows) into an e4m3 table with per-(page, K|V, head) scales.  Algorithmic bytes: every row read
+    once (2 bytes per element) and written once (1 byte); the kernels read the rows twice (absmax pass, quantise pass)."""
+    from recsdk_amd import kvcache
+    cfg = W.kv_append_config(0, users=32, heads=4, dim=128, prev_lo=0, prev_hi=0, new_lo=1024, new_hi=4096, page_size=64)
+    dev = W.to_device(cfg)
+    n = cfg["nnz"]
+    bi = torch.empty(n, dtype=torch.int32, device="cuda")
+    pos = torch.empty_like(bi)
+    kvcache.get_paged_batch_indices_positions(dev["append_indptr"], dev["seq_lens"], bi, pos)
+    pages = cfg["kv_cache"].shape[0]
+    cache8 = torch.zeros(pages, 2, 64, 4, 128, dtype=torch.uint8, device="cuda")
+    scales = torch.ones(pages, 2, 4, device="cuda")
+    ws = torch.empty(pages * 9 * 4, dtype=torch.uint8, device="cuda")
+
+    def fn():
+        kvcache.append_kvcache_fp8(dev["append_key"], dev["append_value"], bi, pos, dev["offsets"], dev["nnz_dev"], n, cache8, scales,
+                                   dev["kv_indices"], dev["kv_indptr"], workspace=ws)
+    for _ in range(args.warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    kern_ms = e0.elapsed_time(e1) / args.steps
+    elems = n * 2 * 4 * 128
+    alg = elems * 3 + pages * 8 * 4 + n * 2 * 4
+    out = {
+        "metric": "paged_kv_append_fp8_gbps", "value": round(alg / (ms * 1e-3) / 1e9, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u8", "data": "synthetic", "us_per_call": round(ms * 1e3, 2),
+        "config": {"workload": f"fp8 append of {n} new tokens (32 users x U[1024,4096]) x 4 heads x 128 from bf16, 64-token pages, seed 0",
+                   "algorithmic_bytes_per_call": alg, "entry": "hstu_hip_kv_append_fp8 (C ABI): init, scan, scale, write kernels"},
+        "roofline": {"bound": "hbm", "kernel": "hstu_kv_fp8_scan_kernel + hstu_kv_fp8_write_kernel (+ 2 small kernels; all inside the events)",
+                     "achieved": round(alg / (kern_ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(alg / (kern_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                     "kernel_us": round(kern_ms * 1e3, 2)},
+    }
+    if not args.no_cpu_baseline:
+        from oracle import kvcache_oracle as KO
+        users = 2
+        last = int(cfg["append_indptr"][users])
+        c8, sc = torch.zeros(pages, 2, 64, 4, 128, dtype=torch.uint8), torch.ones(pages, 2, 4)
+        b_, p_ = KO.paged_batch_indices_positions(cfg["append_indptr"][: users + 1].numpy(), cfg["seq_lens"][:users].numpy())
+        t0 = time.perf_counter()
+        KO.append_paged_kvcache_fp8(c8, sc, cfg["append_key"], cfg["append_value"], b_, p_, cfg["offsets"].numpy(), last, cfg["kv_indices"].numpy(),
+                                    cfg["kv_indptr"].numpy())
+        dt = time.perf_counter() - t0
+        out["cpu_baseline"] = {"value": round(alg * last / n / dt / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"the first {users} users ({last} tokens) once, page loop in torch, {dt:.2f} s"}
     print(json.dumps(out), flush=True)
 
 

@@ -55,42 +55,51 @@ __global__ __launch_bounds__(256) void hstu_kv_fp8_init_kernel(unsigned* unit_ma
     if (i < pages) first_slot[i] = KF_NOSLOT;
 }
 
-// one lane = 8 elements of one (token, K|V, head) row; the dim / 8 lanes of a row sit side by side in a wave
+// one lane = the same 8 elements of the K row and of the V row of one (token, head); the dim / 8 lanes of a row sit
+// side by side in a wave.  IDX: type of the flat lane index, 32 bits whenever nnz_max * lanes per token fits
+template <typename IDX>
 __global__ __launch_bounds__(256) void hstu_kv_fp8_scan_kernel(const hstu_kv_append_fp8_params p, unsigned* unit_max, int* first_slot) {
     const unsigned cph = (unsigned)p.head_dim / 8;
-    const unsigned cpt = cph * (unsigned)p.num_heads * 2;
+    const unsigned cpt = cph * (unsigned)p.num_heads;
     const int nnz = min(max(*p.nnz_dev, 0), p.nnz_max);
-    const unsigned long long total = (unsigned long long)nnz * cpt;
-    const unsigned long long stride = (unsigned long long)gridDim.x * 256;
+    const IDX total = (IDX)nnz * cpt;
+    const IDX stride = (IDX)gridDim.x * 256;
     const int bf16 = p.src_dtype == HSTU_BF16;
     // every lane of a wave runs the same number of rounds: the shuffles below need all lanes of a row present
-    const unsigned long long rounds = (total + stride - 1) / stride;
-    for (unsigned long long r = 0; r < rounds; r++) {
-        const unsigned long long gidx = r * stride + (unsigned long long)blockIdx.x * 256 + threadIdx.x;
-        float amax = 0.f;
+    const IDX rounds = (total + stride - 1) / stride;
+    for (IDX r = 0; r < rounds; r++) {
+        const IDX gidx = r * stride + (IDX)blockIdx.x * 256 + threadIdx.x;
+        float kmax = 0.f, vmax = 0.f;
         bool ok = false;
-        int page = 0, slot = 0, kv = 0;
+        int page = 0, slot = 0;
         unsigned head = 0, c = 0;
         if (gidx < total) {
             const unsigned i = (unsigned)(gidx / cpt), rem = (unsigned)(gidx % cpt);
-            kv = (int)(rem / (cph * p.num_heads));
-            head = rem / cph % (unsigned)p.num_heads;
+            head = rem / cph;
             c = rem % cph;
             int64_t row;
             ok = kf_route(p, i, page, slot, row);
             if (ok) {
-                const unsigned short* src = reinterpret_cast<const unsigned short*>(kv ? p.append_value : p.append_key);
-                const int64_t sn = kv ? p.append_v_stride_n : p.append_k_stride_n, sh = kv ? p.append_v_stride_h : p.append_k_stride_h;
-                const kf_u32x4 x = *reinterpret_cast<const kf_u32x4*>(src + row * sn + head * sh + 8 * c);
+                const kf_u32x4 kx = *reinterpret_cast<const kf_u32x4*>(reinterpret_cast<const unsigned short*>(p.append_key) +
+                                                                       row * p.append_k_stride_n + head * p.append_k_stride_h + 8 * c);
+                const kf_u32x4 vx = *reinterpret_cast<const kf_u32x4*>(reinterpret_cast<const unsigned short*>(p.append_value) +
+                                                                       row * p.append_v_stride_n + head * p.append_v_stride_h + 8 * c);
 #pragma unroll
-                for (int e = 0; e < 4; e++) amax = fmaxf(amax, fmaxf(fabsf(kf_elem(x[e], 0, bf16)), fabsf(kf_elem(x[e], 1, bf16))));
+                for (int e = 0; e < 4; e++) {
+                    kmax = fmaxf(kmax, fmaxf(fabsf(kf_elem(kx[e], 0, bf16)), fabsf(kf_elem(kx[e], 1, bf16))));
+                    vmax = fmaxf(vmax, fmaxf(fabsf(kf_elem(vx[e], 0, bf16)), fabsf(kf_elem(vx[e], 1, bf16))));
+                }
             }
         }
-        for (unsigned o = 1; o < cph; o <<= 1) amax = fmaxf(amax, __shfl_xor(amax, (int)o));
+        for (unsigned o = 1; o < cph; o <<= 1) {
+            kmax = fmaxf(kmax, __shfl_xor(kmax, (int)o));
+            vmax = fmaxf(vmax, __shfl_xor(vmax, (int)o));
+        }
         if (ok && c == 0) {
             // non-negative floats order like their bit patterns
-            atomicMax(unit_max + ((int64_t)page * 2 + kv) * p.num_heads + head, __builtin_bit_cast(unsigned, amax));
-            if (kv == 0 && head == 0) atomicMin(first_slot + page, slot);
+            atomicMax(unit_max + ((int64_t)page * 2 + 0) * p.num_heads + head, __builtin_bit_cast(unsigned, kmax));
+            atomicMax(unit_max + ((int64_t)page * 2 + 1) * p.num_heads + head, __builtin_bit_cast(unsigned, vmax));
+            if (head == 0) atomicMin(first_slot + page, slot);
         }
     }
 }
@@ -118,30 +127,34 @@ __global__ __launch_bounds__(256) void hstu_kv_fp8_scale_kernel(const hstu_kv_ap
     if (threadIdx.x == 0) p.kv_scales[unit] = s;
 }
 
+template <typename IDX>
 __global__ __launch_bounds__(256) void hstu_kv_fp8_write_kernel(const hstu_kv_append_fp8_params p) {
     const unsigned cph = (unsigned)p.head_dim / 8;
-    const unsigned cpt = cph * (unsigned)p.num_heads * 2;
+    const unsigned cpt = cph * (unsigned)p.num_heads;
     const int nnz = min(max(*p.nnz_dev, 0), p.nnz_max);
-    const unsigned long long total = (unsigned long long)nnz * cpt;
-    const unsigned long long stride = (unsigned long long)gridDim.x * 256;
+    const IDX total = (IDX)nnz * cpt;
+    const IDX stride = (IDX)gridDim.x * 256;
     const int bf16 = p.src_dtype == HSTU_BF16;
-    for (unsigned long long gidx = (unsigned long long)blockIdx.x * 256 + threadIdx.x; gidx < total; gidx += stride) {
+    for (IDX gidx = (IDX)blockIdx.x * 256 + threadIdx.x; gidx < total; gidx += stride) {
         const unsigned i = (unsigned)(gidx / cpt), rem = (unsigned)(gidx % cpt);
-        const int kv = (int)(rem / (cph * p.num_heads));
-        const unsigned head = rem / cph % (unsigned)p.num_heads, c = rem % cph;
+        const unsigned head = rem / cph, c = rem % cph;
         int page, slot;
         int64_t row;
         if (!kf_route(p, i, page, slot, row)) continue;
-        const unsigned short* src = reinterpret_cast<const unsigned short*>(kv ? p.append_value : p.append_key);
-        const int64_t sn = kv ? p.append_v_stride_n : p.append_k_stride_n, sh = kv ? p.append_v_stride_h : p.append_k_stride_h;
-        const kf_u32x4 x = *reinterpret_cast<const kf_u32x4*>(src + row * sn + head * sh + 8 * c);
-        const float s = p.kv_scales[((int64_t)page * 2 + kv) * p.num_heads + head];
-        unsigned q[4];
+        const kf_u32x4 kx = *reinterpret_cast<const kf_u32x4*>(reinterpret_cast<const unsigned short*>(p.append_key) + row * p.append_k_stride_n +
+                                                               head * p.append_k_stride_h + 8 * c);
+        const kf_u32x4 vx = *reinterpret_cast<const kf_u32x4*>(reinterpret_cast<const unsigned short*>(p.append_value) + row * p.append_v_stride_n +
+                                                               head * p.append_v_stride_h + 8 * c);
+        const float sk = p.kv_scales[((int64_t)page * 2 + 0) * p.num_heads + head], sv = p.kv_scales[((int64_t)page * 2 + 1) * p.num_heads + head];
+        unsigned qk[4], qv[4];
 #pragma unroll
-        for (int e = 0; e < 4; e++) q[e] = kf_quant2(kf_elem(x[e], 0, bf16), kf_elem(x[e], 1, bf16), s);
-        const kf_u32x2 out = {q[0] | (q[1] << 16), q[2] | (q[3] << 16)};
-        uint8_t* dst = p.kv_cache + ((((int64_t)page * 2 + kv) * p.page_size + slot) * p.num_heads + head) * p.head_dim + 8 * c;
-        *reinterpret_cast<kf_u32x2*>(dst) = out;
+        for (int e = 0; e < 4; e++) {
+            qk[e] = kf_quant2(kf_elem(kx[e], 0, bf16), kf_elem(kx[e], 1, bf16), sk);
+            qv[e] = kf_quant2(kf_elem(vx[e], 0, bf16), kf_elem(vx[e], 1, bf16), sv);
+        }
+        uint8_t* dst = p.kv_cache + ((((int64_t)page * 2) * p.page_size + slot) * p.num_heads + head) * p.head_dim + 8 * c;
+        *reinterpret_cast<kf_u32x2*>(dst) = kf_u32x2{qk[0] | (qk[1] << 16), qk[2] | (qk[3] << 16)};
+        *reinterpret_cast<kf_u32x2*>(dst + (int64_t)p.page_size * p.num_heads * p.head_dim) = kf_u32x2{qv[0] | (qv[1] << 16), qv[2] | (qv[3] << 16)};
     }
 }
 
@@ -194,12 +207,15 @@ extern "C" int hstu_hip_kv_append_fp8(const hstu_kv_append_fp8_params* p, void* 
     int* first_slot = reinterpret_cast<int*>(unit_max + units);
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     hipLaunchKernelGGL(hstu_kv_fp8_init_kernel, dim3((unsigned)((units + 255) / 256)), dim3(256), 0, st, unit_max, units, first_slot, p->num_pages);
-    const int64_t lanes = (int64_t)p->nnz_max * 2 * p->num_heads * (p->head_dim / 8);
+    const int64_t lanes = (int64_t)p->nnz_max * p->num_heads * (p->head_dim / 8);
     const int64_t want = (lanes + 255) / 256;
     const unsigned grid = (unsigned)(want < 1 ? 1 : (want > 65536 ? 65536 : want));
-    hipLaunchKernelGGL(hstu_kv_fp8_scan_kernel, dim3(grid), dim3(256), 0, st, *p, unit_max, first_slot);
+    const bool small = lanes + 2 * (int64_t)grid * 256 < (int64_t)1 << 32;
+    if (small) hipLaunchKernelGGL(hstu_kv_fp8_scan_kernel<unsigned>, dim3(grid), dim3(256), 0, st, *p, unit_max, first_slot);
+    else hipLaunchKernelGGL(hstu_kv_fp8_scan_kernel<unsigned long long>, dim3(grid), dim3(256), 0, st, *p, unit_max, first_slot);
     hipLaunchKernelGGL(hstu_kv_fp8_scale_kernel, dim3((unsigned)units), dim3(256), 0, st, *p, unit_max, first_slot);
-    hipLaunchKernelGGL(hstu_kv_fp8_write_kernel, dim3(grid), dim3(256), 0, st, *p);
+    if (small) hipLaunchKernelGGL(hstu_kv_fp8_write_kernel<unsigned>, dim3(grid), dim3(256), 0, st, *p);
+    else hipLaunchKernelGGL(hstu_kv_fp8_write_kernel<unsigned long long>, dim3(grid), dim3(256), 0, st, *p);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString(e));
     return HSTU_OK;
