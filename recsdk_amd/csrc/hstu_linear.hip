@@ -6,8 +6,8 @@
 //   workgroup = 128 rows m x 64 columns n; wave w = rows 32 w .. 32 w + 31, all 64 columns (two 32 x 32 blocks: at 73
 //   registers and 4.5 KiB of LDS per wave six waves share a SIMD, which is what keeps the stores flowing; four blocks
 //   per wave measured 9 % slower, one block 23 % slower)
-//   out^T block = W x^T: v_mfma_f32_32x32x16 with A = W fragment, B = x fragment, both straight from global memory
-//   (each lane reads 16 contiguous bytes of a row: x and W are k-contiguous, which is what both operands want)
+//   out^T block = W x^T: v_mfma_f32_32x32x16 with A = W fragment, B = x fragment; both operands are staged through LDS
+//   64 columns of k at a time (loads of 128 contiguous bytes per row; a fragment is one 16-byte LDS read)
 //   epilogue: + bias, round -> linear_output; silu of the rounded value, round -> the four outputs; both leave through
 //   a per-wave LDS tile so that a lane stores 16 bytes of one output row and a wave instruction covers eight 128-byte runs
 // Definition: cust_op/test/in_linear_silu_test/test_in_linear_silu.py:31-45.
@@ -40,6 +40,7 @@ template <> struct IlsMM<_Float16> {
 constexpr int ILS_NB = 2;                                   // 32 x 32 blocks side by side per wave
 constexpr int ILS_BM = 128, ILS_BN = 32 * ILS_NB, ILS_NT = 256;
 constexpr int ILS_LPR = ILS_BN / 8, ILS_RPI = 64 / ILS_LPR;   // store phase: lanes per row, rows per instruction
+constexpr int ILS_KC = 64, ILS_SROW = ILS_KC * 2 + 16;   // k columns per staging round; bytes of one staged operand row
 constexpr int ILS_ROW = ILS_BN * 2 + 16;   // bytes of one parked row: + 16 keeps the 8-byte column writes of 32 rows off one bank
 
 struct IlsArgs {
@@ -50,7 +51,10 @@ struct IlsArgs {
 template <typename T>
 __global__ __launch_bounds__(ILS_NT) void hstu_in_linear_silu_kernel(const IlsArgs a) {
     typedef typename IlsMM<T>::v8 v8;
-    __shared__ __attribute__((aligned(16))) char park_all[(ILS_NT / 64) * 32 * ILS_ROW];
+    // operand staging of the k loop (x rows of the four waves, then the W rows they share) and, after it, the parked
+    // output tiles of the epilogue share one buffer
+    static_assert(ILS_SROW == ILS_ROW, "a wave's parked tile takes the place of its staged x rows");
+    __shared__ __attribute__((aligned(16))) char park_all[(ILS_BM + ILS_BN) * ILS_SROW];
     const hstu_in_linear_silu_params& p = a.p;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int g = lane >> 5, l32 = lane & 31;
@@ -70,35 +74,51 @@ __global__ __launch_bounds__(ILS_NT) void hstu_in_linear_silu_kernel(const IlsAr
     }
     const int n0 = tn * ILS_BN;
     const int64_t m0 = (int64_t)tm * ILS_BM + 32 * w;
-    if (m0 >= p.m) return;   // whole wave; nothing below synchronises across waves
     const T* x = reinterpret_cast<const T*>(p.x);
     const T* wt = reinterpret_cast<const T*>(p.weight);
-    // operand rows of this lane, clamped into the tensors (what is read for rows past the end is never stored)
-    const T* xrow = x + (m0 + l32 < p.m ? m0 + l32 : p.m - 1) * K + 8 * g;
-    const T* wrow[ILS_NB];
-#pragma unroll
-    for (int nb = 0; nb < ILS_NB; nb++) wrow[nb] = wt + (int64_t)min(n0 + 32 * nb + l32, N - 1) * K + 8 * g;
     ils_f32x16 acc[ILS_NB];
 #pragma unroll
     for (int nb = 0; nb < ILS_NB; nb++)
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[nb][r] = 0.f;
-    auto step = [&](int k0) __attribute__((always_inline)) {
-        const v8 xf = *reinterpret_cast<const v8*>(xrow + k0);
-        v8 wf[ILS_NB];
+    // Operands come in through LDS: eight lanes read 128 contiguous bytes of a row (x and W are k-contiguous), a wave
+    // its own 32 rows of x and a quarter of the 64 rows of W that the four waves share; an MFMA fragment is then one
+    // 16-byte LDS read (row stride 144 bytes: conflict-free).  Rows past the end repeat the last one (never stored),
+    // columns past k are zero.
+    {
+        const int chunk = lane & 7, lrow = lane >> 3;
+        char* xs = park_all + w * (32 * ILS_SROW);
+        char* wsh = park_all + ILS_BM * ILS_SROW;
+        const T* xsrc[4];
+        const T* wsrc[2];
 #pragma unroll
-        for (int nb = 0; nb < ILS_NB; nb++) wf[nb] = *reinterpret_cast<const v8*>(wrow[nb] + k0);
+        for (int i = 0; i < 4; i++) xsrc[i] = x + (m0 + lrow + 8 * i < p.m ? m0 + lrow + 8 * i : p.m - 1) * K + 8 * chunk;
 #pragma unroll
-        for (int nb = 0; nb < ILS_NB; nb++) acc[nb] = IlsMM<T>::mfma(wf[nb], xf, acc[nb]);
-    };
-    int k0 = 0;
-    for (; k0 + 64 <= K; k0 += 64) {   // four steps' loads in flight together
-        step(k0);
-        step(k0 + 16);
-        step(k0 + 32);
-        step(k0 + 48);
+        for (int i = 0; i < 2; i++) wsrc[i] = wt + (int64_t)min(n0 + 16 * w + lrow + 8 * i, N - 1) * K + 8 * chunk;
+        for (int k0 = 0; k0 < K; k0 += ILS_KC) {
+            const bool in = k0 + 8 * chunk < K;
+            v8 xv[4], wv[2];
+#pragma unroll
+            for (int i = 0; i < 4; i++) xv[i] = in ? *reinterpret_cast<const v8*>(xsrc[i] + k0) : v8{};
+#pragma unroll
+            for (int i = 0; i < 2; i++) wv[i] = in ? *reinterpret_cast<const v8*>(wsrc[i] + k0) : v8{};
+#pragma unroll
+            for (int i = 0; i < 4; i++) *reinterpret_cast<v8*>(xs + (lrow + 8 * i) * ILS_SROW + chunk * 16) = xv[i];
+#pragma unroll
+            for (int i = 0; i < 2; i++) *reinterpret_cast<v8*>(wsh + (16 * w + lrow + 8 * i) * ILS_SROW + chunk * 16) = wv[i];
+            __syncthreads();
+#pragma unroll
+            for (int s = 0; s < ILS_KC / 16; s++) {
+                const v8 xf = *reinterpret_cast<const v8*>(xs + l32 * ILS_SROW + (16 * s + 8 * g) * 2);
+#pragma unroll
+                for (int nb = 0; nb < ILS_NB; nb++) {
+                    const v8 wf = *reinterpret_cast<const v8*>(wsh + (32 * nb + l32) * ILS_SROW + (16 * s + 8 * g) * 2);
+                    acc[nb] = IlsMM<T>::mfma(wf, xf, acc[nb]);
+                }
+            }
+            __syncthreads();
+        }
     }
-    for (; k0 < K; k0 += 16) step(k0);
     // accumulator register r of block nb holds column n0 + 32 nb + 8 (r / 4) + 4 g + r % 4 of row m0 + l32
     char* park = park_all + w * (32 * ILS_ROW);
     T lin[ILS_NB][16];
