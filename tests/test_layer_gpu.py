@@ -247,3 +247,36 @@ def test_in_linear_silu_autograd():
     want = LO.in_linear_silu_backward(grads, x, w, outs[4].detach().cpu())
     _ilb_close(leaves[0].grad, want[0], dtype, "x.grad")
     _ilb_close(leaves[1].grad, want[1], dtype, "weight.grad")
+
+
+def test_in_linear_silu_backward_largest_reference_shape():
+    """k = 8160, n = 32640 at m = 511 (test_in_linear_silu_backward.py:169-176): 64 blocks of k per workgroup column, one
+    range of m.  Too large for the fp64 oracle in a test; checked against the same formula evaluated with torch's own
+    GPU routines in fp32 (sigmoid, rounding of dlin to bf16, two matrix products) -- a checker, not a code path of the op."""
+    m, k, n, dtype = 511, 8160, 32640, torch.bfloat16
+    say("in_linear_silu_backward largest", m, k, n)
+    g = torch.Generator(device="cuda").manual_seed(0)
+    sp = [n // 4] * 4
+    grads = [torch.rand(m, s_, generator=g, device="cuda").to(dtype) for s_ in sp]
+    u = lambda *s: (torch.rand(*s, generator=g, device="cuda") * 2 - 1).to(dtype)
+    x, w, lin = u(m, k), u(n, k), u(m, n)
+    bias = torch.zeros(n, device="cuda")
+    got = torch.ops.mxrec.in_linear_silu_backward(x, w, bias, *grads, lin, sp)
+    torch.cuda.synchronize()
+    z = lin.float()
+    sg = torch.sigmoid(z)
+    dlin = torch.cat(grads, dim=-1).float() * (sg * (1 + z * (1 - sg)))
+    want_b = dlin.sum(dim=0)
+    dl = dlin.to(dtype).float()
+    prev = torch.backends.cuda.matmul.allow_tf32
+    torch.backends.cuda.matmul.allow_tf32 = False
+    try:
+        want_x, want_w = dl @ w.float(), dl.t() @ x.float()
+    finally:
+        torch.backends.cuda.matmul.allow_tf32 = prev
+    for name, a, wnt, f32 in (("x_grad", got[0], want_x, False), ("weight_grad", got[1], want_w, False), ("bias_grad", got[2], want_b, True)):
+        a, wnt = a.double(), wnt.double()
+        scale = float(wnt.abs().max())
+        lim = (0.0 if f32 else 2.0 ** -8) * wnt.abs() * 1.001 + 2e-4 * scale
+        d = (a - wnt).abs()
+        assert bool((d <= lim).all()), f"{name}: worst {float((d / lim).max()):.2f} x the limit, scale {scale:.3e}"
