@@ -136,7 +136,7 @@ class HstuInLinearSiluParams(C.Structure):
 class HstuInLinearSiluBwdParams(C.Structure):
     _fields_ = [
         ("struct_size", C.c_uint32), ("dtype", C.c_int32), ("m", C.c_int64), ("k", C.c_int32), ("n", C.c_int32),
-        ("split", C.c_int32 * 4), ("grad_dtype", C.c_int32), ("reserved", C.c_int32),
+        ("split", C.c_int32 * 4), ("grad_dtype", C.c_int32), ("algorithm", C.c_int32),
         ("x", C.c_void_p), ("weight", C.c_void_p), ("grad", C.c_void_p * 4), ("linear_output", C.c_void_p),
         ("x_grad", C.c_void_p), ("weight_grad", C.c_void_p), ("bias_grad", C.c_void_p),
     ]

@@ -223,24 +223,30 @@ __global__ __launch_bounds__(ILB_NT) void hstu_ilb_xgrad_kernel(const IlbArgs a)
 }
 
 // weight_grad and bias_grad partial sums.  grid = (ceil(n / 256), ceil(k / KC), S), 4 waves of 64 columns n each.
-template <typename T, int KC>
+// FUSED (k <= 64 only, on request: it halves the HBM traffic but measured no faster, the two workgroup barriers per
+// tile and 171 registers cost what the second pass over the inputs costs): the parked tile is also multiplied by the wave's 64 rows of W, which stay in registers; the
+// four waves' products meet in LDS and leave as this workgroup's partial x_grad of the tile (one slab per 256 columns
+// of n, added up by hstu_ilb_reduce_kernel), so that the gradients and linear_output are streamed once instead of twice.
+template <typename T, int KC, bool FUSED>
 __global__ __launch_bounds__(ILB_NT) void hstu_ilb_wgrad_kernel(const IlbArgs a) {
     typedef typename IlbMM<T>::v8 v8;
     constexpr int KB = KC / 32;
     __shared__ __attribute__((aligned(16))) char park_all[(ILB_NT / 64) * 32 * ILB_PARK];
+    __shared__ float red[FUSED ? 4 : 1][FUSED ? 32 : 1][KC + 1];
     const hstu_in_linear_silu_bwd_params& p = a.p;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int g = lane >> 5, l32 = lane & 31;
     const int N = p.n, K = p.k;
     const int nw = blockIdx.x * 256 + 64 * w;     // first column of this wave
-    if (nw >= N) return;                          // whole wave; nothing below synchronises across waves
+    const bool wave_on = nw < N;
+    if (!FUSED && !wave_on) return;               // whole wave; without FUSED nothing below synchronises across waves
     const int k0 = blockIdx.y * KC;
     const int64_t mbeg = (int64_t)blockIdx.z * a.rows_per_part;
     const int64_t mend = mbeg + a.rows_per_part < p.m ? mbeg + a.rows_per_part : p.m;
     // load phase: lane = 8 consecutive columns (chunk) of the rows lrow, lrow + 8, lrow + 16, lrow + 24 of a tile
     const int chunk = lane & 7, lrow = lane >> 3;
     const int ncol = nw + 8 * chunk;
-    const bool live = ncol < N;
+    const bool live = wave_on && ncol < N;
     const int ncl = live ? ncol : 0;
     int sel = 0;
 #pragma unroll
@@ -275,6 +281,15 @@ __global__ __launch_bounds__(ILB_NT) void hstu_ilb_wgrad_kernel(const IlbArgs a)
             lf[i] = *reinterpret_cast<const v8*>(lptr + rc * N);
         }
     };
+    v8 wf[FUSED ? 4 : 1][KB];   // FUSED: W^T, columns nw + 16 s + 8 g .. + 7 (a step past n repeats the last one against zeros)
+    if constexpr (FUSED) {
+#pragma unroll
+        for (int s = 0; s < 4; s++)
+#pragma unroll
+            for (int kb = 0; kb < KB; kb++)
+                wf[s][kb] = *reinterpret_cast<const v8*>(reinterpret_cast<const T*>(a.wt) +
+                                                         (((int64_t)min(nw / 16 + s, N / 16 - 1) * a.kbt + min(kb, a.kbt - 1)) * 64 + lane) * 8);
+    }
     v8 gf[4], lf[4];
     fetch(mbeg, gf, lf);
     for (int64_t m0 = mbeg; m0 < mend; m0 += 32) {
@@ -313,6 +328,32 @@ __global__ __launch_bounds__(ILB_NT) void hstu_ilb_wgrad_kernel(const IlbArgs a)
 #pragma unroll
                 for (int kb = 0; kb < KB; kb++) acc[nb][kb] = IlbMM<T>::mfma(af, xf[ks][kb], acc[nb][kb]);
             }
+        }
+        if constexpr (FUSED) {
+            ilb_f32x16 ax[KB];
+#pragma unroll
+            for (int kb = 0; kb < KB; kb++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) ax[kb][r] = 0.f;
+#pragma unroll
+            for (int s = 0; s < 4; s++) {
+                // row m0 + l32 of dlin, columns nw + 16 s + 8 g .. + 7
+                const v8 bf = *reinterpret_cast<const v8*>(park + l32 * ILB_PARK + (16 * s + 8 * g) * 2);
+#pragma unroll
+                for (int kb = 0; kb < KB; kb++) ax[kb] = IlbMM<T>::mfma(wf[s][kb], bf, ax[kb]);
+            }
+            // register r of block kb: column 32 kb + 8 (r / 4) + 4 g + r % 4 of row m0 + l32
+#pragma unroll
+            for (int kb = 0; kb < KB; kb++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) red[w][l32][32 * kb + 8 * (r / 4) + 4 * g + (r % 4)] = ax[kb][r];
+            __syncthreads();
+            float* xp = a.xpart + ((int64_t)blockIdx.x * p.m + m0) * K;
+            for (int i = threadIdx.x; i < 32 * KC; i += ILB_NT) {
+                const int r = i / KC, c = i % KC;
+                if (m0 + r < mend && c < K) xp[(int64_t)r * K + c] = ((red[0][r][c] + red[1][r][c]) + red[2][r][c]) + red[3][r][c];
+            }
+            __syncthreads();
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -370,6 +411,7 @@ struct IlbPlan {
     int kc;               // k columns per workgroup: 64 or 128
     int parts;
     int kbt, nparts, cols_per_part;
+    bool fused;
     int64_t rows_per_part, mpad;
     uint64_t off_xt, off_wt, off_wpart, off_bpart, off_xpart, total;
 };
@@ -405,8 +447,15 @@ static IlbPlan ilb_plan(const hstu_in_linear_silu_bwd_params* p) {
     if (nparts < 1) nparts = 1;
     pl.cols_per_part = (int)((rounds + nparts - 1) / nparts) * 256;
     pl.nparts = (p->n + pl.cols_per_part - 1) / pl.cols_per_part;
+    // on request (k <= 64): one pass over the inputs, x_grad as one partial slab per 256 columns of n
+    const uint64_t slabs = (uint64_t)rounds;
+    pl.fused = p->algorithm == 2;
+    if (pl.fused) {
+        pl.nparts = (int)slabs;
+        pl.cols_per_part = 256;
+    }
     pl.off_xpart = o;
-    if (pl.nparts > 1) o = ilb_align(o + (uint64_t)pl.nparts * p->m * p->k * 4);
+    if (pl.nparts > 1 || pl.fused) o = ilb_align(o + (uint64_t)pl.nparts * p->m * p->k * 4);
     pl.total = o;
     return pl;
 }
@@ -429,6 +478,8 @@ static int ilb_check(const hstu_in_linear_silu_bwd_params* p) {
     if (p->n < 64 || p->n > 32768 || p->n % 16) return fail(HSTU_ERR_INVALID_ARGUMENT, "weight dim[0] must in range[64, 32768] and multiples of 16.");
     if (total != p->n) return fail(HSTU_ERR_INVALID_ARGUMENT, "weight_dim[0] must equal to sum(splitList).");
     if (p->n % (4 * p->k)) return fail(HSTU_ERR_INVALID_ARGUMENT, "weight dim[0] must be a multiple of 4 x dim[1]");
+    if (p->algorithm < 0 || p->algorithm > 2) return fail(HSTU_ERR_INVALID_ARGUMENT, "algorithm expect 0, 1 or 2, but value is %d", p->algorithm);
+    if (p->algorithm == 2 && p->k > 64) return fail(HSTU_ERR_INVALID_ARGUMENT, "algorithm 2 (one pass) needs x dim[1] <= 64, but got %d", p->k);
     return HSTU_OK;
 }
 
@@ -454,14 +505,16 @@ static void ilb_launch(const IlbArgs& a, const IlbPlan& pl, hipStream_t st) {
                        p.k, pl.kbt, xunits, reinterpret_cast<uint16_t*>(const_cast<void*>(a.xt)));
     const unsigned kchunks = (unsigned)((p.k + pl.kc - 1) / pl.kc);
     const dim3 gx((unsigned)(pl.mpad / 32), kchunks, (unsigned)pl.nparts), gw((unsigned)((p.n + 255) / 256), kchunks, (unsigned)pl.parts);
-    if (pl.kc == 64) {
+    if (pl.fused) {
+        hipLaunchKernelGGL((hstu_ilb_wgrad_kernel<T, 64, true>), gw, dim3(ILB_NT), 0, st, a);
+    } else if (pl.kc == 64) {
         hipLaunchKernelGGL((hstu_ilb_xgrad_kernel<T, 64>), gx, dim3(ILB_NT), 0, st, a);
-        hipLaunchKernelGGL((hstu_ilb_wgrad_kernel<T, 64>), gw, dim3(ILB_NT), 0, st, a);
+        hipLaunchKernelGGL((hstu_ilb_wgrad_kernel<T, 64, false>), gw, dim3(ILB_NT), 0, st, a);
     } else {
         hipLaunchKernelGGL((hstu_ilb_xgrad_kernel<T, 128>), gx, dim3(ILB_NT), 0, st, a);
-        hipLaunchKernelGGL((hstu_ilb_wgrad_kernel<T, 128>), gw, dim3(ILB_NT), 0, st, a);
+        hipLaunchKernelGGL((hstu_ilb_wgrad_kernel<T, 128, false>), gw, dim3(ILB_NT), 0, st, a);
     }
-    if (pl.nparts > 1) {
+    if (pl.nparts > 1 || pl.fused) {
         const int64_t cx = p.m * p.k;
         hipLaunchKernelGGL(hstu_ilb_reduce_kernel<T>, dim3((unsigned)((cx / 4 + 255) / 256)), dim3(256), 0, st, a.xpart, pl.nparts, cx, p.x_grad,
                            (int)(p.grad_dtype == HSTU_F32));

@@ -122,7 +122,7 @@ def test_in_linear_silu_backward_validation_and_workspace():
                        (dict(split=[16, 16, 32, 32]), "weight_dim[0] must equal to sum(splitList)"), (dict(k=24), "x dim[1] must in range"),
                        (dict(k=32), "weight dim[0] must be a multiple of 4 x dim[1]"), (dict(dtype=_capi.HSTU_F32), "dtype expect float16 or bfloat16"),
                        (dict(grad_dtype=_capi.HSTU_F16), "grad_dtype expect float32 or the dtype of x"), (dict(m=0), "x dim[0] must in range"),
-                       (dict(x_grad=None), "must not be NULL")):
+                       (dict(algorithm=3), "algorithm expect 0, 1 or 2"), (dict(algorithm=2, k=128, n=512, split=[128] * 4), "needs x dim[1] <= 64"), (dict(x_grad=None), "must not be NULL")):
         rc, msg = call(**over)
         assert rc == -1 and text in msg, (over, msg)
     rc, msg = call(bias_grad=0x1004)
@@ -139,8 +139,11 @@ def test_in_linear_silu_backward_validation_and_workspace():
     assert need.value == al(128 // 16 * 1024) + al(64 // 16 * 1024) + al(parts * 64 * 16 * 4) + al(parts * 64 * 4)
     big = mk(m=16384, k=64, n=16384, split=[4096] * 4)
     assert L.hstu_hip_in_linear_silu_backward_get_workspace_size(C.byref(big), C.byref(need)) == 0
-    # 16 ranges of m for weight_grad, 2 ranges of n for x_grad
+    # 16 ranges of m for weight_grad; x_grad: 2 ranges of n with the two product kernels, 64 slabs in one pass
     assert need.value == al(64 * 16384 * 2) * 2 + al(16 * 16384 * 64 * 4) + al(16 * 16384 * 4) + al(2 * 16384 * 64 * 4)
+    big.algorithm = 2
+    assert L.hstu_hip_in_linear_silu_backward_get_workspace_size(C.byref(big), C.byref(need)) == 0
+    assert need.value == al(64 * 16384 * 2) * 2 + al(16 * 16384 * 64 * 4) + al(16 * 16384 * 4) + al(64 * 16384 * 64 * 4)
     m = torch.ops.mxrec
     assert str(m.in_linear_silu.default._schema) == "mxrec::in_linear_silu(Tensor x, Tensor weight, Tensor bias, int[] attr_dict) -> Tensor[]"
     assert str(m.in_linear_silu_backward.default._schema) == ("mxrec::in_linear_silu_backward(Tensor x, Tensor weight, Tensor? bias, Tensor user_grad, "

@@ -280,3 +280,49 @@ def test_in_linear_silu_backward_largest_reference_shape():
         lim = (0.0 if f32 else 2.0 ** -8) * wnt.abs() * 1.001 + 2e-4 * scale
         d = (a - wnt).abs()
         assert bool((d <= lim).all()), f"{name}: worst {float((d / lim).max()):.2f} x the limit, scale {scale:.3e}"
+
+
+def _ilb_capi(grads, x, w, lin, sp, algorithm, dtype_code):
+    import ctypes as C
+    from recsdk_amd import _capi
+    m, k, n = x.shape[0], x.shape[1], w.shape[0]
+    dev = [t.cuda() for t in grads]
+    xd, wd, ld = x.cuda(), w.cuda(), lin.cuda()
+    xg = torch.full((m, k), float("nan"), device="cuda")
+    wg = torch.full((n, k), float("nan"), device="cuda")
+    bg = torch.full((n,), float("nan"), device="cuda")
+    L = _capi.lib()
+    p = _capi.HstuInLinearSiluBwdParams()
+    p.struct_size = C.sizeof(p)
+    p.dtype, p.grad_dtype, p.m, p.k, p.n, p.algorithm = dtype_code, _capi.HSTU_F32, m, k, n, algorithm
+    for i in range(4):
+        p.split[i] = sp[i]
+        p.grad[i] = dev[i].data_ptr()
+    p.x, p.weight, p.linear_output = xd.data_ptr(), wd.data_ptr(), ld.data_ptr()
+    p.x_grad, p.weight_grad, p.bias_grad = xg.data_ptr(), wg.data_ptr(), bg.data_ptr()
+    need = C.c_uint64(0)
+    assert L.hstu_hip_in_linear_silu_backward_get_workspace_size(C.byref(p), C.byref(need)) == 0
+    ws = torch.empty(need.value, dtype=torch.uint8, device="cuda")
+    rc = L.hstu_hip_in_linear_silu_backward(C.byref(p), ws.data_ptr(), need.value, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, L.hstu_hip_last_error().decode()
+    torch.cuda.synchronize()
+    return xg.cpu(), wg.cpu(), bg.cpu()
+
+
+@pytest.mark.parametrize("m,k,n,diff", [(1123, 64, 512, True), (2048, 32, 1152, False), (77, 16, 64, False)])
+def test_in_linear_silu_backward_one_pass_against_two_product_kernels(m, k, n, diff):
+    """`algorithm` = 2 runs one pass over the inputs (x_grad as partial slabs per 256 columns of n) instead of the two
+    product kernels.  Same roundings, different order of the fp32 sums: both against the oracle, and against each other
+    to the accumulation error alone; weight_grad and bias_grad (same code) bit for bit."""
+    from recsdk_amd import _capi
+    say("in_linear_silu_backward one pass vs two", m, k, n, diff)
+    dtype = torch.bfloat16
+    grads, x, w, lin, bias, sp = _ilb_inputs(m, k, n, dtype, diff)
+    one = _ilb_capi(grads, x, w, lin, sp, 2, _capi.HSTU_BF16)
+    two = _ilb_capi(grads, x, w, lin, sp, 0, _capi.HSTU_BF16)
+    want = LO.in_linear_silu_backward(grads, x, w, lin)
+    for name, a, b, wnt in zip(("x_grad", "weight_grad", "bias_grad"), one, two, want):
+        _ilb_close(a, wnt, dtype, name + " (one pass)", f32=True)
+        _ilb_close(b, wnt, dtype, name + " (two kernels)", f32=True)
+    assert torch.equal(one[1], two[1]) and torch.equal(one[2], two[2])
+    assert float((one[0] - two[0]).abs().max()) <= 1e-5 * float(want[0].abs().max())
