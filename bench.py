@@ -63,8 +63,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
-        raise SystemExit("bench.py: this build runs on ONE GPU (the path is single-device; see DESIGN.md for how it "
-                         "would shard). Run with --gpus 1.")
+        raise SystemExit("bench.py: this build runs on ONE GPU: (sequence, head) work units are independent, so several GPUs "
+                         "would each take a share of the sequences with no exchange between them. Run with --gpus 1.")
     import torch
     import recsdk_amd  # noqa: F401  (fails loudly if the HIP libraries are missing)
     from recsdk_amd import _capi, workloads as W
