@@ -105,7 +105,8 @@ def test_dropout_under_the_mask_the_op_returns(dim1, dtype, ratio):
 @pytest.mark.parametrize("m,n,k,split,dtype", [
     (2789, 9216, 64, None, torch.bfloat16), (256, 1024, 16, None, torch.float16), (2561, 1024, 128, "diff", torch.bfloat16),
     (512, 4096, 32, None, torch.float16), (1000, 9216, 48, "diff", torch.float16), (100, 64, 16, None, torch.bfloat16),
-    (129, 2048, 256, "diff", torch.bfloat16), (33, 192, 48, None, torch.float16)])
+    (129, 2048, 256, "diff", torch.bfloat16), (33, 192, 48, None, torch.float16), (300, 3072, 768, None, torch.bfloat16),
+    (65, 960, 240, "diff", torch.float16)])
 def test_in_linear_silu_forward(m, n, k, split, dtype):
     """The reference's generators (test_in_linear_silu.py:70-99): integer x in [-100, 100], Xavier-uniform W, bias of ones;
     equal splits or (s - 16, s - 16, s + 16, s + 16).  Against the oracle's exactly rounded values the fp32 accumulation
