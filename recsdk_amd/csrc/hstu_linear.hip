@@ -3,9 +3,9 @@
 // (thousands), so at 2 * k FLOPs per output element against 4 bytes written the op is bounded by the HBM writes of
 // its two [m, n] results, not by the matrix cores: the kernel is an MFMA GEMM without any pipelining of the k loop,
 // built around its stores.
-//   workgroup = 128 rows m x 64 columns n; wave w = rows 32 w .. 32 w + 31, all 64 columns (two 32 x 32 blocks: at 73
-//   registers and 4.5 KiB of LDS per wave six waves share a SIMD, which is what keeps the stores flowing; four blocks
-//   per wave measured 9 % slower, one block 23 % slower)
+//   workgroup = 64 rows m x 128 columns n as 2 x 2 waves; a wave = 32 rows x 64 columns (two 32 x 32 blocks: at 74
+//   registers and 6.75 KiB of LDS per wave five waves share a SIMD, which is what keeps the stores flowing; four blocks
+//   per wave measured 9 % slower, one block 23 % slower; 4 x 1 waves the same, 1 x 4 waves 8 % slower)
 //   out^T block = W x^T: v_mfma_f32_32x32x16 with A = W fragment, B = x fragment; both operands are staged through LDS
 //   64 columns of k at a time (loads of 128 contiguous bytes per row; a fragment is one 16-byte LDS read)
 //   epilogue: + bias, round -> linear_output; silu of the rounded value, round -> the four outputs; both leave through
@@ -38,10 +38,12 @@ template <> struct IlsMM<_Float16> {
 };
 
 constexpr int ILS_NB = 2;                                   // 32 x 32 blocks side by side per wave
-constexpr int ILS_BM = 128, ILS_BN = 32 * ILS_NB, ILS_NT = 256;
-constexpr int ILS_LPR = ILS_BN / 8, ILS_RPI = 64 / ILS_LPR;   // store phase: lanes per row, rows per instruction
+constexpr int ILS_WCOLS = 32 * ILS_NB;                      // columns of a wave
+constexpr int ILS_WN = 2, ILS_WM = 4 / ILS_WN;              // waves of a workgroup along n and along m
+constexpr int ILS_BM = 32 * ILS_WM, ILS_BN = ILS_WCOLS * ILS_WN, ILS_NT = 256;
+constexpr int ILS_LPR = ILS_WCOLS / 8, ILS_RPI = 64 / ILS_LPR;   // store phase: lanes per row, rows per instruction
 constexpr int ILS_KC = 64, ILS_SROW = ILS_KC * 2 + 16;   // k columns per staging round; bytes of one staged operand row
-constexpr int ILS_ROW = ILS_BN * 2 + 16;   // bytes of one parked row: + 16 keeps the 8-byte column writes of 32 rows off one bank
+constexpr int ILS_ROW = ILS_WCOLS * 2 + 16;   // bytes of one parked row: + 16 keeps the 8-byte column writes of 32 rows off one bank
 
 struct IlsArgs {
     hstu_in_linear_silu_params p;
@@ -53,7 +55,7 @@ __global__ __launch_bounds__(ILS_NT) void hstu_in_linear_silu_kernel(const IlsAr
     typedef typename IlsMM<T>::v8 v8;
     // operand staging of the k loop (x rows of the four waves, then the W rows they share) and, after it, the parked
     // output tiles of the epilogue share one buffer
-    static_assert(ILS_SROW == ILS_ROW, "a wave's parked tile takes the place of its staged x rows");
+    static_assert(4 * 32 * ILS_ROW <= (ILS_BM + ILS_BN) * ILS_SROW, "the four parked tiles fit into the staging buffer");
     __shared__ __attribute__((aligned(16))) char park_all[(ILS_BM + ILS_BN) * ILS_SROW];
     const hstu_in_linear_silu_params& p = a.p;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
@@ -72,8 +74,9 @@ __global__ __launch_bounds__(ILS_NT) void hstu_in_linear_silu_kernel(const IlsAr
         tn = blockIdx.x % nt;
         tm = blockIdx.x / nt;
     }
-    const int n0 = tn * ILS_BN;
-    const int64_t m0 = (int64_t)tm * ILS_BM + 32 * w;
+    const int wn = w % ILS_WN, wm = w / ILS_WN;
+    const int n0 = tn * ILS_BN + ILS_WCOLS * wn;          // first column and row of this wave
+    const int64_t m0 = (int64_t)tm * ILS_BM + 32 * wm;
     const T* x = reinterpret_cast<const T*>(p.x);
     const T* wt = reinterpret_cast<const T*>(p.weight);
     ils_f32x16 acc[ILS_NB];
@@ -81,38 +84,44 @@ __global__ __launch_bounds__(ILS_NT) void hstu_in_linear_silu_kernel(const IlsAr
     for (int nb = 0; nb < ILS_NB; nb++)
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[nb][r] = 0.f;
-    // Operands come in through LDS: eight lanes read 128 contiguous bytes of a row (x and W are k-contiguous), a wave
-    // its own 32 rows of x and a quarter of the 64 rows of W that the four waves share; an MFMA fragment is then one
+    // Operands come in through LDS: eight lanes read 128 contiguous bytes of a row (x and W are k-contiguous), each wave
+    // a quarter of the workgroup's rows of x and of W; an MFMA fragment is then one
     // 16-byte LDS read (row stride 144 bytes: conflict-free).  Rows past the end repeat the last one (never stored),
     // columns past k are zero.
     {
         const int chunk = lane & 7, lrow = lane >> 3;
-        char* xs = park_all + w * (32 * ILS_SROW);
+        constexpr int XR = ILS_BM / 4, WR = ILS_BN / 4;   // rows of x and of W that one wave brings in
+        char* xsh = park_all;
         char* wsh = park_all + ILS_BM * ILS_SROW;
-        const T* xsrc[4];
-        const T* wsrc[2];
+        const int64_t mt = (int64_t)tm * ILS_BM;
+        const int ntile = tn * ILS_BN;
+        const T* xsrc[XR / 8];
+        const T* wsrc[WR / 8];
 #pragma unroll
-        for (int i = 0; i < 4; i++) xsrc[i] = x + (m0 + lrow + 8 * i < p.m ? m0 + lrow + 8 * i : p.m - 1) * K + 8 * chunk;
+        for (int i = 0; i < XR / 8; i++) {
+            const int64_t r = mt + XR * w + lrow + 8 * i;
+            xsrc[i] = x + (r < p.m ? r : p.m - 1) * K + 8 * chunk;
+        }
 #pragma unroll
-        for (int i = 0; i < 2; i++) wsrc[i] = wt + (int64_t)min(n0 + 16 * w + lrow + 8 * i, N - 1) * K + 8 * chunk;
+        for (int i = 0; i < WR / 8; i++) wsrc[i] = wt + (int64_t)min(ntile + WR * w + lrow + 8 * i, N - 1) * K + 8 * chunk;
         for (int k0 = 0; k0 < K; k0 += ILS_KC) {
             const bool in = k0 + 8 * chunk < K;
-            v8 xv[4], wv[2];
+            v8 xv[XR / 8], wv[WR / 8];
 #pragma unroll
-            for (int i = 0; i < 4; i++) xv[i] = in ? *reinterpret_cast<const v8*>(xsrc[i] + k0) : v8{};
+            for (int i = 0; i < XR / 8; i++) xv[i] = in ? *reinterpret_cast<const v8*>(xsrc[i] + k0) : v8{};
 #pragma unroll
-            for (int i = 0; i < 2; i++) wv[i] = in ? *reinterpret_cast<const v8*>(wsrc[i] + k0) : v8{};
+            for (int i = 0; i < WR / 8; i++) wv[i] = in ? *reinterpret_cast<const v8*>(wsrc[i] + k0) : v8{};
 #pragma unroll
-            for (int i = 0; i < 4; i++) *reinterpret_cast<v8*>(xs + (lrow + 8 * i) * ILS_SROW + chunk * 16) = xv[i];
+            for (int i = 0; i < XR / 8; i++) *reinterpret_cast<v8*>(xsh + (XR * w + lrow + 8 * i) * ILS_SROW + chunk * 16) = xv[i];
 #pragma unroll
-            for (int i = 0; i < 2; i++) *reinterpret_cast<v8*>(wsh + (16 * w + lrow + 8 * i) * ILS_SROW + chunk * 16) = wv[i];
+            for (int i = 0; i < WR / 8; i++) *reinterpret_cast<v8*>(wsh + (WR * w + lrow + 8 * i) * ILS_SROW + chunk * 16) = wv[i];
             __syncthreads();
 #pragma unroll
             for (int s = 0; s < ILS_KC / 16; s++) {
-                const v8 xf = *reinterpret_cast<const v8*>(xs + l32 * ILS_SROW + (16 * s + 8 * g) * 2);
+                const v8 xf = *reinterpret_cast<const v8*>(xsh + (32 * wm + l32) * ILS_SROW + (16 * s + 8 * g) * 2);
 #pragma unroll
                 for (int nb = 0; nb < ILS_NB; nb++) {
-                    const v8 wf = *reinterpret_cast<const v8*>(wsh + (32 * nb + l32) * ILS_SROW + (16 * s + 8 * g) * 2);
+                    const v8 wf = *reinterpret_cast<const v8*>(wsh + (ILS_WCOLS * wn + 32 * nb + l32) * ILS_SROW + (16 * s + 8 * g) * 2);
                     acc[nb] = IlsMM<T>::mfma(wf, xf, acc[nb]);
                 }
             }
