@@ -349,8 +349,6 @@ def bias_bench(args, torch):
     """The standalone bias producers at the reference's evaluation shape (test_relative_attn_bias.py:106-113): 8 layers,
     train_len 2000 + 600 candidates -> s = 2300, 4 users, fp16 tables, int32 timestamps.  HBM-bound: the (2s)^2 outputs
     (the gradient input for the backward) dominate the bytes."""
-    import torch.nn.functional as F  # noqa: F401
-    from oracle import bias_oracle as BO
     n, bs, train, cand = 8, 4, 2000, 600
     s = train + cand // 2
     g = torch.Generator().manual_seed(0)
@@ -373,8 +371,9 @@ def bias_bench(args, torch):
         sample = "the whole call once (oracle in torch)"
     elif args.workload == "rab_time_bwd":
         grad = (torch.randn(n, bs, 2 * s, 2 * s, generator=g, dtype=torch.float16) * 1e-2).cuda()
-        ids = BO.time_buckets(ts).to(torch.int32)
-        idd = ids.cuda()
+        # the bucket ids the backward consumes come from this library's forward
+        idd = m.relative_attn_bias_time_with_index(ts.cuda(), w.cuda(), 0.301)[1].to(torch.int32)
+        ids = idd.cpu()
         fn = lambda: m.relative_attn_bias_time_backward(grad, idd, 129)
         alg = n * bs * 4 * s * s * esz + bs * s * s * 4
         kernel, desc = "hstu_rab_time_bwd_kernel", "grad [8,4,4600,4600] fp16 and ids [4,2300,2300] int32 read (algorithmic: once each)"
@@ -418,6 +417,7 @@ def bias_bench(args, torch):
                      "kernel_us": round(kern_ms * 1e3, 2)},
     }
     if not args.no_cpu_baseline:
+        from oracle import bias_oracle as BO
         t0 = time.perf_counter()
         cpu()
         dt = time.perf_counter() - t0
@@ -430,7 +430,6 @@ def nmd_bench(args, torch):
     """norm_multiply_dropout at the shape of the reference's sample (README of the op: 262144 x 512, bf16, eps 1e-5), with
     dropout 0.3 so that the mask is written and read.  HBM-bound: forward reads x, u and writes y (+ mask, mean, var);
     backward reads d_out, x, u (+ mask, mean, var) and writes d_x, d_u."""
-    from oracle import layer_oracle as LO
     rows, cols, ratio, eps = 262144, 512, 0.3, 1e-5
     g = torch.Generator().manual_seed(321)
     mk = lambda *s: (torch.rand(*s, generator=g) * 2 - 1).to(torch.bfloat16)
@@ -477,6 +476,7 @@ def nmd_bench(args, torch):
                      "kernel_us": round(kern_ms * 1e3, 2)},
     }
     if not args.no_cpu_baseline:
+        from oracle import layer_oracle as LO
         t0 = time.perf_counter()
         cpu()
         dt = time.perf_counter() - t0
@@ -489,7 +489,6 @@ def in_linear_silu_bench(args, torch):
     """The input projection at the largest shape of the reference's tests (test_in_linear_silu.py:101-109): m = 16384,
     n = 16384, k = 64, bf16, equal splits.  4 bytes written per output element against 2 k = 128 FLOPs: bounded by the HBM
     writes of linear_output and the four split outputs."""
-    from oracle import layer_oracle as LO
     m_, n, k = 16384, 16384, 64
     g = torch.Generator().manual_seed(13)
     x = torch.randint(-100, 101, (m_, k), generator=g).to(torch.bfloat16)
@@ -524,6 +523,7 @@ def in_linear_silu_bench(args, torch):
                      "kernel_us": round(kern_ms * 1e3, 2)},
     }
     if not args.no_cpu_baseline:
+        from oracle import layer_oracle as LO
         rows = 4096
         t0 = time.perf_counter()
         LO.in_linear_silu(x[:rows], w, bias, sp)
@@ -539,7 +539,6 @@ def in_linear_silu_bwd_bench(args, torch):
     read once (2 m n esize), x and W read, x_grad, weight_grad and bias_grad written."""
     import ctypes as C
     from recsdk_amd import _capi
-    from oracle import layer_oracle as LO
     m_, n, k = 16384, 16384, 64
     g = torch.Generator().manual_seed(13)
     sp = [n // 4] * 4
@@ -594,6 +593,7 @@ def in_linear_silu_bwd_bench(args, torch):
                      "kernel_us": round(kern_ms * 1e3, 2)},
     }
     if not args.no_cpu_baseline:
+        from oracle import layer_oracle as LO
         rows = 2048
         t0 = time.perf_counter()
         LO.in_linear_silu_backward([t[:rows] for t in grads], x[:rows], w, lin[:rows])
