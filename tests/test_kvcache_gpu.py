@@ -212,3 +212,36 @@ def test_fp8_prefill_equals_whole_page_quantisation_and_feeds_paged_fp8():
     touched[c["kv_indices"].long()] = True
     assert torch.equal(sc.cpu()[touched], want_s[touched])
     assert torch.equal(cache8.cpu()[touched], want8.view(torch.uint8)[touched])
+
+
+def test_fp8_prefill_at_the_bench_shape_against_torch_on_the_gpu():
+    """Config 5's history (32 users x U[1024, 4096] tokens, 4 heads x 128, 64-token pages) is too long for the token loop
+    of the oracle; the prefill is checked through what it must equal: the 2-byte table written by the 2-byte append
+    (bit-exact against the oracle at smaller sizes), quantised page by page with torch's own GPU routines."""
+    say("kv append fp8 at the bench shape")
+    c = W.kv_append_config(0, users=32, heads=4, dim=128, prev_lo=0, prev_hi=0, new_lo=1024, new_hi=4096, page_size=64)
+    d = W.to_device(c)
+    n = c["nnz"]
+    bi = torch.empty(n, dtype=torch.int32, device="cuda")
+    pos = torch.empty_like(bi)
+    kvcache.get_paged_batch_indices_positions(d["append_indptr"], d["seq_lens"], bi, pos)
+    table = d["kv_cache"]
+    kc, vc = table.unbind(1)
+    kvcache.append_kvcache(d["append_key"], d["append_value"], bi, pos, d["offsets"], d["nnz_dev"], n, kc, vc, d["kv_indices"], d["kv_indptr"],
+                           d["kv_last_page_len"], 0)
+    cache8 = torch.zeros(table.shape, dtype=torch.uint8, device="cuda")
+    sc = torch.ones(table.shape[0], 2, table.shape[3], device="cuda")
+    kvcache.append_kvcache_fp8(d["append_key"], d["append_value"], bi, pos, d["offsets"], d["nnz_dev"], n, cache8, sc, d["kv_indices"], d["kv_indptr"])
+    torch.cuda.synchronize()
+    x = table.float()
+    amax = x.abs().amax(dim=(2, 4))
+    # tensor / tensor: torch divides for real there (a tensor over a Python number is multiplied by its rounded reciprocal)
+    want_s = torch.where(amax > 0, amax / torch.full_like(amax, 448.0), torch.ones_like(amax))
+    assert torch.equal(sc, want_s)
+    want8 = (x / want_s[:, :, None, :, None]).clamp(-448.0, 448.0).to(torch.float8_e4m3fn).view(torch.uint8)
+    diff = cache8 != want8
+    assert not bool(diff.any()), f"{int(diff.sum())} of {diff.numel()} bytes differ"
+    # and back: every stored value within the e4m3 step of the original
+    deq = cache8.view(torch.float8_e4m3fn).float() * sc[:, :, None, :, None]
+    lim = x.abs() * 2.0 ** -4 + sc[:, :, None, :, None] * 2.0 ** -10
+    assert bool(((deq - x).abs() <= lim * 1.001).all())

@@ -250,11 +250,13 @@ def test_in_linear_silu_autograd():
     _ilb_close(leaves[1].grad, want[1], dtype, "weight.grad")
 
 
-def test_in_linear_silu_backward_largest_reference_shape():
+@pytest.mark.parametrize("m,k,n", [(511, 8160, 32640), (16384, 64, 16384), (20480, 48, 9216)])
+def test_in_linear_silu_backward_largest_reference_shape(m, k, n):
     """k = 8160, n = 32640 at m = 511 (test_in_linear_silu_backward.py:169-176): 64 blocks of k per workgroup column, one
-    range of m.  Too large for the fp64 oracle in a test; checked against the same formula evaluated with torch's own
-    GPU routines in fp32 (sigmoid, rounding of dlin to bf16, two matrix products) -- a checker, not a code path of the op."""
-    m, k, n, dtype = 511, 8160, 32640, torch.bfloat16
+    range of m; the bench shape m = n = 16384, k = 64; the longest m of the reference's tests.  Too large for the fp64
+    oracle in a test; checked against the same formula evaluated with torch's own GPU routines in fp32 (sigmoid, rounding
+    of dlin to bf16, two matrix products) -- a checker, not a code path of the op."""
+    dtype = torch.bfloat16
     say("in_linear_silu_backward largest", m, k, n)
     g = torch.Generator(device="cuda").manual_seed(0)
     sp = [n // 4] * 4
@@ -327,3 +329,36 @@ def test_in_linear_silu_backward_one_pass_against_two_product_kernels(m, k, n, d
         _ilb_close(b, wnt, dtype, name + " (two kernels)", f32=True)
     assert torch.equal(one[1], two[1]) and torch.equal(one[2], two[2])
     assert float((one[0] - two[0]).abs().max()) <= 1e-5 * float(want[0].abs().max())
+
+
+@pytest.mark.parametrize("m,n,k", [(16384, 16384, 64), (20480, 9216, 48)])
+def test_in_linear_silu_forward_largest_reference_shapes(m, n, k):
+    """The largest shapes of the reference's forward tests (test_in_linear_silu.py:110-127), too large for the fp64 oracle
+    in a test: linear_output against torch's fp32 product on the GPU (one unit in the last place of bf16: the order of
+    the fp32 sums differs), the four outputs against SiLU of the linear_output the kernel itself wrote."""
+    dtype = torch.bfloat16
+    say("in_linear_silu forward largest", m, n, k)
+    g = torch.Generator(device="cuda").manual_seed(13)
+    x = torch.randint(-100, 101, (m, k), generator=g, device="cuda").to(dtype)
+    w = ((torch.rand(n, k, generator=g, device="cuda") * 2 - 1) * (6.0 / (n + k)) ** 0.5).to(dtype)
+    bias = torch.ones(n, device="cuda")
+    sp = [n // 4] * 4
+    got = torch.ops.mxrec.distance_in_linear_silu(x, w, bias, sp)
+    torch.cuda.synchronize()
+    prev = torch.backends.cuda.matmul.allow_tf32
+    torch.backends.cuda.matmul.allow_tf32 = False
+    try:
+        want = x.float() @ w.float().t() + bias
+    finally:
+        torch.backends.cuda.matmul.allow_tf32 = prev
+    lin = got[4].float()
+    acc_err = 2.0 ** -20 * float((x.float().abs() @ w.float().abs().t()).max())
+    d = (lin - want).abs()
+    lim = 2.0 ** -7 * want.abs().clamp(min=2.0 ** -14) * 1.001 + acc_err
+    assert bool((d <= lim).all()), f"linear_output: worst {float((d / lim).max()):.2f} x the limit"
+    del d, lim, want
+    act = torch.cat(got[:4], dim=-1).float()
+    ref = lin * torch.sigmoid(lin)
+    d = (act - ref).abs()
+    assert bool((d <= 2.0 ** -7 * ref.abs().clamp(min=2.0 ** -14) * 1.001).all()), "outputs: more than one unit in the last place of silu(linear_output)"
+    assert [t.shape[1] for t in got] == sp + [n]
