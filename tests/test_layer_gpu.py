@@ -362,3 +362,38 @@ def test_in_linear_silu_forward_largest_reference_shapes(m, n, k):
     d = (act - ref).abs()
     assert bool((d <= 2.0 ** -7 * ref.abs().clamp(min=2.0 ** -14) * 1.001).all()), "outputs: more than one unit in the last place of silu(linear_output)"
     assert [t.shape[1] for t in got] == sp + [n]
+
+
+def test_norm_multiply_dropout_at_the_bench_shape():
+    """262144 x 512 bf16 (the shape of the reference's sample), without dropout: forward against torch's own layer_norm
+    on the GPU in fp32, backward against autograd through it; with dropout 0.3: the kept fraction and that dropped
+    positions (read from the mask bits) are exactly zero in y and in d_u."""
+    import torch.nn.functional as F
+    rows, cols, dtype = 262144, 512, torch.bfloat16
+    say("nmd at the bench shape", rows, cols)
+    g = torch.Generator(device="cuda").manual_seed(321)
+    mk = lambda *s: (torch.rand(*s, generator=g, device="cuda") * 2 - 1).to(dtype)
+    x, u, w, b, dy = mk(rows, cols), mk(rows, cols), mk(cols), mk(cols), mk(rows, cols)
+    leaves = [t.clone().requires_grad_(True) for t in (x, u, w, b)]
+    y = torch.ops.mxrec.norm_multiply_dropout(*leaves, EPS, 0.0)[0]
+    y.backward(dy)
+    ref = [t.float().requires_grad_(True) for t in (x, u, w, b)]
+    yr = F.layer_norm(ref[0], (cols,), ref[2], ref[3], EPS) * ref[1]
+    yr.backward(dy.float())
+    assert torch.allclose(y.float(), yr, rtol=2e-2, atol=2e-2)
+    assert torch.allclose(leaves[0].grad.float(), ref[0].grad, rtol=2e-2, atol=2e-2)
+    assert torch.allclose(leaves[1].grad.float(), ref[1].grad, rtol=2e-2, atol=2e-2)
+    for a, r in ((leaves[2].grad, ref[2].grad), (leaves[3].grad, ref[3].grad)):   # sums over 262144 rows, handed over in bf16
+        assert float((a.float() - r).abs().max()) <= 1e-2 * float(r.abs().max())
+    del ref, yr
+    outs = torch.ops.mxrec.norm_multiply_dropout_forward(x, u, w, b, EPS, 0.3)
+    # bit e % 8 of mask byte e / 8 = element e kept
+    bits = (outs[3][: rows * cols // 8, None] >> torch.arange(8, device="cuda", dtype=torch.uint8)) & 1
+    keep = bits.reshape(rows, cols).bool()
+    assert abs(float(keep.float().mean()) - 0.7) < 2e-3
+    assert not bool(outs[0][~keep].any())
+    gr = torch.ops.mxrec.norm_multiply_dropout_backward(dy, x, u, w, b, outs[1], outs[2], outs[3], EPS, 0.3)
+    assert not bool(gr[1][~keep].any())
+    # kept elements are the undropped result scaled by 1 / (1 - p), up to the one rounding
+    y0 = torch.ops.mxrec.norm_multiply_dropout_forward(x, u, w, b, EPS, 0.0)[0]
+    assert torch.allclose(outs[0][keep].float(), y0[keep].float() / 0.7, rtol=2e-2, atol=2e-2)
