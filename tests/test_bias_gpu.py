@@ -147,3 +147,37 @@ def test_rab_time_feeds_hstu_jagged_as_attn_bias():
                                                        None, 0, L, L, 0.0, off.cuda(), off.cuda(), None, None, 0, 0.125, DIV)
     # the dense path rounds the bias to bf16 first, the fused path adds the fp32 table entry
     T.assert_parity(out_dense.cpu(), out_fused.cpu().double(), torch.bfloat16, what="dense bias from the producer vs fused table")
+
+
+def test_rab_time_at_the_evaluation_shape():
+    """8 layers, 4 users, s = 2300 (train 2000 + 600 candidates), fp16 (test_relative_attn_bias.py:106-113): too large for
+    the oracle's Python-side repeat in a test, so checked through what must hold at any size -- the output is the table
+    gathered at the returned ids and repeated 2 x 2, the ids are symmetric with a zero diagonal and equal the oracle's on
+    a slice; the weight gradient equals an index_add over the same ids (torch on the GPU, fp32)."""
+    say("rab_time at the evaluation shape")
+    n, bs, train, cand = 8, 4, 2000, 600
+    s = train + cand // 2
+    g = torch.Generator().manual_seed(0)
+    lens = torch.randint(0, train, (bs,), generator=g).tolist()
+    ts = _timestamps(train, cand, lens, torch.int32)
+    w = (torch.arange(NUM_BUCKETS + 1, dtype=torch.float32).repeat(n).reshape(n, -1) + torch.randn(n, NUM_BUCKETS + 1, generator=g)).half()
+    out, ids = torch.ops.mxrec.relative_attn_bias_time_with_index(ts.cuda(), w.cuda(), DIV)
+    assert out.shape == (n, bs, 2 * s, 2 * s) and ids.shape == (bs, s, s)
+    assert torch.equal(ids, ids.transpose(1, 2)) and not bool(torch.diagonal(ids, dim1=1, dim2=2).any())
+    assert int(ids.min()) >= 0 and int(ids.max()) <= NUM_BUCKETS
+    _, want_ids = BO.rab_time(ts[:1, :300], w[:1], DIV)
+    assert torch.equal(ids[:1, :300, :300].cpu(), want_ids)
+    wd = w.cuda()
+    for layer in range(n):
+        gathered = wd[layer][ids.long()]                                   # [bs, s, s]
+        for a in (0, 1):
+            for c in (0, 1):
+                assert torch.equal(out[layer, :, a::2, c::2], gathered)
+    grad = (torch.randn(n, bs, 2 * s, 2 * s, generator=g, dtype=torch.float16) * 1e-2).cuda()
+    gw = torch.ops.mxrec.relative_attn_bias_time_backward(grad, ids, NUM_BUCKETS + 1)
+    summed = (grad[:, :, 0::2, 0::2].float() + grad[:, :, 0::2, 1::2].float()) + (grad[:, :, 1::2, 0::2].float() + grad[:, :, 1::2, 1::2].float())
+    want = torch.zeros(n, NUM_BUCKETS + 1, device="cuda", dtype=torch.float64)
+    flat = ids.reshape(-1).long()
+    for layer in range(n):
+        want[layer].index_add_(0, flat, summed[layer].reshape(-1).double())
+    assert float((gw.double() - want).abs().max()) <= 1e-3 * float(want.abs().max())
