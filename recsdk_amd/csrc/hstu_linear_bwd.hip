@@ -151,8 +151,8 @@ __global__ __launch_bounds__(ILB_NT) void hstu_ilb_xgrad_kernel(const IlbArgs a)
             if (ncl >= a.base[i]) gwidth = a.p.split[i];
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            gf[i] = *reinterpret_cast<const v8*>(gp + rows[i] * gwidth);
-            lf[i] = *reinterpret_cast<const v8*>(lin + rows[i] * N + ncl);
+            gf[i] = __builtin_nontemporal_load(reinterpret_cast<const v8*>(gp + rows[i] * gwidth));
+            lf[i] = __builtin_nontemporal_load(reinterpret_cast<const v8*>(lin + rows[i] * N + ncl));
         }
     };
     v8 gf[4], lf[4];
@@ -277,8 +277,8 @@ __global__ __launch_bounds__(ILB_NT) void hstu_ilb_wgrad_kernel(const IlbArgs a)
         for (int i = 0; i < 4; i++) {
             const int64_t r = m0 + lrow + 8 * i;
             const int64_t rc = r < mend ? r : mend - 1;
-            gf[i] = *reinterpret_cast<const v8*>(gptr + rc * gwidth);
-            lf[i] = *reinterpret_cast<const v8*>(lptr + rc * N);
+            gf[i] = __builtin_nontemporal_load(reinterpret_cast<const v8*>(gptr + rc * gwidth));
+            lf[i] = __builtin_nontemporal_load(reinterpret_cast<const v8*>(lptr + rc * N));
         }
     };
     v8 wf[FUSED ? 4 : 1][KB];   // FUSED: W^T, columns nw + 16 s + 8 g .. + 7 (a step past n repeats the last one against zeros)
