@@ -23,7 +23,7 @@ PEAK_HBM_GBS = 8000.0
 # HBM-side bytes per launch from rocprofv3 FETCH_SIZE/WRITE_SIZE, each scaled by what the same counter reads for the
 # plain 256 MiB copy of `--workload copy` (factors 2.000 and 1.000); see profiles/*.md
 MEASURED_TRAFFIC_BYTES = {"config2": 184.3e6, "kv_append": 351.9e6, "rab_time": 1479.8e6, "rab_time_bwd": 2242.4e6, "rab_pos": 305.2e6,
-                          "nmd_fwd": 827.4e6, "nmd_bwd": 1382.0e6, "in_linear_silu": 1092.8e6, "in_linear_silu_bwd": 2405.4e6, "kv_append_fp8": 455.0e6}
+                          "nmd_fwd": 826.4e6, "nmd_bwd": 1380.0e6, "in_linear_silu": 1092.8e6, "in_linear_silu_bwd": 2405.4e6, "kv_append_fp8": 455.0e6}
 
 
 def build_workload(name, torch, W):
