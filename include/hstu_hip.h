@@ -143,6 +143,22 @@ typedef struct hstu_fwd_params {
 int hstu_hip_jagged_forward_get_workspace_size(const hstu_fwd_params* p, uint64_t* workspace_bytes);
 int hstu_hip_jagged_forward(const hstu_fwd_params* p, void* workspace, uint64_t workspace_bytes, void* stream);
 
+/*
+ * hstu_hip_jagged_forward for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and results as
+ * hstu_hip_jagged_forward without a workspace: the work list lives in a fixed array of HSTU_NOALLOC_SCRATCH_BYTES
+ * that the library holds in the memory of every GPU it runs on until the process ends.  The call allocates nothing
+ * (the first call on a GPU looks the array's address up once; make that call outside a capture).
+ *   - a batch whose work list does not fit is rejected with HSTU_ERR_WORKSPACE (the list takes about 64 bytes per
+ *     128-row Q tile and head: the array holds about 30 000 of them);
+ *   - every Q tile stays one work item (hstu_hip_jagged_forward splits the K range of serving-shaped batches and adds
+ *     the parts through its workspace), and HSTU_FLAG_REUSE_WORKSPACE is ignored: the list is rebuilt by every call;
+ *   - all calls on one GPU share the array: calls that overlap on one GPU (two streams, two threads) race.
+ *     Calls on one stream are ordered and safe.
+ */
+#define HSTU_NOALLOC_SCRATCH_BYTES (2u << 20)
+int hstu_hip_jagged_forward_noalloc(const hstu_fwd_params* p, void* stream);
+
 /* replaces aclnnHstuPagedForwardGetWorkspaceSize / aclnnHstuPagedForward (hstu_paged.cpp:67-69) */
 int hstu_hip_paged_forward_get_workspace_size(const hstu_fwd_params* p, uint64_t* workspace_bytes);
 int hstu_hip_paged_forward(const hstu_fwd_params* p, void* workspace, uint64_t workspace_bytes, void* stream);

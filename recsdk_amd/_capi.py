@@ -21,7 +21,7 @@ MASK_TRIL, MASK_TRIU, MASK_NONE, MASK_CUSTOM = 0, 1, 2, 3
 FLAG_DETERMINISTIC, FLAG_FORCE_GENERIC, FLAG_REUSE_WORKSPACE = 1, 2, 4
 
 EXPORTS = [
-    "hstu_hip_jagged_forward_get_workspace_size", "hstu_hip_jagged_forward",
+    "hstu_hip_jagged_forward_get_workspace_size", "hstu_hip_jagged_forward", "hstu_hip_jagged_forward_noalloc",
     "hstu_hip_paged_forward_get_workspace_size", "hstu_hip_paged_forward",
     "hstu_hip_dense_forward_get_workspace_size", "hstu_hip_dense_forward",
     "hstu_hip_jagged_backward_get_workspace_size", "hstu_hip_jagged_backward",
@@ -161,6 +161,7 @@ def lib() -> C.CDLL:
         for n in ("jagged", "paged", "dense"):
             getattr(_lib, f"hstu_hip_{n}_forward").argtypes = [C.POINTER(HstuFwdParams), C.c_void_p, C.c_uint64, C.c_void_p]
             getattr(_lib, f"hstu_hip_{n}_forward_get_workspace_size").argtypes = [C.POINTER(HstuFwdParams), C.POINTER(C.c_uint64)]
+        _lib.hstu_hip_jagged_forward_noalloc.argtypes = [C.POINTER(HstuFwdParams), C.c_void_p]
         for n in ("jagged", "dense"):
             getattr(_lib, f"hstu_hip_{n}_backward").argtypes = [C.POINTER(HstuBwdParams), C.c_void_p, C.c_uint64, C.c_void_p]
             getattr(_lib, f"hstu_hip_{n}_backward_get_workspace_size").argtypes = [C.POINTER(HstuBwdParams), C.POINTER(C.c_uint64)]
@@ -262,6 +263,14 @@ def run(op: str, params: HstuFwdParams, stream=None):
     ws = torch.empty(n.value, dtype=torch.uint8, device="cuda") if n.value else None
     _check(getattr(L, f"hstu_hip_{op}_forward")(C.byref(params), _ptr(ws), n.value, stream if stream is not None else _stream()))
     return ws
+
+
+def run_noalloc(params: HstuFwdParams, stream=None):
+    """The jagged forward through the entry point that allocates nothing (work list in the library's fixed array)."""
+    _check(lib().hstu_hip_jagged_forward_noalloc(C.byref(params), stream if stream is not None else _stream()))
+
+
+NOALLOC_SCRATCH_BYTES = 2 << 20
 
 
 def make_backward_params(fwd: HstuFwdParams, grad_out, grad_q, grad_k, grad_v, grad_bias=None) -> HstuBwdParams:

@@ -5,6 +5,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <string>
 
 #include "hstu_internal.h"
@@ -24,6 +25,31 @@ int fail(int code, const char* fmt, ...) {
 }
 
 static bool in_range(int64_t v, int64_t lo, int64_t hi) { return v >= lo && v <= hi; }
+
+// Work list of hstu_hip_jagged_forward_noalloc: a fixed array in every GPU's memory instead of a caller workspace.
+// Host code never uses the array's name as an address: scratch_of_current_device() asks the runtime for the
+// device address once per GPU and every launch gets that pointer.
+static __device__ __align__(256) unsigned char scratch[HSTU_NOALLOC_SCRATCH_BYTES];
+constexpr int MAX_DEVICES = 64;
+static void* g_scratch_ptr[MAX_DEVICES];
+static std::mutex g_scratch_mutex;
+
+static int scratch_of_current_device(void** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "hipGetDevice failed: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= MAX_DEVICES) return fail(HSTU_ERR_UNSUPPORTED, "device index %d outside [0, %d)", dev, MAX_DEVICES);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr)
+            return fail(HSTU_ERR_LAUNCH, "hipGetSymbolAddress(scratch) failed on device %d: %s", dev, hipGetErrorString(e));
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return HSTU_OK;
+}
 
 static int validate(const hstu_fwd_params* p, int op, KArgs* out, bool need_out = true) {
     if (!p) return fail(HSTU_ERR_INVALID_ARGUMENT, "params is NULL");
@@ -95,6 +121,7 @@ static int validate(const hstu_fwd_params* p, int op, KArgs* out, bool need_out 
     }
 
     out->p = *p;
+    out->p.flags &= HSTU_FLAG_DETERMINISTIC | HSTU_FLAG_FORCE_GENERIC | HSTU_FLAG_REUSE_WORKSPACE;   // the rest is the library's own
     out->op = op;
     out->head_ratio = p->heads_q / p->heads_k;
     out->out_scale = p->alpha * p->silu_scale;
@@ -165,6 +192,34 @@ extern "C" {
 
 int hstu_hip_jagged_forward_get_workspace_size(const hstu_fwd_params* p, uint64_t* b) { return ws_size(p, OP_JAGGED, b); }
 int hstu_hip_jagged_forward(const hstu_fwd_params* p, void* ws, uint64_t n, void* s) { return run(p, OP_JAGGED, ws, n, s); }
+
+int hstu_hip_jagged_forward_noalloc(const hstu_fwd_params* p, void* stream) {
+    KArgs a;
+    int rc = validate(p, OP_JAGGED, &a);
+    if (rc != HSTU_OK) return rc;
+    if (p->total_q == 0) return HSTU_OK;
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    const char* name = nullptr;
+    hipError_t e;
+    if (!(a.p.flags & HSTU_FLAG_FORCE_GENERIC) && mfma_supported(a, &name)) {
+        // whole Q tiles only (no partial sums of split K ranges, which would need a buffer that grows with the batch); the
+        // list is rebuilt by every call because the array is shared by all callers of this GPU
+        a.p.flags = (a.p.flags & ~HSTU_FLAG_REUSE_WORKSPACE) | FLAG_WHOLE_TILES;
+        const uint64_t need = mfma_workspace_bytes(a);
+        if (need > HSTU_NOALLOC_SCRATCH_BYTES)
+            return fail(HSTU_ERR_WORKSPACE, "the work list of this batch needs %llu bytes, hstu_hip_jagged_forward_noalloc holds %u: "
+                        "use hstu_hip_jagged_forward with a caller workspace", (unsigned long long)need, (unsigned)HSTU_NOALLOC_SCRATCH_BYTES);
+        void* ptr = nullptr;
+        rc = scratch_of_current_device(&ptr);
+        if (rc != HSTU_OK) return rc;
+        e = launch_mfma(a, ptr, st);
+    } else {
+        e = launch_generic(a, st);   // uses no device memory beyond its arguments
+    }
+    if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString(e));
+    return HSTU_OK;
+}
+
 int hstu_hip_paged_forward_get_workspace_size(const hstu_fwd_params* p, uint64_t* b) { return ws_size(p, OP_PAGED, b); }
 int hstu_hip_paged_forward(const hstu_fwd_params* p, void* ws, uint64_t n, void* s) { return run(p, OP_PAGED, ws, n, s); }
 int hstu_hip_dense_forward_get_workspace_size(const hstu_fwd_params* p, uint64_t* b) { return ws_size(p, OP_DENSE, b); }

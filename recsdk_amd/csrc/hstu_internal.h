@@ -10,6 +10,10 @@ namespace hstu {
 // records the message hstu_hip_last_error() returns to the calling thread; returns `code`
 int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 
+// private bit of hstu_fwd_params.flags inside the library (callers' copies of it are cleared): every Q tile stays one
+// item, no K ranges with partial sums
+constexpr uint32_t FLAG_WHOLE_TILES = 0x80000000u;
+
 enum OpKind : int32_t { OP_JAGGED = 0, OP_PAGED = 1, OP_DENSE = 2 };
 
 // Kernel argument block: the caller's parameters plus what the host derives from them.

@@ -186,7 +186,7 @@ static SchedDims sched_dims(const hstu_fwd_params& p, bool whole_tiles = false) 
     // they simply add up) go through the workspace and a small reduction kernel.
     d.nsplit = 1;
     const int ktiles = (p.max_seq_len_k + BN - 1) / BN;
-    if (!whole_tiles && d.bound < 384 && ktiles >= 16) {
+    if (!whole_tiles && !(p.flags & FLAG_WHOLE_TILES) && d.bound < 384 && ktiles >= 16) {
         int s = 768 / (int)(d.bound ? d.bound : 1);
         if (s > 4) s = 4;
         if (s > ktiles / 4) s = ktiles / 4;

@@ -56,6 +56,16 @@ def _ws(p, op="jagged"):
     return rc, n.value, _capi.lib().hstu_hip_last_error().decode()
 
 
+def test_noalloc_entry_rejects_a_work_list_beyond_its_fixed_array():
+    # host checks only: nothing is launched and no device is touched before the size check
+    p = _params(batch=2048, heads_q=16, heads_k=16, max_seq_len_q=20480, max_seq_len_k=20480, total_q=2048 * 20480, total_k=2048 * 20480)
+    assert _capi.lib().hstu_hip_jagged_forward_noalloc(C.byref(p), None) == -3
+    msg = _capi.lib().hstu_hip_last_error().decode()
+    assert "hstu_hip_jagged_forward_noalloc holds %d" % _capi.NOALLOC_SCRATCH_BYTES in msg
+    # and the ordinary validation comes first
+    assert _capi.lib().hstu_hip_jagged_forward_noalloc(C.byref(_params(batch=0)), None) == -1
+
+
 def test_struct_layout_matches_and_workspace_size():
     rc, n, msg = _ws(_params())
     # a size mismatch between ctypes and C would be rejected here.  MFMA kernels keep their work list in the
