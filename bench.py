@@ -50,6 +50,16 @@ def build_workload(name, torch, W):
         kv = sum(c["hist"]) * 2 * 4 * 128
         qo = 2 * 32 * 256 * 4 * 128 * 2
         return c, "paged", flops, kv + 2 * qo, "config5 paged fp8-KV: 32 users x 256 candidates, hist~U[1024,4096], 64-token pages"
+    if name in ("ref_bias", "ref_nobias"):
+        c = W.reference_benchmark_config(has_rab=name == "ref_bias")
+        flops = W.headline_flops(c["lens"], 8, 128)
+        t = sum(c["lens"])
+        b = 4 * t * 8 * 128 * 2
+        # of the dense bias only the causal half is needed: sum over sequences and heads of L (L + 1) / 2 two-byte values
+        if name == "ref_bias":
+            b += sum(8 * l * (l + 1) // 2 * 2 for l in c["lens"])
+        return c, "jagged", flops, b, ("reference benchmark shape (test_forward_op_benchmark.py:246-259): B=32 h=8 d=128 S=2048, every length "
+                                      "0.9 S, alpha=0.5, silu_scale=1/1024, bf16, causal, " + ("dense attn_bias [B,h,S,S]" if name == "ref_bias" else "no bias"))
     raise SystemExit(f"unknown workload {name}")
 
 
@@ -58,7 +68,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=1000)
-    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "config2_bwd", "kv_append", "kv_append_fp8", "rab_time", "rab_time_bwd", "rab_pos", "nmd_fwd", "nmd_bwd", "in_linear_silu", "in_linear_silu_bwd", "copy"],
+    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "ref_bias", "ref_nobias", "config2_bwd", "kv_append", "kv_append_fp8", "rab_time", "rab_time_bwd", "rab_pos", "nmd_fwd", "nmd_bwd", "in_linear_silu", "in_linear_silu_bwd", "copy"],
                     help="'copy' runs a plain 256 MiB device copy: the known-size kernel the FETCH_SIZE/WRITE_SIZE counters are scaled by")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
@@ -92,6 +102,7 @@ def main():
     out = torch.empty_like(q)
     kw = dict(seq_offset_q=dev["seq_offset"], seq_offset_k=dev.get("seq_offset_k"), max_seq_len_q=cfg["max_seq_len"],
               max_seq_len_k=cfg.get("max_seq_len_k"), mask_type=0, alpha=cfg["alpha"], num_target=dev.get("num_target"),
+              attn_bias=dev.get("attn_bias"), silu_scale=cfg.get("silu_scale", 0.0),
               target_group_size=cfg.get("target_group_size", 0), pos_table=dev.get("pos_table"),
               ts_table=dev.get("ts_table"), timestamps=dev.get("timestamps"))
     if cfg.get("ts_table") is not None:

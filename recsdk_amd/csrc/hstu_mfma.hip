@@ -13,9 +13,6 @@
 // Element-wise order follows the reference (vector_score_inter.h:299-323): x = alpha*(S+bias), SiLU,
 // then scale*mask; P is rounded to the I/O dtype before PV as there (vector_score_inter.h:177-184),
 // S itself stays in fp32.
-#include <cstdio>
-#include <cstdlib>
-
 #include "hstu_device.h"
 
 namespace hstu {
@@ -48,6 +45,14 @@ template <> struct MM<_Float16> {
         f16x2 r; r[0] = (_Float16)x; r[1] = (_Float16)y; return __builtin_bit_cast(unsigned, r);
     }
 };
+
+// 16-bit half `hi` (0 / 1) of a 32-bit word as float
+template <typename T> __device__ __forceinline__ float half_to_float(unsigned w, int hi);
+template <> __device__ __forceinline__ float half_to_float<__bf16>(unsigned w, int hi) { return __builtin_bit_cast(float, hi ? (w & 0xffff0000u) : (w << 16)); }
+template <> __device__ __forceinline__ float half_to_float<_Float16>(unsigned w, int hi) {
+    const f16x2 v = __builtin_bit_cast(f16x2, w);
+    return (float)v[hi];
+}
 
 constexpr int BM = 128;  // Q rows per workgroup
 constexpr int BN = 64;   // K columns per step
@@ -239,12 +244,6 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
     unsigned* list = ws + WS_HEADER;
     unsigned* ovf = list + REC * 8 * (size_t)d.cap;
 
-#ifdef HSTU_SCHED_TIMING
-    unsigned long long ts0 = __builtin_amdgcn_s_memrealtime(), ts1 = 0, ts2 = 0, ts3 = 0, ts4 = 0;
-#define SST(x) x = __builtin_amdgcn_s_memrealtime()
-#else
-#define SST(x)
-#endif
     for (size_t i = tid; i < 8 * (size_t)d.cap; i += nthr) list[REC * i] = ITEM_EMPTY;
     if (tid < 256) s_hist[tid] = 0;
     if (tid == 0) s_ovf = 0;
@@ -271,7 +270,6 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
         atomicAdd(&s_hist[key], 1u);
     }
     __syncthreads();
-    SST(ts1);
     if (p.batch <= 32) {
         // small batch: rank by counting (ties by batch index, so the order is reproducible), one barrier
         if (tid < p.batch) {
@@ -307,8 +305,6 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
         for (int b = tid; b < p.batch; b += nthr) s_order[atomicAdd(&s_base[s_key[b]], 1u)] = (unsigned short)b;
         __syncthreads();
     }
-
-    SST(ts2);
     // groups r = rank * heads + head; exclusive prefix of the tile counts inside each XCD's list.  A chunk of
     // 1024 consecutive groups is scanned with stride 16 (one scan per residue class r % 16); XCD x owns the
     // classes x and 15 - x, class x first.
@@ -371,7 +367,6 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
     }
     if (tid < 8) s_len[tid] = cb;   // entries of list x = classes x and 15 - x
     __syncthreads();
-    SST(ts3);
     // items that did not fit their XCD's list move to the free slots at the end of the other lists
     const unsigned novf = s_ovf;
     for (unsigned i = tid; i < novf; i += nthr) {
@@ -393,22 +388,8 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
         const int64_t owned = p.seq_offset_q ? ld_idx(p.seq_offset_q, p.batch, p.index_type == HSTU_I64) : p.total_q;
         *reinterpret_cast<int64_t*>(ws + 2) = owned;
     }
-#ifdef HSTU_SCHED_TIMING
-    SST(ts4);
-    if (tid == 0) { ws[8] = (unsigned)(ts1 - ts0); ws[9] = (unsigned)(ts2 - ts1); ws[10] = (unsigned)(ts3 - ts2); ws[11] = (unsigned)(ts4 - ts3); }
-#endif
 }
 
-#ifdef HSTU_ITEM_TIMING
-// Development aid (not part of the normal build): per workgroup of the main kernel {start, time to the first tile in
-// LDS, time to the end, hardware id, K tiles}, in 10 ns ticks of the constant clock.
-__device__ unsigned g_item_times[8 * 32768];
-}  // namespace hstu
-extern "C" int hstu_hip_debug_item_times(void* dst, size_t bytes) {
-    return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(hstu::g_item_times), bytes);
-}
-namespace hstu {
-#endif
 
 // EXTRA: 0 = no bias / built-in mask only, 1 = dense bias and/or custom mask (tables, if any, gathered from
 // global memory), 2 / 3 / 4 = bias tables only, gathered from LDS-resident copies: position table / time table /
@@ -431,10 +412,7 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
     typedef Shape<D, EXTRA, PAGED> SH;
     constexpr int BNT = SH::BNT;
     constexpr bool LEAN = SH::WAVES == 3;          // register-tight variants read V fragments right before use
-#ifndef HSTU_PARK_OUT
-#define HSTU_PARK_OUT LEAN
-#endif
-    constexpr bool PARK_OUT = HSTU_PARK_OUT;
+    constexpr bool PARK_OUT = LEAN;                // output tiles leave through LDS as whole rows
     constexpr int NBLK4 = BNT / 4;                 // 4-row blocks per tile
     typedef typename MM<T>::v8 v8;
     const hstu_fwd_params& p = a.p;
@@ -461,17 +439,18 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
     // paged: page ids of this user and, for an fp8 cache, the (K, V) scales of this kv head
     __shared__ int lds_pid[PAGED ? MAXP : 1];
     __shared__ float lds_psc[PAGED ? 2 * MAXP : 1];
+    // dense bias / custom mask: every wave takes its 32 x 32 block in as whole 64-byte row pieces (16 bytes per lane, four
+    // lanes per row) and reads it back from this private tile in the layout of the score registers; loading it in that
+    // layout directly would touch 64 cache lines per instruction.  Row stride 72 bytes.
+    constexpr int XRS = 72;
+    constexpr bool XTILE = EXTRA == 1 && !PAGED;   // (the paged variant with a dense bias has no registers or LDS to spare for it)
+    __shared__ __attribute__((aligned(16))) char lds_x[XTILE ? 4 * 32 * XRS : 16];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave index, kept in a scalar register
     const int g = lane >> 5, l32 = lane & 31;
 
-#ifdef HSTU_ITEM_TIMING
-    const unsigned long long it0 = __builtin_amdgcn_s_memrealtime();
-    unsigned long long it1 = it0, it_loop = it0;
-    int it_ntk = 0;
-#endif
     // blockIdx -> record of the work list (see above)
     unsigned rw[REC];
     {
@@ -501,6 +480,9 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
     s.delta = s.lk - s.lq; s.hist_q = s.lq - s.tgt; s.hist_k = s.lk - s.tgt; s.cand_row = s.q_start + s.hist_q;
     const bool tril = p.mask_type == HSTU_MASK_TRIL;
     const int tgs = p.target_group_size;
+    // rows of attn_bias / mask start on 16-byte boundaries
+    const bool x_rows16 = XTILE && p.max_seq_len_k % 8 == 0 && ((reinterpret_cast<uintptr_t>(p.attn_bias) | reinterpret_cast<uintptr_t>(p.mask)) & 15) == 0;
+    const bool x_mask = EXTRA == 1 && p.mask_type == HSTU_MASK_CUSTOM;
     const T* qbase = reinterpret_cast<const T*>(p.q);
     T* obase = reinterpret_cast<T*>(p.out);
 
@@ -702,10 +684,6 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
         const int kt0 = part * per, kt1 = min(ntk, kt0 + per);
         if (kt0 < kt1) fetch(kt0, lds0);
         stash(kt0, lds0);
-#ifdef HSTU_ITEM_TIMING
-        it1 = __builtin_amdgcn_s_memrealtime();
-        it_ntk += kt1 - kt0;
-#endif
 
         auto iteration = [&](int kt, const char* cur, char* nxt) __attribute__((always_inline)) {
             const int buf = kt & 1;
@@ -719,6 +697,22 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                 if (cls == BLK_SKIP) continue;  // wave-uniform
                 // ---- S^T block: 32 keys x 32 Q rows.  All K fragments are requested before the first
                 // MFMA so that the LDS latency is paid once per block, not once per instruction.
+                // dense bias / mask block: rows r0 + lane / 4 and 16 more, columns c0 + 8 * (lane % 4) .. + 7 per lane; requested
+                // here, used after the S^T products.  (Requesting it one block ahead costs more in spilled registers than
+                // the latency it hides: measured.)
+                u32x4 xb[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}}, xm[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
+                if (XTILE && x_rows16) {
+                    const int col = c0 + 8 * (lane & 3);
+#pragma unroll
+                    for (int i = 0; i < 2; i++) {
+                        const int row = r0 + (lane >> 2) + 16 * i;
+                        if (row < p.max_seq_len_q && col < p.max_seq_len_k) {   // outside the attribute's square: no bias, mask 0
+                            const int64_t at = (((int64_t)b * p.heads_q + h) * p.max_seq_len_q + row) * (int64_t)p.max_seq_len_k + col;
+                            if (p.attn_bias) xb[i] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const T*>(p.attn_bias) + at);
+                            if (x_mask) xm[i] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const T*>(p.mask) + at);
+                        }
+                    }
+                }
                 v8 kf[D / 16];
 #pragma unroll
                 for (int ds = 0; ds < D / 16; ds++) kf[ds] = read_kf(cur, kb, ds);
@@ -738,6 +732,25 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                         vhi[db] = read_vf(cur, kb, db, 1);
                     }
                 }
+                // the bias (and mask) block in the layout of the score registers: 4 consecutive keys per 8-byte read
+                u32x2 xbr[4], xmr[4];
+                if (XTILE && x_rows16) {
+                    char* tile = lds_x + w * (32 * XRS);
+                    auto through_tile = [&](const u32x4* in, u32x2* out) __attribute__((always_inline)) {
+#pragma unroll
+                        for (int i = 0; i < 2; i++) {
+                            char* at = tile + ((lane >> 2) + 16 * i) * XRS + 16 * (lane & 3);
+                            *reinterpret_cast<u32x2*>(at) = (u32x2){in[i][0], in[i][1]};
+                            *reinterpret_cast<u32x2*>(at + 8) = (u32x2){in[i][2], in[i][3]};
+                        }
+                        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                        for (int q = 0; q < 4; q++) out[q] = *reinterpret_cast<const u32x2*>(tile + l32 * XRS + (8 * q + 4 * g) * 2);
+                        __builtin_amdgcn_wave_barrier();
+                    };
+                    if (p.attn_bias) through_tile(xb, xbr);
+                    if (x_mask) through_tile(xm, xmr);
+                }
                 // ---- P = s * sigmoid(alpha * s) (scale folded into the epilogue), masked
                 // accumulator register r holds key c0 + 8*(r/4) + 4*g + r%4 for Q row qi
                 float pf[16];
@@ -749,7 +762,11 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                     if (EXTRA == 1) {
                         const bool in_attr = qi < p.max_seq_len_q && j < p.max_seq_len_k;
                         const int64_t bm = (((int64_t)b * p.heads_q + h) * p.max_seq_len_q + qi) * (int64_t)p.max_seq_len_k + j;
-                        if (p.attn_bias && in_attr) x += to_float(reinterpret_cast<const T*>(p.attn_bias)[bm]);
+                        if (x_rows16) {
+                            if (p.attn_bias) x += half_to_float<T>(xbr[r >> 2][(r >> 1) & 1], r & 1);
+                        } else if (p.attn_bias && in_attr) {
+                            x += to_float(reinterpret_cast<const T*>(p.attn_bias)[bm]);
+                        }
                         if (p.pos_table) {
                             const int idx = (p.max_seq_len_k - 1) + j - (qi + s.delta);
                             if (idx >= 0 && idx < 2 * p.max_seq_len_k - 1) x += p.pos_table[idx];
@@ -758,7 +775,7 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                             float dt = abs_dt_as_float(tq, p.timestamps[s.k_start + j]);
                             x += p.ts_table[ts_bucket(p.ts_bounds, p.num_buckets, dt)];
                         }
-                        if (p.mask_type == HSTU_MASK_CUSTOM) mval = in_attr ? to_float(reinterpret_cast<const T*>(p.mask)[bm]) : 0.f;
+                        if (x_mask) mval = x_rows16 ? half_to_float<T>(xmr[r >> 2][(r >> 1) & 1], r & 1) : (in_attr ? to_float(reinterpret_cast<const T*>(p.mask)[bm]) : 0.f);
                     }
                     if (TAB) {
                         const int jj = 32 * kb + 8 * (r >> 2) + 4 * g + (r & 3);        // j - k0
@@ -873,9 +890,6 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
             if (kt + 1 < kt1) iteration(kt + 1, lds1, lds0);
         }
 
-#ifdef HSTU_ITEM_TIMING
-        it_loop = __builtin_amdgcn_s_memrealtime();
-#endif
         // ---- epilogue: O^T accumulator register r of block db holds d = 32*db + 8*(r/4) + 4*g + r%4 for row qi
         if (PARK_OUT && nsplit == 1) {
             // Through LDS, so that the stores are whole rows: each wave parks its 32 x D tile in the K/V stage that
@@ -934,16 +948,6 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
         __syncthreads();   // the next tile's loads overwrite the stages the output tiles were parked in
     }
 
-#ifdef HSTU_ITEM_TIMING
-    if (tid == 0 && blockIdx.x < 32768) {
-        const unsigned long long it2 = __builtin_amdgcn_s_memrealtime();
-        unsigned* o = g_item_times + 8 * blockIdx.x;
-        o[0] = (unsigned)it0; o[1] = (unsigned)(it1 - it0); o[2] = (unsigned)(it2 - it0);
-        o[3] = __builtin_amdgcn_s_getreg((31 << 11) | 4);     // HW_ID: CU 11:8, SH 12, SE 14:13
-        o[4] = (unsigned)it_ntk; o[5] = item; o[7] = (unsigned)(it_loop - it0);
-        o[6] = __builtin_amdgcn_s_getreg((3 << 11) | 20);     // XCC_ID
-    }
-#endif
     // rows past the last offset are zero (the reference zero-fills its output: hstu_jagged.cpp:56-59)
     if (owned_rows < p.total_q) {
         const int64_t n = (p.total_q - owned_rows) * p.heads_q * (int64_t)D;
@@ -1020,11 +1024,6 @@ static hipError_t launch_td(const KArgs& a, unsigned* ws, hipStream_t stream) {
     }
     dim3 grid(8 * d.cap), block(NT);   // the overflow list starts at entry gridDim.x of the lists
     const float* part = reinterpret_cast<const float*>(reinterpret_cast<const char*>(ws) + list_bytes(d));
-    if (getenv("HSTU_HIP_DEBUG")) {
-        int nb = -1;
-        e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, hstu_mfma_kernel<T, D, 0, false>, NT, 0);
-        fprintf(stderr, "[hstu_hip] mfma d=%d grid=%u workgroups/CU=%d (%s)\n", D, grid.x, nb, hipGetErrorString(e));
-    }
 #define HSTU_LAUNCH(E, P) hipLaunchKernelGGL((hstu_mfma_kernel<T, D, E, P>), grid, block, 0, stream, a, ws, part)
     if (paged) {
         if (extra == 0) HSTU_LAUNCH(0, true);

@@ -81,6 +81,51 @@ def test_mfma_bias_and_custom_mask(dtype):
 
 @pytest.mark.parametrize("dtype", LOWP)
 @pytest.mark.parametrize("d", [64, 128])
+def test_mfma_dense_bias_row_pieces(d, dtype):
+    """attn_bias / mask whose rows start on 16-byte boundaries (max_seq_len_k % 8 == 0): the blocks are taken in as whole
+    row pieces through the per-wave tile.  Square, delta-q with GQA, and an attribute smaller than the longest sequence
+    (rows and columns behind it get no bias and mask 0)."""
+    say("mfma_bias_rows16", dtype, d)
+    lens = [137, 64, 296]
+    cfg, rng = _jag(61, lens, 2, 2, d, d, dtype)
+    b, n, m = 3, 2, 296
+    cfg["attn_bias"] = torch.from_numpy(rng.normal(0, 0.7, (b, n, m, m)).astype(np.float32)).to(dtype)
+    _check(cfg, dtype, "dense bias, 16-byte rows")
+    cfg["mask"] = torch.from_numpy(rng.integers(0, 2, (b, n, m, m)).astype(np.float32)).to(dtype)
+    cfg["mask_type"] = 3
+    _check(cfg, dtype, "dense bias + custom mask, 16-byte rows")
+    cfg2, rng = _jag(62, [70, 200, 33], 4, 2, d, d, dtype, lens_k=[130, 200, 97])
+    mq, mk = 200, 200
+    cfg2["attn_bias"] = torch.from_numpy(rng.normal(0, 0.7, (3, 4, mq, mk)).astype(np.float32)).to(dtype)
+    _check(cfg2, dtype, "dense bias, delta-q + GQA")
+    cfg3, rng = _jag(63, [300, 140], 2, 2, d, d, dtype)
+    cfg3["max_seq_len"] = 104
+    cfg3["attn_bias"] = torch.from_numpy(rng.normal(0, 0.7, (2, 2, 104, 104)).astype(np.float32)).to(dtype)
+    # (the goldens have no such case: both kernels of this library give rows and columns behind the attribute no bias)
+    out, name = T.run_capi(cfg3)
+    assert name.startswith("mfma_"), name
+    gen, _ = T.run_capi(cfg3, flags=FORCE_GENERIC)
+    T.assert_parity(out, gen.float(), dtype, what="dense bias, attribute smaller than the sequences, vs generic kernel")
+
+
+def test_reference_benchmark_shape_with_dense_bias():
+    """The reference's own benchmark shape with its dense bias (B=32, h=8, d=128, S=2048, lengths 0.9 S, alpha 0.5,
+    silu_scale 1/1024): the whole batch against the plain-FMA kernel, its first two sequences against the oracle."""
+    say("ref_bias")
+    dtype = torch.bfloat16
+    cfg = W.reference_benchmark_config()
+    out, name = T.run_capi(cfg)
+    assert name == "mfma_bf16_d128", name
+    gen, _ = T.run_capi(cfg, flags=FORCE_GENERIC)
+    T.assert_parity(out, gen.float(), dtype, what="reference benchmark shape vs generic kernel")
+    l = cfg["lens"][0]
+    sub = dict(cfg, q=cfg["q"][:2 * l], k=cfg["k"][:2 * l], v=cfg["v"][:2 * l], seq_offset=cfg["seq_offset"][:3], lens=cfg["lens"][:2],
+               attn_bias=cfg["attn_bias"][:2])
+    T.assert_parity(out[:2 * l], T.oracle_jagged(sub), dtype, what="reference benchmark shape vs oracle")
+
+
+@pytest.mark.parametrize("dtype", LOWP)
+@pytest.mark.parametrize("d", [64, 128])
 def test_mfma_table_bias(d, dtype):
     say("mfma_tables", dtype, d)
     rng = np.random.default_rng(27)
