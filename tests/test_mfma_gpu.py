@@ -232,6 +232,78 @@ def test_config5_paged_fp8():
     T.assert_parity(out8, T.oracle_paged(cfg), torch.bfloat16, tol=5e-2, what="config5 vs unquantised oracle")
 
 
+def test_config4_full_size_properties():
+    """Config 4 at its full batch (B=128: 512 groups, the schedule kernel's 512-thread shape): MFMA kernel against the
+    plain-FMA kernel, plus what holds at any size: linear in V, and a candidate row sees the history and itself only
+    (changing another candidate's K/V leaves it alone, changing a history row does not)."""
+    cfg = W.config4()
+    say("config4_full", sum(cfg["lens"]))
+    dtype = torch.bfloat16
+    out, name = T.run_capi(cfg)
+    assert name == "mfma_bf16_d64"
+    gen, _ = T.run_capi(cfg, flags=FORCE_GENERIC)
+    T.assert_parity(out, gen.float(), dtype, what="config4 full size vs generic kernel")
+    assert torch.equal(T.run_op(cfg, op="table"), out)
+    out2, _ = T.run_capi(cfg, v=(cfg["v"].float() * 2).to(dtype))
+    assert torch.allclose(out2.float(), 2 * out.float(), rtol=2e-2, atol=1e-6)
+    o = cfg["seq_offset"].tolist()
+    b = 5
+    cand0 = o[b + 1] - 64                      # first candidate row of sequence b
+    k3, v3 = cfg["k"].clone(), cfg["v"].clone()
+    k3[cand0 + 10] += 1; v3[cand0 + 10] -= 1   # candidate 10 of sequence b
+    out3, _ = T.run_capi(cfg, k=k3, v=v3)
+    changed = (out3 != out).flatten(1).any(1).nonzero().flatten().tolist()
+    assert changed == [cand0 + 10], changed
+    k4, v4 = cfg["k"].clone(), cfg["v"].clone()
+    k4[o[b] + 3] += 1; v4[o[b] + 3] -= 1       # history row 3: every later row of the sequence sees it
+    out4, _ = T.run_capi(cfg, k=k4, v=v4)
+    changed = (out4 != out).flatten(1).any(1).nonzero().flatten()
+    assert changed.min().item() == o[b] + 3 and changed.max().item() < o[b + 1] and changed.numel() > 64
+
+
+def test_config5_full_size_properties():
+    """Config 5 at its full batch (32 users: three K ranges per Q tile, where 8 users get four): MFMA kernel against the
+    plain-FMA kernel, linear in the values (candidate V rows and the cache's scales of the V planes doubled), candidates
+    isolated from each other, and no causal order inside the history (its last row reaches every candidate)."""
+    cfg = W.config5()
+    say("config5_full", len(cfg["hist"]))
+    dtype = torch.bfloat16
+    out, name = T.run_capi(cfg, op="paged", use_fp8=True)
+    assert name == "mfma_bf16_d128"
+    gen, _ = T.run_capi(cfg, op="paged", use_fp8=True, flags=FORCE_GENERIC)
+    T.assert_parity(out, gen.float(), dtype, what="config5 full size vs generic kernel")
+    sc2 = cfg["kv_scales"].clone()
+    sc2[:, 1] *= 2
+    out2, _ = T.run_capi(cfg, op="paged", use_fp8=True, v=(cfg["v"].float() * 2).to(dtype), kv_scales=sc2)
+    assert torch.allclose(out2.float(), 2 * out.float(), rtol=2e-2, atol=1e-6)
+    u = 7
+    k3, v3 = cfg["k"].clone(), cfg["v"].clone()
+    k3[256 * u + 100] += 1; v3[256 * u + 100] -= 1          # candidate 100 of user u
+    out3, _ = T.run_capi(cfg, op="paged", use_fp8=True, k=k3, v=v3)
+    changed = (out3 != out).flatten(1).any(1).nonzero().flatten().tolist()
+    assert changed == [256 * u + 100], changed
+    page = int(cfg["page_ids"][int(cfg["page_offsets"][u + 1]) - 1])     # last history page of user u
+    slot = (cfg["hist"][u] - 1) % 64
+    c4 = cfg["kv_cache_fp8"].clone().view(torch.uint8)
+    c4[page, :, slot] ^= 0x40                                # another e4m3 value in the last history row
+    out4, _ = T.run_capi(dict(cfg, kv_cache_fp8=c4), op="paged", use_fp8=True)
+    changed = (out4 != out).flatten(1).any(1).nonzero().flatten()
+    assert changed.min().item() >= 256 * u and changed.max().item() < 256 * (u + 1) and changed.numel() > 200
+
+
+def test_reference_user_shape_long_sequences():
+    """The reference benchmark's user case B=128, h=4, d=128, S=7621 with lengths int(0.9 S) = 6858
+    (test_forward_op_benchmark.py:185-199), a quarter of its batch (the plain-FMA kernel it is checked against runs 10 x
+    longer): bf16, no bias, causal."""
+    say("ref_user_shape")
+    dtype = torch.bfloat16
+    cfg = W.reference_benchmark_config(batch=32, heads=4, dim=128, max_seq_len=7621, has_rab=False)
+    out, name = T.run_capi(cfg)
+    assert name == "mfma_bf16_d128", name
+    gen, _ = T.run_capi(cfg, flags=FORCE_GENERIC)
+    T.assert_parity(out, gen.float(), dtype, what="reference user shape vs generic kernel")
+
+
 # ---- work list (schedule kernel) -----------------------------------------------------------------
 def test_work_list_overflow_path():
     """Sequences sorted by K length but with very uneven Q lengths: one XCD list gets more tiles than its
