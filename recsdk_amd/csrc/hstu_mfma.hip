@@ -402,7 +402,8 @@ template <int D, int EXTRA, bool PAGED> struct Shape {
     static constexpr bool DMA = !PAGED && D == 128;
     static constexpr bool LEAN = DMA && EXTRA == 0;
     static constexpr int BNT = LEAN ? 32 : 64;     // K columns per step
-    static constexpr int WAVES = (LEAN || (D == 64 && EXTRA != 1)) ? 3 : 2;     // waves per SIMD
+    // waves per SIMD; head dim 256 needs the registers of a whole SIMD lane for its 32 x 256 accumulator and Q fragments
+    static constexpr int WAVES = D == 256 ? 1 : ((LEAN || (D <= 64 && EXTRA != 1)) ? 3 : 2);
 };
 
 template <typename T, int D, int EXTRA, bool PAGED>
@@ -983,11 +984,13 @@ bool mfma_supported(const KArgs& a, const char** name) {
     const hstu_fwd_params& p = a.p;
     *name = nullptr;
     if (p.dtype != HSTU_BF16 && p.dtype != HSTU_F16) return false;
-    if (p.dim_qk != p.dim_v || (p.dim_qk != 64 && p.dim_qk != 128)) return false;
+    const int d = p.dim_qk;
+    if (d != p.dim_v || (d != 32 && d != 64 && d != 128 && d != 256)) return false;
+    if (a.op == OP_PAGED && (d == 32 || d == 256)) return false;   // paged K/V: head dims 64 and 128 only
     if (a.op == OP_PAGED && (p.max_seq_len_k + p.page_size - 1) / p.page_size > MAXP) return false;  // page ids of a user must fit the LDS copy
     const bool bf = p.dtype == HSTU_BF16;
-    if (p.dim_qk == 128) *name = bf ? "mfma_bf16_d128" : "mfma_f16_d128";
-    else *name = bf ? "mfma_bf16_d64" : "mfma_f16_d64";
+    *name = d == 32 ? (bf ? "mfma_bf16_d32" : "mfma_f16_d32") : d == 64 ? (bf ? "mfma_bf16_d64" : "mfma_f16_d64")
+          : d == 128 ? (bf ? "mfma_bf16_d128" : "mfma_f16_d128") : (bf ? "mfma_bf16_d256" : "mfma_f16_d256");
     return true;
 }
 
@@ -1025,7 +1028,12 @@ static hipError_t launch_td(const KArgs& a, unsigned* ws, hipStream_t stream) {
     dim3 grid(8 * d.cap), block(NT);   // the overflow list starts at entry gridDim.x of the lists
     const float* part = reinterpret_cast<const float*>(reinterpret_cast<const char*>(ws) + list_bytes(d));
 #define HSTU_LAUNCH(E, P) hipLaunchKernelGGL((hstu_mfma_kernel<T, D, E, P>), grid, block, 0, stream, a, ws, part)
-    if (paged) {
+    if constexpr (D == 32 || D == 256) {
+        // the head dims at the ends of the reference's sweep: plain and general variants only (bias tables are gathered
+        // from global memory by the general one)
+        if (extra == 0) HSTU_LAUNCH(0, false);
+        else HSTU_LAUNCH(1, false);
+    } else if (paged) {
         if (extra == 0) HSTU_LAUNCH(0, true);
         else HSTU_LAUNCH(1, true);      // paged + bias: the general gather path
     } else {
@@ -1047,8 +1055,20 @@ static hipError_t launch_td(const KArgs& a, unsigned* ws, hipStream_t stream) {
 hipError_t launch_mfma(const KArgs& a, void* workspace, hipStream_t stream) {
     const hstu_fwd_params& p = a.p;
     unsigned* ws = reinterpret_cast<unsigned*>(workspace);
-    if (p.dtype == HSTU_BF16) return p.dim_qk == 128 ? launch_td<__bf16, 128>(a, ws, stream) : launch_td<__bf16, 64>(a, ws, stream);
-    return p.dim_qk == 128 ? launch_td<_Float16, 128>(a, ws, stream) : launch_td<_Float16, 64>(a, ws, stream);
+    if (p.dtype == HSTU_BF16) {
+        switch (p.dim_qk) {
+            case 32: return launch_td<__bf16, 32>(a, ws, stream);
+            case 64: return launch_td<__bf16, 64>(a, ws, stream);
+            case 128: return launch_td<__bf16, 128>(a, ws, stream);
+            default: return launch_td<__bf16, 256>(a, ws, stream);
+        }
+    }
+    switch (p.dim_qk) {
+        case 32: return launch_td<_Float16, 32>(a, ws, stream);
+        case 64: return launch_td<_Float16, 64>(a, ws, stream);
+        case 128: return launch_td<_Float16, 128>(a, ws, stream);
+        default: return launch_td<_Float16, 256>(a, ws, stream);
+    }
 }
 
 }  // namespace hstu

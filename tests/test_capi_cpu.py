@@ -130,6 +130,8 @@ def test_describe_kernel_selection():
     lib = _capi.lib()
     for over, want in [(dict(), "mfma_bf16_d128"), (dict(dim_qk=64, dim_v=64, dtype=_capi.HSTU_F16), "mfma_f16_d64"),
                        (dict(dtype=_capi.HSTU_F32), "generic_f32"), (dict(dim_v=64), "generic_bf16"),
+                       (dict(dim_qk=32, dim_v=32), "mfma_bf16_d32"), (dict(dim_qk=256, dim_v=256, dtype=_capi.HSTU_F16), "mfma_f16_d256"),
+                       (dict(dim_qk=96, dim_v=96), "generic_bf16"),
                        (dict(flags=_capi.FLAG_FORCE_GENERIC), "generic_bf16")]:
         p = _params(**over)
         assert lib.hstu_hip_describe_kernel(C.byref(p), buf, 64) == 0
@@ -138,7 +140,8 @@ def test_describe_kernel_selection():
     paged = dict(kv_cache=0x1000, page_offsets=0x1000, page_ids=0x1000, last_page_len=0x1000, cache_dtype=_capi.HSTU_BF16)
     for over, want in [(dict(page_size=64, max_seq_len_k=20480), "mfma_bf16_d128"),
                        (dict(page_size=8, max_seq_len_k=2560), "mfma_bf16_d128"),
-                       (dict(page_size=8, max_seq_len_k=2561), "generic_bf16")]:
+                       (dict(page_size=8, max_seq_len_k=2561), "generic_bf16"),
+                       (dict(page_size=64, dim_qk=256, dim_v=256), "generic_bf16")]:
         p = _params(**paged, **over)
         assert lib.hstu_hip_describe_kernel(C.byref(p), buf, 64) == 0
         assert buf.value.decode() == want, over

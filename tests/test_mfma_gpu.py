@@ -28,7 +28,7 @@ def _check(cfg, dtype, what, op="jagged", oracle=None, tol=None, **kw):
 
 
 @pytest.mark.parametrize("dtype", LOWP)
-@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("d", [32, 64, 128, 256])
 @pytest.mark.parametrize("lens", [[1], [31, 32, 33], [63, 64, 65, 127, 128, 129], [300, 0, 17, 0], [513, 257]])
 def test_mfma_causal_shapes(lens, d, dtype):
     say("mfma_causal", dtype, d, lens)
@@ -37,7 +37,7 @@ def test_mfma_causal_shapes(lens, d, dtype):
 
 
 @pytest.mark.parametrize("dtype", LOWP)
-@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("d", [32, 64, 128, 256])
 def test_mfma_gqa_delta_int32_tail(d, dtype):
     say("mfma_gqa_delta", dtype, d)
     cfg, _ = _jag(22, [70, 200, 33], 8, 2, d, d, dtype, lens_k=[130, 200, 97], index_dtype=torch.int32, extra_rows=7)
@@ -80,7 +80,7 @@ def test_mfma_bias_and_custom_mask(dtype):
 
 
 @pytest.mark.parametrize("dtype", LOWP)
-@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("d", [32, 64, 128, 256])
 def test_mfma_dense_bias_row_pieces(d, dtype):
     """attn_bias / mask whose rows start on 16-byte boundaries (max_seq_len_k % 8 == 0): the blocks are taken in as whole
     row pieces through the per-wave tile.  Square, delta-q with GQA, and an attribute smaller than the longest sequence
@@ -125,7 +125,7 @@ def test_reference_benchmark_shape_with_dense_bias():
 
 
 @pytest.mark.parametrize("dtype", LOWP)
-@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("d", [32, 64, 128, 256])
 def test_mfma_table_bias(d, dtype):
     say("mfma_tables", dtype, d)
     rng = np.random.default_rng(27)
@@ -347,7 +347,7 @@ def test_work_list_reuse_across_calls():
 
 
 @pytest.mark.parametrize("dtype", LOWP)
-@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("d", [32, 64, 128, 256])
 def test_split_k_ranges(d, dtype):
     """Few Q tiles against long K: each tile's K range is split over several workgroups, partial sums are reduced by
     a second kernel.  Causal (early tiles have empty ranges), delta-q with targets, and a tail of unused rows."""
