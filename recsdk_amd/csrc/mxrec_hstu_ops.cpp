@@ -87,6 +87,87 @@ static void run_abi(int (*ws_fn)(const hstu_fwd_params*, uint64_t*), int (*fn)(c
 }
 
 // ---------------------------------------------------------------------------------------------
+// The layers of one model call the jagged op on one batch geometry: same offset tensors, same shapes and
+// attributes, other q/k/v.  The work list in the workspace depends on the geometry only, so the last workspace of every
+// (device, stream) is kept together with what it was built from, and a call that matches passes
+// HSTU_FLAG_REUSE_WORKSPACE instead of building the list again.  The entry holds references to the offset / count
+// tensors themselves: their storage cannot be handed to another tensor while it is cached, and an in-place write
+// shows in their version counters.  Calls on one stream are ordered, so sharing the workspace between them is safe.
+// ---------------------------------------------------------------------------------------------
+struct ListCacheEntry {
+    at::Tensor ws;
+    std::vector<at::Tensor> geo;            // seq_offset, seq_offset_k, num_context, num_target (undefined where absent)
+    std::vector<uint32_t> versions;
+    hstu_fwd_params shape;                  // the scalar fields of the call that built it (pointers zeroed)
+    void* stream = nullptr;
+    int device = -1;
+};
+
+static hstu_fwd_params scalar_fields(hstu_fwd_params p) {
+    p.q = p.k = p.v = nullptr; p.out = nullptr; p.mask = p.attn_bias = nullptr;
+    p.seq_offset_q = p.seq_offset_k = p.num_context = p.num_target = nullptr;
+    p.kv_cache = p.page_offsets = p.page_ids = p.last_page_len = nullptr; p.kv_scales = nullptr;
+    p.pos_table = p.ts_table = p.ts_bounds = nullptr; p.timestamps = nullptr;
+    p.silu_scale = 0.f; p.alpha = 0.f; p.flags = 0;
+    return p;
+}
+
+static void run_abi_cached(const hstu_fwd_params& p0, const at::Tensor& q, const std::vector<at::Tensor>& geo, const char* op) {
+    static std::mutex mu;
+    static std::vector<ListCacheEntry> cache;   // a handful of (device, stream) pairs
+    hstu_fwd_params p = p0;
+    uint64_t ws_bytes = 0;
+    int rc = hstu_hip_jagged_forward_get_workspace_size(&p, &ws_bytes);
+    TORCH_CHECK(rc == HSTU_OK, "mxrec::", op, ": ", hstu_hip_last_error());
+    require_gpu(q, op);
+    c10::hip::OptionalHIPGuardMasqueradingAsCUDA guard(q.device());
+    auto stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA();
+    if (ws_bytes == 0) {
+        rc = hstu_hip_jagged_forward(&p, nullptr, 0, (void*)stream.stream());
+        TORCH_CHECK(rc == HSTU_OK, "mxrec::", op, ": ", hstu_hip_last_error());
+        return;
+    }
+    // what the list depends on besides the offsets: every scalar field, and which optional inputs are there
+    hstu_fwd_params shape = scalar_fields(p);
+    shape.flags = (p.attn_bias ? 1u : 0u) | (p.mask ? 2u : 0u) | (p.pos_table ? 4u : 0u) | (p.ts_table ? 8u : 0u);
+    std::lock_guard<std::mutex> lock(mu);
+    ListCacheEntry* hit = nullptr;
+    ListCacheEntry* slot = nullptr;
+    for (auto& e : cache)
+        if (e.device == q.device().index() && e.stream == (void*)stream.stream()) slot = &e;
+    if (slot && slot->ws.defined() && (uint64_t)slot->ws.numel() >= ws_bytes && std::memcmp(&slot->shape, &shape, sizeof(shape)) == 0) {
+        bool same = true;
+        for (size_t i = 0; i < geo.size(); i++) {
+            const at::Tensor& a = slot->geo[i];
+            same = same && a.defined() == geo[i].defined() &&
+                   (!a.defined() || (a.is_same(geo[i]) && slot->versions[i] == geo[i]._version()));
+        }
+        if (same) hit = slot;
+    }
+    if (hit) {
+        p.flags |= HSTU_FLAG_REUSE_WORKSPACE;
+        rc = hstu_hip_jagged_forward(&p, hit->ws.data_ptr(), ws_bytes, (void*)stream.stream());
+        TORCH_CHECK(rc == HSTU_OK, "mxrec::", op, ": ", hstu_hip_last_error());
+        return;
+    }
+    if (!slot) {
+        if (cache.size() >= 8) cache.erase(cache.begin());
+        cache.emplace_back();
+        slot = &cache.back();
+    }
+    slot->ws = at::empty({(int64_t)ws_bytes}, q.options().dtype(at::kByte));
+    slot->geo = geo;
+    slot->versions.clear();
+    for (const auto& t : geo) slot->versions.push_back(t.defined() ? t._version() : 0u);
+    slot->shape = shape;
+    slot->stream = (void*)stream.stream();
+    slot->device = q.device().index();
+    rc = hstu_hip_jagged_forward(&p, slot->ws.data_ptr(), ws_bytes, (void*)stream.stream());
+    if (rc != HSTU_OK) slot->ws = at::Tensor();
+    TORCH_CHECK(rc == HSTU_OK, "mxrec::", op, ": ", hstu_hip_last_error());
+}
+
+// ---------------------------------------------------------------------------------------------
 // Smallest fp32 |dt| of every time bucket, from the reference formula
 //   bucket = trunc(log(clamp(|dt|, 1, e^(nb*div))) / div)   (cust_op/test/relative_attn_bias/torch/utils.py:115-123)
 // evaluated with ATen's own CPU log so that the integer ids agree bit for bit with a torch evaluation
@@ -284,7 +365,12 @@ static at::Tensor jagged_forward_impl(const at::Tensor& q, const at::Tensor& k, 
         *grads = std::make_tuple(gq, gk, gv, gb);
         return at::Tensor();
     }
-    run_abi(hstu_hip_jagged_forward_get_workspace_size, hstu_hip_jagged_forward, p, dq, op);
+    // the tensors the caller handed in (not converted copies, which are new objects every call) identify the geometry
+    auto opt = [](const c10::optional<at::Tensor>& t) { return t.has_value() ? *t : at::Tensor(); };
+    const bool caller_owns = off_q.is_same(seq_offset) && off_k.is_same(seq_offset_k) &&
+                             (!ctx.defined() || ctx.is_same(opt(num_context))) && (!tgt.defined() || tgt.is_same(opt(num_target)));
+    if (caller_owns) run_abi_cached(p, dq, {off_q, off_k, ctx, tgt}, op);
+    else run_abi(hstu_hip_jagged_forward_get_workspace_size, hstu_hip_jagged_forward, p, dq, op);
     return out;
 }
 

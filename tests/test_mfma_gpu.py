@@ -346,6 +346,29 @@ def test_work_list_reuse_across_calls():
     T.assert_parity(out, T.oracle_jagged(cfg_b), dtype, what="reused work list vs oracle")
 
 
+def test_torch_op_keeps_the_work_list_of_an_unchanged_geometry():
+    """torch.ops.mxrec.hstu_jagged called again with the same offset tensors (the other layers of a model) reuses the work
+    list it built; new q/k/v give new results, an in-place change of the offsets is noticed, and so is another tensor."""
+    say("op_list_cache")
+    dtype = torch.bfloat16
+    lens = [300, 40, 513, 129]
+    cfg_a, _ = _jag(71, lens, 4, 2, 128, 128, dtype)
+    cfg_b, _ = _jag(72, lens, 4, 2, 128, 128, dtype)
+    off = cfg_a["seq_offset"].cuda()
+    first = T.run_op(dict(cfg_a, seq_offset=off))
+    again = T.run_op(dict(cfg_b, seq_offset=off))          # same geometry, other data: list reused
+    want_b, _ = T.run_capi(cfg_b)
+    assert torch.equal(first, T.run_capi(cfg_a)[0]) and torch.equal(again, want_b)
+    # the same tensor object with other contents: sequences [300, 40, 513, 129] -> [340, 0, 513, 129]
+    off[1] = 340
+    off[2] = 340
+    lens2 = [340, 0, 513, 129]
+    changed = T.run_op(dict(cfg_b, seq_offset=off))
+    cfg_c = dict(cfg_b, seq_offset=W.offsets(lens2), lens=lens2)
+    assert torch.equal(changed, T.run_capi(cfg_c)[0])
+    T.assert_parity(changed, T.oracle_jagged(cfg_c), dtype, what="offsets changed in place")
+
+
 @pytest.mark.parametrize("dtype", LOWP)
 @pytest.mark.parametrize("d", [32, 64, 128, 256])
 def test_split_k_ranges(d, dtype):
