@@ -205,8 +205,17 @@ int hstu_hip_dense_backward(const hstu_bwd_params* p, void* workspace, uint64_t 
 const char* hstu_hip_last_error(void);
 
 /* Name of the kernel variant the given arguments select ("mfma_bf16_d128", "generic_f32", ...);
- * written NUL-terminated into buf.  Diagnostic: lets a caller assert that the MFMA path is the one in use. */
+ * written NUL-terminated into buf.  Diagnostic: lets a caller assert that the MFMA path is the one in use.  The
+ * matrix-core kernels take bf16 / fp16 with dim_qk == dim_v in {32, 64, 128, 256} (paged: 64 or 128, and at most 320 pages
+ * per user) and buffers on 16-byte boundaries; everything else (fp32, other head dims, dim_qk != dim_v) runs the plain
+ * fp32-FMA kernel, which is an order of magnitude slower. */
 int hstu_hip_describe_kernel(const hstu_fwd_params* p, char* buf, size_t buf_bytes);
+
+/* The same for the backward: "mfma_bwd_bf16_d128", "mfma_bwd_f16_d64_bias", "generic_bwd_f32", ...  The matrix-core
+ * kernels take bf16 / fp16, head dim 64 or 128 (dim_qk == dim_v), the built-in mask or none, an optional dense attn_bias
+ * whose rows hold a multiple of 8 elements, and buffers on 16-byte boundaries; everything else (fp32, other head dims, a
+ * custom mask) runs the plain fp32-FMA kernels, which are an order of magnitude slower. */
+int hstu_hip_describe_backward_kernel(const hstu_bwd_params* p, char* buf, size_t buf_bytes);
 
 int hstu_hip_abi_version(void);
 

@@ -26,7 +26,7 @@ EXPORTS = [
     "hstu_hip_dense_forward_get_workspace_size", "hstu_hip_dense_forward",
     "hstu_hip_jagged_backward_get_workspace_size", "hstu_hip_jagged_backward",
     "hstu_hip_dense_backward_get_workspace_size", "hstu_hip_dense_backward",
-    "hstu_hip_last_error", "hstu_hip_describe_kernel", "hstu_hip_abi_version",
+    "hstu_hip_last_error", "hstu_hip_describe_kernel", "hstu_hip_describe_backward_kernel", "hstu_hip_abi_version",
     "hstu_hip_kv_append", "hstu_hip_kv_token_positions", "hstu_hip_kv_append_fp8", "hstu_hip_kv_append_fp8_get_workspace_size",
     "hstu_hip_rab_time", "hstu_hip_rab_time_backward", "hstu_hip_rab_pos",
     "hstu_hip_norm_multiply_dropout", "hstu_hip_norm_multiply_dropout_backward",
@@ -166,6 +166,7 @@ def lib() -> C.CDLL:
             getattr(_lib, f"hstu_hip_{n}_backward").argtypes = [C.POINTER(HstuBwdParams), C.c_void_p, C.c_uint64, C.c_void_p]
             getattr(_lib, f"hstu_hip_{n}_backward_get_workspace_size").argtypes = [C.POINTER(HstuBwdParams), C.POINTER(C.c_uint64)]
         _lib.hstu_hip_describe_kernel.argtypes = [C.POINTER(HstuFwdParams), C.c_char_p, C.c_size_t]
+        _lib.hstu_hip_describe_backward_kernel.argtypes = [C.POINTER(HstuBwdParams), C.c_char_p, C.c_size_t]
         _lib.hstu_hip_kv_append.argtypes = [C.POINTER(HstuKvAppendParams), C.c_void_p]
         _lib.hstu_hip_kv_append_fp8.argtypes = [C.POINTER(HstuKvAppendFp8Params), C.c_void_p, C.c_uint64, C.c_void_p]
         _lib.hstu_hip_kv_append_fp8_get_workspace_size.argtypes = [C.POINTER(HstuKvAppendFp8Params), C.POINTER(C.c_uint64)]
@@ -291,6 +292,12 @@ def run_backward(params: HstuBwdParams, stream=None, op: str = "jagged"):
     ws = torch.empty(n.value, dtype=torch.uint8, device="cuda") if n.value else None
     _check(getattr(L, f"hstu_hip_{op}_backward")(C.byref(params), _ptr(ws), n.value, stream if stream is not None else _stream()))
     return ws
+
+
+def describe_backward_kernel(params: HstuBwdParams) -> str:
+    buf = C.create_string_buffer(64)
+    _check(lib().hstu_hip_describe_backward_kernel(C.byref(params), buf, 64))
+    return buf.value.decode()
 
 
 def describe_kernel(params: HstuFwdParams) -> str:

@@ -275,6 +275,18 @@ int hstu_hip_describe_kernel(const hstu_fwd_params* p, char* buf, size_t n) {
     return HSTU_OK;
 }
 
+int hstu_hip_describe_backward_kernel(const hstu_bwd_params* p, char* buf, size_t n) {
+    if (!buf || n == 0) return fail(HSTU_ERR_INVALID_ARGUMENT, "buf is NULL");
+    BArgs a;
+    int rc = validate_backward(p, (p && !p->fwd.seq_offset_q) ? OP_DENSE : OP_JAGGED, &a);
+    if (rc != HSTU_OK) return rc;
+    const bool mfma = !(p->fwd.flags & HSTU_FLAG_FORCE_GENERIC) && mfma_backward_supported(a);
+    const char* dt = p->fwd.dtype == HSTU_F32 ? "f32" : (p->fwd.dtype == HSTU_F16 ? "f16" : "bf16");
+    if (mfma) snprintf(buf, n, "mfma_bwd_%s_d%d%s", dt, p->fwd.dim_qk, p->fwd.attn_bias ? "_bias" : "");
+    else snprintf(buf, n, "generic_bwd_%s", dt);
+    return HSTU_OK;
+}
+
 int hstu_hip_abi_version(void) { return HSTU_HIP_ABI_VERSION; }
 
 }  // extern "C"

@@ -987,6 +987,11 @@ bool mfma_supported(const KArgs& a, const char** name) {
     const int d = p.dim_qk;
     if (d != p.dim_v || (d != 32 && d != 64 && d != 128 && d != 256)) return false;
     if (a.op == OP_PAGED && (d == 32 || d == 256)) return false;   // paged K/V: head dims 64 and 128 only
+    // rows are read and written 16 bytes at a time (vector loads, direct copies into LDS): buffers that do not start on
+    // such a boundary take the plain kernel
+    const uintptr_t all = reinterpret_cast<uintptr_t>(p.q) | reinterpret_cast<uintptr_t>(p.k) | reinterpret_cast<uintptr_t>(p.v) |
+                          reinterpret_cast<uintptr_t>(p.out) | reinterpret_cast<uintptr_t>(p.kv_cache);
+    if (all & 15) return false;
     if (a.op == OP_PAGED && (p.max_seq_len_k + p.page_size - 1) / p.page_size > MAXP) return false;  // page ids of a user must fit the LDS copy
     const bool bf = p.dtype == HSTU_BF16;
     *name = d == 32 ? (bf ? "mfma_bf16_d32" : "mfma_f16_d32") : d == 64 ? (bf ? "mfma_bf16_d64" : "mfma_f16_d64")

@@ -1,4 +1,5 @@
-// Jagged HSTU backward on the gfx950 matrix cores (bf16 / fp16, head dim 64 or 128, built-in mask, no bias).
+// Jagged HSTU backward on the gfx950 matrix cores (bf16 / fp16, head dim 64 or 128, built-in mask, optional dense attn_bias
+// with its gradient).
 //
 // Three kernels from one template, each a variation of the forward kernel's scheme: the rows a wave owns sit in
 // registers as B operands, the other side streams through LDS in 64-row tiles, the 32x32 score block is produced by
@@ -12,6 +13,9 @@
 // alpha * silu_scale factors out of the sums and is applied once to the fp32 accumulators; P and dS are rounded to the
 // I/O dtype when they are packed for the second GEMM, as P in the forward.  Every gradient element has one producing
 // workgroup (with GQA the K-side kernels loop over the query heads of their K/V head): no atomics, deterministic.
+// With a dense attn_bias (BIAS) the scores are S + bias, read from [batch, heads, max_q, max_k] next to every block, and
+// the dQ kernel, which owns whole Q rows, also writes dBias = dS (hstu_jagged.cpp:69-138: the only case that produces it)
+// into a buffer that a fill kernel has zeroed: blocks the mask hides are never visited.
 #include "hstu_device.h"
 
 namespace hstu {
@@ -48,7 +52,17 @@ enum { MODE_DQ = 0, MODE_DK = 1, MODE_DV = 2 };
 constexpr int WBM = 128;   // rows a workgroup owns
 constexpr int WBN = 64;    // rows of the other side per step
 
-template <typename T, int D, int MODE>
+template <typename T> __global__ __launch_bounds__(256) void hstu_bwd_zero_kernel(T* out, int64_t n8) {
+    const b_u32x4 z = {0, 0, 0, 0};
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n8; i += (int64_t)gridDim.x * 256) reinterpret_cast<b_u32x4*>(out)[i] = z;
+}
+
+// 16-bit half `hi` (0 / 1) of a 32-bit word as float
+template <typename T> __device__ __forceinline__ float bwd_half(unsigned w, int hi);
+template <> __device__ __forceinline__ float bwd_half<__bf16>(unsigned w, int hi) { return __builtin_bit_cast(float, hi ? (w & 0xffff0000u) : (w << 16)); }
+template <> __device__ __forceinline__ float bwd_half<_Float16>(unsigned w, int hi) { return (float)__builtin_bit_cast(b_f16x2, w)[hi]; }
+
+template <typename T, int D, int MODE, bool BIAS>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
     typedef typename BMM<T>::v8 v8;
@@ -198,10 +212,32 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
                         }
                     }
                     // accumulator register r holds streamed row c0 + 8*(r/4) + 4*g + r%4 for the owned row of this lane
+                    // dense bias of this lane's 16 elements: the dQ kernel owns the row and takes four 8-byte pieces of it, the
+                    // K-side kernels own the column and take 16 single values (the lanes of a wave then read along a row)
+                    float bias_f[BIAS ? 16 : 1];
+                    const T* bias_bh = reinterpret_cast<const T*>(p.attn_bias) + ((int64_t)b * p.heads_q + h) * p.max_seq_len_q * (int64_t)p.max_seq_len_k;
+                    if (BIAS) {
+                        if (MODE == MODE_DQ) {
+#pragma unroll
+                            for (int q = 0; q < 4; q++) {
+                                const int j = c0 + 8 * q + 4 * g;
+                                b_u32x2 raw = {0, 0};
+                                if (orow < p.max_seq_len_q && j < p.max_seq_len_k) raw = *reinterpret_cast<const b_u32x2*>(bias_bh + orow * (int64_t)p.max_seq_len_k + j);
+#pragma unroll
+                                for (int i = 0; i < 4; i++) bias_f[4 * q + i] = bwd_half<T>(raw[i >> 1], i & 1);
+                            }
+                        } else {
+#pragma unroll
+                            for (int r = 0; r < 16; r++) {
+                                const int i = c0 + 8 * (r >> 2) + 4 * g + (r & 3);
+                                bias_f[r] = (i < p.max_seq_len_q && orow < p.max_seq_len_k) ? to_float(bias_bh[i * (int64_t)p.max_seq_len_k + orow]) : 0.f;
+                            }
+                        }
+                    }
                     float wv[16];
 #pragma unroll
                     for (int r = 0; r < 16; r++) {
-                        const float sv = sacc[r];
+                        const float sv = BIAS ? sacc[r] + bias_f[r] : sacc[r];
                         const float e = __builtin_amdgcn_exp2f(sv * a.f.exp_scale);
                         const float sg = __builtin_amdgcn_rcpf(1.0f + e);
                         if (TWO) {
@@ -217,6 +253,8 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
                         pk0[x] = BMM<T>::pack2(wv[2 * x], wv[2 * x + 1]);
                         pk1[x] = BMM<T>::pack2(wv[8 + 2 * x], wv[8 + 2 * x + 1]);
                     }
+                    // visibility of this lane's 16 elements as masks of the packed pairs
+                    b_u32x4 m0 = {~0u, ~0u, ~0u, ~0u}, m1 = m0;
                     if (diag) {
                         // visible iff j <= i + delta; t runs over this lane's 16 streamed rows
                         auto vis = [&](int r) __attribute__((always_inline)) -> bool {
@@ -225,8 +263,8 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
                         };
 #pragma unroll
                         for (int x = 0; x < 4; x++) {
-                            pk0[x] &= (vis(2 * x) ? 0xffffu : 0u) | (vis(2 * x + 1) ? 0xffff0000u : 0u);
-                            pk1[x] &= (vis(8 + 2 * x) ? 0xffffu : 0u) | (vis(9 + 2 * x) ? 0xffff0000u : 0u);
+                            m0[x] = (vis(2 * x) ? 0xffffu : 0u) | (vis(2 * x + 1) ? 0xffff0000u : 0u);
+                            m1[x] = (vis(8 + 2 * x) ? 0xffffu : 0u) | (vis(9 + 2 * x) ? 0xffff0000u : 0u);
                         }
                     } else if (pred) {
                         // branch-free form of builtin_visible() for this lane's 16 elements
@@ -240,8 +278,28 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
                         };
 #pragma unroll
                         for (int x = 0; x < 4; x++) {
-                            pk0[x] &= (vis(2 * x) ? 0xffffu : 0u) | (vis(2 * x + 1) ? 0xffff0000u : 0u);
-                            pk1[x] &= (vis(8 + 2 * x) ? 0xffffu : 0u) | (vis(9 + 2 * x) ? 0xffff0000u : 0u);
+                            m0[x] = (vis(2 * x) ? 0xffffu : 0u) | (vis(2 * x + 1) ? 0xffff0000u : 0u);
+                            m1[x] = (vis(8 + 2 * x) ? 0xffffu : 0u) | (vis(9 + 2 * x) ? 0xffff0000u : 0u);
+                        }
+                    }
+                    if (diag || pred) {
+#pragma unroll
+                        for (int x = 0; x < 4; x++) { pk0[x] &= m0[x]; pk1[x] &= m1[x]; }
+                    }
+                    if (BIAS && MODE == MODE_DQ) {
+                        // dBias = dS with its scale, rounded once, zero where the mask hides the element and behind the sequence;
+                        // pair x of the first half holds this lane's streamed rows 8*(x/2) + 2*(x%2) and + 1, the second half 16 more
+                        T* gbias = reinterpret_cast<T*>(a.grad_bias) + ((int64_t)b * p.heads_q + h) * p.max_seq_len_q * (int64_t)p.max_seq_len_k;
+                        const float sc = a.f.out_scale;
+#pragma unroll
+                        for (int q = 0; q < 4; q++) {
+                            const int j = c0 + 8 * q + 4 * g;
+                            const b_u32x4& mm = q < 2 ? m0 : m1;
+                            const int x0 = 2 * (q & 1);
+                            b_u32x2 o;
+                            o[0] = BMM<T>::pack2(wv[4 * q] * sc, wv[4 * q + 1] * sc) & mm[x0];
+                            o[1] = BMM<T>::pack2(wv[4 * q + 2] * sc, wv[4 * q + 3] * sc) & mm[x0 + 1];
+                            if (ovalid && orow < p.max_seq_len_q && j < p.max_seq_len_k) *reinterpret_cast<b_u32x2*>(gbias + orow * (int64_t)p.max_seq_len_k + j) = o;
                         }
                     }
                     // OUT^T += (tile)^T W: transposing LDS reads, 4 streamed rows of one head-dim column per lane
@@ -303,7 +361,15 @@ bool mfma_backward_supported(const BArgs& a) {
     const hstu_fwd_params& p = a.f.p;
     if (p.dtype != HSTU_BF16 && p.dtype != HSTU_F16) return false;
     if (p.dim_qk != p.dim_v || (p.dim_qk != 64 && p.dim_qk != 128)) return false;
-    if (p.attn_bias || p.mask_type == HSTU_MASK_CUSTOM) return false;
+    if (p.mask_type == HSTU_MASK_CUSTOM) return false;
+    // a dense bias is read 8 bytes at a time along its rows, its gradient written the same way
+    if (p.attn_bias && (p.max_seq_len_k % 8 != 0 || ((reinterpret_cast<uintptr_t>(p.attn_bias) | reinterpret_cast<uintptr_t>(a.grad_bias)) & 15)))
+        return false;
+    // rows are read and written 16 bytes at a time: buffers that do not start on such a boundary take the plain kernels
+    const uintptr_t all = reinterpret_cast<uintptr_t>(p.q) | reinterpret_cast<uintptr_t>(p.k) | reinterpret_cast<uintptr_t>(p.v) |
+                          reinterpret_cast<uintptr_t>(a.grad_out) | reinterpret_cast<uintptr_t>(a.grad_q) |
+                          reinterpret_cast<uintptr_t>(a.grad_k) | reinterpret_cast<uintptr_t>(a.grad_v);
+    if (all & 15) return false;
     return true;
 }
 
@@ -347,13 +413,30 @@ static hipError_t launch_bwd_td(const BArgs& a, unsigned* ws, hipStream_t stream
         e = launch_work_list(kside, wsk, false, stream);   // tile costs are only roughly those of the K tiles: no pairs
         if (e != hipSuccess) return e;
     }
-    hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DQ>), dim3(lq.grid), dim3(256), 0, stream, a, wsq);
+    if (a.f.p.attn_bias) {
+        // dBias: zero everywhere, then the dQ kernel writes the blocks the mask lets it visit
+        const hstu_fwd_params& p = a.f.p;
+        const int64_t n8 = (int64_t)p.batch * p.heads_q * p.max_seq_len_q * (int64_t)p.max_seq_len_k / 8;   // max_seq_len_k % 8 == 0
+        const unsigned zgrid = (unsigned)(n8 / 256 + 1 < 8192 ? n8 / 256 + 1 : 8192);
+        hipLaunchKernelGGL(hstu_bwd_zero_kernel<T>, dim3(zgrid), dim3(256), 0, stream, reinterpret_cast<T*>(a.grad_bias), n8);
+        e = hipGetLastError();
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DQ, true>), dim3(lq.grid), dim3(256), 0, stream, a, wsq);
+        e = hipGetLastError();
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DK, true>), dim3(lk.grid), dim3(256), 0, stream, a, wsk);
+        e = hipGetLastError();
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DV, true>), dim3(lk.grid), dim3(256), 0, stream, a, wsk);
+        return hipGetLastError();
+    }
+    hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DQ, false>), dim3(lq.grid), dim3(256), 0, stream, a, wsq);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DK>), dim3(lk.grid), dim3(256), 0, stream, a, wsk);
+    hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DK, false>), dim3(lk.grid), dim3(256), 0, stream, a, wsk);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DV>), dim3(lk.grid), dim3(256), 0, stream, a, wsk);
+    hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DV, false>), dim3(lk.grid), dim3(256), 0, stream, a, wsk);
     return hipGetLastError();
 }
 

@@ -48,8 +48,9 @@ def append_kvcache(append_key, append_value, batch_indices, positions, seqlen_of
     ``kv_indices[kv_indptr[b] + positions[i] // page_size]``, slot ``positions[i] % page_size``; its source row is
     ``i + seqlen_offsets[b]``.  ``paged_k_cache`` / ``paged_v_cache`` are the ``unbind(1)`` views of a
     ``[pages, 2, page_size, heads, dim]`` table (``kv_layout`` 0, NHD) or ``[pages, heads, page_size, dim]`` views
-    (``kv_layout`` 1, HND); strides are taken from the tensors.  ``nnz`` (host) bounds the launch; the reference accepts
-    and ignores it (pybind.cpp:57-61), here it may also be larger than ``nnz_npu[0]``.
+    (``kv_layout`` 1, HND); strides are taken from the tensors.  ``nnz`` (host) is accepted and ignored like in the reference
+    (pybind.cpp:57-61): the launch covers ``min(len(batch_indices), len(positions))`` tokens and ``nnz_npu[0]`` says how many of
+    them exist.
     """
     device = append_key.device
     _check_kv_2byte(append_key, device, 3, "append_key")
@@ -78,7 +79,9 @@ def append_kvcache(append_key, append_value, batch_indices, positions, seqlen_of
         raise RuntimeError("the head_dim axis of the caches and of append_key / append_value must be contiguous")
     if tuple(append_key.shape[1:]) != (num_heads, head_dim):
         raise RuntimeError(f"append_key shape {tuple(append_key.shape)} mismatch with cache heads {num_heads}, head_dim {head_dim}")
-    n = min(int(nnz), batch_indices.numel(), positions.numel())
+    # the reference's binding takes the host `nnz` and ignores it (pybind.cpp:57-61; its kernel reads nnz_npu only): a stale
+    # or zero value must not lose tokens, so the launch is sized by the index arrays and the device count does the rest
+    n = min(batch_indices.numel(), positions.numel())
     p = _capi.HstuKvAppendParams()
     p.struct_size = C.sizeof(_capi.HstuKvAppendParams)
     p.elem_bytes = 2
@@ -144,7 +147,7 @@ def append_kvcache_fp8(append_key, append_value, batch_indices, positions, seqle
     p.append_v_stride_n, p.append_v_stride_h = append_value.stride(0), append_value.stride(1)
     p.append_rows = append_key.size(0)
     p.batch_indices, p.positions, p.offsets = batch_indices.data_ptr(), positions.data_ptr(), seqlen_offsets.data_ptr()
-    p.nnz_dev, p.nnz_max = nnz_npu.data_ptr(), min(int(nnz), batch_indices.numel(), positions.numel())
+    p.nnz_dev, p.nnz_max = nnz_npu.data_ptr(), min(batch_indices.numel(), positions.numel())   # host nnz: a hint only, as above
     need = C.c_uint64(0)
     _capi._check(_capi.lib().hstu_hip_kv_append_fp8_get_workspace_size(C.byref(p), C.byref(need)))
     _require_gpu(append_key, "append_kvcache_fp8")

@@ -76,9 +76,14 @@ def run_capi_backward(cfg, grad, flags=0, op="jagged", **over):
     dq, dk, dv = torch.full_like(q, nan), torch.full_like(k, nan), torch.full_like(v, nan)
     db = None if bias is None else torch.full_like(bias, nan)
     p = _capi.make_backward_params(fwd, g, dq, dk, dv, db)
+    global last_backward_kernel
+    last_backward_kernel = _capi.describe_backward_kernel(p)
     _capi.run_backward(p, op=op)
     torch.cuda.synchronize()
     return dq.cpu(), dk.cpu(), dv.cpu(), None if db is None else db.cpu()
+
+
+last_backward_kernel = None   # name of the kernel variant the last run_capi_backward call selected
 
 
 def run_op(cfg, *, op="jagged", **over):

@@ -142,6 +142,12 @@ MFMA_CASES = [
     dict(lens_q=[260, 150], nq=2, nk=2, d=64, dtype=torch.bfloat16, ctx=[5, 0], tgt=[40, 17], tgs=3),  # context rows + target groups
     dict(lens_q=[190, 33], nq=1, nk=1, d=128, dtype=torch.float16, mask="none"),
     dict(lens_q=[515], nq=2, nk=2, d=64, dtype=torch.bfloat16, ctx=[130], tgt=[0], tgs=1),             # context rows across tiles
+    # dense attn_bias (rows of max_seq_len_k % 8 == 0 elements): the scores take it in, the dQ kernel writes dBias
+    dict(lens_q=[296, 129, 64, 1, 0, 257], nq=2, nk=2, d=128, dtype=torch.bfloat16, bias=True),
+    dict(lens_q=[200, 77], nq=4, nk=2, d=64, dtype=torch.float16, bias=True),                          # GQA
+    dict(lens_q=[130, 40], nq=2, nk=1, d=128, dtype=torch.bfloat16, lens_k=[336, 40], bias=True),      # delta-q + GQA
+    dict(lens_q=[264, 150], nq=2, nk=2, d=64, dtype=torch.bfloat16, ctx=[5, 0], tgt=[40, 17], tgs=3, bias=True),
+    dict(lens_q=[192, 33], nq=1, nk=1, d=128, dtype=torch.float16, mask="none", bias=True),
 ]
 
 
@@ -152,11 +158,17 @@ def test_backward_mfma_kernels(c):
     dtype, d = c.pop("dtype"), c.pop("d")
     cfg, grad = _case(11, c.pop("lens_q"), c.pop("nq"), c.pop("nk"), d, d, dtype, **c)
     got = T.run_capi_backward(cfg, grad)
+    assert T.last_backward_kernel.startswith("mfma_bwd_"), T.last_backward_kernel
     want = _oracle(cfg, grad)
     gen = T.run_capi_backward(cfg, grad, flags=2)   # the plain-FMA kernels
-    for name, g, w, x in zip(("dq", "dk", "dv"), got, want, gen):
+    assert T.last_backward_kernel.startswith("generic_bwd_"), T.last_backward_kernel
+    names = ("dq", "dk", "dv", "dbias") if cfg.get("attn_bias") is not None else ("dq", "dk", "dv")
+    for name, g, w, x in zip(names, got, want, gen):
         T.assert_parity(g, w, dtype, what=f"mfma backward {name}")
         T.assert_parity(g, x.double(), dtype, what=f"mfma vs plain kernels {name}")
+    if cfg.get("attn_bias") is not None:
+        # dBias is written completely: exact zeros wherever the oracle has none (behind the sequences, under the mask)
+        assert bool((got[3][want[3] == 0] == 0).all())
 
 
 def test_backward_mfma_sequences_longer_than_the_attribute():

@@ -132,6 +132,7 @@ def test_describe_kernel_selection():
                        (dict(dtype=_capi.HSTU_F32), "generic_f32"), (dict(dim_v=64), "generic_bf16"),
                        (dict(dim_qk=32, dim_v=32), "mfma_bf16_d32"), (dict(dim_qk=256, dim_v=256, dtype=_capi.HSTU_F16), "mfma_f16_d256"),
                        (dict(dim_qk=96, dim_v=96), "generic_bf16"),
+                       (dict(q=0x1002), "generic_bf16"), (dict(out=0x1008), "generic_bf16"),   # not on a 16-byte boundary
                        (dict(flags=_capi.FLAG_FORCE_GENERIC), "generic_bf16")]:
         p = _params(**over)
         assert lib.hstu_hip_describe_kernel(C.byref(p), buf, 64) == 0
@@ -286,7 +287,11 @@ def test_backward_validation_and_workspace():
     rc, n, msg = _bwd_ws(_bwd_params(dtype=_capi.HSTU_F32))  # plain kernels: nothing to stage
     assert rc == 0 and n == 0, msg
     rc, n, msg = _bwd_ws(_bwd_params(attn_bias=0x1000, grad_bias=0x1000))
-    assert rc == 0 and n == 0, msg                           # dense bias -> plain kernels
+    assert rc == 0 and n == 1024, msg                        # dense bias whose rows are a multiple of 8 elements: MFMA kernels too
+    rc, n, msg = _bwd_ws(_bwd_params(attn_bias=0x1000, grad_bias=0x1000, max_seq_len_q=60, max_seq_len_k=60))
+    assert rc == 0 and n == 0, msg                           # rows of 60 elements -> plain kernels
+    rc, n, msg = _bwd_ws(_bwd_params(mask=0x1000, mask_type=3))
+    assert rc == 0 and n == 0, msg                           # custom mask -> plain kernels
     rc, _, msg = _bwd_ws(_bwd_params(attn_bias=0x1000))
     assert rc == -1 and "grad_bias must be given exactly when attn_bias is" in msg
     rc, _, msg = _bwd_ws(_bwd_params(grad_bias=0x1000))

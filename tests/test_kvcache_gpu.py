@@ -88,6 +88,10 @@ def test_append_skips_what_points_outside_and_honours_the_device_count():
     table = c["kv_cache"].cuda()
     _append(short, bi, pos, table)
     assert np.array_equal(table.cpu().view(torch.int16).numpy(), want)
+    # the host-side nnz is only a hint (the reference's binding ignores it, pybind.cpp:57-61): a stale 0 loses nothing
+    table = c["kv_cache"].cuda()
+    _append(c, bi, pos, table, nnz=0)
+    assert np.array_equal(table.cpu().view(torch.int16).numpy(), _oracle(c)[2])
     # corrupt three tokens of a fresh append
     bad = dict(c, kv_indices=c["kv_indices"].clone())
     first_page_u0 = int(bad["kv_indices"][0])

@@ -217,6 +217,27 @@ def test_paged_fp8_cache():
     assert torch.equal(T.run_op(cfg, op="paged_fp8"), T.run_capi(cfg, op="paged", use_fp8=True)[0])
 
 
+def test_buffers_off_a_16_byte_boundary_take_the_plain_kernel():
+    """q (or any of k, v, out) starting 2 bytes past a 16-byte boundary: the MFMA kernels' 16-byte accesses do not apply,
+    the call is routed to the plain kernel and the result is the same."""
+    say("misaligned")
+    from recsdk_amd import _capi
+    dtype = torch.bfloat16
+    cfg, _ = _jag(81, [70, 200, 33], 2, 2, 128, 128, dtype)
+    q = cfg["q"].cuda()
+    buf = torch.empty(q.numel() + 8, dtype=dtype, device="cuda")
+    q_off = buf[1:1 + q.numel()].view_as(q)
+    q_off.copy_(q)
+    assert q_off.data_ptr() % 16 == 2
+    out = torch.full_like(q, float("nan"))
+    p, keep = _capi.make_params(q_off, cfg["k"].cuda(), cfg["v"].cuda(), out, seq_offset_q=cfg["seq_offset"].cuda(),
+                                max_seq_len_q=cfg["max_seq_len"], alpha=cfg["alpha"])
+    assert _capi.describe_kernel(p) == "generic_bf16"
+    _capi.run("jagged", p)
+    torch.cuda.synchronize()
+    T.assert_parity(out.cpu(), T.oracle_jagged(cfg), dtype, what="misaligned q")
+
+
 def test_error_paths_on_device():
     """Host rejections surface as RuntimeError with the reference's messages (test_hstu_jagged_forward.py:508-711)."""
     say("errors")
