@@ -19,6 +19,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_FP8_TFLOPS = 5000.0    # MI355X dense fp8 MFMA
 PEAK_HBM_GBS = 8000.0
 # HBM-side bytes per launch from rocprofv3 FETCH_SIZE/WRITE_SIZE, each scaled by what the same counter reads for the
 # plain 256 MiB copy of `--workload copy` (factors 2.000 and 1.000); see profiles/*.md
@@ -32,6 +33,15 @@ MEASURED_TRAFFIC_BYTES = {"config2": 184.3e6, "kv_append": 351.9e6, "rab_time": 
 
 
 def build_workload(name, torch, W):
+    if name.endswith("_fp8"):
+        # the same geometry with float8_e4m3fn q / k / v drawn like the reference's fp8 tests (uniform(-1, 1) rounded to
+        # e4m3, test_hstu_jagged_forward.py:61-86) and fp16 output: 3 one-byte rows in, 1 two-byte row out
+        c, op, flops, b, desc = build_workload(name[:-4], torch, W)
+        g = torch.Generator().manual_seed(11)
+        for x in "qkv":
+            c[x] = (torch.rand(c[x].shape, generator=g) * 2 - 1).to(torch.float8_e4m3fn)
+        c.setdefault("silu_scale", 1.0 / 64)   # keeps P above the subnormals of e4m3
+        return c, op, flops, b * 5 // 8, desc.replace("bf16", "float8_e4m3fn in / fp16 out") + ", uniform(-1,1) data, silu_scale=" + f"{c['silu_scale']:.6f}"
     if name == "config2":
         c = W.config2()
         flops = W.headline_flops(c["lens"], 4, 128)
@@ -73,7 +83,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=1000)
-    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "ref_bias", "ref_nobias", "config2_bwd", "kv_append", "kv_append_fp8", "rab_time", "rab_time_bwd", "rab_pos", "nmd_fwd", "nmd_bwd", "in_linear_silu", "in_linear_silu_bwd", "copy"],
+    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "ref_bias", "ref_nobias", "config2_fp8", "ref_nobias_fp8", "config2_bwd", "kv_append", "kv_append_fp8", "rab_time", "rab_time_bwd", "rab_pos", "nmd_fwd", "nmd_bwd", "in_linear_silu", "in_linear_silu_bwd", "copy"],
                     help="'copy' runs a plain 256 MiB device copy: the known-size kernel the FETCH_SIZE/WRITE_SIZE counters are scaled by")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--settle-ms", type=float, default=80.0,
@@ -107,7 +117,9 @@ def main():
     cfg, op, flops, alg_bytes, desc = build_workload(args.workload, torch, W)
     dev = W.to_device(cfg)
     q, k, v = dev["q"], dev["k"], dev["v"]
-    out = torch.empty_like(q)
+    out = torch.empty(q.shape, dtype=_capi.out_dtype(q.dtype), device=q.device)
+    fp8 = q.dtype == torch.float8_e4m3fn
+    peak = PEAK_FP8_TFLOPS if fp8 else PEAK_BF16_TFLOPS
     kw = dict(seq_offset_q=dev["seq_offset"], seq_offset_k=dev.get("seq_offset_k"), max_seq_len_q=cfg["max_seq_len"],
               max_seq_len_k=cfg.get("max_seq_len_k"), mask_type=0, alpha=cfg["alpha"], num_target=dev.get("num_target"),
               attn_bias=dev.get("attn_bias"), silu_scale=cfg.get("silu_scale", 0.0),
@@ -157,12 +169,12 @@ def main():
     result = {
         "metric": "hstu_jagged_attn_fwd_tflops", "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "us_per_call": round(ms_per_step * 1e3, 2), "pct_bf16_mfma_peak": round(100 * tflops / PEAK_BF16_TFLOPS, 2),
+        "scaling": "weak", "vs_baseline": None, "dtype": "fp8_e4m3" if fp8 else "bf16", "data": "synthetic",
+        "us_per_call": round(ms_per_step * 1e3, 2), ("pct_fp8_mfma_peak" if fp8 else "pct_bf16_mfma_peak"): round(100 * tflops / peak, 2),
         "config": {"workload": desc, "kernel": kernel, "flops_per_call": flops, "algorithmic_bytes_per_call": alg_bytes,
                    "entry": f"hstu_hip_{op}_forward (C ABI)", "l2_flushed_between_calls": False},
-        "roofline": {"bound": "mfma", "achieved": round(kern_tflops, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(kern_tflops / PEAK_BF16_TFLOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+        "roofline": {"bound": "mfma", "achieved": round(kern_tflops, 2), "peak": peak, "unit": "TFLOP/s",
+                     "frac": round(kern_tflops / peak, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
                      "traffic_source": TRAFFIC_SOURCE.get(args.workload),
                      "kernel_us": round(kern_ms * 1e3, 2),
                      "hbm_algorithmic_gbs": round(alg_bytes / (kern_ms * 1e-3) / 1e9, 1),
@@ -688,7 +700,7 @@ def cpu_baseline(cfg, op, flops, torch, workload, W):
         f = (lambda: T.oracle_paged(cfg)) if op == "paged" else (lambda: T.oracle_jagged(cfg, mode="lowp"))
         sec = _median_seconds(f, runs=2 if op == "paged" else 5)
         return {"value": round(flops / sec / 1e12, 4), "unit": "TFLOP/s", "cores": n, "kind": "port",
-                "sample": f"the whole batch of this workload once (bf16 I/O, the golden's rounding points), {sec:.2f} s on {n} threads",
+                "sample": f"the whole batch of this workload once (its I/O dtype, the golden's rounding points), {sec:.2f} s on {n} threads",
                 "seconds_per_call": round(sec, 3)}
     detail = {}
     c1 = W.config1()

@@ -20,6 +20,9 @@ Definition followed (reference file:line):
 * built-in mask (causal with delta = Lk-Lq, context rows, target groups)
   -- cust_op/test/hstu_dense/torch/test_target_mask.py:260-288 and
   .../op_kernel/hstu_dense_causal_mask.h:63-117,204-237
+* fp8 inputs (float8_e4m3fn q/k/v, the reference's Ascend-950 path): operands up-cast to fp32, score math in
+  fp32, P (after silu_scale and mask) rounded to e4m3 and back, PV in fp32, fp16 out
+  -- test_hstu_jagged_forward.py:150-189 (``use_float8``), plugin hstu_jagged.cpp:53-54
 * GQA = repeat_interleave of K/V heads -- test_hstu_jagged_forward.py:155-159
 * defaults ``silu_scale==0 -> 1/max_seq_len_q``, ``alpha -> 1.0``
   -- cust_op/framework/torch_plugin/torch_library/hstu/hstu_jagged.cpp:43-61
@@ -42,6 +45,9 @@ formulas; the checks live in tests/test_oracle_*.py):
   (linearity in V and silu_scale, alpha=0, batch permutation, causality,
   B=1 dense==jagged, explicit tril mask == mask_type 0, GQA ==
   repeat_interleave).                                                     PINNED
+* fp8 branch of ``hstu_jagged_forward`` (mode "lowp" on float8_e4m3fn inputs): brute-force loop whose e4m3
+  rounding is an independent numpy implementation (round to nearest even on the 3-bit mantissa grid,
+  subnormals below 2^-6), tests/test_oracle_forward.py.                    PINNED
 * ``hstu_paged_forward``: equivalence with the delta-q jagged op on the
   de-paged K/V.                                                           PINNED
 * ``hstu_jagged_backward``: torch.autograd of ``hstu_jagged_forward`` in
@@ -231,6 +237,12 @@ def hstu_jagged_forward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, seq_o
     if mask_type == MASK_CUSTOM and mask is None:
         raise ValueError("custom mask needs a mask tensor")
     io_dtype = q.dtype
+    fp8 = io_dtype == torch.float8_e4m3fn
+    if fp8:
+        # the reference's use_float8 golden: fp32 operands, P through e4m3, fp16 out (test_hstu_jagged_forward.py:150-189)
+        q, k, v = q.to(torch.float32), k.to(torch.float32), v.to(torch.float32)
+        if attn_bias is not None:
+            attn_bias = attn_bias.to(torch.float32)
     nq, nk, dv = q.shape[1], k.shape[1], v.shape[2]
     assert nq % nk == 0
     ratio = nq // nk
@@ -242,7 +254,7 @@ def hstu_jagged_forward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, seq_o
 
     exact = mode == "exact"
     cd = compute_dtype if exact else torch.float32
-    out = torch.zeros(q.shape[0], nq, dv, dtype=cd if exact else io_dtype)
+    out = torch.zeros(q.shape[0], nq, dv, dtype=cd if exact else (torch.float32 if fp8 else io_dtype))
     for b in range(nb):
         lq, lk = int(oq[b + 1] - oq[b]), int(okk[b + 1] - okk[b])
         if lq == 0 or lk == 0:
@@ -264,10 +276,14 @@ def hstu_jagged_forward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, seq_o
         else:
             s = torch.matmul(qb, kb.transpose(1, 2)).to(torch.float32)
             p = _score_to_p(s, bias, alpha, scale, m).to(io_dtype)
+            if fp8:
+                p = p.to(torch.float32)
             ob = torch.matmul(p, vb)
         out[oq[b]: oq[b] + lq] = ob.permute(1, 0, 2)
     if out_dtype is not None:
         out = out.to(out_dtype)
+    elif fp8 and not exact:
+        out = out.to(torch.float16)
     return out
 
 

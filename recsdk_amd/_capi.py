@@ -183,7 +183,12 @@ def lib() -> C.CDLL:
     return _lib
 
 
-_DT = {torch.float32: HSTU_F32, torch.float16: HSTU_F16, torch.bfloat16: HSTU_BF16}
+_DT = {torch.float32: HSTU_F32, torch.float16: HSTU_F16, torch.bfloat16: HSTU_BF16, torch.float8_e4m3fn: HSTU_FP8_E4M3}
+
+
+def out_dtype(in_dtype):
+    """dtype of the forward's output for q/k/v of ``in_dtype`` (fp16 for float8_e4m3fn, reference hstu_jagged.cpp:53-54)."""
+    return torch.float16 if in_dtype == torch.float8_e4m3fn else in_dtype
 
 
 def _ptr(t):

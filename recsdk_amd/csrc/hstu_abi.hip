@@ -56,8 +56,10 @@ static int validate(const hstu_fwd_params* p, int op, KArgs* out, bool need_out 
     if (p->struct_size != sizeof(hstu_fwd_params))
         return fail(HSTU_ERR_INVALID_ARGUMENT, "hstu_fwd_params size mismatch: caller %u, library %zu (ABI version %d)",
                     p->struct_size, sizeof(hstu_fwd_params), HSTU_HIP_ABI_VERSION);
-    if (p->dtype != HSTU_F32 && p->dtype != HSTU_F16 && p->dtype != HSTU_BF16)
-        return fail(HSTU_ERR_INVALID_ARGUMENT, "dtype expect float32, float16 or bfloat16, but value is %d", p->dtype);
+    if (p->dtype != HSTU_F32 && p->dtype != HSTU_F16 && p->dtype != HSTU_BF16 && p->dtype != HSTU_FP8_E4M3)
+        return fail(HSTU_ERR_INVALID_ARGUMENT, "dtype expect float32, float16, bfloat16 or float8_e4m3fn, but value is %d", p->dtype);
+    if (p->dtype == HSTU_FP8_E4M3 && op == OP_PAGED)
+        return fail(HSTU_ERR_UNSUPPORTED, "float8_e4m3fn q/k/v are taken by the jagged and dense forward only (the paged op takes an fp8 cache)");
     if (p->index_type != HSTU_I32 && p->index_type != HSTU_I64)
         return fail(HSTU_ERR_INVALID_ARGUMENT, "index_type expect int32 or int64, but value is %d", p->index_type);
     if (!p->q || !p->k || !p->v || (need_out && !p->out)) return fail(HSTU_ERR_INVALID_ARGUMENT, "q, k, v and out must not be NULL");
@@ -170,6 +172,7 @@ static int validate_backward(const hstu_bwd_params* p, int op, BArgs* out) {
                     p->struct_size, sizeof(hstu_bwd_params), HSTU_HIP_ABI_VERSION);
     int rc = validate(&p->fwd, op, &out->f, false);
     if (rc != HSTU_OK) return rc;
+    if (p->fwd.dtype == HSTU_FP8_E4M3) return fail(HSTU_ERR_UNSUPPORTED, "the backward takes float32, float16 or bfloat16 (float8_e4m3fn is forward only)");
     if (p->fwd.pos_table || p->fwd.ts_table)
         return fail(HSTU_ERR_UNSUPPORTED, "the backward takes a dense attn_bias only (no bias tables)");
     if (!p->grad_out || !p->grad_q || !p->grad_k || !p->grad_v)
@@ -269,7 +272,7 @@ int hstu_hip_describe_kernel(const hstu_fwd_params* p, char* buf, size_t n) {
     if (rc != HSTU_OK) return rc;
     const char* name = nullptr;
     if ((p->flags & HSTU_FLAG_FORCE_GENERIC) || !mfma_supported(a, &name)) {
-        name = p->dtype == HSTU_F32 ? "generic_f32" : (p->dtype == HSTU_F16 ? "generic_f16" : "generic_bf16");
+        name = p->dtype == HSTU_F32 ? "generic_f32" : (p->dtype == HSTU_F16 ? "generic_f16" : (p->dtype == HSTU_BF16 ? "generic_bf16" : "generic_fp8"));
     }
     snprintf(buf, n, "%s", name);
     return HSTU_OK;

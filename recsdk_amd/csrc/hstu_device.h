@@ -16,6 +16,22 @@ __device__ __forceinline__ float to_float(_Float16 x) { return (float)x; }
 __device__ __forceinline__ float to_float(__bf16 x) { return (float)x; }
 template <typename T> __device__ __forceinline__ T from_float(float x) { return (T)x; }
 
+// float8_e4m3fn element of q / k / v / mask / attn_bias (the reference's fp8 path: hstu_jagged.cpp:53-54): scores and
+// sums stay in fp32, P is rounded to e4m3 (to nearest even) before P*V, the output is fp16.
+struct fp8e4 { uint8_t v; };
+__device__ __forceinline__ float to_float(fp8e4 x) {
+    f32x2 r = __builtin_amdgcn_cvt_pk_f32_fp8((int)x.v, false);
+    return r[0];
+}
+template <> __device__ __forceinline__ fp8e4 from_float<fp8e4>(float x) {
+    fp8e4 r;
+    r.v = (uint8_t)(__builtin_amdgcn_cvt_pk_fp8_f32(x, 0.f, 0, false) & 0xff);
+    return r;
+}
+// element type of `out` for inputs of type T
+template <typename T> struct OutOf { typedef T type; };
+template <> struct OutOf<fp8e4> { typedef _Float16 type; };
+
 // Geometry of one sequence.  Q row i sits at K position i + delta.
 struct Seq {
     int64_t q_start;   // first row of the sequence in q / out

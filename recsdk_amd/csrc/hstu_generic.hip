@@ -1,7 +1,7 @@
 // Full-feature HSTU forward kernel in plain fp32 FMA arithmetic.
 //
-// Covers everything the op accepts (fp32/fp16/bf16 I/O, any head dim <= 512, Dqk != Dv, GQA, delta-q,
-// context/target masks, custom mask, dense bias, bias tables, paged and fp8 caches).  It is the path
+// Covers everything the op accepts (fp32/fp16/bf16 I/O, float8_e4m3fn inputs with fp16 output, any head dim <= 512,
+// Dqk != Dv, GQA, delta-q, context/target masks, custom mask, dense bias, bias tables, paged and fp8 caches).  It is the path
 // for fp32 I/O (where bf16 MFMA cannot meet 1e-5) and for shapes the MFMA kernels do not specialise.
 // Element-wise order follows the reference's vector pass (vector_score_inter.h:299-323,186-212):
 //   x = alpha*(S + bias);  p = x*sigmoid(x);  p *= silu_scale*mask;  P = round_to_io_dtype(p).
@@ -70,7 +70,8 @@ __global__ __launch_bounds__(256) void hstu_generic_kernel(const KArgs a) {
     const int hk = h / a.head_ratio;
     const Seq s = load_seq(a, b);
     const T* q = reinterpret_cast<const T*>(p.q);
-    T* out = reinterpret_cast<T*>(p.out);
+    typedef typename OutOf<T>::type OT;
+    OT* out = reinterpret_cast<OT*>(p.out);
     const int r = tid / 16, cb = tid % 16;
     const int is_tril = p.mask_type == HSTU_MASK_TRIL;
     const int64_t bh = (int64_t)b * p.heads_q + h;
@@ -185,7 +186,7 @@ __global__ __launch_bounds__(256) void hstu_generic_kernel(const KArgs a) {
 #pragma unroll
                 for (int jj = 0; jj < 4; jj++) {
                     int d = ch * GDC + cb + 16 * jj;
-                    if (d < p.dim_v) out[((s.q_start + i) * p.heads_q + h) * (int64_t)p.dim_v + d] = from_float<T>(oacc[ch * 4 + jj]);
+                    if (d < p.dim_v) out[((s.q_start + i) * p.heads_q + h) * (int64_t)p.dim_v + d] = from_float<OT>(oacc[ch * 4 + jj]);
                 }
             }
         }
@@ -201,8 +202,8 @@ __global__ __launch_bounds__(256) void hstu_generic_kernel(const KArgs a) {
             int64_t n = (p.total_q - tail) * p.heads_q * (int64_t)p.dim_v;
             int64_t nblk = (int64_t)gridDim.x * gridDim.y * gridDim.z;
             int64_t blk = ((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
-            T* o = out + tail * p.heads_q * (int64_t)p.dim_v;
-            for (int64_t e = blk * 256 + tid; e < n; e += nblk * 256) o[e] = from_float<T>(0.f);
+            OT* o = out + tail * p.heads_q * (int64_t)p.dim_v;
+            for (int64_t e = blk * 256 + tid; e < n; e += nblk * 256) o[e] = from_float<OT>(0.f);
         }
     }
 }
@@ -217,6 +218,7 @@ hipError_t launch_generic(const KArgs& a, hipStream_t stream) {
         case HSTU_F32: hipLaunchKernelGGL(hstu_generic_kernel<float>, grid, dim3(256), lds, stream, a); break;
         case HSTU_F16: hipLaunchKernelGGL(hstu_generic_kernel<_Float16>, grid, dim3(256), lds, stream, a); break;
         case HSTU_BF16: hipLaunchKernelGGL(hstu_generic_kernel<__bf16>, grid, dim3(256), lds, stream, a); break;
+        case HSTU_FP8_E4M3: hipLaunchKernelGGL(hstu_generic_kernel<fp8e4>, grid, dim3(256), lds, stream, a); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

@@ -31,6 +31,10 @@ bool mfma_supported(const KArgs& a, const char** name);
 // bytes of device workspace the MFMA path needs for its work list; the buffer needs no initialisation
 uint64_t mfma_workspace_bytes(const KArgs& a);
 hipError_t launch_mfma(const KArgs& a, void* workspace, hipStream_t stream);
+// the same three for float8_e4m3fn q / k / v (reached through the three above)
+bool mfma_fp8_supported(const KArgs& a, const char** name);
+uint64_t mfma_fp8_workspace_bytes(const KArgs& a);
+hipError_t launch_mfma_fp8(const KArgs& a, void* workspace, hipStream_t stream);
 
 // The device-built work list of the MFMA kernels, for kernels outside hstu_mfma.hip.  Layout (uint32 words): 16 header
 // words ([2..3] = rows the sequences own, int64), then `grid` records of 8 words, read by workgroup index:

@@ -208,6 +208,7 @@ static uint64_t list_bytes(const SchedDims& d) {
 }
 
 uint64_t mfma_workspace_bytes(const KArgs& a) {
+    if (a.p.dtype == HSTU_FP8_E4M3) return mfma_fp8_workspace_bytes(a);
     const SchedDims d = sched_dims(a.p);
     uint64_t b = list_bytes(d);
     if (d.nsplit > 1) b += (uint64_t)d.nsplit * a.p.total_q * a.p.heads_q * a.p.dim_v * sizeof(float);   // partial sums
@@ -983,6 +984,7 @@ void hstu_reduce_kernel(const KArgs a, const float* __restrict__ part, const int
 bool mfma_supported(const KArgs& a, const char** name) {
     const hstu_fwd_params& p = a.p;
     *name = nullptr;
+    if (p.dtype == HSTU_FP8_E4M3) return mfma_fp8_supported(a, name);
     if (p.dtype != HSTU_BF16 && p.dtype != HSTU_F16) return false;
     const int d = p.dim_qk;
     if (d != p.dim_v || (d != 32 && d != 64 && d != 128 && d != 256)) return false;
@@ -1060,6 +1062,7 @@ static hipError_t launch_td(const KArgs& a, unsigned* ws, hipStream_t stream) {
 hipError_t launch_mfma(const KArgs& a, void* workspace, hipStream_t stream) {
     const hstu_fwd_params& p = a.p;
     unsigned* ws = reinterpret_cast<unsigned*>(workspace);
+    if (p.dtype == HSTU_FP8_E4M3) return launch_mfma_fp8(a, workspace, stream);
     if (p.dtype == HSTU_BF16) {
         switch (p.dim_qk) {
             case 32: return launch_td<__bf16, 32>(a, ws, stream);

@@ -1,0 +1,304 @@
+// HSTU forward for float8_e4m3fn q / k / v on the gfx950 matrix cores (head dim 64, 128 or 256, built-in mask or none,
+// GQA, delta-q; fp16 output).  The reference's fp8 path: hstu_jagged.cpp:53-54 (fp16 output for fp8 inputs), golden
+// test_hstu_jagged_forward.py:150-189: operands up-cast exactly, scores and sums in fp32, P = silu(alpha * S) * silu_scale
+// * mask rounded to e4m3 before P V.
+//
+// Same scheme as the 16-bit kernel, on v_mfma_f32_32x32x64_f8f6f4 (64 products per lane and instruction, twice the
+// 16-bit rate): a workgroup (4 waves) owns a 128-row Q tile of one (sequence, head), wave w rows 32w..32w+31; K and V
+// tiles of 64 keys stream through LDS (two stages, fetched into registers one tile ahead, one barrier per tile).
+// Per tile and wave:
+//     S^T = K Q^T      two 32-key blocks; A = K rows (32 bytes of the head dim per lane: 2 x ds_read_b128), B = Q rows
+//                      (registers).  Lane half g of both operands holds head-dim bytes 64t + 32g .. + 31: the k index of a
+//                      (lane half, byte) is the same for A and B, which is all a dot product needs.
+//     P                s * sigmoid(alpha * s) * alpha * silu_scale in fp32, rounded to e4m3 (v_cvt_pk_fp8_f32), masked
+//     O^T += V^T P^T   one instruction per 32 head-dim columns covers all 64 keys: B = the 32 P bytes of the lane, A = V^T
+//                      from four transposing reads (ds_read_b64_tr_b8: 8 consecutive keys of one column per lane)
+// A-row rho of an S^T block holds key (rho with bits 2 and 3 swapped): accumulator registers 8u..8u+7 of lane half g are
+// then keys 16u + 8g .. + 7 of the block, 8 consecutive keys per transposing read.  alpha * silu_scale cannot move to the
+// epilogue here: it decides where P falls on the e4m3 grid.
+#include "hstu_device.h"
+
+namespace hstu {
+
+typedef __attribute__((ext_vector_type(8))) int q_i32x8;
+typedef __attribute__((ext_vector_type(2))) int q_i32x2;
+typedef __attribute__((ext_vector_type(4))) unsigned int q_u32x4;
+typedef __attribute__((ext_vector_type(2))) unsigned int q_u32x2;
+typedef __attribute__((ext_vector_type(16))) float q_f32x16;
+typedef __attribute__((ext_vector_type(2))) _Float16 q_f16x2;
+
+#define FP8_LDS_PTR(type, p) ((__attribute__((address_space(3))) type*)(p))
+
+constexpr int FBM = 128;   // Q rows per workgroup
+constexpr int FBN = 64;    // keys per step
+
+enum { FBLK_ALL = 0, FBLK_CAUSAL = 1, FBLK_PRED = 2, FBLK_SKIP = 3 };
+
+// visibility class of Q rows r0..r0+31 against keys c0..c0+31 under the built-in mask
+__device__ __forceinline__ int fp8_classify(const Seq& s, int tgs, int r0, int c0) {
+    const bool has_ctx = s.ctx > 0 && r0 < s.ctx;
+    const bool has_tgt = s.tgt > 0 && tgs > 0 && r0 + 31 >= s.hist_q && c0 + 31 >= s.hist_k;
+    if (!has_ctx && c0 > r0 + 31 + s.delta) return FBLK_SKIP;
+    if (has_ctx || has_tgt) return FBLK_PRED;
+    if (c0 + 31 <= r0 + s.delta) return FBLK_ALL;
+    return FBLK_CAUSAL;
+}
+
+template <int D>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 1 : 2, D == 256 ? 1 : 2)))
+void hstu_mfma_fp8_kernel(const KArgs a, const unsigned* __restrict__ ws) {
+    const hstu_fwd_params& p = a.p;
+    // row strides in bytes: +16 keeps the 16-byte row-wise reads of 16 K rows on distinct banks, +32 does the same for
+    // the 8-row transposing reads of V
+    constexpr int KS = D + 16, VS = D + 32;
+    constexpr int NCH = D / 64;          // 16-byte chunks per thread, tile and tensor
+    constexpr int CPR = D / 16;          // chunks per row
+    __shared__ __attribute__((aligned(16))) unsigned char kst[2][FBN * KS];
+    __shared__ __attribute__((aligned(16))) unsigned char vst[2][FBN * VS];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int g = lane >> 5, l32 = lane & 31;
+
+    // workgroup -> record of the device-built work list
+    unsigned rw[WORK_RECORD_WORDS];
+    {
+        const unsigned* rec = ws + WORK_HEADER_WORDS + WORK_RECORD_WORDS * (size_t)blockIdx.x;
+#pragma unroll
+        for (int i = 0; i < WORK_RECORD_WORDS; i++) rw[i] = rec[i];
+    }
+    const int64_t owned_rows = *reinterpret_cast<const int64_t*>(ws + 2);
+    const unsigned item = rw[0];
+    const bool active = item != WORK_ITEM_EMPTY;
+    const int b = active ? (int)(item & 0xfff) : 0, h = active ? (int)((item >> 12) & 0xf) : 0;
+    const int tile0 = (int)((item >> 16) & 0xff);
+    const int tile_last = ((item >> 24) & 1) ? 0x7fffff : tile0 + (int)((item >> 25) & 7);
+    const int hk = h / a.head_ratio;
+    Seq s;
+    s.q_start = active ? (int)rw[1] : 0; s.lq = active ? (int)rw[2] : 0;
+    s.k_start = active ? (int)rw[3] : 0; s.lk = active ? (int)rw[4] : 0;
+    s.ctx = active ? (int)rw[5] : 0; s.tgt = active ? (int)rw[6] : 0; s.page0 = 0;
+    s.delta = s.lk - s.lq; s.hist_q = s.lq - s.tgt; s.hist_k = s.lk - s.tgt; s.cand_row = s.q_start + s.hist_q;
+    (void)b;
+    const bool tril = p.mask_type == HSTU_MASK_TRIL;
+    const int tgs = p.target_group_size;
+    const unsigned char* qbase = reinterpret_cast<const unsigned char*>(p.q);
+    const unsigned char* kbase = reinterpret_cast<const unsigned char*>(p.k);
+    const unsigned char* vbase = reinterpret_cast<const unsigned char*>(p.v);
+    _Float16* obase = reinterpret_cast<_Float16*>(p.out);
+
+    // K fragment: A-row l32 holds key (l32 with bits 2 and 3 swapped) of the block
+    const int krow = (l32 & 0x13) | ((l32 & 4) << 1) | ((l32 & 8) >> 1);
+    const int kfrag_off = krow * KS + 32 * g;
+    // V^T fragment: lane i of a 16-lane group addresses 8 bytes of key row i / 2; the group receives columns
+    // 16 * (group % 2) .. + 15, keys 8 * g .. + 7 of the 16-key step
+    const int vfrag_off = (8 * g + ((lane & 15) >> 1)) * VS + 16 * ((lane >> 4) & 1) + 8 * (lane & 1);
+
+    for (int tile = tile0; active && tile <= tile_last && tile * FBM < s.lq; tile++) {
+        const int i0 = tile * FBM;
+        const int kend = (s.lk > 0) ? k_extent(a, s, i0, min(i0 + FBM, s.lq)) : 0;
+        const int ntk = (kend + FBN - 1) / FBN;
+        const int r0 = i0 + 32 * w;
+        const int qi = r0 + l32;
+        const bool qvalid = qi < s.lq;
+
+        // Q fragments (B operand of S^T = K Q^T): column = Q row, lane half g holds head-dim bytes 64t + 32g .. + 31
+        q_i32x8 qf[D / 64];
+        {
+            const unsigned char* qp = qbase + ((s.q_start + min(qi, s.lq - 1)) * p.heads_q + h) * (int64_t)D + 32 * g;
+#pragma unroll
+            for (int t = 0; t < D / 64; t++) {
+                const q_u32x4 z = {0, 0, 0, 0};
+                q_u32x4 x0 = *reinterpret_cast<const q_u32x4*>(qp + 64 * t);
+                q_u32x4 x1 = *reinterpret_cast<const q_u32x4*>(qp + 64 * t + 16);
+                x0 = qvalid ? x0 : z;
+                x1 = qvalid ? x1 : z;
+                qf[t] = (q_i32x8){(int)x0[0], (int)x0[1], (int)x0[2], (int)x0[3], (int)x1[0], (int)x1[1], (int)x1[2], (int)x1[3]};
+            }
+        }
+        q_f32x16 oacc[D / 32];
+#pragma unroll
+        for (int db = 0; db < D / 32; db++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) oacc[db][r] = 0.f;
+
+        q_u32x4 nk[NCH], nv[NCH];
+        auto fetch = [&](int kt) __attribute__((always_inline)) {
+#pragma unroll
+            for (int i = 0; i < NCH; i++) {
+                const int c = tid + 256 * i;
+                const int row = c / CPR, cc = c % CPR;
+                // nothing here waits for the data: rows past the end are zeroed when the tile is written to LDS
+                const int64_t e = ((s.k_start + min(kt * FBN + row, kend - 1)) * p.heads_k + hk) * (int64_t)D + 16 * cc;
+                nk[i] = *reinterpret_cast<const q_u32x4*>(kbase + e);
+                nv[i] = *reinterpret_cast<const q_u32x4*>(vbase + e);
+            }
+        };
+        auto stash = [&](int kt, int stage) __attribute__((always_inline)) {
+#pragma unroll
+            for (int i = 0; i < NCH; i++) {
+                const int c = tid + 256 * i;
+                const int row = c / CPR, cc = c % CPR;
+                const bool ok = kt * FBN + row < kend;   // zero rows: S = 0 gives P = 0, and 0 * V must not meet a NaN
+                const q_u32x4 z = {0, 0, 0, 0};
+                *reinterpret_cast<q_u32x4*>(kst[stage] + row * KS + 16 * cc) = ok ? nk[i] : z;
+                *reinterpret_cast<q_u32x4*>(vst[stage] + row * VS + 16 * cc) = ok ? nv[i] : z;
+            }
+        };
+        __syncthreads();   // every wave is done with the stages of the previous tile
+        if (ntk > 0) {
+            fetch(0);
+            stash(0, 0);
+        }
+        __syncthreads();
+
+        for (int kt = 0; kt < ntk; kt++) {
+            const int stage = kt & 1;
+            const int k0 = kt * FBN;
+            if (kt + 1 < ntk) fetch(kt + 1);
+            int cls[2];
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++) {
+                const int c0 = k0 + 32 * kb;
+                cls[kb] = c0 >= kend ? FBLK_SKIP : (tril ? fp8_classify(s, tgs, r0, c0) : FBLK_ALL);   // wave-uniform
+            }
+            if (cls[0] != FBLK_SKIP || cls[1] != FBLK_SKIP) {
+                const unsigned char* kt_lds = kst[stage];
+                const unsigned char* vt_lds = vst[stage];
+                unsigned pq[8];   // P of this lane's Q row: byte 8c + s = key k0 + 16c + 8g + s
+#pragma unroll
+                for (int kb = 0; kb < 2; kb++) {
+                    if (cls[kb] == FBLK_SKIP) {
+#pragma unroll
+                        for (int x = 0; x < 4; x++) pq[4 * kb + x] = 0u;
+                        continue;
+                    }
+                    q_i32x8 kf[D / 64];
+#pragma unroll
+                    for (int t = 0; t < D / 64; t++) {
+                        const unsigned char* at = kt_lds + 32 * kb * KS + kfrag_off + 64 * t;
+                        const q_u32x4 x0 = *reinterpret_cast<const q_u32x4*>(at);
+                        const q_u32x4 x1 = *reinterpret_cast<const q_u32x4*>(at + 16);
+                        kf[t] = (q_i32x8){(int)x0[0], (int)x0[1], (int)x0[2], (int)x0[3], (int)x1[0], (int)x1[1], (int)x1[2], (int)x1[3]};
+                    }
+                    q_f32x16 sacc;
+#pragma unroll
+                    for (int r = 0; r < 16; r++) sacc[r] = 0.f;
+#pragma unroll
+                    for (int t = 0; t < D / 64; t++)
+                        sacc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf[t], qf[t], sacc, 0, 0, 0, 0, 0, 0);
+                    // P = x * sigmoid(alpha * x) * alpha * silu_scale, to e4m3: register 8u + i of the block -> byte i of step u
+#pragma unroll
+                    for (int x = 0; x < 4; x++) {
+                        float pv[4];
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            const float sc = sacc[4 * x + i];
+                            const float e = __builtin_amdgcn_exp2f(sc * a.exp_scale);
+                            pv[i] = sc * __builtin_amdgcn_rcpf(1.0f + e) * a.out_scale;
+                        }
+                        int word = __builtin_amdgcn_cvt_pk_fp8_f32(pv[0], pv[1], 0, false);
+                        word = __builtin_amdgcn_cvt_pk_fp8_f32(pv[2], pv[3], word, true);
+                        pq[4 * kb + x] = (unsigned)word;
+                    }
+                    // word x of the block covers keys c0 + 16 * (x / 2) + 8g + 4 * (x % 2) .. + 3
+                    const int c0 = k0 + 32 * kb;
+                    if (cls[kb] == FBLK_CAUSAL) {
+#pragma unroll
+                        for (int x = 0; x < 4; x++) {
+                            const int lim = qi + s.delta - (c0 + 16 * (x >> 1) + 8 * g + 4 * (x & 1));   // key offset o of the word is visible iff o <= lim
+                            pq[4 * kb + x] &= lim >= 3 ? 0xffffffffu : (lim < 0 ? 0u : (0xffffffffu >> (8 * (3 - lim))));
+                        }
+                    } else if (cls[kb] == FBLK_PRED) {
+                        // branch-free form of builtin_visible()
+                        const bool ctx_row = s.ctx > 0 && qi < s.ctx;
+                        const bool tgt_row = tgs > 0 && s.tgt > 0 && qi >= s.hist_q;
+                        const int left = tgt_row ? s.hist_k + ((qi - s.hist_q) / tgs) * tgs : 0;   // first visible target column
+                        const int jmax = qi + s.delta;
+#pragma unroll
+                        for (int x = 0; x < 4; x++) {
+                            unsigned m = 0;
+#pragma unroll
+                            for (int i = 0; i < 4; i++) {
+                                const int j = c0 + 16 * (x >> 1) + 8 * g + 4 * (x & 1) + i;
+                                const bool vis = (ctx_row & (j < s.hist_k)) | ((j <= jmax) & !(tgt_row & (j >= s.hist_k) & (j < left)));
+                                m |= vis ? (0xffu << (8 * i)) : 0u;
+                            }
+                            pq[4 * kb + x] &= m;
+                        }
+                    }
+                }
+                const q_i32x8 pb = {(int)pq[0], (int)pq[1], (int)pq[2], (int)pq[3], (int)pq[4], (int)pq[5], (int)pq[6], (int)pq[7]};
+                // ---- O^T += V^T P^T: 64 keys per instruction
+#pragma unroll
+                for (int db = 0; db < D / 32; db++) {
+                    q_i32x2 vq[4];
+#pragma unroll
+                    for (int c = 0; c < 4; c++)
+                        vq[c] = __builtin_amdgcn_ds_read_tr8_b64_v2i32(FP8_LDS_PTR(q_i32x2, vt_lds + 16 * c * VS + vfrag_off + 32 * db));
+                    const q_i32x8 va = {vq[0][0], vq[0][1], vq[1][0], vq[1][1], vq[2][0], vq[2][1], vq[3][0], vq[3][1]};
+                    oacc[db] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(va, pb, oacc[db], 0, 0, 0, 0, 0, 0);
+                }
+            }
+            if (kt + 1 < ntk) stash(kt + 1, stage ^ 1);
+            __syncthreads();
+        }
+
+        // epilogue: O^T accumulator register r of block db holds d = 32 * db + 8 * (r / 4) + 4g + r % 4 of row qi
+        if (qvalid) {
+            _Float16* op = obase + ((s.q_start + qi) * p.heads_q + h) * (int64_t)D + 4 * g;
+#pragma unroll
+            for (int db = 0; db < D / 32; db++) {
+#pragma unroll
+                for (int rr = 0; rr < 4; rr++) {
+                    q_f16x2 lo, hi;
+                    lo[0] = (_Float16)oacc[db][4 * rr]; lo[1] = (_Float16)oacc[db][4 * rr + 1];
+                    hi[0] = (_Float16)oacc[db][4 * rr + 2]; hi[1] = (_Float16)oacc[db][4 * rr + 3];
+                    const q_u32x2 o = {__builtin_bit_cast(unsigned, lo), __builtin_bit_cast(unsigned, hi)};
+                    *reinterpret_cast<q_u32x2*>(op + 32 * db + 8 * rr) = o;
+                }
+            }
+        }
+    }
+
+    // rows past the last offset are zero (the reference zero-fills its output: hstu_jagged.cpp:56-59)
+    if (owned_rows < p.total_q) {
+        const int64_t n = (p.total_q - owned_rows) * p.heads_q * (int64_t)D;
+        _Float16* o = obase + owned_rows * p.heads_q * (int64_t)D;
+        for (int64_t e = (int64_t)blockIdx.x * 256 + tid; e < n; e += (int64_t)gridDim.x * 256) o[e] = (_Float16)0.f;
+    }
+}
+
+bool mfma_fp8_supported(const KArgs& a, const char** name) {
+    const hstu_fwd_params& p = a.p;
+    *name = nullptr;
+    if (p.dtype != HSTU_FP8_E4M3 || a.op == OP_PAGED) return false;
+    const int d = p.dim_qk;
+    if (d != p.dim_v || (d != 64 && d != 128 && d != 256)) return false;
+    if (p.attn_bias || p.pos_table || p.ts_table || p.mask_type == HSTU_MASK_CUSTOM) return false;   // the plain kernel's
+    const uintptr_t all = reinterpret_cast<uintptr_t>(p.q) | reinterpret_cast<uintptr_t>(p.k) | reinterpret_cast<uintptr_t>(p.v) |
+                          reinterpret_cast<uintptr_t>(p.out);
+    if (all & 15) return false;   // rows are read 16 bytes at a time
+    *name = d == 64 ? "mfma_fp8_d64" : (d == 128 ? "mfma_fp8_d128" : "mfma_fp8_d256");
+    return true;
+}
+
+uint64_t mfma_fp8_workspace_bytes(const KArgs& a) { return work_list_shape(a.p).bytes; }
+
+hipError_t launch_mfma_fp8(const KArgs& a, void* workspace, hipStream_t stream) {
+    const hstu_fwd_params& p = a.p;
+    unsigned* ws = reinterpret_cast<unsigned*>(workspace);
+    if (!(p.flags & HSTU_FLAG_REUSE_WORKSPACE)) {
+        const hipError_t e = launch_work_list(a, ws, true, stream);
+        if (e != hipSuccess) return e;
+    }
+    const dim3 grid(work_list_shape(p).grid), block(256);
+    switch (p.dim_qk) {
+        case 64: hipLaunchKernelGGL(hstu_mfma_fp8_kernel<64>, grid, block, 0, stream, a, ws); break;
+        case 128: hipLaunchKernelGGL(hstu_mfma_fp8_kernel<128>, grid, block, 0, stream, a, ws); break;
+        default: hipLaunchKernelGGL(hstu_mfma_fp8_kernel<256>, grid, block, 0, stream, a, ws); break;
+    }
+    return hipGetLastError();
+}
+
+}  // namespace hstu

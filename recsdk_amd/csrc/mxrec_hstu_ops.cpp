@@ -38,15 +38,20 @@ static void max_seq_len_check(int64_t n) {
     TORCH_CHECK(n >= kMinSeqLen && n <= kMaxSeqLen, "maxSeqLen expect in [1, 20480], but value is ", n);
 }
 
-static int32_t io_dtype(const at::Tensor& t, const char* what) {
+// `fp8`: float8_e4m3fn is taken too (the forward of the jagged and dense ops: hstu_jagged.cpp:53-54, output in fp16)
+static int32_t io_dtype(const at::Tensor& t, const char* what, bool fp8 = false) {
     switch (t.scalar_type()) {
         case at::kFloat: return HSTU_F32;
         case at::kHalf: return HSTU_F16;
         case at::kBFloat16: return HSTU_BF16;
-        default: TORCH_CHECK(false, what, " dtype expect float32, float16 or bfloat16, but get ", t.scalar_type());
+        case at::kFloat8_e4m3fn:
+            if (fp8) return HSTU_FP8_E4M3;
+            [[fallthrough]];
+        default: TORCH_CHECK(false, what, " dtype expect float32, float16 or bfloat16", fp8 ? " or float8_e4m3fn" : "", ", but get ", t.scalar_type());
     }
     return -1;
 }
+static at::ScalarType out_type_of(const at::Tensor& q) { return q.scalar_type() == at::kFloat8_e4m3fn ? at::kHalf : q.scalar_type(); }
 
 static const void* ptr_or_null(const at::Tensor& t) { return t.defined() ? t.const_data_ptr() : nullptr; }
 
@@ -258,7 +263,7 @@ static at::Tensor jagged_forward_impl(const at::Tensor& q, const at::Tensor& k, 
     const bool mask_defined = mask.has_value() && mask->defined();
     mask_check(mask_type, mask_defined);
 
-    const int32_t dt = io_dtype(dq, "q");
+    const int32_t dt = io_dtype(dq, "q", grad == nullptr);
     TORCH_CHECK(dk.scalar_type() == dq.scalar_type() && dv.scalar_type() == dq.scalar_type(), "q, k, v dtype mismatch");
     TORCH_CHECK(dk.size(0) == dv.size(0), "K, V seqLens mismatch");
     TORCH_CHECK(dk.size(1) == dv.size(1), "K, V headNum mismatch");
@@ -318,7 +323,7 @@ static at::Tensor jagged_forward_impl(const at::Tensor& q, const at::Tensor& k, 
         TORCH_CHECK(!t->defined() || t->device() == dq.device(), "all tensors must be on the device of q");
 
     at::Tensor out;
-    if (!grad) out = at::empty({dq.size(0), dq.size(1), dv.size(2)}, dq.options());
+    if (!grad) out = at::empty({dq.size(0), dq.size(1), dv.size(2)}, dq.options().dtype(out_type_of(dq)));
     p.q = dq.const_data_ptr();
     p.k = dk.const_data_ptr();
     p.v = dv.const_data_ptr();
@@ -660,7 +665,7 @@ static at::Tensor dense_impl(const at::Tensor& q, const at::Tensor& k, const at:
     max_seq_len_check(max_seq_len);
     const bool mask_defined = mask.has_value() && mask->defined();
     mask_check(mask_type, mask_defined);
-    const int32_t dt = io_dtype(dq, "q");
+    const int32_t dt = io_dtype(dq, "q", grad == nullptr);
     TORCH_CHECK(dk.scalar_type() == dq.scalar_type() && dv.scalar_type() == dq.scalar_type(), "q, k, v dtype mismatch");
     TORCH_CHECK(dq.sizes() == dk.sizes() && dq.sizes() == dv.sizes(), "dense layout needs q, k and v of one shape");
     TORCH_CHECK(dq.size(1) == max_seq_len, "dense layout: max_seq_len must equal the sequence dimension of q (", dq.size(1), ")");
@@ -733,7 +738,7 @@ static at::Tensor dense_impl(const at::Tensor& q, const at::Tensor& k, const at:
         *grads = std::make_tuple(gq, gk, gv, gb);
         return at::Tensor();
     }
-    auto out = at::empty_like(dq);
+    auto out = at::empty(dq.sizes(), dq.options().dtype(out_type_of(dq)));
     p.out = out.data_ptr();
     run_abi(hstu_hip_dense_forward_get_workspace_size, hstu_hip_dense_forward, p, dq, op);
     return out;

@@ -21,10 +21,11 @@ def run_capi(cfg, *, op="jagged", flags=0, reuse_from=None, **over):
     c.update(over)
     q, k, v = _dev(c["q"]), _dev(c["k"]), _dev(c["v"])
     dense = op == "dense"
+    odt = _capi.out_dtype(q.dtype)
     if dense:
-        out = torch.full_like(q, float("nan"))
+        out = torch.full(q.shape, float("nan"), dtype=odt, device="cuda")
     else:
-        out = torch.full((q.shape[0], q.shape[1], v.shape[2]), float("nan"), dtype=q.dtype, device="cuda")
+        out = torch.full((q.shape[0], q.shape[1], v.shape[2]), float("nan"), dtype=odt, device="cuda")
     kw = dict(max_seq_len_q=c["max_seq_len"], max_seq_len_k=c.get("max_seq_len_k"), mask_type=c.get("mask_type", 0),
               mask=_dev(c.get("mask")), attn_bias=_dev(c.get("attn_bias")), silu_scale=c.get("silu_scale", 0.0),
               alpha=c.get("alpha", 1.0), num_context=_dev(c.get("num_context")), num_target=_dev(c.get("num_target")),

@@ -148,6 +148,37 @@ def test_describe_kernel_selection():
         assert buf.value.decode() == want, over
 
 
+def test_fp8_inputs_selection_and_rejections():
+    """float8_e4m3fn q / k / v: forward of the jagged and dense layouts only; matrix-core kernel for head dims 64 / 128 / 256
+    without bias or custom mask, else the plain kernel; the work list is the only workspace."""
+    buf = C.create_string_buffer(64)
+    lib = _capi.lib()
+    fp8 = dict(dtype=_capi.HSTU_FP8_E4M3)
+    for over, want in [(dict(), "mfma_fp8_d128"), (dict(dim_qk=64, dim_v=64), "mfma_fp8_d64"), (dict(dim_qk=256, dim_v=256), "mfma_fp8_d256"),
+                       (dict(dim_qk=32, dim_v=32), "generic_fp8"), (dict(dim_qk=96, dim_v=80), "generic_fp8"),
+                       (dict(attn_bias=0x1000), "generic_fp8"), (dict(mask_type=3, mask=0x1000), "generic_fp8"),
+                       (dict(mask_type=2), "mfma_fp8_d128"), (dict(k=0x1008), "generic_fp8"),
+                       (dict(flags=_capi.FLAG_FORCE_GENERIC), "generic_fp8")]:
+        p = _params(**fp8, **over)
+        assert lib.hstu_hip_describe_kernel(C.byref(p), buf, 64) == 0, lib.hstu_hip_last_error()
+        assert buf.value.decode() == want, over
+    rc, n, _ = _ws(_params(**fp8))
+    assert rc == 0 and n > 0 and n % 256 == 0
+    rc, n, _ = _ws(_params(**fp8, attn_bias=0x1000))
+    assert rc == 0 and n == 0
+    paged = dict(kv_cache=0x1000, page_offsets=0x1000, page_ids=0x1000, last_page_len=0x1000, cache_dtype=_capi.HSTU_FP8_E4M3,
+                 kv_scales=0x1000, page_size=64)
+    rc, _, msg = _ws(_params(**fp8, **paged), op="paged")
+    assert rc == -2 and "jagged and dense forward only" in msg, (rc, msg)
+    b = _capi.HstuBwdParams()
+    b.struct_size = C.sizeof(_capi.HstuBwdParams)
+    b.fwd = _params(**fp8)
+    b.grad_out = b.grad_q = b.grad_k = b.grad_v = 0x1000
+    n = C.c_uint64(0)
+    assert lib.hstu_hip_jagged_backward_get_workspace_size(C.byref(b), C.byref(n)) == -2
+    assert "forward only" in lib.hstu_hip_last_error().decode()
+
+
 # ---- torch op layer: same checks, same messages, on CPU tensors ------------------------------
 def _call(q, off, mask_type=0, max_len=8, mask=None, **kw):
     return torch.ops.mxrec.hstu_jagged(q, q, q, mask, None, mask_type, max_len, 0.0, off, **kw)

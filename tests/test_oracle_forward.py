@@ -134,6 +134,77 @@ def test_lowp_rounding_points_bf16():
     assert O.double_benchmark_close(lp, lp, ex) and O.mismatch_ratio_close(lp, ex, 5e-3, 5e-3)
 
 
+def _e4m3_round(x: np.ndarray) -> np.ndarray:
+    """float8_e4m3fn rounding written from the format's definition: 3 mantissa bits, exponent bias 7,
+    subnormals in steps of 2^-9 below 2^-6, largest finite value 448, ties to even."""
+    x = np.asarray(x, dtype=np.float64)
+    a = np.abs(x)
+    e = np.floor(np.log2(np.where(a > 0, a, 1.0)))
+    e = np.maximum(e, -6.0)
+    step = np.exp2(e - 3.0)
+    r = np.rint(a / step) * step                       # numpy's rint rounds ties to even
+    r = np.minimum(r, 448.0)
+    return np.sign(x) * r
+
+
+def test_e4m3_rounding_matches_torch_cast():
+    rng = np.random.default_rng(41)
+    x = np.concatenate([rng.normal(0, 1, 4000), rng.normal(0, 1e-2, 4000), rng.uniform(-400, 400, 2000),
+                        [0.0, 2.0 ** -9, 2.0 ** -10, 3 * 2.0 ** -10, 0.4375, 0.46875, 17.0, 18.0, 19.0]])
+    x = x.astype(np.float32)
+    want = torch.from_numpy(x).to(torch.float8_e4m3fn).to(torch.float32).numpy()
+    assert np.array_equal(_e4m3_round(x).astype(np.float32), want)
+
+
+@pytest.mark.parametrize("case", [
+    dict(lens_q=[7, 3], nq=2, nk=2, d=8),
+    dict(lens_q=[5, 0, 9], nq=4, nk=2, d=8),                              # empty sequence, GQA
+    dict(lens_q=[2, 3], lens_k=[6, 5], nq=2, nk=1, d=4),                  # delta-q
+    dict(lens_q=[9], nq=1, nk=1, d=8, ctx=[2], tgt=[3], tgs=2, bias=True),
+])
+def test_fp8_inputs_follow_the_goldens_rounding_points(case):
+    """float8_e4m3fn q/k/v: fp32 scores, P through e4m3 after silu_scale and mask, fp32 PV, fp16 out
+    (reference golden test_hstu_jagged_forward.py:150-189), against scalar loops with ``_e4m3_round``."""
+    rng = np.random.default_rng(17)
+    lens_q, lens_k, d = case["lens_q"], case.get("lens_k", case["lens_q"]), case["d"]
+    q, k, v, oq, ok = _jag(rng, lens_q, case["nq"], case["nk"], d, d, lens_k=lens_k)
+    q, k, v = (t.mul(2.0).to(torch.float8_e4m3fn) for t in (q, k, v))
+    ctx, tgt, tgs = case.get("ctx"), case.get("tgt"), case.get("tgs", 0)
+    mq, mk = max(lens_q), max(lens_k)
+    bias = None
+    if case.get("bias"):
+        bias = torch.from_numpy(rng.normal(0, 0.5, (len(lens_q), case["nq"], mq, mk))).float()
+    kw = dict(max_seq_len_q=mq, silu_scale=0.37, alpha=0.8, attn_bias=bias,
+              num_context=None if ctx is None else torch.tensor(ctx), num_target=None if tgt is None else torch.tensor(tgt),
+              target_group_size=tgs)
+    got = O.hstu_jagged_forward(q, k, v, oq, ok, max_seq_len_k=mk, mode="lowp", **kw)
+    assert got.dtype == torch.float16
+    qf, kf, vf = (t.to(torch.float32).numpy().astype(np.float64) for t in (q, k, v))
+    ratio = case["nq"] // case["nk"]
+    want = np.zeros((sum(lens_q), case["nq"], d))
+    oql, okl = oq.tolist(), ok.tolist()
+    for b in range(len(lens_q)):
+        lq, lk = lens_q[b], lens_k[b]
+        for h in range(case["nq"]):
+            for i in range(lq):
+                for j in range(lk):
+                    mv = O.mask_point(i, j, lq, lk, 0 if ctx is None else ctx[b], 0 if tgt is None else tgt[b], tgs)
+                    s = float(np.float32(qf[oql[b] + i, h] @ kf[okl[b] + j, h // ratio]))
+                    if bias is not None:
+                        s += float(bias[b, h, i, j])
+                    x = 0.8 * s
+                    p = _e4m3_round(np.float32(x / (1.0 + math.exp(-x)) * 0.37 * mv))
+                    want[oql[b] + i, h] += p * vf[okl[b] + j, h // ratio]
+    want16 = torch.from_numpy(want).to(torch.float16)
+    # a score within an fp32 ulp of an e4m3 tie may round the other way: allow one e4m3 step of P on a few outputs
+    diff = (got.float() - want16.float()).abs()
+    assert float(diff.max()) <= 2.0 ** -4 * float(vf.__abs__().max()) * 0.5 + 1e-3
+    assert float((diff > 2e-3).float().mean()) < 0.02
+    # P really goes through e4m3: the exact path differs visibly
+    ex = O.hstu_jagged_forward(q.float(), k.float(), v.float(), oq, ok, max_seq_len_k=mk, **kw)
+    assert float((ex - want16.float()).abs().max()) > 1e-3
+
+
 # ---- paged ---------------------------------------------------------------
 def _paged_case(rng, users, ps, nq, nk, d, dtype=torch.float32):
     hist = [int(x) for x in rng.integers(1, 3 * ps, users)]
