@@ -44,8 +44,12 @@ __device__ __forceinline__ int fp8_classify(const Seq& s, int tgs, int r0, int c
     return FBLK_CAUSAL;
 }
 
+// Waves per SIMD: as many as the registers allow (each more hides more of the LDS and matrix-core latency: measured 14 %
+// from 2 to 3 at head dim 64 and 11 % at 128, 4 % from 3 to 4 at 64); head dim 256 needs a whole SIMD lane's registers.
+template <int D> struct Fp8Shape { static constexpr int WAVES = D == 64 ? 4 : (D == 128 ? 3 : 1); };
+
 template <int D>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 1 : 2, D == 256 ? 1 : 2)))
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(Fp8Shape<D>::WAVES, Fp8Shape<D>::WAVES)))
 void hstu_mfma_fp8_kernel(const KArgs a, const unsigned* __restrict__ ws) {
     const hstu_fwd_params& p = a.p;
     // row strides in bytes: +16 keeps the 16-byte row-wise reads of 16 K rows on distinct banks, +32 does the same for
@@ -82,6 +86,7 @@ void hstu_mfma_fp8_kernel(const KArgs a, const unsigned* __restrict__ ws) {
     (void)b;
     const bool tril = p.mask_type == HSTU_MASK_TRIL;
     const int tgs = p.target_group_size;
+    const float inv_scale = 1.0f / a.out_scale;   // +-inf when alpha is 0: P = x * rcp(inf) = 0, as x * sigmoid(0) * 0
     const unsigned char* qbase = reinterpret_cast<const unsigned char*>(p.q);
     const unsigned char* kbase = reinterpret_cast<const unsigned char*>(p.k);
     const unsigned char* vbase = reinterpret_cast<const unsigned char*>(p.v);
@@ -122,27 +127,42 @@ void hstu_mfma_fp8_kernel(const KArgs a, const unsigned* __restrict__ ws) {
 #pragma unroll
             for (int r = 0; r < 16; r++) oacc[db][r] = 0.f;
 
+        // tile loader: thread t copies 16-byte chunk t % CPR of rows t / CPR (+ 256 / CPR per further chunk) of K and of V.
+        // Offsets are 32-bit, relative to the first row of this sequence and kv head (a sequence spans at most
+        // 20480 * 16 * 256 bytes)
+        const unsigned rowstride = (unsigned)p.heads_k * D;
+        const unsigned char* kseq = kbase + (s.k_start * p.heads_k + hk) * (int64_t)D;
+        const unsigned char* vseq = vbase + (s.k_start * p.heads_k + hk) * (int64_t)D;
+        const int lrow = tid / CPR, lcc = tid % CPR;
         q_u32x4 nk[NCH], nv[NCH];
         auto fetch = [&](int kt) __attribute__((always_inline)) {
 #pragma unroll
             for (int i = 0; i < NCH; i++) {
-                const int c = tid + 256 * i;
-                const int row = c / CPR, cc = c % CPR;
-                // nothing here waits for the data: rows past the end are zeroed when the tile is written to LDS
-                const int64_t e = ((s.k_start + min(kt * FBN + row, kend - 1)) * p.heads_k + hk) * (int64_t)D + 16 * cc;
-                nk[i] = *reinterpret_cast<const q_u32x4*>(kbase + e);
-                nv[i] = *reinterpret_cast<const q_u32x4*>(vbase + e);
+                // nothing here waits for the data; rows past the end are read from the last row and zeroed in stash()
+                const int row = min(kt * FBN + lrow + (256 / CPR) * i, kend - 1);
+                const unsigned e = __umul24((unsigned)row, rowstride) + 16u * lcc;
+                nk[i] = *reinterpret_cast<const q_u32x4*>(kseq + e);
+                nv[i] = *reinterpret_cast<const q_u32x4*>(vseq + e);
             }
         };
         auto stash = [&](int kt, int stage) __attribute__((always_inline)) {
+            unsigned char* kd = kst[stage] + lrow * KS + 16 * lcc;
+            unsigned char* vd = vst[stage] + lrow * VS + 16 * lcc;
+            if ((kt + 1) * FBN <= kend) {   // wave-uniform: every row of the tile exists
 #pragma unroll
-            for (int i = 0; i < NCH; i++) {
-                const int c = tid + 256 * i;
-                const int row = c / CPR, cc = c % CPR;
-                const bool ok = kt * FBN + row < kend;   // zero rows: S = 0 gives P = 0, and 0 * V must not meet a NaN
-                const q_u32x4 z = {0, 0, 0, 0};
-                *reinterpret_cast<q_u32x4*>(kst[stage] + row * KS + 16 * cc) = ok ? nk[i] : z;
-                *reinterpret_cast<q_u32x4*>(vst[stage] + row * VS + 16 * cc) = ok ? nv[i] : z;
+                for (int i = 0; i < NCH; i++) {
+                    *reinterpret_cast<q_u32x4*>(kd + (256 / CPR) * i * KS) = nk[i];
+                    *reinterpret_cast<q_u32x4*>(vd + (256 / CPR) * i * VS) = nv[i];
+                }
+            } else {
+                // the last tile: zero rows past the end (S = 0 gives P = 0, and 0 * V must not meet a NaN)
+#pragma unroll
+                for (int i = 0; i < NCH; i++) {
+                    const bool ok = kt * FBN + lrow + (256 / CPR) * i < kend;
+                    const q_u32x4 z = {0, 0, 0, 0};
+                    *reinterpret_cast<q_u32x4*>(kd + (256 / CPR) * i * KS) = ok ? nk[i] : z;
+                    *reinterpret_cast<q_u32x4*>(vd + (256 / CPR) * i * VS) = ok ? nv[i] : z;
+                }
             }
         };
         __syncthreads();   // every wave is done with the stages of the previous tile
@@ -156,48 +176,67 @@ void hstu_mfma_fp8_kernel(const KArgs a, const unsigned* __restrict__ ws) {
             const int stage = kt & 1;
             const int k0 = kt * FBN;
             if (kt + 1 < ntk) fetch(kt + 1);
+            // visibility class of the two 32-key blocks (wave-uniform).  A block past the K extent holds zero rows (P = 0
+            // without a mask); a block the causal mask hides completely is masked like one it cuts (all bytes to zero), so
+            // that the tile is straight-line code
             int cls[2];
+            bool any = false;
 #pragma unroll
             for (int kb = 0; kb < 2; kb++) {
                 const int c0 = k0 + 32 * kb;
-                cls[kb] = c0 >= kend ? FBLK_SKIP : (tril ? fp8_classify(s, tgs, r0, c0) : FBLK_ALL);   // wave-uniform
+                const int c = (c0 >= kend || !tril) ? FBLK_ALL : fp8_classify(s, tgs, r0, c0);
+                any |= c0 < kend && c != FBLK_SKIP;
+                cls[kb] = c == FBLK_SKIP ? FBLK_CAUSAL : c;
             }
-            if (cls[0] != FBLK_SKIP || cls[1] != FBLK_SKIP) {
+            if (any) {
                 const unsigned char* kt_lds = kst[stage];
                 const unsigned char* vt_lds = vst[stage];
-                unsigned pq[8];   // P of this lane's Q row: byte 8c + s = key k0 + 16c + 8g + s
+                // ---- S^T of both blocks: all K fragments are requested before the first product
+                q_i32x8 kf[2][D / 64];
 #pragma unroll
-                for (int kb = 0; kb < 2; kb++) {
-                    if (cls[kb] == FBLK_SKIP) {
-#pragma unroll
-                        for (int x = 0; x < 4; x++) pq[4 * kb + x] = 0u;
-                        continue;
-                    }
-                    q_i32x8 kf[D / 64];
+                for (int kb = 0; kb < 2; kb++)
 #pragma unroll
                     for (int t = 0; t < D / 64; t++) {
                         const unsigned char* at = kt_lds + 32 * kb * KS + kfrag_off + 64 * t;
                         const q_u32x4 x0 = *reinterpret_cast<const q_u32x4*>(at);
                         const q_u32x4 x1 = *reinterpret_cast<const q_u32x4*>(at + 16);
-                        kf[t] = (q_i32x8){(int)x0[0], (int)x0[1], (int)x0[2], (int)x0[3], (int)x1[0], (int)x1[1], (int)x1[2], (int)x1[3]};
+                        kf[kb][t] = (q_i32x8){(int)x0[0], (int)x0[1], (int)x0[2], (int)x0[3], (int)x1[0], (int)x1[1], (int)x1[2], (int)x1[3]};
                     }
-                    q_f32x16 sacc;
+                q_f32x16 sacc[2];
 #pragma unroll
-                    for (int r = 0; r < 16; r++) sacc[r] = 0.f;
+                for (int kb = 0; kb < 2; kb++) {
+#pragma unroll
+                    for (int r = 0; r < 16; r++) sacc[kb][r] = 0.f;
 #pragma unroll
                     for (int t = 0; t < D / 64; t++)
-                        sacc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf[t], qf[t], sacc, 0, 0, 0, 0, 0, 0);
-                    // P = x * sigmoid(alpha * x) * alpha * silu_scale, to e4m3: register 8u + i of the block -> byte i of step u
+                        sacc[kb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf[kb][t], qf[t], sacc[kb], 0, 0, 0, 0, 0, 0);
+                }
+                // V^T fragments: at head dim 64 requested now and used after the SiLU pass; the wider ones have no registers to
+                // hold them that long
+                q_i32x2 vq[D / 32][4];
+                if (D <= 64) {
+#pragma unroll
+                    for (int db = 0; db < D / 32; db++)
+#pragma unroll
+                        for (int c = 0; c < 4; c++)
+                            vq[db][c] = __builtin_amdgcn_ds_read_tr8_b64_v2i32(FP8_LDS_PTR(q_i32x2, vt_lds + 16 * c * VS + vfrag_off + 32 * db));
+                }
+                // ---- P = x * sigmoid(alpha * x) * alpha * silu_scale = x / ((1 + e) / (alpha * silu_scale)), to e4m3: register
+                // 8u + i of block kb -> byte i of step 2 kb + u
+                unsigned pq[8];   // P of this lane's Q row: byte 8c + i = key k0 + 16c + 8g + i
+#pragma unroll
+                for (int kb = 0; kb < 2; kb++) {
 #pragma unroll
                     for (int x = 0; x < 4; x++) {
                         float pv[4];
 #pragma unroll
                         for (int i = 0; i < 4; i++) {
-                            const float sc = sacc[4 * x + i];
+                            const float sc = sacc[kb][4 * x + i];
                             const float e = __builtin_amdgcn_exp2f(sc * a.exp_scale);
-                            pv[i] = sc * __builtin_amdgcn_rcpf(1.0f + e) * a.out_scale;
+                            pv[i] = sc * __builtin_amdgcn_rcpf(__builtin_fmaf(e, inv_scale, inv_scale));
                         }
-                        int word = __builtin_amdgcn_cvt_pk_fp8_f32(pv[0], pv[1], 0, false);
+                        // both halves of the word are written: its initial value is irrelevant, and a live register saves a move
+                        int word = __builtin_amdgcn_cvt_pk_fp8_f32(pv[0], pv[1], __builtin_bit_cast(int, pv[0]), false);
                         word = __builtin_amdgcn_cvt_pk_fp8_f32(pv[2], pv[3], word, true);
                         pq[4 * kb + x] = (unsigned)word;
                     }
@@ -232,11 +271,12 @@ void hstu_mfma_fp8_kernel(const KArgs a, const unsigned* __restrict__ ws) {
                 // ---- O^T += V^T P^T: 64 keys per instruction
 #pragma unroll
                 for (int db = 0; db < D / 32; db++) {
-                    q_i32x2 vq[4];
+                    if (D > 64) {
 #pragma unroll
-                    for (int c = 0; c < 4; c++)
-                        vq[c] = __builtin_amdgcn_ds_read_tr8_b64_v2i32(FP8_LDS_PTR(q_i32x2, vt_lds + 16 * c * VS + vfrag_off + 32 * db));
-                    const q_i32x8 va = {vq[0][0], vq[0][1], vq[1][0], vq[1][1], vq[2][0], vq[2][1], vq[3][0], vq[3][1]};
+                        for (int c = 0; c < 4; c++)
+                            vq[db][c] = __builtin_amdgcn_ds_read_tr8_b64_v2i32(FP8_LDS_PTR(q_i32x2, vt_lds + 16 * c * VS + vfrag_off + 32 * db));
+                    }
+                    const q_i32x8 va = {vq[db][0][0], vq[db][0][1], vq[db][1][0], vq[db][1][1], vq[db][2][0], vq[db][2][1], vq[db][3][0], vq[db][3][1]};
                     oacc[db] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(va, pb, oacc[db], 0, 0, 0, 0, 0, 0);
                 }
             }
