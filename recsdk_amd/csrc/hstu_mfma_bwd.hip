@@ -253,7 +253,9 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
                         pk0[x] = BMM<T>::pack2(wv[2 * x], wv[2 * x + 1]);
                         pk1[x] = BMM<T>::pack2(wv[8 + 2 * x], wv[8 + 2 * x + 1]);
                     }
-                    // visibility of this lane's 16 elements as masks of the packed pairs
+                    // visibility of this lane's 16 elements as masks of the packed pairs: applied to them at once, kept only where
+                    // dBias needs them too (holding them in every variant costs the dK kernel 70 spilled registers)
+                    constexpr bool KEEP_MASK = BIAS && MODE == MODE_DQ;
                     b_u32x4 m0 = {~0u, ~0u, ~0u, ~0u}, m1 = m0;
                     if (diag) {
                         // visible iff j <= i + delta; t runs over this lane's 16 streamed rows
@@ -263,8 +265,11 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
                         };
 #pragma unroll
                         for (int x = 0; x < 4; x++) {
-                            m0[x] = (vis(2 * x) ? 0xffffu : 0u) | (vis(2 * x + 1) ? 0xffff0000u : 0u);
-                            m1[x] = (vis(8 + 2 * x) ? 0xffffu : 0u) | (vis(9 + 2 * x) ? 0xffff0000u : 0u);
+                            const unsigned v0 = (vis(2 * x) ? 0xffffu : 0u) | (vis(2 * x + 1) ? 0xffff0000u : 0u);
+                            const unsigned v1 = (vis(8 + 2 * x) ? 0xffffu : 0u) | (vis(9 + 2 * x) ? 0xffff0000u : 0u);
+                            pk0[x] &= v0;
+                            pk1[x] &= v1;
+                            if (KEEP_MASK) { m0[x] = v0; m1[x] = v1; }
                         }
                     } else if (pred) {
                         // branch-free form of builtin_visible() for this lane's 16 elements
@@ -278,13 +283,12 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
                         };
 #pragma unroll
                         for (int x = 0; x < 4; x++) {
-                            m0[x] = (vis(2 * x) ? 0xffffu : 0u) | (vis(2 * x + 1) ? 0xffff0000u : 0u);
-                            m1[x] = (vis(8 + 2 * x) ? 0xffffu : 0u) | (vis(9 + 2 * x) ? 0xffff0000u : 0u);
+                            const unsigned v0 = (vis(2 * x) ? 0xffffu : 0u) | (vis(2 * x + 1) ? 0xffff0000u : 0u);
+                            const unsigned v1 = (vis(8 + 2 * x) ? 0xffffu : 0u) | (vis(9 + 2 * x) ? 0xffff0000u : 0u);
+                            pk0[x] &= v0;
+                            pk1[x] &= v1;
+                            if (KEEP_MASK) { m0[x] = v0; m1[x] = v1; }
                         }
-                    }
-                    if (diag || pred) {
-#pragma unroll
-                        for (int x = 0; x < 4; x++) { pk0[x] &= m0[x]; pk1[x] &= m1[x]; }
                     }
                     if (BIAS && MODE == MODE_DQ) {
                         // dBias = dS with its scale, rounded once, zero where the mask hides the element and behind the sequence;
