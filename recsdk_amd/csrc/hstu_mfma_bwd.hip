@@ -214,7 +214,8 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
                     // accumulator register r holds streamed row c0 + 8*(r/4) + 4*g + r%4 for the owned row of this lane
                     // dense bias of this lane's 16 elements: the dQ kernel owns the row and takes four 8-byte pieces of it, the
                     // K-side kernels own the column and take 16 single values (the lanes of a wave then read along a row)
-                    float bias_f[BIAS ? 16 : 1];
+                    // kept as 8 words of two 16-bit values (pair x = elements 2x, 2x + 1) and widened where they are used
+                    unsigned bias_w[BIAS ? 8 : 1];
                     const T* bias_bh = reinterpret_cast<const T*>(p.attn_bias) + ((int64_t)b * p.heads_q + h) * p.max_seq_len_q * (int64_t)p.max_seq_len_k;
                     if (BIAS) {
                         if (MODE == MODE_DQ) {
@@ -222,22 +223,29 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
                             for (int q = 0; q < 4; q++) {
                                 const int j = c0 + 8 * q + 4 * g;
                                 b_u32x2 raw = {0, 0};
-                                if (orow < p.max_seq_len_q && j < p.max_seq_len_k) raw = *reinterpret_cast<const b_u32x2*>(bias_bh + orow * (int64_t)p.max_seq_len_k + j);
-#pragma unroll
-                                for (int i = 0; i < 4; i++) bias_f[4 * q + i] = bwd_half<T>(raw[i >> 1], i & 1);
+                                if (orow < p.max_seq_len_q && j < p.max_seq_len_k) raw = *reinterpret_cast<const b_u32x2*>(bias_bh + ((unsigned)orow * (unsigned)p.max_seq_len_k + (unsigned)j));
+                                bias_w[2 * q] = raw[0];
+                                bias_w[2 * q + 1] = raw[1];
                             }
                         } else {
+                            typedef __attribute__((ext_vector_type(2))) T T2;
+                            const bool col_ok = orow < p.max_seq_len_k;
 #pragma unroll
-                            for (int r = 0; r < 16; r++) {
-                                const int i = c0 + 8 * (r >> 2) + 4 * g + (r & 3);
-                                bias_f[r] = (i < p.max_seq_len_q && orow < p.max_seq_len_k) ? to_float(bias_bh[i * (int64_t)p.max_seq_len_k + orow]) : 0.f;
+                            for (int x = 0; x < 8; x++) {
+                                const int i = c0 + 8 * (x >> 1) + 4 * g + 2 * (x & 1);
+                                T2 v = {(T)0.f, (T)0.f};
+                                // 32-bit element offsets: one (batch, head) plane holds at most 20480^2 values
+                                const unsigned at = (unsigned)i * (unsigned)p.max_seq_len_k + (unsigned)orow;
+                                if (col_ok && i < p.max_seq_len_q) v[0] = bias_bh[at];
+                                if (col_ok && i + 1 < p.max_seq_len_q) v[1] = bias_bh[at + (unsigned)p.max_seq_len_k];
+                                bias_w[x] = __builtin_bit_cast(unsigned, v);
                             }
                         }
                     }
                     float wv[16];
 #pragma unroll
                     for (int r = 0; r < 16; r++) {
-                        const float sv = BIAS ? sacc[r] + bias_f[r] : sacc[r];
+                        const float sv = BIAS ? sacc[r] + bwd_half<T>(bias_w[r >> 1], r & 1) : sacc[r];
                         const float e = __builtin_amdgcn_exp2f(sv * a.f.exp_scale);
                         const float sg = __builtin_amdgcn_rcpf(1.0f + e);
                         if (TWO) {
@@ -303,7 +311,7 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
                             b_u32x2 o;
                             o[0] = BMM<T>::pack2(wv[4 * q] * sc, wv[4 * q + 1] * sc) & mm[x0];
                             o[1] = BMM<T>::pack2(wv[4 * q + 2] * sc, wv[4 * q + 3] * sc) & mm[x0 + 1];
-                            if (ovalid && orow < p.max_seq_len_q && j < p.max_seq_len_k) *reinterpret_cast<b_u32x2*>(gbias + orow * (int64_t)p.max_seq_len_k + j) = o;
+                            if (ovalid && orow < p.max_seq_len_q && j < p.max_seq_len_k) *reinterpret_cast<b_u32x2*>(gbias + ((unsigned)orow * (unsigned)p.max_seq_len_k + (unsigned)j)) = o;
                         }
                     }
                     // OUT^T += (tile)^T W: transposing LDS reads, 4 streamed rows of one head-dim column per lane
