@@ -23,12 +23,13 @@ PEAK_FP8_TFLOPS = 5000.0    # MI355X dense fp8 MFMA
 PEAK_HBM_GBS = 8000.0
 # HBM-side bytes per launch from rocprofv3 FETCH_SIZE/WRITE_SIZE, each scaled by what the same counter reads for the
 # plain 256 MiB copy of `--workload copy` (factors 2.000 and 1.000); see profiles/*.md
-TRAFFIC_SOURCE = {"config2": "profiles/hstu_mfma_kernel_configs2-5.md", "kv_append": "profiles/hstu_kv_append_kernel.md",
+TRAFFIC_SOURCE = {"config2": "profiles/hstu_mfma_kernel_configs2-5.md", "config2_fp8": "profiles/hstu_mfma_fp8_kernel.md",
+                  "ref_bias": "profiles/hstu_mfma_kernel_reference_benchmark_shape.md", "kv_append": "profiles/hstu_kv_append_kernel.md",
                   "rab_time": "profiles/hstu_rab_kernels.md", "rab_time_bwd": "profiles/hstu_rab_kernels.md", "rab_pos": "profiles/hstu_rab_kernels.md",
                   "nmd_fwd": "profiles/hstu_nmd_kernels.md", "nmd_bwd": "profiles/hstu_nmd_kernels.md",
                   "in_linear_silu": "profiles/hstu_in_linear_silu_kernel.md", "in_linear_silu_bwd": "profiles/hstu_in_linear_silu_backward_kernels.md",
                   "kv_append_fp8": "profiles/hstu_kv_append_fp8_kernels.md"}
-MEASURED_TRAFFIC_BYTES = {"config2": 184.3e6, "kv_append": 351.9e6, "rab_time": 1479.8e6, "rab_time_bwd": 2242.4e6, "rab_pos": 305.2e6,
+MEASURED_TRAFFIC_BYTES = {"config2": 184.5e6, "config2_fp8": 116.5e6, "ref_bias": 1503.6e6, "kv_append": 351.9e6, "rab_time": 1479.8e6, "rab_time_bwd": 2242.4e6, "rab_pos": 305.2e6,
                           "nmd_fwd": 826.4e6, "nmd_bwd": 1380.0e6, "in_linear_silu": 1092.8e6, "in_linear_silu_bwd": 2405.4e6, "kv_append_fp8": 455.0e6}
 
 
@@ -65,15 +66,16 @@ def build_workload(name, torch, W):
         kv = sum(c["hist"]) * 2 * 4 * 128
         qo = 2 * 32 * 256 * 4 * 128 * 2
         return c, "paged", flops, kv + 2 * qo, "config5 paged fp8-KV: 32 users x 256 candidates, hist~U[1024,4096], 64-token pages"
-    if name in ("ref_bias", "ref_nobias"):
-        c = W.reference_benchmark_config(has_rab=name == "ref_bias")
-        flops = W.headline_flops(c["lens"], 8, 128)
+    if name in ("ref_bias", "ref_nobias", "ref_nobias_d32", "ref_nobias_d64", "ref_nobias_d256"):
+        dim = int(name.split("_d")[1]) if "_d" in name else 128   # the ends and the middle of the reference's head-dim sweep
+        c = W.reference_benchmark_config(has_rab=name == "ref_bias", dim=dim)
+        flops = W.headline_flops(c["lens"], 8, dim)
         t = sum(c["lens"])
-        b = 4 * t * 8 * 128 * 2
+        b = 4 * t * 8 * dim * 2
         # of the dense bias only the causal half is needed: sum over sequences and heads of L (L + 1) / 2 two-byte values
         if name == "ref_bias":
             b += sum(8 * l * (l + 1) // 2 * 2 for l in c["lens"])
-        return c, "jagged", flops, b, ("reference benchmark shape (test_forward_op_benchmark.py:246-259): B=32 h=8 d=128 S=2048, every length "
+        return c, "jagged", flops, b, ("reference benchmark shape (test_forward_op_benchmark.py:246-259): B=32 h=8 d=" + str(dim) + " S=2048, every length "
                                       "0.9 S, alpha=0.5, silu_scale=1/1024, bf16, causal, " + ("dense attn_bias [B,h,S,S]" if name == "ref_bias" else "no bias"))
     raise SystemExit(f"unknown workload {name}")
 
@@ -83,7 +85,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=1000)
-    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "ref_bias", "ref_nobias", "config2_fp8", "ref_nobias_fp8", "config2_bwd", "kv_append", "kv_append_fp8", "rab_time", "rab_time_bwd", "rab_pos", "nmd_fwd", "nmd_bwd", "in_linear_silu", "in_linear_silu_bwd", "copy"],
+    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "ref_bias", "ref_nobias", "ref_nobias_d32", "ref_nobias_d64", "ref_nobias_d256", "config2_fp8", "ref_nobias_fp8", "config2_bwd", "ref_bias_bwd", "kv_append", "kv_append_fp8", "rab_time", "rab_time_bwd", "rab_pos", "nmd_fwd", "nmd_bwd", "in_linear_silu", "in_linear_silu_bwd", "copy"],
                     help="'copy' runs a plain 256 MiB device copy: the known-size kernel the FETCH_SIZE/WRITE_SIZE counters are scaled by")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--settle-ms", type=float, default=80.0,
@@ -100,7 +102,7 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs the MI355X"
     if args.workload == "copy":
         return copy_calibration(args, torch)
-    if args.workload == "config2_bwd":
+    if args.workload in ("config2_bwd", "ref_bias_bwd"):
         return backward_bench(args, torch, W, _capi)
     if args.workload == "kv_append":
         return kv_append_bench(args, torch, W)
@@ -205,18 +207,26 @@ def backward_bench(args, torch, W, _capi):
     """The jagged backward (dQ, dK, dV) on the headline configuration: five GEMM-shaped products of L^2 * h * d
     multiply-adds each under the causal mask (S, dO V^T, dV, dK, dQ) = 2.5 x the forward's FLOPs."""
     import ctypes as C
-    cfg = W.config2()
+    with_bias = args.workload == "ref_bias_bwd"
+    # ref_bias_bwd: the reference's benchmark shape (B=32 h=8 d=128 S=2048, lengths 0.9 S) with a dense attn_bias, whose
+    # gradient (the same 2.1 GB again) the call also produces
+    cfg = W.reference_benchmark_config(has_rab=True) if with_bias else W.config2()
+    heads = 8 if with_bias else 4
     dev = W.to_device(cfg)
     q, k, v = dev["q"], dev["k"], dev["v"]
+    bias = dev.get("attn_bias")
     g = torch.Generator(device="cuda").manual_seed(1)
     grad = torch.randn(q.shape, generator=g, device="cuda", dtype=torch.float32).to(q.dtype)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-    fwd, keep = _capi.make_params(q, k, v, q, seq_offset_q=dev["seq_offset"], max_seq_len_q=cfg["max_seq_len"], alpha=cfg["alpha"])
+    dbias = None if bias is None else torch.empty_like(bias)
+    fwd, keep = _capi.make_params(q, k, v, q, seq_offset_q=dev["seq_offset"], max_seq_len_q=cfg["max_seq_len"], alpha=cfg["alpha"],
+                                  attn_bias=bias, silu_scale=cfg.get("silu_scale", 0.0))
     fwd.out = None
-    p = _capi.make_backward_params(fwd, grad, dq, dk, dv)
+    p = _capi.make_backward_params(fwd, grad, dq, dk, dv, dbias)
+    kernel = _capi.describe_backward_kernel(p)
     L = _capi.lib()
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
-    flops = 2.5 * W.headline_flops(cfg["lens"], 4, 128)
+    flops = 2.5 * W.headline_flops(cfg["lens"], heads, 128)
 
     nws = C.c_uint64(0)
     if L.hstu_hip_jagged_backward_get_workspace_size(C.byref(p), C.byref(nws)) != 0:
@@ -243,13 +253,20 @@ def backward_bench(args, torch, W, _capi):
     kern_ms = e0.elapsed_time(e1) / args.steps
     tflops = flops / (ms * 1e-3) / 1e12
     t = sum(cfg["lens"])
-    alg_bytes = 7 * t * 4 * 128 * 2   # Q, K, V, dO read once; dQ, dK, dV written once
+    alg_bytes = 7 * t * heads * 128 * 2   # Q, K, V, dO read once; dQ, dK, dV written once
+    if with_bias:
+        # the causal half of the bias is read by each of the three kernels' producers once (counted once), the whole
+        # gradient buffer is zero-filled and its causal half written again
+        half = sum(heads * l * (l + 1) // 2 * 2 for l in cfg["lens"])
+        alg_bytes += half + bias.numel() * 2 + half
+    desc = ("reference benchmark shape, backward with dense attn_bias and its gradient: B=32 h=8 d=128 S=2048, every length 0.9 S, bf16, causal"
+            if with_bias else "config2 shapes, backward: B=64 h=4 d=128 L~U[256,1024] bf16 causal no-bias seed0")
     print(json.dumps({
         "metric": "hstu_jagged_attn_bwd_tflops", "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic", "us_per_call": round(ms * 1e3, 2),
         "pct_bf16_mfma_peak": round(100 * tflops / PEAK_BF16_TFLOPS, 2),
-        "config": {"workload": "config2 shapes, backward: B=64 h=4 d=128 L~U[256,1024] bf16 causal no-bias seed0",
+        "config": {"workload": desc, "kernel": kernel,
                    "flops_per_call": flops, "algorithmic_bytes_per_call": alg_bytes, "entry": "hstu_hip_jagged_backward (C ABI)"},
         "roofline": {"bound": "mfma", "achieved": round(flops / (kern_ms * 1e-3) / 1e12, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(flops / (kern_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4), "traffic": None,
