@@ -58,7 +58,7 @@ enum { HSTU_MASK_TRIL = 0, HSTU_MASK_TRIU = 1, HSTU_MASK_NONE = 2, HSTU_MASK_CUS
  * One argument block for the three forward ops.  Pointers are device pointers unless stated.
  * Layouts (row-major, innermost last):
  *   q   [total_q, heads_q, dim_qk]     k [total_k, heads_k, dim_qk]     v [total_k, heads_k, dim_v]
- *   out [total_q, heads_q, dim_v]      same dtype as q
+ *   out [total_q, heads_q, dim_v]      same dtype as q; fp16 when q / k / v are FP8_E4M3 (reference: hstu_jagged.cpp:53-54)
  *   seq_offset_q / seq_offset_k  [batch+1] of index_type; sequence b owns rows off[b]..off[b+1]-1.
  *     Q row i of a sequence sits at position i + (Lk - Lq) of its K timeline ("delta-q").
  *     Both NULL = dense layout: every sequence has max_seq_len_q (= max_seq_len_k) rows.
@@ -69,7 +69,8 @@ enum { HSTU_MASK_TRIL = 0, HSTU_MASK_TRIU = 1, HSTU_MASK_NONE = 2, HSTU_MASK_CUS
 typedef struct hstu_fwd_params {
     uint32_t struct_size; /* sizeof(hstu_fwd_params) of the caller, for ABI checking */
     uint32_t flags;
-    int32_t dtype;      /* hstu_dtype of q/k/v/out/mask/attn_bias: F32, F16 or BF16 */
+    int32_t dtype;      /* hstu_dtype of q/k/v/out/mask/attn_bias: F32, F16 or BF16; FP8_E4M3 (float8_e4m3fn q/k/v/mask/attn_bias,
+                           fp16 out, scores and sums in fp32, P rounded to e4m3 before P*V) in the jagged and dense forward only */
     int32_t index_type; /* hstu_index_type of every integer tensor */
 
     const void* q;
@@ -207,8 +208,9 @@ const char* hstu_hip_last_error(void);
 /* Name of the kernel variant the given arguments select ("mfma_bf16_d128", "generic_f32", ...);
  * written NUL-terminated into buf.  Diagnostic: lets a caller assert that the MFMA path is the one in use.  The
  * matrix-core kernels take bf16 / fp16 with dim_qk == dim_v in {32, 64, 128, 256} (paged: 64 or 128, and at most 320 pages
- * per user) and buffers on 16-byte boundaries; everything else (fp32, other head dims, dim_qk != dim_v) runs the plain
- * fp32-FMA kernel, which is an order of magnitude slower. */
+ * per user) and buffers on 16-byte boundaries, and FP8_E4M3 with dim_qk == dim_v in {64, 128, 256}, the built-in mask or
+ * none and no bias ("mfma_fp8_d128"); everything else (fp32, other head dims, dim_qk != dim_v, fp8 bias or custom mask)
+ * runs the plain fp32-FMA kernel, which is an order of magnitude slower. */
 int hstu_hip_describe_kernel(const hstu_fwd_params* p, char* buf, size_t buf_bytes);
 
 /* The same for the backward: "mfma_bwd_bf16_d128", "mfma_bwd_f16_d64_bias", "generic_bwd_f32", ...  The matrix-core
