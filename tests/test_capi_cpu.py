@@ -349,3 +349,12 @@ def test_dense_backward_validation():
     assert rc == 0 and n > 0 and n % 256 == 0, msg           # bf16 d=128: the MFMA kernels with one work list
     rc = _capi.lib().hstu_hip_dense_backward(C.byref(d), None, 0, None)
     assert rc == -3 and "workspace" in _capi.lib().hstu_hip_last_error().decode()
+
+
+def test_rate_diagnostics_reject_bad_arguments():
+    # host checks only: nothing is launched
+    lib = _capi.lib()
+    assert lib.hstu_hip_measure_block_rates(0, 1, 10, None, None, None, None) == -1          # no buffers
+    for mode, waves in [(1, 4), (2, 4), (3, 3), (0, 5), (0, 0), (9, 1)]:
+        assert lib.hstu_hip_measure_block_rates(mode, waves, 10, 0x1000, 0x1000, 0x1000, None) == -1, (mode, waves)
+    assert lib.hstu_hip_measure_block_rates(0, 1, 0, 0x1000, 0x1000, 0x1000, None) == -1      # no iterations
