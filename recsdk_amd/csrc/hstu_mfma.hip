@@ -392,7 +392,9 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
 }
 
 
-// EXTRA: 0 = no bias / built-in mask only, 1 = dense bias and/or custom mask (tables, if any, gathered from
+// EXTRA: 5 = a dense bias whose rows start on 16-byte boundaries and nothing else (built-in mask or none): the general
+// variant's per-score code carries every option as a run-time test and runs 2.7 x slower than this one on the same input;
+// 0 = no bias / built-in mask only, 1 = dense bias and/or custom mask (tables, if any, gathered from
 // global memory), 2 / 3 / 4 = bias tables only, gathered from LDS-resident copies: position table / time table /
 // both (compile-time so that the per-score code is branch-free)
 // The plain variant (head dim 128, built-in mask, no bias, rows straight from k/v) fits 168 registers and 34 KB of
@@ -432,7 +434,8 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
     // table mode: per K tile a window of the position table and the key timestamps (double buffered with the
     // K/V tiles), plus the whole time table and its bucket bounds as (lower, upper) pairs
     constexpr int PW = BM + BN;   // window entries: (j - k0) - (qi - i0) + BM - 1 in [0, BM + BN - 2]
-    constexpr bool TAB = EXTRA >= 2, tab_pos = EXTRA == 2 || EXTRA == 4, tab_ts = EXTRA == 3 || EXTRA == 4;
+    constexpr bool TAB = EXTRA >= 2 && EXTRA <= 4, tab_pos = EXTRA == 2 || EXTRA == 4, tab_ts = EXTRA == 3 || EXTRA == 4;
+    constexpr bool BIAS_ONLY = EXTRA == 5;   // attn_bias given, rows on 16-byte boundaries, no custom mask, no tables (host-checked)
     __shared__ float lds_pos[tab_pos ? 2 * PW : 1];
     __shared__ __attribute__((aligned(8))) double lds_tk[tab_ts ? 2 * BN : 1];
     // entry f of the time table: {bounds[f], table[f - 1], table[f]}: a score whose rounded log estimate is f sits in
@@ -445,7 +448,7 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
     // lanes per row) and reads it back from this private tile in the layout of the score registers; loading it in that
     // layout directly would touch 64 cache lines per instruction.  Row stride 72 bytes.
     constexpr int XRS = 72;
-    constexpr bool XTILE = EXTRA == 1 && !PAGED;   // (the paged variant with a dense bias has no registers or LDS to spare for it)
+    constexpr bool XTILE = (EXTRA == 1 || BIAS_ONLY) && !PAGED;   // (the paged variant with a dense bias has no registers or LDS to spare for it)
     __shared__ __attribute__((aligned(16))) char lds_x[XTILE ? 4 * 32 * XRS : 16];
 
     const int tid = threadIdx.x;
@@ -483,7 +486,7 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
     const bool tril = p.mask_type == HSTU_MASK_TRIL;
     const int tgs = p.target_group_size;
     // rows of attn_bias / mask start on 16-byte boundaries
-    const bool x_rows16 = XTILE && p.max_seq_len_k % 8 == 0 && ((reinterpret_cast<uintptr_t>(p.attn_bias) | reinterpret_cast<uintptr_t>(p.mask)) & 15) == 0;
+    const bool x_rows16 = BIAS_ONLY || XTILE && p.max_seq_len_k % 8 == 0 && ((reinterpret_cast<uintptr_t>(p.attn_bias) | reinterpret_cast<uintptr_t>(p.mask)) & 15) == 0;
     const bool x_mask = EXTRA == 1 && p.mask_type == HSTU_MASK_CUSTOM;
     const T* qbase = reinterpret_cast<const T*>(p.q);
     T* obase = reinterpret_cast<T*>(p.out);
@@ -527,7 +530,7 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
             for (int r = 0; r < 16; r++) oacc[db][r] = 0.f;
 
         int64_t tq = 0;
-        if (EXTRA && p.ts_table && qvalid && qi + s.delta >= 0) tq = p.timestamps[s.k_start + qi + s.delta];
+        if (EXTRA && !BIAS_ONLY && p.ts_table && qvalid && qi + s.delta >= 0) tq = p.timestamps[s.k_start + qi + s.delta];
         // LDS-table mode works on timestamps relative to the first one of the sequence, held as doubles: the
         // difference of two of them and its rounding to fp32 equal (float)|t_i - t_j| of the int64 values as long as
         // the timestamps of one sequence span less than 2^53
@@ -710,7 +713,7 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                         const int row = r0 + (lane >> 2) + 16 * i;
                         if (row < p.max_seq_len_q && col < p.max_seq_len_k) {   // outside the attribute's square: no bias, mask 0
                             const int64_t at = (((int64_t)b * p.heads_q + h) * p.max_seq_len_q + row) * (int64_t)p.max_seq_len_k + col;
-                            if (p.attn_bias) xb[i] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const T*>(p.attn_bias) + at);
+                            if (BIAS_ONLY || p.attn_bias) xb[i] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const T*>(p.attn_bias) + at);
                             if (x_mask) xm[i] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const T*>(p.mask) + at);
                         }
                     }
@@ -750,7 +753,7 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                         for (int q = 0; q < 4; q++) out[q] = *reinterpret_cast<const u32x2*>(tile + l32 * XRS + (8 * q + 4 * g) * 2);
                         __builtin_amdgcn_wave_barrier();
                     };
-                    if (p.attn_bias) through_tile(xb, xbr);
+                    if (BIAS_ONLY || p.attn_bias) through_tile(xb, xbr);
                     if (x_mask) through_tile(xm, xmr);
                 }
                 // ---- P = s * sigmoid(alpha * s) (scale folded into the epilogue), masked
@@ -761,6 +764,7 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                     float x = sacc[r];
                     const int j = c0 + 8 * (r >> 2) + 4 * g + (r & 3);
                     float mval = 1.f;
+                    if (BIAS_ONLY) x += half_to_float<T>(xbr[r >> 2][(r >> 1) & 1], r & 1);
                     if (EXTRA == 1) {
                         const bool in_attr = qi < p.max_seq_len_q && j < p.max_seq_len_k;
                         const int64_t bm = (((int64_t)b * p.heads_q + h) * p.max_seq_len_q + qi) * (int64_t)p.max_seq_len_k + j;
@@ -1018,8 +1022,12 @@ static hipError_t launch_td(const KArgs& a, unsigned* ws, hipStream_t stream) {
     // the time table is used from LDS when it fits and the search hint is there; else the general path searches the
     // bounds in global memory
     const bool ts_in_lds = p.ts_table && p.num_buckets <= 128 && p.ts_log2_scale > 0.f;
+    // a dense bias alone, rows on 16-byte boundaries: the variant without the other options
+    const bool bias_only = p.attn_bias && p.mask_type != HSTU_MASK_CUSTOM && !p.pos_table && !p.ts_table && a.op != OP_PAGED &&
+                           p.max_seq_len_k % 8 == 0 && (reinterpret_cast<uintptr_t>(p.attn_bias) & 15) == 0;
     int extra = 0;
-    if (dense_extra || (p.ts_table && !ts_in_lds)) extra = 1;
+    if (bias_only) extra = 5;
+    else if (dense_extra || (p.ts_table && !ts_in_lds)) extra = 1;
     else if (p.pos_table && p.ts_table) extra = 4;
     else if (p.ts_table) extra = 3;
     else if (p.pos_table) extra = 2;
@@ -1039,6 +1047,7 @@ static hipError_t launch_td(const KArgs& a, unsigned* ws, hipStream_t stream) {
         // the head dims at the ends of the reference's sweep: plain and general variants only (bias tables are gathered
         // from global memory by the general one)
         if (extra == 0) HSTU_LAUNCH(0, false);
+        else if (extra == 5) HSTU_LAUNCH(5, false);
         else HSTU_LAUNCH(1, false);
     } else if (paged) {
         if (extra == 0) HSTU_LAUNCH(0, true);
@@ -1048,6 +1057,7 @@ static hipError_t launch_td(const KArgs& a, unsigned* ws, hipStream_t stream) {
         else if (extra == 1) HSTU_LAUNCH(1, false);
         else if (extra == 2) HSTU_LAUNCH(2, false);
         else if (extra == 3) HSTU_LAUNCH(3, false);
+        else if (extra == 5) HSTU_LAUNCH(5, false);
         else HSTU_LAUNCH(4, false);
     }
 #undef HSTU_LAUNCH
