@@ -404,7 +404,9 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
 template <int D, int EXTRA, bool PAGED> struct Shape {
     static constexpr bool DMA = !PAGED && D == 128;
     static constexpr bool LEAN = DMA && EXTRA == 0;
-    static constexpr int BNT = LEAN ? 32 : 64;     // K columns per step
+    // a dense bias alone next to direct K/V copies: its blocks are copied into LDS the same way, one tile ahead
+    static constexpr bool XDMA = DMA && EXTRA == 5;
+    static constexpr int BNT = (LEAN || XDMA) ? 32 : 64;     // K columns per step
     // waves per SIMD; head dim 256 needs the registers of a whole SIMD lane for its 32 x 256 accumulator and Q fragments
     static constexpr int WAVES = D == 256 ? 1 : ((LEAN || (D <= 64 && EXTRA != 1)) ? 3 : 2);
 };
@@ -450,6 +452,15 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
     constexpr int XRS = 72;
     constexpr bool XTILE = (EXTRA == 1 || BIAS_ONLY) && !PAGED;   // (the paged variant with a dense bias has no registers or LDS to spare for it)
     __shared__ __attribute__((aligned(16))) char lds_x[XTILE ? 4 * 32 * XRS : 16];
+    // Direct copies of the bias (or, without a bias, the mask) block of every wave: 32 rows x 32 columns = 2 KB per wave and
+    // K tile, two stages.  One wave instruction copies 16 rows of 64 bytes (lane L: row L / 4, 16-byte slot L % 4); slot s of
+    // row r holds piece s ^ (r / 4 % 4) of the row, which spreads the 8-byte reads in register layout below over all banks.
+    constexpr bool XDMA = SH::XDMA;
+    // Two stages in two separate arrays, like the K/V tiles: the compiler then does not make the reads of one stage wait for
+    // the copy in flight into the other.
+    constexpr int XDW = 2048, XDS = 4 * XDW;   // bytes per wave and per stage
+    __shared__ __attribute__((aligned(1024))) char lds_xd0[XDMA ? XDS : 16];
+    __shared__ __attribute__((aligned(1024))) char lds_xd1[XDMA ? XDS : 16];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -488,6 +499,10 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
     // rows of attn_bias / mask start on 16-byte boundaries
     const bool x_rows16 = BIAS_ONLY || XTILE && p.max_seq_len_k % 8 == 0 && ((reinterpret_cast<uintptr_t>(p.attn_bias) | reinterpret_cast<uintptr_t>(p.mask)) & 15) == 0;
     const bool x_mask = EXTRA == 1 && p.mask_type == HSTU_MASK_CUSTOM;
+    // the direct copies carry the bias of the bias-only variant at head dim 128
+    constexpr bool xd_bias = XDMA, xd_mask = false;
+    const unsigned xd_plane_bytes = (unsigned)p.max_seq_len_q * (unsigned)p.max_seq_len_k * (unsigned)sizeof(T);   // <= 20480^2 * 2
+    const char* xd_plane = reinterpret_cast<const char*>(xd_bias ? p.attn_bias : p.mask) + ((int64_t)b * p.heads_q + h) * (int64_t)xd_plane_bytes;
     const T* qbase = reinterpret_cast<const T*>(p.q);
     T* obase = reinterpret_cast<T*>(p.out);
 
@@ -636,6 +651,26 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                 if (tab_ts && tid < BN) tk_reg = (double)(p.timestamps[s.k_start + min(k0 + tid, s.lk - 1)] - tbase);
             }
         };
+        // direct copy of this wave's block of the bias (mask) for tile kt into a stage, unless the built-in mask hides the
+        // block (wave-uniform).  Pieces outside the [max_q, max_k] square get an offset past the view and arrive as zeros.
+        auto fetch_x = [&](int kt, char* xstage) __attribute__((always_inline)) -> bool {
+            if constexpr (XDMA) {
+                const int k0 = kt * BNT;
+                if (!(xd_bias || xd_mask) || k0 >= kend || (tril && classify_block(s, tgs, i0 + 32 * w, k0) == BLK_SKIP)) return false;
+                __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void*)xd_plane, 0, (int)xd_plane_bytes, 0x00020000);
+                char* xdst = xstage + w * XDW;
+#pragma unroll
+                for (int n = 0; n < 2; n++) {
+                    const int rr = 16 * n + (lane >> 2);                    // row of the block
+                    const int row = i0 + 32 * w + rr, col = k0 + 8 * ((lane & 3) ^ ((rr >> 2) & 3));
+                    const unsigned off = (row < p.max_seq_len_q && col < p.max_seq_len_k)
+                                             ? ((unsigned)row * (unsigned)p.max_seq_len_k + (unsigned)col) * (unsigned)sizeof(T) : 0x80000000u;
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, LDS_PTR(void, xdst + n * 1024), 16, off, 0, 0, 0);
+                }
+                return true;
+            }
+            return false;
+        };
         // second half of the register path, and the table windows; ends with the tile being complete in LDS
         auto stash = [&](int kt, char* dst) __attribute__((always_inline)) {
             const int k0 = kt * BNT;
@@ -688,12 +723,14 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
         const int per = (ntk + nsplit - 1) / nsplit;
         const int kt0 = part * per, kt1 = min(ntk, kt0 + per);
         if (kt0 < kt1) fetch(kt0, lds0);
+        if (XDMA && kt0 < kt1) fetch_x(kt0, lds_xd0);
         stash(kt0, lds0);
 
-        auto iteration = [&](int kt, const char* cur, char* nxt) __attribute__((always_inline)) {
+        auto iteration = [&](int kt, const char* cur, char* nxt, const char* xcur, char* xnxt) __attribute__((always_inline)) {
             const int buf = kt & 1;
             const int k0 = kt * BNT;
             if (kt + 1 < kt1) fetch(kt + 1, nxt);
+            if (XDMA && kt + 1 < kt1) fetch_x(kt + 1, xnxt);
 
 #pragma unroll
             for (int kb = 0; kb < BNT / 32; kb++) {
@@ -706,7 +743,7 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                 // here, used after the S^T products.  (Requesting it one block ahead costs more in spilled registers than
                 // the latency it hides: measured.)
                 u32x4 xb[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}}, xm[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
-                if (XTILE && x_rows16) {
+                if (XTILE && x_rows16 && !xd_bias) {
                     const int col = c0 + 8 * (lane & 3);
 #pragma unroll
                     for (int i = 0; i < 2; i++) {
@@ -753,8 +790,15 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                         for (int q = 0; q < 4; q++) out[q] = *reinterpret_cast<const u32x2*>(tile + l32 * XRS + (8 * q + 4 * g) * 2);
                         __builtin_amdgcn_wave_barrier();
                     };
-                    if (BIAS_ONLY || p.attn_bias) through_tile(xb, xbr);
+                    if ((BIAS_ONLY || p.attn_bias) && !xd_bias) through_tile(xb, xbr);
                     if (x_mask) through_tile(xm, xmr);
+                }
+                if constexpr (XDMA) {
+                    // the copied block in register layout: piece q of row l32 sits in slot q ^ (l32 / 4 % 4)
+                    const char* xt = xcur + w * XDW + l32 * 64 + 8 * g;
+                    const int sw = (l32 >> 2) & 3;
+#pragma unroll
+                    for (int q = 0; q < 4; q++) xbr[q] = *reinterpret_cast<const u32x2*>(xt + 16 * (q ^ sw));
                 }
                 // ---- P = s * sigmoid(alpha * s) (scale folded into the epilogue), masked
                 // accumulator register r holds key c0 + 8*(r/4) + 4*g + r%4 for Q row qi
@@ -892,8 +936,8 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
             stash(kt + 1, nxt);
         };
         for (int kt = kt0; kt < kt1; kt += 2) {
-            iteration(kt, lds0, lds1);
-            if (kt + 1 < kt1) iteration(kt + 1, lds1, lds0);
+            iteration(kt, lds0, lds1, lds_xd0, lds_xd1);
+            if (kt + 1 < kt1) iteration(kt + 1, lds1, lds0, lds_xd1, lds_xd0);
         }
 
         // ---- epilogue: O^T accumulator register r of block db holds d = 32*db + 8*(r/4) + 4*g + r%4 for row qi
