@@ -392,8 +392,8 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
 }
 
 
-// EXTRA: 5 = a dense bias whose rows start on 16-byte boundaries and nothing else (built-in mask or none): the general
-// variant's per-score code carries every option as a run-time test and runs 2.7 x slower than this one on the same input;
+// EXTRA: 5 / 6 / 7 = a dense bias / a custom mask / both, rows on 16-byte boundaries, and nothing else: the general
+// variant's per-score code carries every option as a run-time test and runs 2.7 x slower than these on the same input;
 // 0 = no bias / built-in mask only, 1 = dense bias and/or custom mask (tables, if any, gathered from
 // global memory), 2 / 3 / 4 = bias tables only, gathered from LDS-resident copies: position table / time table /
 // both (compile-time so that the per-score code is branch-free)
@@ -404,8 +404,8 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
 template <int D, int EXTRA, bool PAGED> struct Shape {
     static constexpr bool DMA = !PAGED && D == 128;
     static constexpr bool LEAN = DMA && EXTRA == 0;
-    // a dense bias alone next to direct K/V copies: its blocks are copied into LDS the same way, one tile ahead
-    static constexpr bool XDMA = DMA && EXTRA == 5;
+    // a dense bias (or, without one, a custom mask) next to direct K/V copies: its blocks are copied into LDS the same way, one tile ahead
+    static constexpr bool XDMA = DMA && EXTRA >= 5;
     static constexpr int BNT = (LEAN || XDMA) ? 32 : 64;     // K columns per step
     // waves per SIMD; head dim 256 needs the registers of a whole SIMD lane for its 32 x 256 accumulator and Q fragments
     static constexpr int WAVES = D == 256 ? 1 : ((LEAN || (D <= 64 && EXTRA != 1)) ? 3 : 2);
@@ -437,7 +437,8 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
     // K/V tiles), plus the whole time table and its bucket bounds as (lower, upper) pairs
     constexpr int PW = BM + BN;   // window entries: (j - k0) - (qi - i0) + BM - 1 in [0, BM + BN - 2]
     constexpr bool TAB = EXTRA >= 2 && EXTRA <= 4, tab_pos = EXTRA == 2 || EXTRA == 4, tab_ts = EXTRA == 3 || EXTRA == 4;
-    constexpr bool BIAS_ONLY = EXTRA == 5;   // attn_bias given, rows on 16-byte boundaries, no custom mask, no tables (host-checked)
+    // the dense-only variants: attn_bias (XB) and / or custom mask (XM) given, rows on 16-byte boundaries, no tables (host-checked)
+    constexpr bool DENSE_ONLY = EXTRA >= 5, XB = EXTRA == 5 || EXTRA == 7, XM = EXTRA == 6 || EXTRA == 7;
     __shared__ float lds_pos[tab_pos ? 2 * PW : 1];
     __shared__ __attribute__((aligned(8))) double lds_tk[tab_ts ? 2 * BN : 1];
     // entry f of the time table: {bounds[f], table[f - 1], table[f]}: a score whose rounded log estimate is f sits in
@@ -450,7 +451,7 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
     // lanes per row) and reads it back from this private tile in the layout of the score registers; loading it in that
     // layout directly would touch 64 cache lines per instruction.  Row stride 72 bytes.
     constexpr int XRS = 72;
-    constexpr bool XTILE = (EXTRA == 1 || BIAS_ONLY) && !PAGED;   // (the paged variant with a dense bias has no registers or LDS to spare for it)
+    constexpr bool XTILE = (EXTRA == 1 || DENSE_ONLY) && !PAGED;   // (the paged variant with a dense bias has no registers or LDS to spare for it)
     __shared__ __attribute__((aligned(16))) char lds_x[XTILE ? 4 * 32 * XRS : 16];
     // Direct copies of the bias (or, without a bias, the mask) block of every wave: 32 rows x 32 columns = 2 KB per wave and
     // K tile, two stages.  One wave instruction copies 16 rows of 64 bytes (lane L: row L / 4, 16-byte slot L % 4); slot s of
@@ -497,10 +498,10 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
     const bool tril = p.mask_type == HSTU_MASK_TRIL;
     const int tgs = p.target_group_size;
     // rows of attn_bias / mask start on 16-byte boundaries
-    const bool x_rows16 = BIAS_ONLY || XTILE && p.max_seq_len_k % 8 == 0 && ((reinterpret_cast<uintptr_t>(p.attn_bias) | reinterpret_cast<uintptr_t>(p.mask)) & 15) == 0;
-    const bool x_mask = EXTRA == 1 && p.mask_type == HSTU_MASK_CUSTOM;
-    // the direct copies carry the bias of the bias-only variant at head dim 128
-    constexpr bool xd_bias = XDMA, xd_mask = false;
+    const bool x_rows16 = DENSE_ONLY || XTILE && p.max_seq_len_k % 8 == 0 && ((reinterpret_cast<uintptr_t>(p.attn_bias) | reinterpret_cast<uintptr_t>(p.mask)) & 15) == 0;
+    const bool x_mask = XM || (EXTRA == 1 && p.mask_type == HSTU_MASK_CUSTOM);
+    // the direct copies (head dim 128) carry the bias, or the mask of the variant without a bias; with both the mask keeps the tile path
+    constexpr bool xd_bias = XDMA && XB, xd_mask = XDMA && !XB;
     const unsigned xd_plane_bytes = (unsigned)p.max_seq_len_q * (unsigned)p.max_seq_len_k * (unsigned)sizeof(T);   // <= 20480^2 * 2
     const char* xd_plane = reinterpret_cast<const char*>(xd_bias ? p.attn_bias : p.mask) + ((int64_t)b * p.heads_q + h) * (int64_t)xd_plane_bytes;
     const T* qbase = reinterpret_cast<const T*>(p.q);
@@ -545,7 +546,7 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
             for (int r = 0; r < 16; r++) oacc[db][r] = 0.f;
 
         int64_t tq = 0;
-        if (EXTRA && !BIAS_ONLY && p.ts_table && qvalid && qi + s.delta >= 0) tq = p.timestamps[s.k_start + qi + s.delta];
+        if (EXTRA && !DENSE_ONLY && p.ts_table && qvalid && qi + s.delta >= 0) tq = p.timestamps[s.k_start + qi + s.delta];
         // LDS-table mode works on timestamps relative to the first one of the sequence, held as doubles: the
         // difference of two of them and its rounding to fp32 equal (float)|t_i - t_j| of the int64 values as long as
         // the timestamps of one sequence span less than 2^53
@@ -743,15 +744,15 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                 // here, used after the S^T products.  (Requesting it one block ahead costs more in spilled registers than
                 // the latency it hides: measured.)
                 u32x4 xb[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}}, xm[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
-                if (XTILE && x_rows16 && !xd_bias) {
+                if (XTILE && x_rows16 && !(XDMA && !(XB && XM))) {
                     const int col = c0 + 8 * (lane & 3);
 #pragma unroll
                     for (int i = 0; i < 2; i++) {
                         const int row = r0 + (lane >> 2) + 16 * i;
                         if (row < p.max_seq_len_q && col < p.max_seq_len_k) {   // outside the attribute's square: no bias, mask 0
                             const int64_t at = (((int64_t)b * p.heads_q + h) * p.max_seq_len_q + row) * (int64_t)p.max_seq_len_k + col;
-                            if (BIAS_ONLY || p.attn_bias) xb[i] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const T*>(p.attn_bias) + at);
-                            if (x_mask) xm[i] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const T*>(p.mask) + at);
+                            if ((XB || (EXTRA == 1 && p.attn_bias)) && !xd_bias) xb[i] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const T*>(p.attn_bias) + at);
+                            if (x_mask && !xd_mask) xm[i] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const T*>(p.mask) + at);
                         }
                     }
                 }
@@ -790,15 +791,20 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                         for (int q = 0; q < 4; q++) out[q] = *reinterpret_cast<const u32x2*>(tile + l32 * XRS + (8 * q + 4 * g) * 2);
                         __builtin_amdgcn_wave_barrier();
                     };
-                    if ((BIAS_ONLY || p.attn_bias) && !xd_bias) through_tile(xb, xbr);
-                    if (x_mask) through_tile(xm, xmr);
+                    if ((XB || (EXTRA == 1 && p.attn_bias)) && !xd_bias) through_tile(xb, xbr);
+                    if (x_mask && !xd_mask) through_tile(xm, xmr);
                 }
                 if constexpr (XDMA) {
                     // the copied block in register layout: piece q of row l32 sits in slot q ^ (l32 / 4 % 4)
                     const char* xt = xcur + w * XDW + l32 * 64 + 8 * g;
                     const int sw = (l32 >> 2) & 3;
+                    if constexpr (xd_bias) {
 #pragma unroll
-                    for (int q = 0; q < 4; q++) xbr[q] = *reinterpret_cast<const u32x2*>(xt + 16 * (q ^ sw));
+                        for (int q = 0; q < 4; q++) xbr[q] = *reinterpret_cast<const u32x2*>(xt + 16 * (q ^ sw));
+                    } else {
+#pragma unroll
+                        for (int q = 0; q < 4; q++) xmr[q] = *reinterpret_cast<const u32x2*>(xt + 16 * (q ^ sw));
+                    }
                 }
                 // ---- P = s * sigmoid(alpha * s) (scale folded into the epilogue), masked
                 // accumulator register r holds key c0 + 8*(r/4) + 4*g + r%4 for Q row qi
@@ -808,7 +814,8 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                     float x = sacc[r];
                     const int j = c0 + 8 * (r >> 2) + 4 * g + (r & 3);
                     float mval = 1.f;
-                    if (BIAS_ONLY) x += half_to_float<T>(xbr[r >> 2][(r >> 1) & 1], r & 1);
+                    if (XB) x += half_to_float<T>(xbr[r >> 2][(r >> 1) & 1], r & 1);
+                    if (XM) mval = half_to_float<T>(xmr[r >> 2][(r >> 1) & 1], r & 1);
                     if (EXTRA == 1) {
                         const bool in_attr = qi < p.max_seq_len_q && j < p.max_seq_len_k;
                         const int64_t bm = (((int64_t)b * p.heads_q + h) * p.max_seq_len_q + qi) * (int64_t)p.max_seq_len_k + j;
@@ -841,7 +848,7 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                     }
                     float e = __builtin_amdgcn_exp2f(x * a.exp_scale);
                     float pv = x * __builtin_amdgcn_rcpf(1.0f + e);
-                    if (EXTRA == 1) pv *= mval;
+                    if (EXTRA == 1 || XM) pv *= mval;
                     pf[r] = pv;
                 }
                 // The built-in mask: the two-per-CU variants zero the fp32 values; the register-tight ones mask the packed
@@ -1066,11 +1073,12 @@ static hipError_t launch_td(const KArgs& a, unsigned* ws, hipStream_t stream) {
     // the time table is used from LDS when it fits and the search hint is there; else the general path searches the
     // bounds in global memory
     const bool ts_in_lds = p.ts_table && p.num_buckets <= 128 && p.ts_log2_scale > 0.f;
-    // a dense bias alone, rows on 16-byte boundaries: the variant without the other options
-    const bool bias_only = p.attn_bias && p.mask_type != HSTU_MASK_CUSTOM && !p.pos_table && !p.ts_table && a.op != OP_PAGED &&
-                           p.max_seq_len_k % 8 == 0 && (reinterpret_cast<uintptr_t>(p.attn_bias) & 15) == 0;
+    // a dense bias and / or a custom mask alone, rows on 16-byte boundaries: the variants without the other options
+    const bool custom = p.mask_type == HSTU_MASK_CUSTOM;
+    const bool dense_only = dense_extra && !p.pos_table && !p.ts_table && a.op != OP_PAGED && p.max_seq_len_k % 8 == 0 &&
+                            ((reinterpret_cast<uintptr_t>(p.attn_bias) | (custom ? reinterpret_cast<uintptr_t>(p.mask) : 0)) & 15) == 0;
     int extra = 0;
-    if (bias_only) extra = 5;
+    if (dense_only) extra = p.attn_bias ? (custom ? 7 : 5) : 6;
     else if (dense_extra || (p.ts_table && !ts_in_lds)) extra = 1;
     else if (p.pos_table && p.ts_table) extra = 4;
     else if (p.ts_table) extra = 3;
@@ -1092,6 +1100,8 @@ static hipError_t launch_td(const KArgs& a, unsigned* ws, hipStream_t stream) {
         // from global memory by the general one)
         if (extra == 0) HSTU_LAUNCH(0, false);
         else if (extra == 5) HSTU_LAUNCH(5, false);
+        else if (extra == 6) HSTU_LAUNCH(6, false);
+        else if (extra == 7) HSTU_LAUNCH(7, false);
         else HSTU_LAUNCH(1, false);
     } else if (paged) {
         if (extra == 0) HSTU_LAUNCH(0, true);
@@ -1102,6 +1112,8 @@ static hipError_t launch_td(const KArgs& a, unsigned* ws, hipStream_t stream) {
         else if (extra == 2) HSTU_LAUNCH(2, false);
         else if (extra == 3) HSTU_LAUNCH(3, false);
         else if (extra == 5) HSTU_LAUNCH(5, false);
+        else if (extra == 6) HSTU_LAUNCH(6, false);
+        else if (extra == 7) HSTU_LAUNCH(7, false);
         else HSTU_LAUNCH(4, false);
     }
 #undef HSTU_LAUNCH

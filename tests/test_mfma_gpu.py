@@ -94,10 +94,18 @@ def test_mfma_dense_bias_row_pieces(d, dtype):
     cfg["mask"] = torch.from_numpy(rng.integers(0, 2, (b, n, m, m)).astype(np.float32)).to(dtype)
     cfg["mask_type"] = 3
     _check(cfg, dtype, "dense bias + custom mask, 16-byte rows")
+    del cfg["attn_bias"]
+    _check(cfg, dtype, "custom mask alone, 16-byte rows")
     cfg2, rng = _jag(62, [70, 200, 33], 4, 2, d, d, dtype, lens_k=[130, 200, 97])
     mq, mk = 200, 200
     cfg2["attn_bias"] = torch.from_numpy(rng.normal(0, 0.7, (3, 4, mq, mk)).astype(np.float32)).to(dtype)
     _check(cfg2, dtype, "dense bias, delta-q + GQA")
+    # long enough for the copies of the bias blocks to run several tiles ahead of the products, with context rows and targets
+    cfg4, rng = _jag(64, [700, 391], 2, 1, d, d, dtype)
+    cfg4["num_context"] = torch.tensor([5, 0]); cfg4["num_target"] = torch.tensor([40, 17]); cfg4["target_group_size"] = 2
+    cfg4["attn_bias"] = torch.from_numpy(rng.normal(0, 0.7, (2, 2, 704, 704)).astype(np.float32)).to(dtype)
+    cfg4["max_seq_len"] = 704
+    _check(cfg4, dtype, "dense bias, long sequences, context rows and targets")
     cfg3, rng = _jag(63, [300, 140], 2, 2, d, d, dtype)
     cfg3["max_seq_len"] = 104
     cfg3["attn_bias"] = torch.from_numpy(rng.normal(0, 0.7, (2, 2, 104, 104)).astype(np.float32)).to(dtype)
