@@ -1,4 +1,4 @@
-// HSTU forward on the gfx950 matrix cores (bf16 / fp16 I/O, head dim 64 or 128).
+// HSTU forward on the gfx950 matrix cores (bf16 / fp16 I/O, head dim 32, 64, 128 or 256).
 //
 // One workgroup (4 waves) owns a 128-row Q tile of one (sequence, head); wave w owns rows 32w..32w+31.
 // K and V tiles of 64 columns (32 in the plain head-dim-128 variant, see Shape) stream through LDS, double buffered,
@@ -401,11 +401,13 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
 // LDS with 32-column K/V tiles: three workgroups per CU (3 waves/SIMD), which overlaps the MFMA, SiLU and LDS phases of
 // the waves better than two (measured -8 %).  The head-dim-64 variants other than the dense-bias one fit three per CU
 // with 64-column tiles (-10..15 %).  The rest run 64-column tiles at two workgroups per CU.
+// EXTRA 8 (paged only) = no bias like 0, with 2-byte pages of a multiple of 4 rows copied straight into LDS.
 template <int D, int EXTRA, bool PAGED> struct Shape {
-    static constexpr bool DMA = !PAGED && D == 128;
-    static constexpr bool LEAN = DMA && EXTRA == 0;
+    static constexpr bool PDMA = PAGED && EXTRA == 8 && D == 128;
+    static constexpr bool DMA = (!PAGED && D == 128) || PDMA;
+    static constexpr bool LEAN = DMA && (EXTRA == 0 || EXTRA == 8);
     // a dense bias (or, without one, a custom mask) next to direct K/V copies: its blocks are copied into LDS the same way, one tile ahead
-    static constexpr bool XDMA = DMA && EXTRA >= 5;
+    static constexpr bool XDMA = DMA && EXTRA >= 5 && EXTRA <= 7;
     static constexpr int BNT = (LEAN || XDMA) ? 32 : 64;     // K columns per step
     // waves per SIMD; head dim 256 needs the registers of a whole SIMD lane for its 32 x 256 accumulator and Q fragments
     static constexpr int WAVES = D == 256 ? 1 : ((LEAN || (D <= 64 && EXTRA != 1)) ? 3 : 2);
@@ -438,7 +440,7 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
     constexpr int PW = BM + BN;   // window entries: (j - k0) - (qi - i0) + BM - 1 in [0, BM + BN - 2]
     constexpr bool TAB = EXTRA >= 2 && EXTRA <= 4, tab_pos = EXTRA == 2 || EXTRA == 4, tab_ts = EXTRA == 3 || EXTRA == 4;
     // the dense-only variants: attn_bias (XB) and / or custom mask (XM) given, rows on 16-byte boundaries, no tables (host-checked)
-    constexpr bool DENSE_ONLY = EXTRA >= 5, XB = EXTRA == 5 || EXTRA == 7, XM = EXTRA == 6 || EXTRA == 7;
+    constexpr bool DENSE_ONLY = EXTRA >= 5 && EXTRA <= 7, XB = EXTRA == 5 || EXTRA == 7, XM = EXTRA == 6 || EXTRA == 7;
     __shared__ float lds_pos[tab_pos ? 2 * PW : 1];
     __shared__ __attribute__((aligned(8))) double lds_tk[tab_ts ? 2 * BN : 1];
     // entry f of the time table: {bounds[f], table[f - 1], table[f]}: a score whose rounded log estimate is f sits in
@@ -546,7 +548,7 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
             for (int r = 0; r < 16; r++) oacc[db][r] = 0.f;
 
         int64_t tq = 0;
-        if (EXTRA && !DENSE_ONLY && p.ts_table && qvalid && qi + s.delta >= 0) tq = p.timestamps[s.k_start + qi + s.delta];
+        if (EXTRA && EXTRA <= 4 && p.ts_table && qvalid && qi + s.delta >= 0) tq = p.timestamps[s.k_start + qi + s.delta];
         // LDS-table mode works on timestamps relative to the first one of the sequence, held as doubles: the
         // difference of two of them and its rounding to fp32 equal (float)|t_i - t_j| of the int64 values as long as
         // the timestamps of one sequence span less than 2^53
@@ -585,7 +587,42 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
         const unsigned view_bytes = kend > 0 ? (unsigned)(kend - 1) * rowstride + D * 2 : 0;
         auto fetch = [&](int kt, char* dst) __attribute__((always_inline)) {
             const int k0 = kt * BNT;
-            if constexpr (DMA) {
+            if constexpr (SH::PDMA) {
+                // Paged rows by direct copies.  A block of 4 rows lies in one page (page_size % 4 == 0, host-checked) or behind
+                // the history, in the candidate rows of k / v; lanes of a block that straddles the two take their side under
+                // the execution mask.  Rows past the visible range get an offset past the view and arrive as zeros.
+                const int ps = p.page_size;
+                const unsigned plane_bytes = (unsigned)ps * rowstride;     // the K (or V) half of a page
+                const char* cand_k = reinterpret_cast<const char*>(p.k) + ((int64_t)s.cand_row * p.heads_k + hk) * D * 2;
+                const char* cand_v = reinterpret_cast<const char*>(p.v) + ((int64_t)s.cand_row * p.heads_k + hk) * D * 2;
+                const unsigned chunkK = ((lpos - lrho) & 15) << 4, chunkV = ((lpos - 4 * lrho) & 15) << 4;
+#pragma unroll
+                for (int i = 0; i < NBLK4 / 4; i++) {
+                    const int blk = (NBLK4 / 4) * w + i;
+                    const int j0 = k0 + 4 * blk, j = j0 + lrho;            // first key of the block, this lane's key
+                    const int pq = j0 / ps, slot0 = j0 - pq * ps;          // page of the block in the user's list, its first slot (wave-uniform)
+                    const int pidx = min(pq, MAXP - 1);
+                    const int64_t page = __builtin_amdgcn_readfirstlane(lds_pid[j0 < s.hist_k ? pidx : 0]);
+                    const char* pk = reinterpret_cast<const char*>(p.kv_cache) + page * (int64_t)(2u * plane_bytes) + (unsigned)hk * D * 2;
+                    __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc((void*)pk, 0, 0x7fffffff, 0x00020000);
+                    __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc((void*)(pk + plane_bytes), 0, 0x7fffffff, 0x00020000);
+                    __amdgpu_buffer_rsrc_t ck = __builtin_amdgcn_make_buffer_rsrc((void*)cand_k, 0, 0x7fffffff, 0x00020000);
+                    __amdgpu_buffer_rsrc_t cv = __builtin_amdgcn_make_buffer_rsrc((void*)cand_v, 0, 0x7fffffff, 0x00020000);
+                    char* kd = dst + blk * KBLK;
+                    char* vd = dst + NBLK4 * KBLK + blk * VBLK;
+                    if (j < s.hist_k) {
+                        const unsigned row = (unsigned)(slot0 + lrho) * rowstride;
+                        const unsigned ok = j < kend ? 0u : 0x80000000u;
+                        __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, LDS_PTR(void, kd), 16, (row + chunkK) | ok, 0, 0, 0);
+                        __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, LDS_PTR(void, vd), 16, (row + chunkV) | ok, 0, 0, 0);
+                    } else {
+                        const unsigned row = (unsigned)(j - s.hist_k) * rowstride;
+                        const unsigned ok = j < kend ? 0u : 0x80000000u;
+                        __builtin_amdgcn_raw_ptr_buffer_load_lds(ck, LDS_PTR(void, kd), 16, (row + chunkK) | ok, 0, 0, 0);
+                        __builtin_amdgcn_raw_ptr_buffer_load_lds(cv, LDS_PTR(void, vd), 16, (row + chunkV) | ok, 0, 0, 0);
+                    }
+                }
+            } else if constexpr (DMA) {
                 const unsigned tile_off = (unsigned)k0 * rowstride;
                 __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc((void*)(kview + tile_off), 0, (int)(view_bytes - tile_off), 0x00020000);
                 __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc((void*)(vview + tile_off), 0, (int)(view_bytes - tile_off), 0x00020000);
@@ -1104,7 +1141,10 @@ static hipError_t launch_td(const KArgs& a, unsigned* ws, hipStream_t stream) {
         else if (extra == 7) HSTU_LAUNCH(7, false);
         else HSTU_LAUNCH(1, false);
     } else if (paged) {
-        if (extra == 0) HSTU_LAUNCH(0, true);
+        // pages in the dtype of q with a multiple of 4 rows: rows are copied straight into LDS (head dim 128)
+        const bool page_copies = D == 128 && p.cache_dtype == p.dtype && p.page_size % 4 == 0;
+        if (extra == 0 && page_copies) HSTU_LAUNCH(8, true);
+        else if (extra == 0) HSTU_LAUNCH(0, true);
         else HSTU_LAUNCH(1, true);      // paged + bias: the general gather path
     } else {
         if (extra == 0) HSTU_LAUNCH(0, false);

@@ -151,7 +151,7 @@ def test_mfma_table_bias(d, dtype):
 
 
 @pytest.mark.parametrize("dtype", LOWP)
-@pytest.mark.parametrize("d,page_size,new_hist", [(64, 32, 0), (128, 64, 7), (128, 16, 130)])
+@pytest.mark.parametrize("d,page_size,new_hist", [(64, 32, 0), (128, 64, 7), (128, 16, 130), (128, 12, 5), (128, 10, 3)])
 def test_mfma_paged(d, page_size, new_hist, dtype):
     say("mfma_paged", dtype, d, page_size, new_hist)
     cfg = W.paged_config(28, 5, 2, d, new_hist + 1, 400, 40, page_size, dtype, new_hist=new_hist)
