@@ -401,11 +401,13 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
 // LDS with 32-column K/V tiles: three workgroups per CU (3 waves/SIMD), which overlaps the MFMA, SiLU and LDS phases of
 // the waves better than two (measured -8 %).  The head-dim-64 variants other than the dense-bias one fit three per CU
 // with 64-column tiles (-10..15 %).  The rest run 64-column tiles at two workgroups per CU.
-// EXTRA 8 (paged only) = no bias like 0, with 2-byte pages of a multiple of 4 rows copied straight into LDS.
+// EXTRA 8 (paged only) = no bias like 0, with 2-byte pages of a multiple of 4 rows copied straight into LDS; 9 = the same
+// for fp8 pages of a multiple of 8 rows: the raw bytes are copied into a staging area and widened from there.
 template <int D, int EXTRA, bool PAGED> struct Shape {
-    static constexpr bool PDMA = PAGED && EXTRA == 8 && D == 128;
+    static constexpr bool PDMA8 = PAGED && EXTRA == 9 && D == 128;
+    static constexpr bool PDMA = PAGED && (EXTRA == 8 || EXTRA == 9) && D == 128;
     static constexpr bool DMA = (!PAGED && D == 128) || PDMA;
-    static constexpr bool LEAN = DMA && (EXTRA == 0 || EXTRA == 8);
+    static constexpr bool LEAN = DMA && (EXTRA == 0 || EXTRA == 8 || EXTRA == 9);
     // a dense bias (or, without one, a custom mask) next to direct K/V copies: its blocks are copied into LDS the same way, one tile ahead
     static constexpr bool XDMA = DMA && EXTRA >= 5 && EXTRA <= 7;
     static constexpr int BNT = (LEAN || XDMA) ? 32 : 64;     // K columns per step
@@ -447,6 +449,8 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
     // bucket f or f - 1, and the exact bound decides which
     __shared__ __attribute__((aligned(16))) float lds_tsq[tab_ts ? 4 * 132 : 4];
     // paged: page ids of this user and, for an fp8 cache, the (K, V) scales of this kv head
+    // fp8 pages by direct copies: raw rows of the next tile (32 keys x 128 bytes of K, then of V; wave w owns keys 8w..8w+7)
+    __shared__ __attribute__((aligned(1024))) char lds_raw[SH::PDMA8 ? 2 * 4096 : 16];
     __shared__ int lds_pid[PAGED ? MAXP : 1];
     __shared__ float lds_psc[PAGED ? 2 * MAXP : 1];
     // dense bias / custom mask: every wave takes its 32 x 32 block in as whole 64-byte row pieces (16 bytes per lane, four
@@ -610,7 +614,15 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                     __amdgpu_buffer_rsrc_t cv = __builtin_amdgcn_make_buffer_rsrc((void*)cand_v, 0, 0x7fffffff, 0x00020000);
                     char* kd = dst + blk * KBLK;
                     char* vd = dst + NBLK4 * KBLK + blk * VBLK;
-                    if (j < s.hist_k) {
+                    if constexpr (SH::PDMA8) {
+                        // only the candidate rows (k / v inputs) come in here; the history rows follow below
+                        if (j >= s.hist_k) {
+                            const unsigned row = (unsigned)(j - s.hist_k) * rowstride;
+                            const unsigned ok = j < kend ? 0u : 0x80000000u;
+                            __builtin_amdgcn_raw_ptr_buffer_load_lds(ck, LDS_PTR(void, kd), 16, (row + chunkK) | ok, 0, 0, 0);
+                            __builtin_amdgcn_raw_ptr_buffer_load_lds(cv, LDS_PTR(void, vd), 16, (row + chunkV) | ok, 0, 0, 0);
+                        }
+                    } else if (j < s.hist_k) {
                         const unsigned row = (unsigned)(slot0 + lrho) * rowstride;
                         const unsigned ok = j < kend ? 0u : 0x80000000u;
                         __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, LDS_PTR(void, kd), 16, (row + chunkK) | ok, 0, 0, 0);
@@ -620,6 +632,22 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                         const unsigned ok = j < kend ? 0u : 0x80000000u;
                         __builtin_amdgcn_raw_ptr_buffer_load_lds(ck, LDS_PTR(void, kd), 16, (row + chunkK) | ok, 0, 0, 0);
                         __builtin_amdgcn_raw_ptr_buffer_load_lds(cv, LDS_PTR(void, vd), 16, (row + chunkV) | ok, 0, 0, 0);
+                    }
+                }
+                if constexpr (SH::PDMA8) {
+                    // raw fp8 history rows of this wave's 8 keys (one page: page_size % 8 == 0): lane L = row L / 8, bytes 16 (L % 8) .. + 15
+                    const int j0 = k0 + 8 * w;
+                    if (j0 < s.hist_k) {
+                        const int pq = j0 / ps, slot0 = j0 - pq * ps;
+                        const int64_t page = __builtin_amdgcn_readfirstlane(lds_pid[min(pq, MAXP - 1)]);
+                        const unsigned row8 = (unsigned)p.heads_k * D;           // bytes between consecutive fp8 rows of a page
+                        const unsigned plane8 = (unsigned)ps * row8;
+                        const char* pk = reinterpret_cast<const char*>(p.kv_cache) + page * (int64_t)(2u * plane8) + (unsigned)hk * D;
+                        __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc((void*)pk, 0, 0x7fffffff, 0x00020000);
+                        __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc((void*)(pk + plane8), 0, 0x7fffffff, 0x00020000);
+                        const unsigned off = (j0 + (lane >> 3) < s.hist_k) ? (unsigned)(slot0 + (lane >> 3)) * row8 + 16u * (lane & 7) : 0x80000000u;
+                        __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, LDS_PTR(void, lds_raw + 1024 * w), 16, off, 0, 0, 0);
+                        __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, LDS_PTR(void, lds_raw + 4096 + 1024 * w), 16, off, 0, 0, 0);
                     }
                 }
             } else if constexpr (DMA) {
@@ -736,6 +764,24 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                 if (tab_ts && tid < BN) lds_tk[buf * BN + tid] = tk_reg;
             }
             if constexpr (DMA) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            if constexpr (SH::PDMA8) {
+                // widen this wave's staged history rows (e4m3 x the page's scale, rounded once to the I/O dtype) into the tile:
+                // lane L holds 16 elements of key k0 + 8w + L / 8 = chunks 2 (L % 8) and + 1 of row rho = that key % 4
+                const int j0 = k0 + 8 * w, j = j0 + (lane >> 3);
+                if (k0 < kend && j < s.hist_k) {
+                    const int pc = min(j0 / p.page_size, MAXP - 1);
+                    const float ks = lds_psc[2 * pc], vs = lds_psc[2 * pc + 1];
+                    const u32x4 rk = *reinterpret_cast<const u32x4*>(lds_raw + 1024 * w + 16 * lane);
+                    const u32x4 rv = *reinterpret_cast<const u32x4*>(lds_raw + 4096 + 1024 * w + 16 * lane);
+                    const int blk = 2 * w + (lane >> 5), rho = (lane >> 3) & 3, c = 2 * (lane & 7);
+                    char* kd = dst + blk * KBLK + rho * 256;
+                    char* vd = dst + NBLK4 * KBLK + blk * VBLK + rho * 256;
+                    *reinterpret_cast<u32x4*>(kd + (((c + rho) & 15) << 4)) = dequant_chunk<T>((u32x4){rk[0], rk[1], 0u, 0u}, ks);
+                    *reinterpret_cast<u32x4*>(kd + (((c + 1 + rho) & 15) << 4)) = dequant_chunk<T>((u32x4){rk[2], rk[3], 0u, 0u}, ks);
+                    *reinterpret_cast<u32x4*>(vd + (((c + 4 * rho) & 15) << 4)) = dequant_chunk<T>((u32x4){rv[0], rv[1], 0u, 0u}, vs);
+                    *reinterpret_cast<u32x4*>(vd + (((c + 1 + 4 * rho) & 15) << 4)) = dequant_chunk<T>((u32x4){rv[2], rv[3], 0u, 0u}, vs);
+                }
+            }
             __syncthreads();
         };
         // fragment reads
@@ -1143,7 +1189,9 @@ static hipError_t launch_td(const KArgs& a, unsigned* ws, hipStream_t stream) {
     } else if (paged) {
         // pages in the dtype of q with a multiple of 4 rows: rows are copied straight into LDS (head dim 128)
         const bool page_copies = D == 128 && p.cache_dtype == p.dtype && p.page_size % 4 == 0;
+        const bool page_copies8 = D == 128 && p.cache_dtype == HSTU_FP8_E4M3 && p.page_size % 8 == 0;
         if (extra == 0 && page_copies) HSTU_LAUNCH(8, true);
+        else if (extra == 0 && page_copies8) HSTU_LAUNCH(9, true);
         else if (extra == 0) HSTU_LAUNCH(0, true);
         else HSTU_LAUNCH(1, true);      // paged + bias: the general gather path
     } else {
