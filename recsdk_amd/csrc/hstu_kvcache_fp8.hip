@@ -7,10 +7,12 @@
 //   s = absmax(new rows) / 448 (1 if that is 0) otherwise;  rows already there are requantised from q * s_before
 //   when s grew and are left untouched bit for bit when it did not.
 // A page filled by one append therefore equals quantising the whole page at once.
-// Four small kernels on the stream, nothing read on the host:
-//   init   clears the per-unit maxima and per-page first slots in the workspace
-//   scan   absmax of every new (token, K|V, head) row -> atomic max per unit, atomic min of the slot per page
-//   scale  per touched unit: new scale, requantise the rows below the first new slot if the scale grew
+// Four small kernels on the stream, nothing read on the host, all of them sized by the new tokens and not by the cache
+// (a table of a million pages costs an append of one token no more than a table of ten):
+//   reset  clears the per-unit maxima and the first slot of the pages the new tokens go to, and the list of touched pages
+//   scan   absmax of every new (token, K|V, head) row -> atomic max per unit, atomic min of the slot per page; the token
+//          that finds a page untouched enters it in the list
+//   scale  per unit of a listed page: new scale, requantise the rows below the first new slot if the scale grew
 //   write  quantise the new rows with the unit's scale
 // Byte work bounded by HBM: the new rows are read twice (2 bytes per element) and written once (1 byte).
 #include "hstu_device.h"
@@ -49,16 +51,23 @@ __device__ __forceinline__ bool kf_route(const hstu_kv_append_fp8_params& p, uns
     return page >= 0 && page < p.num_pages && row >= 0 && row < p.append_rows;
 }
 
-__global__ __launch_bounds__(256) void hstu_kv_fp8_init_kernel(unsigned* unit_max, int units, int* first_slot, int pages) {
-    const int i = blockIdx.x * 256 + threadIdx.x;
-    if (i < units) unit_max[i] = 0u;
-    if (i < pages) first_slot[i] = KF_NOSLOT;
+// one thread per new token: the workspace entries of its page start from scratch (several tokens of a page write the same values)
+__global__ __launch_bounds__(256) void hstu_kv_fp8_reset_kernel(const hstu_kv_append_fp8_params p, unsigned* unit_max, int* first_slot, int* touched) {
+    const int nnz = min(max(*p.nnz_dev, 0), p.nnz_max);
+    if (blockIdx.x == 0 && threadIdx.x == 0) touched[0] = 0;
+    for (unsigned i = blockIdx.x * 256 + threadIdx.x; i < (unsigned)nnz; i += gridDim.x * 256) {
+        int page, slot;
+        int64_t row;
+        if (!kf_route(p, i, page, slot, row)) continue;
+        for (int u = 0; u < 2 * p.num_heads; u++) unit_max[(int64_t)page * 2 * p.num_heads + u] = 0u;
+        first_slot[page] = KF_NOSLOT;
+    }
 }
 
 // one lane = the same 8 elements of the K row and of the V row of one (token, head); the dim / 8 lanes of a row sit
 // side by side in a wave.  IDX: type of the flat lane index, 32 bits whenever nnz_max * lanes per token fits
 template <typename IDX>
-__global__ __launch_bounds__(256) void hstu_kv_fp8_scan_kernel(const hstu_kv_append_fp8_params p, unsigned* unit_max, int* first_slot) {
+__global__ __launch_bounds__(256) void hstu_kv_fp8_scan_kernel(const hstu_kv_append_fp8_params p, unsigned* unit_max, int* first_slot, int* touched, int touched_cap) {
     const unsigned cph = (unsigned)p.head_dim / 8;
     const unsigned cpt = cph * (unsigned)p.num_heads;
     const int nnz = min(max(*p.nnz_dev, 0), p.nnz_max);
@@ -99,17 +108,23 @@ __global__ __launch_bounds__(256) void hstu_kv_fp8_scan_kernel(const hstu_kv_app
             // non-negative floats order like their bit patterns
             atomicMax(unit_max + ((int64_t)page * 2 + 0) * p.num_heads + head, __builtin_bit_cast(unsigned, kmax));
             atomicMax(unit_max + ((int64_t)page * 2 + 1) * p.num_heads + head, __builtin_bit_cast(unsigned, vmax));
-            if (head == 0) atomicMin(first_slot + page, slot);
+            // whoever finds the page untouched lists it: touched[0] = count, then the pages
+            if (head == 0 && atomicMin(first_slot + page, slot) == KF_NOSLOT) {
+                const int at = atomicAdd(touched, 1);
+                if (at < touched_cap) touched[1 + at] = page;
+            }
         }
     }
 }
 
-// blockIdx.x = unit (page, K|V, head)
-__global__ __launch_bounds__(256) void hstu_kv_fp8_scale_kernel(const hstu_kv_append_fp8_params p, const unsigned* unit_max, const int* first_slot) {
-    const int unit = blockIdx.x;
-    const int page = unit / (2 * p.num_heads), kv = unit / p.num_heads % 2, head = unit % p.num_heads;
+// blockIdx.x = (entry of the list of touched pages, K|V, head)
+__global__ __launch_bounds__(256) void hstu_kv_fp8_scale_kernel(const hstu_kv_append_fp8_params p, const unsigned* unit_max, const int* first_slot, const int* touched, int touched_cap) {
+    const int entry = blockIdx.x / (2 * p.num_heads);
+    if (entry >= min(touched[0], touched_cap)) return;
+    const int page = touched[1 + entry], kv = blockIdx.x / p.num_heads % 2, head = blockIdx.x % p.num_heads;
+    const int unit = (page * 2 + kv) * p.num_heads + head;
     const int first = first_slot[page];
-    if (first == KF_NOSLOT) return;   // no new token in this page
+    if (first == KF_NOSLOT) return;   // (cannot happen for a listed page)
     const float cand = __builtin_bit_cast(float, unit_max[unit]) / KF_MAX;
     const float s_old = p.kv_scales[unit];
     const float s = first > 0 ? fmaxf(s_old, cand) : (cand > 0.f ? cand : 1.0f);
@@ -158,6 +173,13 @@ __global__ __launch_bounds__(256) void hstu_kv_fp8_write_kernel(const hstu_kv_ap
     }
 }
 
+// pages one call can touch: every new token goes to one page
+static int64_t kf_touched_cap(const hstu_kv_append_fp8_params* p) { return p->nnz_max < p->num_pages ? p->nnz_max : p->num_pages; }
+// per unit a maximum, per page a first slot, then the count and the list of touched pages
+static uint64_t kf_workspace_bytes(const hstu_kv_append_fp8_params* p) {
+    return ((uint64_t)p->num_pages * (2 * p->num_heads + 1) + 1 + (uint64_t)kf_touched_cap(p)) * 4;
+}
+
 static int kf_check(const hstu_kv_append_fp8_params* p) {
     if (!p) return fail(HSTU_ERR_INVALID_ARGUMENT, "params is NULL");
     if (p->struct_size != sizeof(hstu_kv_append_fp8_params))
@@ -181,7 +203,7 @@ extern "C" int hstu_hip_kv_append_fp8_get_workspace_size(const hstu_kv_append_fp
     const int rc = kf_check(p);
     if (rc != HSTU_OK) return rc;
     if (!workspace_bytes) return fail(HSTU_ERR_INVALID_ARGUMENT, "workspace_bytes is NULL");
-    *workspace_bytes = (uint64_t)p->num_pages * (2 * p->num_heads + 1) * 4;
+    *workspace_bytes = kf_workspace_bytes(p);
     return HSTU_OK;
 }
 
@@ -198,7 +220,7 @@ extern "C" int hstu_hip_kv_append_fp8(const hstu_kv_append_fp8_params* p, void* 
         return fail(HSTU_ERR_UNSUPPORTED, "append_key and append_value must be 16-byte aligned");
     if ((reinterpret_cast<uintptr_t>(p->kv_cache) & 7) || (reinterpret_cast<uintptr_t>(p->kv_scales) & 3) || (reinterpret_cast<uintptr_t>(workspace) & 3))
         return fail(HSTU_ERR_UNSUPPORTED, "kv_cache must be 8-byte aligned, kv_scales and the workspace 4-byte aligned");
-    const uint64_t need = (uint64_t)p->num_pages * (2 * p->num_heads + 1) * 4;
+    const uint64_t need = kf_workspace_bytes(p);
     if (!workspace || workspace_bytes < need)
         return fail(HSTU_ERR_WORKSPACE, "workspace of %llu bytes needed, %llu given", (unsigned long long)need, (unsigned long long)workspace_bytes);
     if (p->nnz_max == 0) return HSTU_OK;
@@ -206,14 +228,17 @@ extern "C" int hstu_hip_kv_append_fp8(const hstu_kv_append_fp8_params* p, void* 
     unsigned* unit_max = reinterpret_cast<unsigned*>(workspace);
     int* first_slot = reinterpret_cast<int*>(unit_max + units);
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    hipLaunchKernelGGL(hstu_kv_fp8_init_kernel, dim3((unsigned)((units + 255) / 256)), dim3(256), 0, st, unit_max, units, first_slot, p->num_pages);
+    int* touched = first_slot + p->num_pages;
+    const int touched_cap = (int)kf_touched_cap(p);
+    const unsigned reset_grid = (unsigned)(((int64_t)p->nnz_max + 255) / 256 > 4096 ? 4096 : ((int64_t)p->nnz_max + 255) / 256);
+    hipLaunchKernelGGL(hstu_kv_fp8_reset_kernel, dim3(reset_grid), dim3(256), 0, st, *p, unit_max, first_slot, touched);
     const int64_t lanes = (int64_t)p->nnz_max * p->num_heads * (p->head_dim / 8);
     const int64_t want = (lanes + 255) / 256;
     const unsigned grid = (unsigned)(want < 1 ? 1 : (want > 65536 ? 65536 : want));
     const bool small = lanes + 2 * (int64_t)grid * 256 < (int64_t)1 << 32;
-    if (small) hipLaunchKernelGGL(hstu_kv_fp8_scan_kernel<unsigned>, dim3(grid), dim3(256), 0, st, *p, unit_max, first_slot);
-    else hipLaunchKernelGGL(hstu_kv_fp8_scan_kernel<unsigned long long>, dim3(grid), dim3(256), 0, st, *p, unit_max, first_slot);
-    hipLaunchKernelGGL(hstu_kv_fp8_scale_kernel, dim3((unsigned)units), dim3(256), 0, st, *p, unit_max, first_slot);
+    if (small) hipLaunchKernelGGL(hstu_kv_fp8_scan_kernel<unsigned>, dim3(grid), dim3(256), 0, st, *p, unit_max, first_slot, touched, touched_cap);
+    else hipLaunchKernelGGL(hstu_kv_fp8_scan_kernel<unsigned long long>, dim3(grid), dim3(256), 0, st, *p, unit_max, first_slot, touched, touched_cap);
+    hipLaunchKernelGGL(hstu_kv_fp8_scale_kernel, dim3((unsigned)(touched_cap * 2 * p->num_heads)), dim3(256), 0, st, *p, unit_max, first_slot, touched, touched_cap);
     if (small) hipLaunchKernelGGL(hstu_kv_fp8_write_kernel<unsigned>, dim3(grid), dim3(256), 0, st, *p);
     else hipLaunchKernelGGL(hstu_kv_fp8_write_kernel<unsigned long long>, dim3(grid), dim3(256), 0, st, *p);
     const hipError_t e = hipGetLastError();

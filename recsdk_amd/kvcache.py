@@ -111,7 +111,7 @@ def append_kvcache_fp8(append_key, append_value, batch_indices, positions, seqle
     reference): ``kv_cache_fp8`` is ``[pages, 2, page_size, heads, dim]`` (uint8 or float8_e4m3fn, contiguous),
     ``kv_scales`` ``[pages, 2, heads]`` fp32.  The new rows are quantised with one scale per (page, K|V, head); a page
     that already holds rows keeps its scale unless the new rows need a larger one, in which case its old rows are
-    requantised.  ``workspace`` (uint8, at least ``pages * (2 * heads + 1) * 4`` bytes) is allocated when not given;
+    requantised.  ``workspace`` (uint8, size from ``hstu_hip_kv_append_fp8_get_workspace_size``) is allocated when not given;
     returns it for reuse."""
     device = append_key.device
     _check_kv_2byte(append_key, device, 3, "append_key")

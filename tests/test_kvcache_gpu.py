@@ -195,6 +195,39 @@ def test_fp8_append_matches_oracle_bit_for_bit(dim, heads, page, dtype):
     assert int((cache != 0).sum()) > 0
 
 
+def test_fp8_append_of_a_few_tokens_into_a_large_table_with_a_dirty_workspace():
+    """The work of a call follows the new tokens: a 20000-page table, 11 new tokens of two users, a workspace full of
+    arbitrary bytes.  Only the touched pages and their scales change."""
+    say("kv append fp8, large table")
+    pages, page, heads, dim = 20000, 8, 1, 8
+    g = torch.Generator().manual_seed(77)
+    kv_indices = torch.tensor([17, 19999, 4, 12345, 6], dtype=torch.int32)      # user 0: pages 17, 19999, 4; user 1: 12345, 6
+    kv_indptr = torch.tensor([0, 3, 5], dtype=torch.int32)
+    append_indptr = torch.tensor([0, 7, 11], dtype=torch.int32)                # 7 and 4 new tokens
+    seq_lens = torch.tensor([19, 12], dtype=torch.int32)                       # lengths after the append: positions 12..18 and 8..11
+    key = torch.randn(11, heads, dim, generator=g).to(torch.bfloat16)
+    value = torch.randn(11, heads, dim, generator=g).to(torch.bfloat16)
+    cache = torch.zeros(pages, 2, page, heads, dim, dtype=torch.uint8)
+    scales = torch.ones(pages, 2, heads)
+    bi, pos = KO.paged_batch_indices_positions(append_indptr.numpy(), seq_lens.numpy())
+    zeros = torch.zeros(2, dtype=torch.int32)
+    KO.append_paged_kvcache_fp8(cache, scales, key, value, bi, pos, zeros.numpy(), 11, kv_indices.numpy(), kv_indptr.numpy())
+    dc, ds = torch.zeros_like(cache).cuda(), torch.ones_like(scales).cuda()
+    dbi = torch.empty(11, dtype=torch.int32, device="cuda")
+    dpos = torch.empty_like(dbi)
+    kvcache.get_paged_batch_indices_positions(append_indptr.cuda(), seq_lens.cuda(), dbi, dpos)
+    ws = torch.full((pages * (2 * heads + 1) * 4 + 4096,), 0xA5, dtype=torch.uint8, device="cuda")
+    kvcache.append_kvcache_fp8(key.cuda(), value.cuda(), dbi, dpos, zeros.cuda(), torch.tensor([11], dtype=torch.int32, device="cuda"), 11,
+                               dc, ds, kv_indices.cuda(), kv_indptr.cuda(), workspace=ws)
+    torch.cuda.synchronize()
+    assert torch.equal(ds.cpu(), scales) and torch.equal(dc.cpu(), cache)
+    touched = sorted({int(kv_indices[int(kv_indptr[b]) + int(p) // page]) for b, p in zip(bi[:11], pos[:11])})
+    assert touched == [4, 6, 19999], touched     # positions 12..18 of user 0 -> its second and third page; 8..11 of user 1 -> its second
+    rest = torch.ones(pages, dtype=torch.bool)
+    rest[touched] = False
+    assert int((dc.cpu()[rest] != 0).sum()) == 0 and bool((ds.cpu()[rest] == 1).all())
+
+
 def test_fp8_prefill_equals_whole_page_quantisation_and_feeds_paged_fp8():
     """One append into an empty table = quantising the 2-byte table (appended by the 2-byte kernel) page by page, which
     is what the hstu_paged_fp8 tests feed the attention with."""
