@@ -85,7 +85,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=1000)
-    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "ref_bias", "ref_nobias", "ref_nobias_d32", "ref_nobias_d64", "ref_nobias_d256", "config2_fp8", "ref_nobias_fp8", "config2_bwd", "ref_bias_bwd", "kv_append", "kv_append_fp8", "rab_time", "rab_time_bwd", "rab_pos", "nmd_fwd", "nmd_bwd", "in_linear_silu", "in_linear_silu_bwd", "copy", "rates"],
+    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "ref_bias", "ref_nobias", "ref_nobias_d32", "ref_nobias_d64", "ref_nobias_d256", "config2_fp8", "ref_nobias_fp8", "config2_bwd", "ref_bias_bwd", "ref_nobias_bwd", "ref_nobias_d32_bwd", "ref_nobias_d64_bwd", "ref_nobias_d256_bwd", "kv_append", "kv_append_fp8", "rab_time", "rab_time_bwd", "rab_pos", "nmd_fwd", "nmd_bwd", "in_linear_silu", "in_linear_silu_bwd", "copy", "rates"],
                     help="'copy' runs a plain 256 MiB device copy: the known-size kernel the FETCH_SIZE/WRITE_SIZE counters are scaled by")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--settle-ms", type=float, default=80.0,
@@ -104,7 +104,7 @@ def main():
         return copy_calibration(args, torch)
     if args.workload == "rates":
         return issue_rates(args, torch, _capi)
-    if args.workload in ("config2_bwd", "ref_bias_bwd"):
+    if args.workload.endswith("_bwd"):
         return backward_bench(args, torch, W, _capi)
     if args.workload == "kv_append":
         return kv_append_bench(args, torch, W)
@@ -210,10 +210,12 @@ def backward_bench(args, torch, W, _capi):
     multiply-adds each under the causal mask (S, dO V^T, dV, dK, dQ) = 2.5 x the forward's FLOPs."""
     import ctypes as C
     with_bias = args.workload == "ref_bias_bwd"
-    # ref_bias_bwd: the reference's benchmark shape (B=32 h=8 d=128 S=2048, lengths 0.9 S) with a dense attn_bias, whose
-    # gradient (the same 2.1 GB again) the call also produces
-    cfg = W.reference_benchmark_config(has_rab=True) if with_bias else W.config2()
-    heads = 8 if with_bias else 4
+    ref_shape = args.workload.startswith("ref_")
+    dim = int(args.workload.split("_d")[1].split("_")[0]) if "_d" in args.workload else 128
+    # ref_*_bwd: the reference's benchmark shape (test_backward_op_benchmark.py: B=32 h=8 S=2048, lengths 0.9 S, head dims
+    # 32 .. 256); ref_bias_bwd with a dense attn_bias, whose gradient (the same 2.1 GB again) the call also produces
+    cfg = W.reference_benchmark_config(has_rab=with_bias, dim=dim) if ref_shape else W.config2()
+    heads = 8 if ref_shape else 4
     dev = W.to_device(cfg)
     q, k, v = dev["q"], dev["k"], dev["v"]
     bias = dev.get("attn_bias")
@@ -228,7 +230,7 @@ def backward_bench(args, torch, W, _capi):
     kernel = _capi.describe_backward_kernel(p)
     L = _capi.lib()
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
-    flops = 2.5 * W.headline_flops(cfg["lens"], heads, 128)
+    flops = 2.5 * W.headline_flops(cfg["lens"], heads, dim)
 
     nws = C.c_uint64(0)
     if L.hstu_hip_jagged_backward_get_workspace_size(C.byref(p), C.byref(nws)) != 0:
@@ -255,14 +257,15 @@ def backward_bench(args, torch, W, _capi):
     kern_ms = e0.elapsed_time(e1) / args.steps
     tflops = flops / (ms * 1e-3) / 1e12
     t = sum(cfg["lens"])
-    alg_bytes = 7 * t * heads * 128 * 2   # Q, K, V, dO read once; dQ, dK, dV written once
+    alg_bytes = 7 * t * heads * dim * 2   # Q, K, V, dO read once; dQ, dK, dV written once
     if with_bias:
         # the causal half of the bias is read by each of the three kernels' producers once (counted once), the whole
         # gradient buffer is zero-filled and its causal half written again
         half = sum(heads * l * (l + 1) // 2 * 2 for l in cfg["lens"])
         alg_bytes += half + bias.numel() * 2 + half
     desc = ("reference benchmark shape, backward with dense attn_bias and its gradient: B=32 h=8 d=128 S=2048, every length 0.9 S, bf16, causal"
-            if with_bias else "config2 shapes, backward: B=64 h=4 d=128 L~U[256,1024] bf16 causal no-bias seed0")
+            if with_bias else (f"reference benchmark shape, backward: B=32 h=8 d={dim} S=2048, every length 0.9 S, bf16, causal, no bias" if ref_shape
+                               else "config2 shapes, backward: B=64 h=4 d=128 L~U[256,1024] bf16 causal no-bias seed0"))
     print(json.dumps({
         "metric": "hstu_jagged_attn_bwd_tflops", "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,

@@ -1,4 +1,4 @@
-// Jagged HSTU backward on the gfx950 matrix cores (bf16 / fp16, head dim 64 or 128, built-in mask, optional dense attn_bias
+// Jagged HSTU backward on the gfx950 matrix cores (bf16 / fp16, head dim 32, 64, 128 or 256, built-in mask, optional dense attn_bias
 // with its gradient).
 //
 // Three kernels from one template, each a variation of the forward kernel's scheme: the rows a wave owns sit in
@@ -63,7 +63,8 @@ template <> __device__ __forceinline__ float bwd_half<__bf16>(unsigned w, int hi
 template <> __device__ __forceinline__ float bwd_half<_Float16>(unsigned w, int hi) { return (float)__builtin_bit_cast(b_f16x2, w)[hi]; }
 
 template <typename T, int D, int MODE, bool BIAS>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+// (head dim 256 keeps 32 operand fragments and a 32 x 256 accumulator per wave: one wave per SIMD)
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 1 : (D == 32 ? 3 : 2), D == 256 ? 1 : (D == 32 ? 3 : 2))))
 void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
     typedef typename BMM<T>::v8 v8;
     const hstu_fwd_params& p = a.f.p;
@@ -372,7 +373,7 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
 bool mfma_backward_supported(const BArgs& a) {
     const hstu_fwd_params& p = a.f.p;
     if (p.dtype != HSTU_BF16 && p.dtype != HSTU_F16) return false;
-    if (p.dim_qk != p.dim_v || (p.dim_qk != 64 && p.dim_qk != 128)) return false;
+    if (p.dim_qk != p.dim_v || (p.dim_qk != 32 && p.dim_qk != 64 && p.dim_qk != 128 && p.dim_qk != 256)) return false;
     if (p.mask_type == HSTU_MASK_CUSTOM) return false;
     // a dense bias is read 8 bytes at a time along its rows, its gradient written the same way
     if (p.attn_bias && (p.max_seq_len_k % 8 != 0 || ((reinterpret_cast<uintptr_t>(p.attn_bias) | reinterpret_cast<uintptr_t>(a.grad_bias)) & 15)))
@@ -455,8 +456,20 @@ static hipError_t launch_bwd_td(const BArgs& a, unsigned* ws, hipStream_t stream
 hipError_t launch_backward_mfma(const BArgs& a, void* workspace, hipStream_t stream) {
     const hstu_fwd_params& p = a.f.p;
     unsigned* ws = reinterpret_cast<unsigned*>(workspace);
-    if (p.dtype == HSTU_BF16) return p.dim_qk == 128 ? launch_bwd_td<__bf16, 128>(a, ws, stream) : launch_bwd_td<__bf16, 64>(a, ws, stream);
-    return p.dim_qk == 128 ? launch_bwd_td<_Float16, 128>(a, ws, stream) : launch_bwd_td<_Float16, 64>(a, ws, stream);
+    if (p.dtype == HSTU_BF16) {
+        switch (p.dim_qk) {
+            case 32: return launch_bwd_td<__bf16, 32>(a, ws, stream);
+            case 64: return launch_bwd_td<__bf16, 64>(a, ws, stream);
+            case 128: return launch_bwd_td<__bf16, 128>(a, ws, stream);
+            default: return launch_bwd_td<__bf16, 256>(a, ws, stream);
+        }
+    }
+    switch (p.dim_qk) {
+        case 32: return launch_bwd_td<_Float16, 32>(a, ws, stream);
+        case 64: return launch_bwd_td<_Float16, 64>(a, ws, stream);
+        case 128: return launch_bwd_td<_Float16, 128>(a, ws, stream);
+        default: return launch_bwd_td<_Float16, 256>(a, ws, stream);
+    }
 }
 
 }  // namespace hstu

@@ -148,6 +148,13 @@ MFMA_CASES = [
     dict(lens_q=[130, 40], nq=2, nk=1, d=128, dtype=torch.bfloat16, lens_k=[336, 40], bias=True),      # delta-q + GQA
     dict(lens_q=[264, 150], nq=2, nk=2, d=64, dtype=torch.bfloat16, ctx=[5, 0], tgt=[40, 17], tgs=3, bias=True),
     dict(lens_q=[192, 33], nq=1, nk=1, d=128, dtype=torch.float16, mask="none", bias=True),
+    # the ends of the reference's head-dim sweep (test_backward_op_benchmark.py: head_dims 32 .. 256)
+    dict(lens_q=[300, 129, 64, 1, 0, 257], nq=2, nk=2, d=32, dtype=torch.bfloat16),
+    dict(lens_q=[200, 77], nq=4, nk=2, d=32, dtype=torch.float16, ctx=[3, 0], tgt=[20, 9], tgs=2),
+    dict(lens_q=[264, 150], nq=2, nk=1, d=32, dtype=torch.bfloat16, bias=True),
+    dict(lens_q=[300, 129, 64, 1, 0, 257], nq=2, nk=2, d=256, dtype=torch.bfloat16),
+    dict(lens_q=[130, 40], nq=2, nk=1, d=256, dtype=torch.float16, lens_k=[333, 40]),
+    dict(lens_q=[200, 72], nq=2, nk=2, d=256, dtype=torch.bfloat16, bias=True),
 ]
 
 

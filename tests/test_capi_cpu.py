@@ -323,6 +323,9 @@ def test_backward_validation_and_workspace():
     assert rc == 0 and n == 0, msg                           # rows of 60 elements -> plain kernels
     rc, n, msg = _bwd_ws(_bwd_params(mask=0x1000, mask_type=3))
     assert rc == 0 and n == 0, msg                           # custom mask -> plain kernels
+    for d, want in ((32, True), (256, True), (96, False), (512, False)):
+        rc, n, msg = _bwd_ws(_bwd_params(dim_qk=d, dim_v=d))
+        assert rc == 0 and (n > 0) == want, (d, n, msg)      # head dims 32 / 64 / 128 / 256 have matrix-core kernels
     rc, _, msg = _bwd_ws(_bwd_params(attn_bias=0x1000))
     assert rc == -1 and "grad_bias must be given exactly when attn_bias is" in msg
     rc, _, msg = _bwd_ws(_bwd_params(grad_bias=0x1000))
