@@ -123,11 +123,14 @@ typedef struct hstu_fwd_params {
      *   timestamps [total_k] int64 on the K timeline; ts_table [num_buckets+1] float;
      *   ts_bounds [num_buckets+2] float, ascending, bounds[0] = 0, bounds[num_buckets+1] = +inf:
      *     bucket(i,j) = the b with bounds[b] <= (float)|t_i - t_j| < bounds[b+1];  bias += ts_table[bucket]
-     *   ts_log2_scale: optional search hint.  If non-zero, bounds[b] must sit near 2^(b / ts_log2_scale): the kernel
-     *     rounds log2(|dt|) * ts_log2_scale to the nearest integer f and lets bounds[f] decide between bucket f and
-     *     f - 1, so the estimate only has to be within half a bucket (for the reference's log buckets the scale is
-     *     ln(2)/bucket_divisor).  0 = no hint (binary search over ts_bounds).  With the hint the kernel takes |dt| from
-     *     timestamps held as doubles relative to the sequence's first one: exact while one sequence spans < 2^53 ticks.
+     *   ts_log2_scale: optional search hint.  If non-zero, bounds[b] must sit near 2^(b / ts_log2_scale), within half
+     *     a bucket (for the reference's log buckets the scale is ln(2)/bucket_divisor).  The matrix-core kernels then
+     *     keep a table in LDS that is indexed by the exponent and top three mantissa bits of (float)|dt|: a cell spans at
+     *     most a factor 1.125, so (for ts_log2_scale <= 5, buckets at least 2^(1/5) apart) at most one bound falls into
+     *     it and one comparison with that exact bound picks the bucket; the hint is only used to build the table.
+     *     0, a larger scale, or num_buckets > 62 * ts_log2_scale = binary search over ts_bounds.  With the table the
+     *     kernel takes |dt| from timestamps held as doubles relative to the sequence's first one: exact while one
+     *     sequence spans < 2^53 ticks.
      * Added to attn_bias when both are given.
      */
     const float* pos_table;

@@ -173,10 +173,11 @@ def time_bias(ts_table: torch.Tensor, ts_q: torch.Tensor, ts_k: torch.Tensor, **
 
 def dense_bias_from_tables(seq_offset_q, seq_offset_k, heads_q: int, max_q: int, max_k: int,
                            pos_table: Optional[torch.Tensor] = None, ts_table: Optional[torch.Tensor] = None,
-                           timestamps: Optional[torch.Tensor] = None, dtype=torch.float32) -> torch.Tensor:
+                           timestamps: Optional[torch.Tensor] = None, dtype=torch.float32, **bucket_kw) -> torch.Tensor:
     """The dense ``[B, Nq, max_q, max_k]`` tensor the reference op would be fed:
     position bias + time bias, zero outside ``[:Lq, :Lk]``.  ``timestamps`` is
-    indexed on the K timeline (one value per K row)."""
+    indexed on the K timeline (one value per K row); ``num_buckets`` / ``bucket_divisor``
+    go to :func:`time_bucket_ids`."""
     lq = lengths_from_offsets(seq_offset_q)
     lk = lengths_from_offsets(seq_offset_k)
     ok = seq_offset_k.tolist()
@@ -189,7 +190,7 @@ def dense_bias_from_tables(seq_offset_q, seq_offset_k, heads_q: int, max_q: int,
             bias = bias + rel_pos_bias(pos_table, a, c, max_k)
         if ts_table is not None:
             t = timestamps[ok[b]: ok[b] + c]
-            bias = bias + time_bias(ts_table, t[c - a:], t)
+            bias = bias + time_bias(ts_table, t[c - a:], t, **bucket_kw)
         out[b, :, :a, :c] = bias
     return out.to(dtype)
 

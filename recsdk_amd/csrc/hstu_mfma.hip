@@ -445,9 +445,13 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
     constexpr bool DENSE_ONLY = EXTRA >= 5 && EXTRA <= 7, XB = EXTRA == 5 || EXTRA == 7, XM = EXTRA == 6 || EXTRA == 7;
     __shared__ float lds_pos[tab_pos ? 2 * PW : 1];
     __shared__ __attribute__((aligned(8))) double lds_tk[tab_ts ? 2 * BN : 1];
-    // entry f of the time table: {bounds[f], table[f - 1], table[f]}: a score whose rounded log estimate is f sits in
-    // bucket f or f - 1, and the exact bound decides which
-    __shared__ __attribute__((aligned(16))) float lds_tsq[tab_ts ? 4 * 132 : 4];
+
+    // The time table, indexed by the top bits of (float)|dt| itself (exponent and three mantissa bits, counted from 1.0f):
+    // cell c covers the values whose bits start with 0x3f8 + c, a range no wider than a factor 1.125, so at most one
+    // bucket bound falls inside it (host-checked through the spacing the hint promises).  Entry {that bound or the next
+    // one above the cell, table[bucket below it], table[bucket from it on]}: one read and one comparison give the bias.
+    constexpr int TS_CELLS = 512;
+    __shared__ __attribute__((aligned(16))) float lds_tsq[tab_ts ? 4 * TS_CELLS : 4];
     // paged: page ids of this user and, for an fp8 cache, the (K, V) scales of this kv head
     // fp8 pages by direct copies: raw rows of the next tile (32 keys x 128 bytes of K, then of V; wave w owns keys 8w..8w+7)
     __shared__ __attribute__((aligned(1024))) char lds_raw[SH::PDMA8 ? 2 * 4096 : 16];
@@ -559,9 +563,18 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
         int64_t tbase = 0;
         if (tab_ts && s.lk > 0) tbase = p.timestamps[s.k_start];
         const double tqd = (double)(tq - tbase);
-        if (tab_ts && tid <= p.num_buckets + 1) {
-            const f32x4 entry = {p.ts_bounds[tid], p.ts_table[max(tid - 1, 0)], p.ts_table[min(tid, p.num_buckets)], 0.f};
-            *reinterpret_cast<f32x4*>(lds_tsq + 4 * tid) = entry;
+        // values from the last bound on share the last bucket: |dt| is clamped to it (and to the last cell)
+        float ts_top = 1.0f;
+        if (tab_ts) {
+            ts_top = fminf(p.ts_bounds[p.num_buckets], __builtin_bit_cast(float, 0x3f800000u + ((unsigned)(TS_CELLS - 1) << 20)));
+            for (int c = tid; c < TS_CELLS; c += NT) {
+                // bucket of the cell's lowest value: the rounded log estimate f or f - 1, the exact bound of f decides
+                const float lo = __builtin_bit_cast(float, 0x3f800000u + ((unsigned)c << 20));
+                const int f = min((int)(__builtin_amdgcn_logf(lo) * p.ts_log2_scale + 0.5f), p.num_buckets + 1);
+                const int bk = max(min(lo >= p.ts_bounds[f] ? f : f - 1, p.num_buckets), 0);
+                const f32x4 entry = {p.ts_bounds[bk + 1], p.ts_table[bk], p.ts_table[min(bk + 1, p.num_buckets)], 0.f};
+                *reinterpret_cast<f32x4*>(lds_tsq + 4 * c) = entry;
+            }
         }
         float pw_reg = 0.f;
         double tk_reg = 0;
@@ -891,6 +904,29 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                 }
                 // ---- P = s * sigmoid(alpha * s) (scale folded into the epilogue), masked
                 // accumulator register r holds key c0 + 8*(r/4) + 4*g + r%4 for Q row qi
+                if (tab_ts && D > 64) {
+                    // time-bucket bias, a batch of scores at a time: all table reads of a batch are in flight before the first is
+                    // used (one read right before its use leaves its whole latency exposed, sixteen times per block)
+                    constexpr int TSB = 4;
+#pragma unroll
+                    for (int r8 = 0; r8 < 16; r8 += TSB) {
+                        float dcv[TSB];
+                        f32x4 ent[TSB];
+#pragma unroll
+                        for (int i = 0; i < TSB; i++) {
+                            const int r = r8 + i;
+                            const int jj = 32 * kb + 8 * (r >> 2) + 4 * g + (r & 3);        // j - k0
+                            const float dt = (float)__builtin_fabs(tqd - lds_tk[buf * BN + jj]);
+                            // the cell of the clamped value; its one bound decides between the two buckets that meet in it
+                            dcv[i] = __builtin_amdgcn_fmed3f(dt, 1.0f, ts_top);
+                            const unsigned cell16 = ((__builtin_bit_cast(unsigned, dcv[i]) >> 16) & 0xfff0u) - 0x3f80u;
+                            ent[i] = *reinterpret_cast<const f32x4*>(reinterpret_cast<const char*>(lds_tsq) + cell16);
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                        for (int i = 0; i < TSB; i++) sacc[r8 + i] += dcv[i] >= ent[i][0] ? ent[i][2] : ent[i][1];
+                    }
+                }
                 float pf[16];
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
@@ -920,13 +956,13 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                     if (TAB) {
                         const int jj = 32 * kb + 8 * (r >> 2) + 4 * g + (r & 3);        // j - k0
                         if (tab_pos) x += lds_pos[buf * PW + jj - (32 * w + l32) + (BM - 1)];
-                        if (tab_ts) {
+                        if (tab_ts && D <= 64) {
+                            // (three waves per SIMD leave no registers for reads in flight: one score at a time)
                             const float dt = (float)__builtin_fabs(tqd - lds_tk[buf * BN + jj]);
-                            // f = log estimate rounded to the nearest bucket boundary; the bucket is f or f - 1 and
-                            // the exact fp32 bound of f decides (the estimate only has to be within half a bucket)
-                            const int f = min((int)(__builtin_amdgcn_logf(fmaxf(dt, 1.0f)) * p.ts_log2_scale + 0.5f), p.num_buckets + 1);
-                            const f32x4 entry = *reinterpret_cast<const f32x4*>(lds_tsq + 4 * f);
-                            x += dt >= entry[0] ? entry[2] : entry[1];
+                            const float dc = __builtin_amdgcn_fmed3f(dt, 1.0f, ts_top);
+                            const unsigned cell16 = ((__builtin_bit_cast(unsigned, dc) >> 16) & 0xfff0u) - 0x3f80u;
+                            const f32x4 entry = *reinterpret_cast<const f32x4*>(reinterpret_cast<const char*>(lds_tsq) + cell16);
+                            x += dc >= entry[0] ? entry[2] : entry[1];
                         }
                     }
                     float e = __builtin_amdgcn_exp2f(x * a.exp_scale);
@@ -1155,7 +1191,8 @@ static hipError_t launch_td(const KArgs& a, unsigned* ws, hipStream_t stream) {
     const bool dense_extra = p.attn_bias || p.mask_type == HSTU_MASK_CUSTOM;
     // the time table is used from LDS when it fits and the search hint is there; else the general path searches the
     // bounds in global memory
-    const bool ts_in_lds = p.ts_table && p.num_buckets <= 128 && p.ts_log2_scale > 0.f;
+    // the LDS time table: buckets at least a factor 2^(1/5) apart (wider than its cells) and the last bound below 2^62
+    const bool ts_in_lds = p.ts_table && p.ts_log2_scale > 0.f && p.ts_log2_scale <= 5.0f && p.num_buckets <= 62.f * p.ts_log2_scale;
     // a dense bias and / or a custom mask alone, rows on 16-byte boundaries: the variants without the other options
     const bool custom = p.mask_type == HSTU_MASK_CUSTOM;
     const bool dense_only = dense_extra && !p.pos_table && !p.ts_table && a.op != OP_PAGED && p.max_seq_len_k % 8 == 0 &&

@@ -34,6 +34,7 @@ def run_capi(cfg, *, op="jagged", flags=0, reuse_from=None, **over):
     if c.get("ts_table") is not None:
         import recsdk_amd
         kw["ts_bounds"] = recsdk_amd.time_bucket_bounds(c["ts_table"].numel() - 1, c.get("bucket_divisor", 0.301)).cuda()
+        kw["bucket_divisor"] = c.get("bucket_divisor", 0.301)
     if not dense:
         kw["seq_offset_q"] = _dev(c["seq_offset"])
         kw["seq_offset_k"] = _dev(c.get("seq_offset_k"))
@@ -143,7 +144,9 @@ def oracle_jagged(cfg, *, mode="exact", compute_dtype=torch.float32, **over):
     if c.get("pos_table") is not None or c.get("ts_table") is not None:
         tb = O.dense_bias_from_tables(c["seq_offset"], ok, c["q"].shape[1], c["max_seq_len"], mk,
                                       pos_table=c.get("pos_table"), ts_table=c.get("ts_table"),
-                                      timestamps=c.get("timestamps"))
+                                      timestamps=c.get("timestamps"),
+                                      **({} if c.get("ts_table") is None else
+                                         dict(num_buckets=c["ts_table"].numel() - 1, bucket_divisor=c.get("bucket_divisor", 0.301))))
         bias = tb if bias is None else bias.float() + tb
     return O.hstu_jagged_forward(c["q"], c["k"], c["v"], c["seq_offset"], ok, max_seq_len_q=c["max_seq_len"],
                                  max_seq_len_k=mk, mask_type=c.get("mask_type", 0), mask=c.get("mask"), attn_bias=bias,

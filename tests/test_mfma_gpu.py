@@ -150,6 +150,26 @@ def test_mfma_table_bias(d, dtype):
     assert torch.equal(T.run_op(cfg, op="table"), out)
 
 
+@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("nb,divisor,gap", [(32, 0.301, 600.0), (128, 0.301, 3e11), (40, 0.6, 50.0), (16, 0.15, 1.0)])
+def test_mfma_time_table_bucket_range(d, nb, divisor, gap):
+    """Time buckets at the ends of the table: differences beyond the last bound (few buckets), differences of 2^40 and more,
+    other bucket widths, many equal timestamps (|dt| = 0 and 1)."""
+    say("mfma_time_table_range", d, nb, divisor, gap)
+    rng = np.random.default_rng(31)
+    lens = [130, 257, 64]
+    cfg, _ = _jag(31, lens, 2, 2, d, d, torch.bfloat16)
+    cfg["ts_table"] = torch.from_numpy(rng.normal(0, 0.5, nb + 1).astype(np.float32))
+    cfg["bucket_divisor"] = divisor
+    ts = [1_700_000_000 + np.cumsum(rng.exponential(gap, l).astype(np.int64)) for l in lens]
+    cfg["timestamps"] = torch.from_numpy(np.concatenate(ts))
+    out, name = T.run_capi(cfg)
+    assert name == f"mfma_bf16_d{d}", name
+    T.assert_parity(out, T.oracle_jagged(cfg), torch.bfloat16, what="time table range")
+    gen, _ = T.run_capi(cfg, flags=FORCE_GENERIC)
+    T.assert_parity(out, gen.float(), torch.bfloat16, what="time table range vs generic kernel")
+
+
 @pytest.mark.parametrize("dtype", LOWP)
 @pytest.mark.parametrize("d,page_size,new_hist", [(64, 32, 0), (128, 64, 7), (128, 16, 130), (128, 12, 5), (128, 10, 3)])
 def test_mfma_paged(d, page_size, new_hist, dtype):
