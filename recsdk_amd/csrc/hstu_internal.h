@@ -49,6 +49,10 @@ constexpr unsigned WORK_ITEM_EMPTY = 0xffffffffu;
 constexpr int WORK_HEADER_WORDS = 16, WORK_RECORD_WORDS = 8;
 WorkList work_list_shape(const hstu_fwd_params& p);
 hipError_t launch_work_list(const KArgs& a, unsigned* ws, bool pair, hipStream_t stream);
+// dV of the backward as a forward pass over reversed rows (head dim 128, plain causal self-attention without GQA):
+// `a` carries K as q, Q as k, dO as v and dV as out; `ws` is a list launch_work_list() built for the same geometry.
+bool reversed_forward_supported(const hstu_fwd_params& p);
+hipError_t launch_reversed_forward(const KArgs& a, const unsigned* ws, hipStream_t stream);
 
 // Backward of the jagged op: the forward's argument block plus the gradient buffers.
 struct BArgs {

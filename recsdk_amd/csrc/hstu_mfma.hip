@@ -407,7 +407,11 @@ template <int D, int EXTRA, bool PAGED> struct Shape {
     static constexpr bool PDMA8 = PAGED && EXTRA == 9 && D == 128;
     static constexpr bool PDMA = PAGED && (EXTRA == 8 || EXTRA == 9) && D == 128;
     static constexpr bool DMA = (!PAGED && D == 128) || PDMA;
-    static constexpr bool LEAN = DMA && (EXTRA == 0 || EXTRA == 8 || EXTRA == 9);
+    static constexpr bool LEAN = DMA && (EXTRA == 0 || EXTRA == 8 || EXTRA == 9 || EXTRA == 10);
+    // EXTRA 10: the plain variant on sequences whose rows are taken in reverse order (row i of q / k / v / out is row
+    // L - 1 - i of its sequence in memory).  With K in the place of q, Q in the place of k and dO in the place of v the
+    // causal forward then computes dV of the backward: dV[j] = sum over i >= j of P[i][j] dO[i].
+    static constexpr bool REV = DMA && EXTRA == 10;
     // a dense bias (or, without one, a custom mask) next to direct K/V copies: its blocks are copied into LDS the same way, one tile ahead
     static constexpr bool XDMA = DMA && EXTRA >= 5 && EXTRA <= 7;
     static constexpr int BNT = (LEAN || XDMA) ? 32 : 64;     // K columns per step
@@ -541,7 +545,8 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
         // Q fragment (B operand of S^T = K Q^T): column = Q row, k = head-dim index
         v8 qf[D / 16];
         {
-            const T* qp = qbase + ((s.q_start + min(qi, s.lq - 1)) * p.heads_q + h) * (int64_t)D + 8 * g;
+            const int qrow = SH::REV ? s.lq - 1 - min(qi, s.lq - 1) : min(qi, s.lq - 1);
+            const T* qp = qbase + ((s.q_start + qrow) * p.heads_q + h) * (int64_t)D + 8 * g;
 #pragma unroll
             for (int ds = 0; ds < D / 16; ds++) {
                 const u32x4 z = {0, 0, 0, 0};
@@ -662,6 +667,20 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                         __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, LDS_PTR(void, lds_raw + 1024 * w), 16, off, 0, 0, 0);
                         __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, LDS_PTR(void, lds_raw + 4096 + 1024 * w), 16, off, 0, 0, 0);
                     }
+                }
+            } else if constexpr (SH::REV) {
+                // the view is the whole sequence; key j sits in row lk - 1 - j, a row before the sequence gets an offset
+                // past the view and arrives as zeros
+                const unsigned all_bytes = s.lk > 0 ? (unsigned)(s.lk - 1) * rowstride + D * 2 : 0;
+                __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc((void*)kview, 0, (int)all_bytes, 0x00020000);
+                __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc((void*)vview, 0, (int)all_bytes, 0x00020000);
+#pragma unroll
+                for (int i = 0; i < NBLK4 / 4; i++) {
+                    const int blk = (NBLK4 / 4) * w + i;
+                    const int prow = s.lk - 1 - (k0 + 4 * blk + lrho);
+                    const unsigned ro = prow >= 0 ? (unsigned)prow * rowstride : 0x80000000u;
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, LDS_PTR(void, dst + blk * KBLK), 16, ro + (ldK - lrho * rowstride), 0, 0, 0);
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, LDS_PTR(void, dst + NBLK4 * KBLK + blk * VBLK), 16, ro + (ldV - lrho * rowstride), 0, 0, 0);
                 }
             } else if constexpr (DMA) {
                 const unsigned tile_off = (unsigned)k0 * rowstride;
@@ -1093,8 +1112,10 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
             for (int i = 0; i < 32 / RPI; i++) {
                 const int row = RPI * i + orow;
                 const u32x4 x = *reinterpret_cast<const u32x4*>(park + row * ORS + ochunk * 16);
-                if (r0 + row < s.lq)
-                    *reinterpret_cast<u32x4*>(obase + ((s.q_start + r0 + row) * p.heads_q + h) * (int64_t)D + ochunk * 8) = x;
+                if (r0 + row < s.lq) {
+                    const int out_row = SH::REV ? s.lq - 1 - (r0 + row) : r0 + row;
+                    *reinterpret_cast<u32x4*>(obase + ((s.q_start + out_row) * p.heads_q + h) * (int64_t)D + ochunk * 8) = x;
+                }
             }
         } else if (qvalid && nsplit == 1) {
             T* op = obase + ((s.q_start + qi) * p.heads_q + h) * (int64_t)D + 4 * g;
@@ -1247,6 +1268,20 @@ static hipError_t launch_td(const KArgs& a, unsigned* ws, hipStream_t stream) {
     const int64_t n4 = p.total_q * p.heads_q * (int64_t)p.dim_v / 4;
     const unsigned rgrid = (unsigned)((n4 + 255) / 256 < 2048 ? (n4 + 255) / 256 : 2048);
     hipLaunchKernelGGL(hstu_reduce_kernel<T>, dim3(rgrid ? rgrid : 1), dim3(256), 0, stream, a, part, d.nsplit);
+    return hipGetLastError();
+}
+
+bool reversed_forward_supported(const hstu_fwd_params& p) {
+    return p.dim_qk == 128 && p.dim_v == 128 && (p.dtype == HSTU_BF16 || p.dtype == HSTU_F16) && p.mask_type == HSTU_MASK_TRIL &&
+           !p.num_context && !p.num_target && !p.attn_bias && !p.pos_table && !p.ts_table && p.heads_q == p.heads_k &&
+           p.seq_offset_q == p.seq_offset_k && p.max_seq_len_q == p.max_seq_len_k && p.total_q == p.total_k;
+}
+
+hipError_t launch_reversed_forward(const KArgs& a, const unsigned* ws, hipStream_t stream) {
+    const SchedDims d = sched_dims(a.p, true);
+    dim3 grid(8 * d.cap), block(NT);
+    if (a.p.dtype == HSTU_BF16) hipLaunchKernelGGL((hstu_mfma_kernel<__bf16, 128, 10, false>), grid, block, 0, stream, a, ws, (const float*)nullptr);
+    else hipLaunchKernelGGL((hstu_mfma_kernel<_Float16, 128, 10, false>), grid, block, 0, stream, a, ws, (const float*)nullptr);
     return hipGetLastError();
 }
 

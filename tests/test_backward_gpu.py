@@ -137,6 +137,7 @@ def test_backward_torch_ops_equal_and_delta_overloads():
 MFMA_CASES = [
     # lens_q, nq, nk, d, dtype, extras
     dict(lens_q=[300, 129, 64, 1, 0, 257], nq=2, nk=2, d=128, dtype=torch.bfloat16),
+    dict(lens_q=[515, 31, 128, 2], nq=3, nk=3, d=128, dtype=torch.float16),                            # (dV by the forward's kernel on reversed rows)
     dict(lens_q=[200, 77], nq=4, nk=2, d=64, dtype=torch.float16),                                    # GQA
     dict(lens_q=[130, 40], nq=2, nk=1, d=128, dtype=torch.bfloat16, lens_k=[333, 40]),                 # delta-q + GQA
     dict(lens_q=[260, 150], nq=2, nk=2, d=64, dtype=torch.bfloat16, ctx=[5, 0], tgt=[40, 17], tgs=3),  # context rows + target groups
@@ -178,10 +179,11 @@ def test_backward_mfma_kernels(c):
         assert bool((got[3][want[3] == 0] == 0).all())
 
 
-def test_backward_mfma_sequences_longer_than_the_attribute():
+@pytest.mark.parametrize("d", [64, 128])
+def test_backward_mfma_sequences_longer_than_the_attribute(d):
     """max_seq_len smaller than the longest sequence: the tiles behind the attribute are still covered."""
-    say("backward mfma, rows behind max_seq_len")
-    cfg, grad = _case(12, [400, 90], 2, 2, 64, 64, torch.bfloat16)
+    say("backward mfma, rows behind max_seq_len", d)
+    cfg, grad = _case(12, [400, 90], 2, 2, d, d, torch.bfloat16)
     cfg["max_seq_len"] = cfg["max_seq_len_k"] = 128
     got = T.run_capi_backward(cfg, grad)
     want = _oracle(cfg, grad)
