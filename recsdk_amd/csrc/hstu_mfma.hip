@@ -411,9 +411,10 @@ template <int D, int EXTRA, bool PAGED> struct Shape {
     // EXTRA 10: the plain variant on sequences whose rows are taken in reverse order (row i of q / k / v / out is row
     // L - 1 - i of its sequence in memory).  With K in the place of q, Q in the place of k and dO in the place of v the
     // causal forward then computes dV of the backward: dV[j] = sum over i >= j of P[i][j] dO[i].
-    static constexpr bool REV = DMA && EXTRA == 10;
+    static constexpr bool REV = EXTRA == 10;
     // a dense bias (or, without one, a custom mask) next to direct K/V copies: its blocks are copied into LDS the same way, one tile ahead
     static constexpr bool XDMA = DMA && EXTRA >= 5 && EXTRA <= 7;
+    static constexpr bool RDMA = DMA && REV;
     static constexpr int BNT = (LEAN || XDMA) ? 32 : 64;     // K columns per step
     // waves per SIMD; head dim 256 needs the registers of a whole SIMD lane for its 32 x 256 accumulator and Q fragments
     static constexpr int WAVES = D == 256 ? 1 : ((LEAN || (D <= 64 && EXTRA != 1)) ? 3 : 2);
@@ -668,7 +669,7 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                         __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, LDS_PTR(void, lds_raw + 4096 + 1024 * w), 16, off, 0, 0, 0);
                     }
                 }
-            } else if constexpr (SH::REV) {
+            } else if constexpr (SH::RDMA) {
                 // the view is the whole sequence; key j sits in row lk - 1 - j, a row before the sequence gets an offset
                 // past the view and arrives as zeros
                 const unsigned all_bytes = s.lk > 0 ? (unsigned)(s.lk - 1) * rowstride + D * 2 : 0;
@@ -728,7 +729,8 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                 for (int i = 0; i < TL::NCH; i++) {
                     const int c = tid + NT * i;
                     const int row = c / (D / 8), cc = c % (D / 8);
-                    const int j = min(k0 + row, kend - 1);
+                    const int jl = min(k0 + row, kend - 1);
+                    const int j = SH::REV ? s.lk - 1 - jl : jl;
                     RowRef<T, PAGED> rk = kv_row_ref<T, PAGED>(a, s, 0, j, hk, D, lds_pid, lds_psc);
                     RowRef<T, PAGED> rv = kv_row_ref<T, PAGED>(a, s, 1, j, hk, D, lds_pid, lds_psc);
                     kreg[i] = load_chunk<T, PAGED>(rk, cc);
@@ -1118,7 +1120,7 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                 }
             }
         } else if (qvalid && nsplit == 1) {
-            T* op = obase + ((s.q_start + qi) * p.heads_q + h) * (int64_t)D + 4 * g;
+            T* op = obase + ((s.q_start + (SH::REV ? s.lq - 1 - qi : qi)) * p.heads_q + h) * (int64_t)D + 4 * g;
 #pragma unroll
             for (int db = 0; db < D / 32; db++) {
 #pragma unroll
@@ -1272,7 +1274,7 @@ static hipError_t launch_td(const KArgs& a, unsigned* ws, hipStream_t stream) {
 }
 
 bool reversed_forward_supported(const hstu_fwd_params& p) {
-    return p.dim_qk == 128 && p.dim_v == 128 && (p.dtype == HSTU_BF16 || p.dtype == HSTU_F16) && p.mask_type == HSTU_MASK_TRIL &&
+    return (p.dim_qk == 64 || p.dim_qk == 128) && p.dim_v == p.dim_qk && (p.dtype == HSTU_BF16 || p.dtype == HSTU_F16) && p.mask_type == HSTU_MASK_TRIL &&
            !p.num_context && !p.num_target && !p.attn_bias && !p.pos_table && !p.ts_table && p.heads_q == p.heads_k &&
            p.seq_offset_q == p.seq_offset_k && p.max_seq_len_q == p.max_seq_len_k && p.total_q == p.total_k;
 }
@@ -1280,8 +1282,14 @@ bool reversed_forward_supported(const hstu_fwd_params& p) {
 hipError_t launch_reversed_forward(const KArgs& a, const unsigned* ws, hipStream_t stream) {
     const SchedDims d = sched_dims(a.p, true);
     dim3 grid(8 * d.cap), block(NT);
-    if (a.p.dtype == HSTU_BF16) hipLaunchKernelGGL((hstu_mfma_kernel<__bf16, 128, 10, false>), grid, block, 0, stream, a, ws, (const float*)nullptr);
-    else hipLaunchKernelGGL((hstu_mfma_kernel<_Float16, 128, 10, false>), grid, block, 0, stream, a, ws, (const float*)nullptr);
+    const float* none = nullptr;
+    if (a.p.dtype == HSTU_BF16) {
+        if (a.p.dim_qk == 128) hipLaunchKernelGGL((hstu_mfma_kernel<__bf16, 128, 10, false>), grid, block, 0, stream, a, ws, none);
+        else hipLaunchKernelGGL((hstu_mfma_kernel<__bf16, 64, 10, false>), grid, block, 0, stream, a, ws, none);
+    } else {
+        if (a.p.dim_qk == 128) hipLaunchKernelGGL((hstu_mfma_kernel<_Float16, 128, 10, false>), grid, block, 0, stream, a, ws, none);
+        else hipLaunchKernelGGL((hstu_mfma_kernel<_Float16, 64, 10, false>), grid, block, 0, stream, a, ws, none);
+    }
     return hipGetLastError();
 }
 

@@ -138,6 +138,7 @@ MFMA_CASES = [
     # lens_q, nq, nk, d, dtype, extras
     dict(lens_q=[300, 129, 64, 1, 0, 257], nq=2, nk=2, d=128, dtype=torch.bfloat16),
     dict(lens_q=[515, 31, 128, 2], nq=3, nk=3, d=128, dtype=torch.float16),                            # (dV by the forward's kernel on reversed rows)
+    dict(lens_q=[300, 129, 64, 1, 0, 257], nq=2, nk=2, d=64, dtype=torch.bfloat16),                   # (the same at head dim 64)
     dict(lens_q=[200, 77], nq=4, nk=2, d=64, dtype=torch.float16),                                    # GQA
     dict(lens_q=[130, 40], nq=2, nk=1, d=128, dtype=torch.bfloat16, lens_k=[333, 40]),                 # delta-q + GQA
     dict(lens_q=[260, 150], nq=2, nk=2, d=64, dtype=torch.bfloat16, ctx=[5, 0], tgt=[40, 17], tgs=3),  # context rows + target groups
