@@ -78,6 +78,11 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
     // two stages: the tiles of the next step are fetched into registers while this step computes, and written to the
     // other stage afterwards (one barrier per step)
     __shared__ __attribute__((aligned(16))) T t1s[2][WBN * TS1];
+    // K-side kernels with a bias: per wave 16 rows x 32 columns of the bias, parked as they lie in memory and read back
+    // transposed (row stride 72 bytes)
+    constexpr int BTS = 72;
+    constexpr bool BIAS_T = BIAS && MODE != MODE_DQ;
+    __shared__ __attribute__((aligned(16))) char bias_tile[BIAS_T ? 4 * 16 * BTS : 16];
     __shared__ __attribute__((aligned(16))) T t2s[2][WBN * TS2];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -197,6 +202,32 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
                         diag = !pred && j_lo + 31 > i_lo + s.delta;
                     }
                     if (c0 >= t_end) continue;
+                    // Dense bias of this block, requested before the MFMAs and without a branch (an element outside the
+                    // [max_q, max_k] square reads offset 0 and becomes 0).  The dQ kernel owns rows: four 8-byte pieces of
+                    // its row.  The K-side kernels own columns: the block comes in as it lies in memory, two times 16 rows of
+                    // 64 bytes (lane L: row L / 4, 16-byte piece L % 4), and is turned in LDS further down.
+                    const T* bias_bh = reinterpret_cast<const T*>(p.attn_bias) + ((int64_t)b * p.heads_q + h) * p.max_seq_len_q * (int64_t)p.max_seq_len_k;
+                    b_u32x2 braw_q[(BIAS && MODE == MODE_DQ) ? 4 : 1];
+                    b_u32x4 braw_k[BIAS_T ? 2 : 1];
+                    if (BIAS && MODE == MODE_DQ) {
+#pragma unroll
+                        for (int q = 0; q < 4; q++) {
+                            const int j = c0 + 8 * q + 4 * g;
+                            const bool ok = orow < p.max_seq_len_q && j < p.max_seq_len_k;
+                            const b_u32x2 x = *reinterpret_cast<const b_u32x2*>(bias_bh + (ok ? (unsigned)orow * (unsigned)p.max_seq_len_k + (unsigned)j : 0u));
+                            braw_q[q] = ok ? x : b_u32x2{0, 0};
+                        }
+                    }
+                    if (BIAS_T) {
+                        const int jcol = r0 + 8 * (lane & 3);
+#pragma unroll
+                        for (int hf = 0; hf < 2; hf++) {
+                            const int i = c0 + 16 * hf + (lane >> 2);
+                            const bool ok = i < p.max_seq_len_q && jcol < p.max_seq_len_k;
+                            const b_u32x4 x = *reinterpret_cast<const b_u32x4*>(bias_bh + (ok ? (unsigned)i * (unsigned)p.max_seq_len_k + (unsigned)jcol : 0u));
+                            braw_k[hf] = ok ? x : b_u32x4{0, 0, 0, 0};
+                        }
+                    }
                     b_f32x16 sacc, gacc;
 #pragma unroll
                     for (int r = 0; r < 16; r++) { sacc[r] = 0.f; gacc[r] = 0.f; }
@@ -213,34 +244,36 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
                         }
                     }
                     // accumulator register r holds streamed row c0 + 8*(r/4) + 4*g + r%4 for the owned row of this lane
-                    // dense bias of this lane's 16 elements: the dQ kernel owns the row and takes four 8-byte pieces of it, the
-                    // K-side kernels own the column and take 16 single values (the lanes of a wave then read along a row)
-                    // kept as 8 words of two 16-bit values (pair x = elements 2x, 2x + 1) and widened where they are used
+                    // the bias of this lane's 16 elements as 8 words of two 16-bit values (pair x = elements 2x, 2x + 1), widened
+                    // where they are used
                     unsigned bias_w[BIAS ? 8 : 1];
-                    const T* bias_bh = reinterpret_cast<const T*>(p.attn_bias) + ((int64_t)b * p.heads_q + h) * p.max_seq_len_q * (int64_t)p.max_seq_len_k;
-                    if (BIAS) {
-                        if (MODE == MODE_DQ) {
+                    if (BIAS && MODE == MODE_DQ) {
 #pragma unroll
-                            for (int q = 0; q < 4; q++) {
-                                const int j = c0 + 8 * q + 4 * g;
-                                b_u32x2 raw = {0, 0};
-                                if (orow < p.max_seq_len_q && j < p.max_seq_len_k) raw = *reinterpret_cast<const b_u32x2*>(bias_bh + ((unsigned)orow * (unsigned)p.max_seq_len_k + (unsigned)j));
-                                bias_w[2 * q] = raw[0];
-                                bias_w[2 * q + 1] = raw[1];
-                            }
-                        } else {
-                            typedef __attribute__((ext_vector_type(2))) T T2;
-                            const bool col_ok = orow < p.max_seq_len_k;
+                        for (int q = 0; q < 4; q++) { bias_w[2 * q] = braw_q[q][0]; bias_w[2 * q + 1] = braw_q[q][1]; }
+                    }
+                    if (BIAS_T) {
+                        char* bt = bias_tile + w * (16 * BTS);
 #pragma unroll
-                            for (int x = 0; x < 8; x++) {
-                                const int i = c0 + 8 * (x >> 1) + 4 * g + 2 * (x & 1);
-                                T2 v = {(T)0.f, (T)0.f};
-                                // 32-bit element offsets: one (batch, head) plane holds at most 20480^2 values
-                                const unsigned at = (unsigned)i * (unsigned)p.max_seq_len_k + (unsigned)orow;
-                                if (col_ok && i < p.max_seq_len_q) v[0] = bias_bh[at];
-                                if (col_ok && i + 1 < p.max_seq_len_q) v[1] = bias_bh[at + (unsigned)p.max_seq_len_k];
-                                bias_w[x] = __builtin_bit_cast(unsigned, v);
+                        for (int hf = 0; hf < 2; hf++) {
+                            char* wp = bt + (lane >> 2) * BTS + (lane & 3) * 16;
+                            *reinterpret_cast<b_u32x2*>(wp) = b_u32x2{braw_k[hf][0], braw_k[hf][1]};
+                            *reinterpret_cast<b_u32x2*>(wp + 8) = b_u32x2{braw_k[hf][2], braw_k[hf][3]};
+                            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                            __builtin_amdgcn_wave_barrier();
+                            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                            // a 16-lane group reads 4 rows x 16 columns and every lane receives 4 consecutive rows of its column:
+                            // streamed rows 16 hf + 8 qq + 4 g + 0..3 = score registers 4 (2 hf + qq) + 0..3
+#pragma unroll
+                            for (int qq = 0; qq < 2; qq++) {
+                                const char* rp = bt + (8 * qq + 4 * g + ((lane & 15) >> 2)) * BTS + (16 * (l32 >> 4) + 4 * (lane & 3)) * 2;
+                                const b_s16x4 t4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(BWD_LDS_PTR(b_s16x4, rp));
+                                const b_u32x2 t2 = __builtin_bit_cast(b_u32x2, t4);
+                                bias_w[2 * (2 * hf + qq)] = t2[0];
+                                bias_w[2 * (2 * hf + qq) + 1] = t2[1];
                             }
+                            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                            __builtin_amdgcn_wave_barrier();
+                            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
                         }
                     }
                     float wv[16];
