@@ -52,9 +52,27 @@ enum { MODE_DQ = 0, MODE_DK = 1, MODE_DV = 2 };
 constexpr int WBM = 128;   // rows a workgroup owns
 constexpr int WBN = 64;    // rows of the other side per step
 
-template <typename T> __global__ __launch_bounds__(256) void hstu_bwd_zero_kernel(T* out, int64_t n8) {
+// Zeroes of the bias gradient ahead of the dQ kernel, which writes every 32 x 32 block it visits: [batch * heads, max_q,
+// max_k], one row per workgroup step, 16 bytes per lane.  Under the plain causal mask (no context rows, no targets) the
+// blocks that lie wholly below the diagonal of a wave's first row are always visited, so their columns are left out;
+// everything else is zeroed, also what the dQ kernel overwrites later (it runs behind this kernel on the stream).
+template <typename T> __global__ __launch_bounds__(256) void hstu_bwd_zero_bias_kernel(const BArgs a) {
+    const hstu_fwd_params& p = a.f.p;
+    const int plane = blockIdx.y, b = plane / p.heads_q;
+    const Seq s = load_seq(a.f, b);
+    const bool plain = p.mask_type == HSTU_MASK_TRIL && s.ctx <= 0 && s.tgt <= 0;
     const b_u32x4 z = {0, 0, 0, 0};
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n8; i += (int64_t)gridDim.x * 256) reinterpret_cast<b_u32x4*>(out)[i] = z;
+    T* base = reinterpret_cast<T*>(a.grad_bias) + (int64_t)plane * p.max_seq_len_q * (int64_t)p.max_seq_len_k;
+    const int nchunk = p.max_seq_len_k / 8;
+    for (int i = blockIdx.x; i < p.max_seq_len_q; i += gridDim.x) {
+        int first = 0;
+        if (plain && i < s.lq) {
+            const int v = i / 32 * 32 + s.delta + 1;   // columns the first row of this wave's 32 rows sees
+            first = v > 0 ? min(v / 32 * 32, p.max_seq_len_k) : 0;
+        }
+        b_u32x4* row = reinterpret_cast<b_u32x4*>(base + (int64_t)i * p.max_seq_len_k);
+        for (int c = first / 8 + threadIdx.x; c < nchunk; c += 256) row[c] = z;
+    }
 }
 
 // 16-bit half `hi` (0 / 1) of a 32-bit word as float
@@ -462,9 +480,8 @@ static hipError_t launch_bwd_td(const BArgs& a, unsigned* ws, hipStream_t stream
     if (a.f.p.attn_bias) {
         // dBias: zero everywhere, then the dQ kernel writes the blocks the mask lets it visit
         const hstu_fwd_params& p = a.f.p;
-        const int64_t n8 = (int64_t)p.batch * p.heads_q * p.max_seq_len_q * (int64_t)p.max_seq_len_k / 8;   // max_seq_len_k % 8 == 0
-        const unsigned zgrid = (unsigned)(n8 / 256 + 1 < 8192 ? n8 / 256 + 1 : 8192);
-        hipLaunchKernelGGL(hstu_bwd_zero_kernel<T>, dim3(zgrid), dim3(256), 0, stream, reinterpret_cast<T*>(a.grad_bias), n8);
+        const unsigned zrows = (unsigned)(p.max_seq_len_q < 512 ? p.max_seq_len_q : 512);   // max_seq_len_k % 8 == 0
+        hipLaunchKernelGGL(hstu_bwd_zero_bias_kernel<T>, dim3(zrows, (unsigned)(p.batch * p.heads_q)), dim3(256), 0, stream, a);
         e = hipGetLastError();
         if (e != hipSuccess) return e;
         hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DQ, true>), dim3(lq.grid), dim3(256), 0, stream, a, wsq);
