@@ -225,15 +225,17 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
                     // its row.  The K-side kernels own columns: the block comes in as it lies in memory, two times 16 rows of
                     // 64 bytes (lane L: row L / 4, 16-byte piece L % 4), and is turned in LDS further down.
                     const T* bias_bh = reinterpret_cast<const T*>(p.attn_bias) + ((int64_t)b * p.heads_q + h) * p.max_seq_len_q * (int64_t)p.max_seq_len_k;
-                    b_u32x2 braw_q[(BIAS && MODE == MODE_DQ) ? 4 : 1];
+                    b_u32x4 braw_q[(BIAS && MODE == MODE_DQ) ? 2 : 1];
                     b_u32x4 braw_k[BIAS_T ? 2 : 1];
                     if (BIAS && MODE == MODE_DQ) {
+                        // 16 bytes per lane: columns c0 + 16 pr + 8 g .. + 7 of its row (the two lanes of a row then cover 32
+                        // contiguous bytes per load); the halves are exchanged between the lanes further down
 #pragma unroll
-                        for (int q = 0; q < 4; q++) {
-                            const int j = c0 + 8 * q + 4 * g;
+                        for (int pr = 0; pr < 2; pr++) {
+                            const int j = c0 + 16 * pr + 8 * g;
                             const bool ok = orow < p.max_seq_len_q && j < p.max_seq_len_k;
-                            const b_u32x2 x = *reinterpret_cast<const b_u32x2*>(bias_bh + (ok ? (unsigned)orow * (unsigned)p.max_seq_len_k + (unsigned)j : 0u));
-                            braw_q[q] = ok ? x : b_u32x2{0, 0};
+                            const b_u32x4 x = *reinterpret_cast<const b_u32x4*>(bias_bh + (ok ? (unsigned)orow * (unsigned)p.max_seq_len_k + (unsigned)j : 0u));
+                            braw_q[pr] = ok ? x : b_u32x4{0, 0, 0, 0};
                         }
                     }
                     if (BIAS_T) {
@@ -266,8 +268,17 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
                     // where they are used
                     unsigned bias_w[BIAS ? 8 : 1];
                     if (BIAS && MODE == MODE_DQ) {
+                        // score registers 4 q .. 4 q + 3 are columns 8 q + 4 g .. + 3: of the 8 columns a lane loaded for q = 2 pr
+                        // and 2 pr + 1, the lane with g = 0 keeps the first four and takes the first four of its partner
+                        // (lane + 32), the lane with g = 1 takes the partner's last four and keeps its own: v_permlane32_swap
+                        // exchanges the upper half of one register with the lower half of another
 #pragma unroll
-                        for (int q = 0; q < 4; q++) { bias_w[2 * q] = braw_q[q][0]; bias_w[2 * q + 1] = braw_q[q][1]; }
+                        for (int pr = 0; pr < 2; pr++) {
+                            const b_u32x2 s0 = __builtin_amdgcn_permlane32_swap(braw_q[pr][0], braw_q[pr][2], false, false);
+                            const b_u32x2 s1 = __builtin_amdgcn_permlane32_swap(braw_q[pr][1], braw_q[pr][3], false, false);
+                            bias_w[4 * pr] = s0[0]; bias_w[4 * pr + 1] = s1[0];
+                            bias_w[4 * pr + 2] = s0[1]; bias_w[4 * pr + 3] = s1[1];
+                        }
                     }
                     if (BIAS_T) {
                         char* bt = bias_tile + w * (16 * BTS);
@@ -356,14 +367,17 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
                         T* gbias = reinterpret_cast<T*>(a.grad_bias) + ((int64_t)b * p.heads_q + h) * p.max_seq_len_q * (int64_t)p.max_seq_len_k;
                         const float sc = a.f.out_scale;
 #pragma unroll
-                        for (int q = 0; q < 4; q++) {
-                            const int j = c0 + 8 * q + 4 * g;
-                            const b_u32x4& mm = q < 2 ? m0 : m1;
-                            const int x0 = 2 * (q & 1);
-                            b_u32x2 o;
-                            o[0] = BMM<T>::pack2(wv[4 * q] * sc, wv[4 * q + 1] * sc) & mm[x0];
-                            o[1] = BMM<T>::pack2(wv[4 * q + 2] * sc, wv[4 * q + 3] * sc) & mm[x0 + 1];
-                            if (ovalid && orow < p.max_seq_len_q && j < p.max_seq_len_k) *reinterpret_cast<b_u32x2*>(gbias + ((unsigned)orow * (unsigned)p.max_seq_len_k + (unsigned)j)) = o;
+                        for (int pr = 0; pr < 2; pr++) {
+                            // the pieces of q = 2 pr and 2 pr + 1 go back through the same exchange and leave as 16 bytes per lane
+                            const b_u32x4& mm = pr == 0 ? m0 : m1;
+                            unsigned o[4];
+#pragma unroll
+                            for (int x = 0; x < 4; x++) o[x] = BMM<T>::pack2(wv[8 * pr + 2 * x] * sc, wv[8 * pr + 2 * x + 1] * sc) & mm[x];
+                            const b_u32x2 s0 = __builtin_amdgcn_permlane32_swap(o[0], o[2], false, false);
+                            const b_u32x2 s1 = __builtin_amdgcn_permlane32_swap(o[1], o[3], false, false);
+                            const b_u32x4 out4 = {s0[0], s1[0], s0[1], s1[1]};
+                            const int j = c0 + 16 * pr + 8 * g;
+                            if (ovalid && orow < p.max_seq_len_q && j < p.max_seq_len_k) *reinterpret_cast<b_u32x4*>(gbias + ((unsigned)orow * (unsigned)p.max_seq_len_k + (unsigned)j)) = out4;
                         }
                     }
                     // OUT^T += (tile)^T W: transposing LDS reads, 4 streamed rows of one head-dim column per lane
