@@ -1119,16 +1119,22 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                     *reinterpret_cast<u32x4*>(obase + ((s.q_start + out_row) * p.heads_q + h) * (int64_t)D + ochunk * 8) = x;
                 }
             }
-        } else if (qvalid && nsplit == 1) {
-            T* op = obase + ((s.q_start + (SH::REV ? s.lq - 1 - qi : qi)) * p.heads_q + h) * (int64_t)D + 4 * g;
+        } else if (nsplit == 1) {
+            // the two lanes of a row hold alternating 8-byte pieces of it: they exchange halves (v_permlane32_swap: upper half of
+            // one register with the lower half of another) and store 16 bytes each
+            const int orow = qvalid ? (SH::REV ? s.lq - 1 - qi : qi) : 0;
+            T* op = obase + ((s.q_start + orow) * p.heads_q + h) * (int64_t)D + 8 * g;
 #pragma unroll
             for (int db = 0; db < D / 32; db++) {
 #pragma unroll
-                for (int rr = 0; rr < 4; rr++) {
-                    u32x2 o;
-                    o[0] = MM<T>::pack2(oacc[db][4 * rr] * a.out_scale, oacc[db][4 * rr + 1] * a.out_scale);
-                    o[1] = MM<T>::pack2(oacc[db][4 * rr + 2] * a.out_scale, oacc[db][4 * rr + 3] * a.out_scale);
-                    *reinterpret_cast<u32x2*>(op + 32 * db + 8 * rr) = o;
+                for (int pr = 0; pr < 2; pr++) {
+                    unsigned o[4];
+#pragma unroll
+                    for (int x = 0; x < 4; x++) o[x] = MM<T>::pack2(oacc[db][8 * pr + 2 * x] * a.out_scale, oacc[db][8 * pr + 2 * x + 1] * a.out_scale);
+                    const u32x2 s0 = __builtin_amdgcn_permlane32_swap(o[0], o[2], false, false);
+                    const u32x2 s1 = __builtin_amdgcn_permlane32_swap(o[1], o[3], false, false);
+                    const u32x4 out4 = {s0[0], s1[0], s0[1], s1[1]};
+                    if (qvalid) *reinterpret_cast<u32x4*>(op + 32 * db + 16 * pr) = out4;
                 }
             }
         } else if (qvalid) {

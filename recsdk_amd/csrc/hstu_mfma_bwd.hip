@@ -400,21 +400,27 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
                 __syncthreads();
             }
         }
-        // accumulator register r of block db holds head-dim index 32*db + 8*(r/4) + 4*g + r%4 for the owned row
-        if (ovalid) {
+        // accumulator register r of block db holds head-dim index 32*db + 8*(r/4) + 4*g + r%4 for the owned row: the two lanes
+        // of a row hold alternating 8-byte pieces of it; they exchange halves (v_permlane32_swap: upper half of one register
+        // with the lower half of another) and store 16 bytes each
+        {
+            const int64_t orc = ovalid ? orow : 0;
             T* out;
-            if (MODE == MODE_DQ) out = reinterpret_cast<T*>(a.grad_q) + ((s.q_start + orow) * p.heads_q + ho) * (int64_t)D;
-            else if (MODE == MODE_DK) out = reinterpret_cast<T*>(a.grad_k) + ((s.k_start + orow) * p.heads_k + ho) * (int64_t)D;
-            else out = reinterpret_cast<T*>(a.grad_v) + ((s.k_start + orow) * p.heads_k + ho) * (int64_t)D;
+            if (MODE == MODE_DQ) out = reinterpret_cast<T*>(a.grad_q) + ((s.q_start + orc) * p.heads_q + ho) * (int64_t)D;
+            else if (MODE == MODE_DK) out = reinterpret_cast<T*>(a.grad_k) + ((s.k_start + orc) * p.heads_k + ho) * (int64_t)D;
+            else out = reinterpret_cast<T*>(a.grad_v) + ((s.k_start + orc) * p.heads_k + ho) * (int64_t)D;
             const float sc = a.f.out_scale;   // alpha * silu_scale
 #pragma unroll
             for (int db = 0; db < D / 32; db++) {
 #pragma unroll
-                for (int rr = 0; rr < 4; rr++) {
-                    b_u32x2 o;
-                    o[0] = BMM<T>::pack2(oacc[db][4 * rr] * sc, oacc[db][4 * rr + 1] * sc);
-                    o[1] = BMM<T>::pack2(oacc[db][4 * rr + 2] * sc, oacc[db][4 * rr + 3] * sc);
-                    *reinterpret_cast<b_u32x2*>(out + 32 * db + 8 * rr + 4 * g) = o;
+                for (int pr = 0; pr < 2; pr++) {
+                    unsigned o[4];
+#pragma unroll
+                    for (int x = 0; x < 4; x++) o[x] = BMM<T>::pack2(oacc[db][8 * pr + 2 * x] * sc, oacc[db][8 * pr + 2 * x + 1] * sc);
+                    const b_u32x2 s0 = __builtin_amdgcn_permlane32_swap(o[0], o[2], false, false);
+                    const b_u32x2 s1 = __builtin_amdgcn_permlane32_swap(o[1], o[3], false, false);
+                    const b_u32x4 out4 = {s0[0], s1[0], s0[1], s1[1]};
+                    if (ovalid) *reinterpret_cast<b_u32x4*>(out + 32 * db + 16 * pr + 8 * g) = out4;
                 }
             }
         }
