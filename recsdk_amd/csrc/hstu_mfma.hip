@@ -417,7 +417,8 @@ template <int D, int EXTRA, bool PAGED> struct Shape {
     static constexpr bool RDMA = DMA && REV;
     static constexpr int BNT = (LEAN || XDMA) ? 32 : 64;     // K columns per step
     // waves per SIMD; head dim 256 needs the registers of a whole SIMD lane for its 32 x 256 accumulator and Q fragments
-    static constexpr int WAVES = D == 256 ? 1 : ((LEAN || (D <= 64 && EXTRA != 1)) ? 3 : 2);
+    // (the variants with a bias or a mask copied by DMA fit three at the price of 7 spilled registers: 2 % faster than two)
+    static constexpr int WAVES = D == 256 ? 1 : ((LEAN || (D <= 64 && EXTRA != 1) || (XDMA && EXTRA != 7)) ? 3 : 2);
 };
 
 template <typename T, int D, int EXTRA, bool PAGED>
