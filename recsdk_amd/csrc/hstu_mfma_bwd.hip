@@ -87,9 +87,10 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
     typedef typename BMM<T>::v8 v8;
     const hstu_fwd_params& p = a.f.p;
     // row strides of the LDS tiles in elements: +16 bytes keeps the 16-byte row-wise reads of 16 rows on distinct banks,
-    // +64 bytes does the same for the 4-row transposing reads; a tile that is read both ways (K for dQ, Q for dK) takes
-    // the second and pays a two-way conflict on its row-wise reads
-    constexpr int TS1 = MODE == MODE_DV ? D + 8 : D + 32;
+    // +64 bytes does the same for the 4-row transposing reads; a tile that is read both ways (K for dQ, Q for dK) takes a
+    // stride of 12 banks modulo 64 (52 at head dim 64), under which the 16 rows of a row-wise read start on 16 different
+    // multiples of 4 banks and the 4 rows of a transposing read lie at least 8 banks apart
+    constexpr int TS1 = MODE == MODE_DV ? D + 8 : D + (D == 64 ? 40 : 24);
     constexpr int TS2 = MODE == MODE_DV ? D + 32 : D + 8;
     constexpr int NCH = D / 32;          // 16-byte chunks per thread and tile
     constexpr bool TWO = MODE != MODE_DV;   // a second score-shaped GEMM (dO V^T)
