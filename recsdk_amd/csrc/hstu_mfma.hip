@@ -926,6 +926,17 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                 }
                 // ---- P = s * sigmoid(alpha * s) (scale folded into the epilogue), masked
                 // accumulator register r holds key c0 + 8*(r/4) + 4*g + r%4 for Q row qi
+                constexpr bool POS_AHEAD = tab_pos && !tab_ts && D > 64;
+                if (POS_AHEAD) {
+                    // position bias alone, two workgroups per CU: all sixteen window entries of the lane are requested before the
+                    // first is added (2.5 % on the skewed configuration; with the time table next to it the registers run out)
+                    float posv[16];
+#pragma unroll
+                    for (int r = 0; r < 16; r++) posv[r] = lds_pos[buf * PW + 32 * kb + 8 * (r >> 2) + 4 * g + (r & 3) - (32 * w + l32) + (BM - 1)];
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int r = 0; r < 16; r++) sacc[r] += posv[r];
+                }
                 if (tab_ts && D > 64) {
                     // time-bucket bias, a batch of scores at a time: all table reads of a batch are in flight before the first is
                     // used (one read right before its use leaves its whole latency exposed, sixteen times per block)
@@ -977,7 +988,7 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                     }
                     if (TAB) {
                         const int jj = 32 * kb + 8 * (r >> 2) + 4 * g + (r & 3);        // j - k0
-                        if (tab_pos) x += lds_pos[buf * PW + jj - (32 * w + l32) + (BM - 1)];
+                        if (tab_pos && !POS_AHEAD) x += lds_pos[buf * PW + jj - (32 * w + l32) + (BM - 1)];
                         if (tab_ts && D <= 64) {
                             // (three waves per SIMD leave no registers for reads in flight: one score at a time)
                             const float dt = (float)__builtin_fabs(tqd - lds_tk[buf * BN + jj]);
