@@ -235,12 +235,13 @@ def _dense_case(seed, b, s, n, d, dtype, bias=False, mask=None):
     return c, mk((b, s, n, d), 1.0)
 
 
-@pytest.mark.parametrize("kind", ["mfma_bf16", "mfma_f16_d64", "bias_f32", "custom_mask_bf16"])
+@pytest.mark.parametrize("kind", ["mfma_bf16", "mfma_f16_d64", "mfma_bias_bf16", "bias_f32", "custom_mask_bf16"])
 def test_dense_backward(kind):
     """hstu_hip_dense_backward ([B, S, N, D] layout, no offsets) against the oracle, for the MFMA and the plain kernels."""
     say("dense backward", kind)
     c, grad = {"mfma_bf16": lambda: _dense_case(21, 3, 200, 2, 128, torch.bfloat16),
                "mfma_f16_d64": lambda: _dense_case(22, 2, 130, 3, 64, torch.float16),
+               "mfma_bias_bf16": lambda: _dense_case(25, 2, 168, 2, 128, torch.bfloat16, bias=True),
                "bias_f32": lambda: _dense_case(23, 2, 45, 2, 32, torch.float32, bias=True),
                "custom_mask_bf16": lambda: _dense_case(24, 2, 70, 2, 64, torch.bfloat16, bias=True, mask="custom")}[kind]()
     dtype = c["q"].dtype
@@ -254,8 +255,10 @@ def test_dense_backward(kind):
         T.assert_parity(g, w, dtype, what=f"dense backward {kind} {name}")
     if kind.startswith("mfma"):
         gen = T.run_capi_backward(c, grad, op="dense", flags=2)
-        for name, g, x in zip(("dq", "dk", "dv"), got, gen):
-            T.assert_parity(g, x.double(), dtype, what=f"dense mfma vs plain kernels {name}")
+        assert T.last_backward_kernel.startswith("generic_bwd_")
+        for name, g, x in zip(("dq", "dk", "dv", "dbias"), got, gen):
+            if x is not None:
+                T.assert_parity(g, x.double(), dtype, what=f"dense mfma vs plain kernels {name}")
         # the same rows as a jagged batch of equal lengths give the same bits
         b, s, n, d = c["q"].shape
         j = dict(c, q=c["q"].reshape(b * s, n, d), k=c["k"].reshape(b * s, n, d), v=c["v"].reshape(b * s, n, d),
