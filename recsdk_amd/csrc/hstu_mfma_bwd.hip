@@ -9,6 +9,7 @@
 //                                                                  dQ^T += K^T dS^T
 //   MODE_DK  owns 128 K rows (and their V rows); streams Q, dO:   S = Q K^T, G = dO V^T, dS = f(S, G), dK^T += Q^T dS
 //   MODE_DV  owns 128 K rows; streams Q, dO:                      S = Q K^T, P = silu(S), dV^T += dO^T P
+//   MODE_DKV (head dim 32 / 64: both accumulators fit) the two K-side kernels in one: S, G, dS and P once per block
 // with f = G * sigmoid(x) * (1 + x * (1 - sigmoid(x))), x = alpha * S (golden: build/presmoke/hstu/hstu_common.py:446-452).
 // alpha * silu_scale factors out of the sums and is applied once to the fp32 accumulators; P and dS are rounded to the
 // I/O dtype when they are packed for the second GEMM, as P in the forward.  Every gradient element has one producing
@@ -48,7 +49,7 @@ template <> struct BMM<_Float16> {
     }
 };
 
-enum { MODE_DQ = 0, MODE_DK = 1, MODE_DV = 2 };
+enum { MODE_DQ = 0, MODE_DK = 1, MODE_DV = 2, MODE_DKV = 3 };
 constexpr int WBM = 128;   // rows a workgroup owns
 constexpr int WBN = 64;    // rows of the other side per step
 
@@ -90,8 +91,9 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
     // +64 bytes does the same for the 4-row transposing reads; a tile that is read both ways (K for dQ, Q for dK) takes a
     // stride of 12 banks modulo 64 (52 at head dim 64), under which the 16 rows of a row-wise read start on 16 different
     // multiples of 4 banks and the 4 rows of a transposing read lie at least 8 banks apart
-    constexpr int TS1 = MODE == MODE_DV ? D + 8 : D + (D == 64 ? 40 : 24);
-    constexpr int TS2 = MODE == MODE_DV ? D + 32 : D + 8;
+    constexpr int BOTH = D + (D == 64 ? 40 : 24);
+    constexpr int TS1 = MODE == MODE_DV ? D + 8 : BOTH;
+    constexpr int TS2 = MODE == MODE_DV ? D + 32 : (MODE == MODE_DKV ? BOTH : D + 8);
     constexpr int NCH = D / 32;          // 16-byte chunks per thread and tile
     constexpr bool TWO = MODE != MODE_DV;   // a second score-shaped GEMM (dO V^T)
     // two stages: the tiles of the next step are fetched into registers while this step computes, and written to the
@@ -153,11 +155,14 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
                 }
             }
         }
-        b_f32x16 oacc[D / 32];
+        b_f32x16 oacc[D / 32], oacc2[MODE == MODE_DKV ? D / 32 : 1];   // (the fused K-side kernel: dK and dV)
 #pragma unroll
         for (int db = 0; db < D / 32; db++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) oacc[db][r] = 0.f;
+            for (int r = 0; r < 16; r++) {
+                oacc[db][r] = 0.f;
+                if constexpr (MODE == MODE_DKV) oacc2[db][r] = 0.f;
+            }
 
         // range of the streamed side
         int t_begin = 0, t_end;
@@ -306,7 +311,7 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
                             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
                         }
                     }
-                    float wv[16];
+                    float wv[16], pv[MODE == MODE_DKV ? 16 : 1];
 #pragma unroll
                     for (int r = 0; r < 16; r++) {
                         const float sv = BIAS ? sacc[r] + bwd_half<T>(bias_w[r >> 1], r & 1) : sacc[r];
@@ -315,15 +320,20 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
                         if (TWO) {
                             const float x = sv * p.alpha;
                             wv[r] = gacc[r] * sg * __builtin_fmaf(x, 1.0f - sg, 1.0f);
+                            if constexpr (MODE == MODE_DKV) pv[r] = sv * sg;
                         } else {
                             wv[r] = sv * sg;
                         }
                     }
-                    b_u32x4 pk0, pk1;
+                    b_u32x4 pk0, pk1, qk0, qk1;   // dS (or, in the dV kernel, P); P of the fused kernel
 #pragma unroll
                     for (int x = 0; x < 4; x++) {
                         pk0[x] = BMM<T>::pack2(wv[2 * x], wv[2 * x + 1]);
                         pk1[x] = BMM<T>::pack2(wv[8 + 2 * x], wv[8 + 2 * x + 1]);
+                        if constexpr (MODE == MODE_DKV) {
+                            qk0[x] = BMM<T>::pack2(pv[2 * x], pv[2 * x + 1]);
+                            qk1[x] = BMM<T>::pack2(pv[8 + 2 * x], pv[8 + 2 * x + 1]);
+                        }
                     }
                     // visibility of this lane's 16 elements as masks of the packed pairs: applied to them at once, kept only where
                     // dBias needs them too (holding them in every variant costs the dK kernel 70 spilled registers)
@@ -341,6 +351,7 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
                             const unsigned v1 = (vis(8 + 2 * x) ? 0xffffu : 0u) | (vis(9 + 2 * x) ? 0xffff0000u : 0u);
                             pk0[x] &= v0;
                             pk1[x] &= v1;
+                            if constexpr (MODE == MODE_DKV) { qk0[x] &= v0; qk1[x] &= v1; }
                             if (KEEP_MASK) { m0[x] = v0; m1[x] = v1; }
                         }
                     } else if (pred) {
@@ -359,6 +370,7 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
                             const unsigned v1 = (vis(8 + 2 * x) ? 0xffffu : 0u) | (vis(9 + 2 * x) ? 0xffff0000u : 0u);
                             pk0[x] &= v0;
                             pk1[x] &= v1;
+                            if constexpr (MODE == MODE_DKV) { qk0[x] &= v0; qk1[x] &= v1; }
                             if (KEEP_MASK) { m0[x] = v0; m1[x] = v1; }
                         }
                     }
@@ -396,6 +408,21 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
                         oacc[db] = BMM<T>::mfma(__builtin_bit_cast(v8, lo), __builtin_bit_cast(v8, pk0), oacc[db]);
                         oacc[db] = BMM<T>::mfma(__builtin_bit_cast(v8, hi), __builtin_bit_cast(v8, pk1), oacc[db]);
                     }
+                    if constexpr (MODE == MODE_DKV) {
+                        // dV^T += dO^T P from the other tile
+#pragma unroll
+                        for (int db = 0; db < D / 32; db++) {
+                            const T* vp = t2 + (32 * kb + 4 * g + ((lane & 15) >> 2)) * TS2 + 16 * (l32 >> 4) + 4 * (lane & 3) + 32 * db;
+                            const b_s16x4 a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(BWD_LDS_PTR(b_s16x4, vp));
+                            const b_s16x4 a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(BWD_LDS_PTR(b_s16x4, vp + 8 * TS2));
+                            const b_s16x4 a2 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(BWD_LDS_PTR(b_s16x4, vp + 16 * TS2));
+                            const b_s16x4 a3 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(BWD_LDS_PTR(b_s16x4, vp + 24 * TS2));
+                            const b_s16x8 lo = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+                            const b_s16x8 hi = {a2[0], a2[1], a2[2], a2[3], a3[0], a3[1], a3[2], a3[3]};
+                            oacc2[db] = BMM<T>::mfma(__builtin_bit_cast(v8, lo), __builtin_bit_cast(v8, qk0), oacc2[db]);
+                            oacc2[db] = BMM<T>::mfma(__builtin_bit_cast(v8, hi), __builtin_bit_cast(v8, qk1), oacc2[db]);
+                        }
+                    }
                 }
                 if (more) stash(t0 + WBN, stage ^ 1);
                 __syncthreads();
@@ -406,24 +433,27 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
         // with the lower half of another) and store 16 bytes each
         {
             const int64_t orc = ovalid ? orow : 0;
-            T* out;
-            if (MODE == MODE_DQ) out = reinterpret_cast<T*>(a.grad_q) + ((s.q_start + orc) * p.heads_q + ho) * (int64_t)D;
-            else if (MODE == MODE_DK) out = reinterpret_cast<T*>(a.grad_k) + ((s.k_start + orc) * p.heads_k + ho) * (int64_t)D;
-            else out = reinterpret_cast<T*>(a.grad_v) + ((s.k_start + orc) * p.heads_k + ho) * (int64_t)D;
             const float sc = a.f.out_scale;   // alpha * silu_scale
+            auto store_rows = [&](T* out, const b_f32x16* acc) __attribute__((always_inline)) {
 #pragma unroll
-            for (int db = 0; db < D / 32; db++) {
+                for (int db = 0; db < D / 32; db++) {
 #pragma unroll
-                for (int pr = 0; pr < 2; pr++) {
-                    unsigned o[4];
+                    for (int pr = 0; pr < 2; pr++) {
+                        unsigned o[4];
 #pragma unroll
-                    for (int x = 0; x < 4; x++) o[x] = BMM<T>::pack2(oacc[db][8 * pr + 2 * x] * sc, oacc[db][8 * pr + 2 * x + 1] * sc);
-                    const b_u32x2 s0 = __builtin_amdgcn_permlane32_swap(o[0], o[2], false, false);
-                    const b_u32x2 s1 = __builtin_amdgcn_permlane32_swap(o[1], o[3], false, false);
-                    const b_u32x4 out4 = {s0[0], s1[0], s0[1], s1[1]};
-                    if (ovalid) *reinterpret_cast<b_u32x4*>(out + 32 * db + 16 * pr + 8 * g) = out4;
+                        for (int x = 0; x < 4; x++) o[x] = BMM<T>::pack2(acc[db][8 * pr + 2 * x] * sc, acc[db][8 * pr + 2 * x + 1] * sc);
+                        const b_u32x2 s0 = __builtin_amdgcn_permlane32_swap(o[0], o[2], false, false);
+                        const b_u32x2 s1 = __builtin_amdgcn_permlane32_swap(o[1], o[3], false, false);
+                        const b_u32x4 out4 = {s0[0], s1[0], s0[1], s1[1]};
+                        if (ovalid) *reinterpret_cast<b_u32x4*>(out + 32 * db + 16 * pr + 8 * g) = out4;
+                    }
                 }
-            }
+            };
+            T* const out_q = reinterpret_cast<T*>(a.grad_q) + ((s.q_start + orc) * p.heads_q + ho) * (int64_t)D;
+            T* const out_k = reinterpret_cast<T*>(a.grad_k) + ((s.k_start + orc) * p.heads_k + ho) * (int64_t)D;
+            T* const out_v = reinterpret_cast<T*>(a.grad_v) + ((s.k_start + orc) * p.heads_k + ho) * (int64_t)D;
+            store_rows(MODE == MODE_DQ ? out_q : (MODE == MODE_DV ? out_v : out_k), oacc);
+            if constexpr (MODE == MODE_DKV) store_rows(out_v, oacc2);
         }
     }
 
@@ -435,9 +465,12 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
         const void* offs = MODE == MODE_DQ ? p.seq_offset_q : p.seq_offset_k;
         const int64_t tail = offs ? ld_idx(offs, p.batch, is64) : total;
         if (tail < total) {
-            T* o = reinterpret_cast<T*>(MODE == MODE_DQ ? a.grad_q : (MODE == MODE_DK ? a.grad_k : a.grad_v)) + tail * heads * (int64_t)D;
+            T* o = reinterpret_cast<T*>(MODE == MODE_DQ ? a.grad_q : (MODE == MODE_DV ? a.grad_v : a.grad_k)) + tail * heads * (int64_t)D;
             const int64_t n = (total - tail) * heads * (int64_t)D;
-            for (int64_t e = (int64_t)blockIdx.x * 256 + tid; e < n; e += (int64_t)gridDim.x * 256) o[e] = (T)0.f;
+            for (int64_t e = (int64_t)blockIdx.x * 256 + tid; e < n; e += (int64_t)gridDim.x * 256) {
+                o[e] = (T)0.f;
+                if constexpr (MODE == MODE_DKV) reinterpret_cast<T*>(a.grad_v)[tail * heads * (int64_t)D + e] = (T)0.f;
+            }
         }
     }
 }
@@ -508,6 +541,10 @@ static hipError_t launch_bwd_td(const BArgs& a, unsigned* ws, hipStream_t stream
         hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DQ, true>), dim3(lq.grid), dim3(256), 0, stream, a, wsq);
         e = hipGetLastError();
         if (e != hipSuccess) return e;
+        if constexpr (D <= 64) {
+            hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DKV, true>), dim3(lk.grid), dim3(256), 0, stream, a, wsk);
+            return hipGetLastError();
+        }
         hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DK, true>), dim3(lk.grid), dim3(256), 0, stream, a, wsk);
         e = hipGetLastError();
         if (e != hipSuccess) return e;
@@ -517,6 +554,11 @@ static hipError_t launch_bwd_td(const BArgs& a, unsigned* ws, hipStream_t stream
     hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DQ, false>), dim3(lq.grid), dim3(256), 0, stream, a, wsq);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
+    if constexpr (D <= 64) {
+        // both K-side accumulators fit: S, G, dS and P once per block
+        hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DKV, false>), dim3(lk.grid), dim3(256), 0, stream, a, wsk);
+        return hipGetLastError();
+    }
     hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DK, false>), dim3(lk.grid), dim3(256), 0, stream, a, wsk);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
