@@ -1292,7 +1292,7 @@ static hipError_t launch_td(const KArgs& a, unsigned* ws, hipStream_t stream) {
 }
 
 bool reversed_forward_supported(const hstu_fwd_params& p) {
-    return (p.dim_qk == 64 || p.dim_qk == 128) && p.dim_v == p.dim_qk && (p.dtype == HSTU_BF16 || p.dtype == HSTU_F16) && p.mask_type == HSTU_MASK_TRIL &&
+    return p.dim_qk == 128 && p.dim_v == 128 && (p.dtype == HSTU_BF16 || p.dtype == HSTU_F16) && p.mask_type == HSTU_MASK_TRIL &&
            !p.num_context && !p.num_target && !p.attn_bias && !p.pos_table && !p.ts_table && p.heads_q == p.heads_k &&
            p.seq_offset_q == p.seq_offset_k && p.max_seq_len_q == p.max_seq_len_k && p.total_q == p.total_k;
 }
@@ -1301,13 +1301,8 @@ hipError_t launch_reversed_forward(const KArgs& a, const unsigned* ws, hipStream
     const SchedDims d = sched_dims(a.p, true);
     dim3 grid(8 * d.cap), block(NT);
     const float* none = nullptr;
-    if (a.p.dtype == HSTU_BF16) {
-        if (a.p.dim_qk == 128) hipLaunchKernelGGL((hstu_mfma_kernel<__bf16, 128, 10, false>), grid, block, 0, stream, a, ws, none);
-        else hipLaunchKernelGGL((hstu_mfma_kernel<__bf16, 64, 10, false>), grid, block, 0, stream, a, ws, none);
-    } else {
-        if (a.p.dim_qk == 128) hipLaunchKernelGGL((hstu_mfma_kernel<_Float16, 128, 10, false>), grid, block, 0, stream, a, ws, none);
-        else hipLaunchKernelGGL((hstu_mfma_kernel<_Float16, 64, 10, false>), grid, block, 0, stream, a, ws, none);
-    }
+    if (a.p.dtype == HSTU_BF16) hipLaunchKernelGGL((hstu_mfma_kernel<__bf16, 128, 10, false>), grid, block, 0, stream, a, ws, none);
+    else hipLaunchKernelGGL((hstu_mfma_kernel<_Float16, 128, 10, false>), grid, block, 0, stream, a, ws, none);
     return hipGetLastError();
 }
 

@@ -562,10 +562,10 @@ static hipError_t launch_bwd_td(const BArgs& a, unsigned* ws, hipStream_t stream
     hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DK, false>), dim3(lk.grid), dim3(256), 0, stream, a, wsk);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
-    if ((D == 64 || D == 128) && shared && reversed_forward_supported(a.f.p)) {
+    if (D == 128 && shared && reversed_forward_supported(a.f.p)) {
         // plain causal self-attention: dV[j] = sum over i >= j of P[i][j] dO[i] is the forward with K as q, Q as k and
-        // dO as v on rows taken in reverse order, and the forward's kernel (three workgroups per CU; at head dim 128 direct
-        // copies into LDS and 32-row tiles) is the faster one
+        // dO as v on rows taken in reverse order, and the forward's kernel for this head dim (direct copies into LDS,
+        // 32-row tiles, three workgroups per CU) is the faster one
         KArgs r = a.f;
         r.p.q = a.f.p.k; r.p.k = a.f.p.q; r.p.v = a.grad_out; r.p.out = a.grad_v;
         return launch_reversed_forward(r, wsq, stream);
