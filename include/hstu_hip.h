@@ -217,7 +217,7 @@ const char* hstu_hip_last_error(void);
 int hstu_hip_describe_kernel(const hstu_fwd_params* p, char* buf, size_t buf_bytes);
 
 /* The same for the backward: "mfma_bwd_bf16_d128", "mfma_bwd_f16_d64_bias", "generic_bwd_f32", ...  The matrix-core
- * kernels take bf16 / fp16, head dim 64 or 128 (dim_qk == dim_v), the built-in mask or none, an optional dense attn_bias
+ * kernels take bf16 / fp16, head dim 32, 64, 128 or 256 (dim_qk == dim_v), the built-in mask or none, an optional dense attn_bias
  * whose rows hold a multiple of 8 elements, and buffers on 16-byte boundaries; everything else (fp32, other head dims, a
  * custom mask) runs the plain fp32-FMA kernels, which are an order of magnitude slower. */
 int hstu_hip_describe_backward_kernel(const hstu_bwd_params* p, char* buf, size_t buf_bytes);
