@@ -1,0 +1,56 @@
+"""The entry points record nothing but kernel launches on the caller's stream (no allocation, no memset, no
+synchronisation), so a layer's forward and backward can be captured in a HIP graph and replayed: every replay, with new
+inputs in the same buffers and eager work between the replays, must equal the eager result bit for bit."""
+import ctypes as C
+
+import pytest
+import torch
+
+from recsdk_amd import _capi, workloads as W
+from tests.test_parity_gpu import say
+
+pytestmark = pytest.mark.gpu
+
+
+def test_forward_and_backward_replayed_from_a_graph():
+    say("graph capture of forward + backward")
+    cfg = W.jagged_config(3, 6, 4, 128, 100, 700, torch.bfloat16, max_seq_len=700)
+    dev = W.to_device(cfg)
+    q, k, v = dev["q"], dev["k"], dev["v"]
+    grad = torch.randn_like(q)
+    out, dq, dk, dv = (torch.empty_like(q) for _ in range(4))
+    L = _capi.lib()
+    fwd, keep = _capi.make_params(q, k, v, out, seq_offset_q=dev["seq_offset"], max_seq_len_q=cfg["max_seq_len"], alpha=cfg["alpha"])
+    bwd = _capi.make_backward_params(fwd, grad, dq, dk, dv, None)
+    nf, nb = C.c_uint64(0), C.c_uint64(0)
+    assert L.hstu_hip_jagged_forward_get_workspace_size(C.byref(fwd), C.byref(nf)) == 0
+    assert L.hstu_hip_jagged_backward_get_workspace_size(C.byref(bwd), C.byref(nb)) == 0
+    wsf = torch.empty(max(nf.value, 16), dtype=torch.uint8, device="cuda")
+    wsb = torch.empty(max(nb.value, 16), dtype=torch.uint8, device="cuda")
+
+    def step(stream):
+        s = C.c_void_p(stream.cuda_stream)
+        assert L.hstu_hip_jagged_forward(C.byref(fwd), wsf.data_ptr(), nf.value, s) == 0, L.hstu_hip_last_error()
+        assert L.hstu_hip_jagged_backward(C.byref(bwd), wsb.data_ptr(), nb.value, s) == 0, L.hstu_hip_last_error()
+
+    def eager():
+        step(torch.cuda.current_stream())
+        torch.cuda.synchronize()
+        return [t.clone() for t in (out, dq, dk, dv)]
+
+    eager()   # everything the first call sets up lazily happens outside the capture
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step(torch.cuda.current_stream())
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    for replay in range(4):
+        for t in (q, k, v, grad):   # new inputs in the captured buffers
+            t.copy_((torch.randn(t.shape, generator=gen, device="cuda") * 0.5).to(t.dtype))
+        want = eager()
+        for t in (out, dq, dk, dv):
+            t.fill_(float("nan"))
+        q.float().square().sum().item()   # unrelated eager work and a synchronisation between the replays
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, got, ref in zip(("out", "dq", "dk", "dv"), (out, dq, dk, dv), want):
+            assert torch.equal(got, ref), f"replay {replay}: {name} differs from the eager call"
