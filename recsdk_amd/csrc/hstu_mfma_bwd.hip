@@ -98,13 +98,25 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
     constexpr bool TWO = MODE != MODE_DV;   // a second score-shaped GEMM (dO V^T)
     // two stages: the tiles of the next step are fetched into registers while this step computes, and written to the
     // other stage afterwards (one barrier per step)
-    __shared__ __attribute__((aligned(16))) T t1s[2][WBN * TS1];
+    // Head dim 128: the streamed tiles are copied global -> LDS by buffer loads with the LDS destination (no registers in
+    // between).  One wave instruction fills 1024 contiguous bytes = 4 rows, so a tile is 16 blocks of 4 rows, 16 bytes of
+    // padding behind each; inside a block row rho keeps its 16-byte chunk c in slot (c + 4 rho) % 16.  The 16 rows of a
+    // row-wise fragment read then start on 16 different multiples of 4 banks and the 4 rows of a transposing read lie 16
+    // banks apart, so one layout serves the tile that is read both ways.  Two stages in separate arrays: the compiler
+    // then does not make the reads of one stage wait for the copy in flight into the other.
+    constexpr bool BDMA = D == 128;
+    constexpr int DBLK = 1040, DTILE = (WBN / 4) * DBLK;
+    __shared__ __attribute__((aligned(16))) char d1a[BDMA ? DTILE : 16];
+    __shared__ __attribute__((aligned(16))) char d1b[BDMA ? DTILE : 16];
+    __shared__ __attribute__((aligned(16))) char d2a[BDMA ? DTILE : 16];
+    __shared__ __attribute__((aligned(16))) char d2b[BDMA ? DTILE : 16];
+    __shared__ __attribute__((aligned(16))) T t1s[BDMA ? 1 : 2][BDMA ? 8 : WBN * TS1];
     // K-side kernels with a bias: per wave 16 rows x 32 columns of the bias, parked as they lie in memory and read back
     // transposed (row stride 72 bytes)
     constexpr int BTS = 72;
     constexpr bool BIAS_T = BIAS && MODE != MODE_DQ;
     __shared__ __attribute__((aligned(16))) char bias_tile[BIAS_T ? 4 * 16 * BTS : 16];
-    __shared__ __attribute__((aligned(16))) T t2s[2][WBN * TS2];
+    __shared__ __attribute__((aligned(16))) T t2s[BDMA ? 1 : 2][BDMA ? 8 : WBN * TS2];
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -176,10 +188,32 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
         const int nheads = MODE == MODE_DQ ? 1 : ratio;
         for (int hq = 0; hq < nheads; hq++) {
             const int h = MODE == MODE_DQ ? ho : ho * ratio + hq;
-            b_u32x4 n1[NCH], n2[NCH];
+            b_u32x4 n1[BDMA ? 1 : NCH], n2[BDMA ? 1 : NCH];
+            // direct copies of the tile that starts at streamed row t0: wave w fills blocks 4 w .. 4 w + 3 of both tiles; lane L
+            // brings slot L % 16 of row L / 16 of a block, i.e. chunk (slot - 4 rho) % 16 of that row; rows past the end get
+            // an offset past the view and arrive as zeros
+            auto dma = [&](int t0, char* d1, char* d2) __attribute__((always_inline)) {
+                if constexpr (BDMA) {
+                    const int sheads = MODE == MODE_DQ ? p.heads_k : p.heads_q, shead = MODE == MODE_DQ ? hk : h;
+                    const unsigned rowstride = (unsigned)sheads * D * 2;
+                    const int64_t first = ((MODE == MODE_DQ ? s.k_start : s.q_start) * (int64_t)sheads + shead) * D;
+                    __amdgpu_buffer_rsrc_t r1 = __builtin_amdgcn_make_buffer_rsrc((void*)((MODE == MODE_DQ ? kb_ : qb) + first), 0, 0x7fffffff, 0x00020000);
+                    __amdgpu_buffer_rsrc_t r2 = __builtin_amdgcn_make_buffer_rsrc((void*)((MODE == MODE_DQ ? vb : gb) + first), 0, 0x7fffffff, 0x00020000);
+                    const int rho = lane >> 4;
+                    const unsigned chunk = (unsigned)(((lane & 15) - 4 * rho) & 15) << 4;
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const int blk = 4 * w + i;
+                        const int row = t0 + 4 * blk + rho;
+                        const unsigned off = row < t_end ? (unsigned)row * rowstride + chunk : 0x80000000u;
+                        __builtin_amdgcn_raw_ptr_buffer_load_lds(r1, BWD_LDS_PTR(void, d1 + blk * DBLK), 16, off, 0, 0, 0);
+                        __builtin_amdgcn_raw_ptr_buffer_load_lds(r2, BWD_LDS_PTR(void, d2 + blk * DBLK), 16, off, 0, 0, 0);
+                    }
+                }
+            };
             auto fetch = [&](int t0) __attribute__((always_inline)) {
 #pragma unroll
-                for (int i = 0; i < NCH; i++) {
+                for (int i = 0; i < (BDMA ? 0 : NCH); i++) {
                     const int c = tid + 256 * i;
                     const int row = c / (D / 8), cc = c % (D / 8);
                     const int64_t grow = (MODE == MODE_DQ ? s.k_start : s.q_start) + min(t0 + row, t_end - 1);
@@ -191,7 +225,7 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
             };
             auto stash = [&](int t0, int stage) __attribute__((always_inline)) {
 #pragma unroll
-                for (int i = 0; i < NCH; i++) {
+                for (int i = 0; i < (BDMA ? 0 : NCH); i++) {
                     const int c = tid + 256 * i;
                     const int row = c / (D / 8), cc = c % (D / 8);
                     const bool ok = t0 + row < t_end;
@@ -202,16 +236,47 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
             };
             __syncthreads();   // every wave is done with the stages of the previous head / tile
             if (t_begin < t_end) {
-                fetch(t_begin);
-                stash(t_begin, 0);
+                if constexpr (BDMA) {
+                    dma(t_begin, d1a, d2a);
+                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                } else {
+                    fetch(t_begin);
+                    stash(t_begin, 0);
+                }
             }
             __syncthreads();
             int stage = 0;
             for (int t0 = t_begin; t0 < t_end; t0 += WBN, stage ^= 1) {
-                const T* t1 = t1s[stage];
-                const T* t2 = t2s[stage];
+                const T* t1 = t1s[BDMA ? 0 : stage];
+                const T* t2 = t2s[BDMA ? 0 : stage];
+                const char* c1 = stage ? d1b : d1a;
+                const char* c2 = stage ? d2b : d2a;
                 const bool more = t0 + WBN < t_end;
-                if (more) fetch(t0 + WBN);
+                if constexpr (BDMA) {
+                    // the other stage was last read before the barrier that ended the previous step
+                    if (more) dma(t0 + WBN, stage ? d1a : d1b, stage ? d2a : d2b);
+                } else {
+                    if (more) fetch(t0 + WBN);
+                }
+                // fragment reads: rows as A operands (row 32 kb + l32, head-dim chunk g + 2 ds), and transposed (4 streamed rows
+                // 32 kb + 8 j + 4 g .. + 3 of head-dim column 32 db + l32 per lane)
+                auto rd_row = [&](const T* tp, const char* tc, int ts, int kb, int ds) __attribute__((always_inline)) -> v8 {
+                    if constexpr (BDMA)
+                        return *reinterpret_cast<const v8*>(tc + (8 * kb + (l32 >> 2)) * DBLK + (l32 & 3) * 256 + (((g + 2 * ds + 4 * (l32 & 3)) & 15) << 4));
+                    else
+                        return *reinterpret_cast<const v8*>(tp + (32 * kb + l32) * ts + 8 * g + 16 * ds);
+                };
+                auto rd_tr = [&](const T* tp, const char* tc, int ts, int kb, int db, int j) __attribute__((always_inline)) -> b_s16x4 {
+                    const int trho = (lane & 15) >> 2;
+                    if constexpr (BDMA) {
+                        const int chunk = 4 * db + 2 * (l32 >> 4) + ((lane & 3) >> 1);
+                        const char* at = tc + (8 * kb + g + 2 * j) * DBLK + trho * 256 + (((chunk + 4 * trho) & 15) << 4) + 8 * (lane & 1);
+                        return __builtin_amdgcn_ds_read_tr16_b64_v4i16(BWD_LDS_PTR(b_s16x4, at));
+                    } else {
+                        const T* vp = tp + (32 * kb + 4 * g + trho + 8 * j) * ts + 16 * (l32 >> 4) + 4 * (lane & 3) + 32 * db;
+                        return __builtin_amdgcn_ds_read_tr16_b64_v4i16(BWD_LDS_PTR(b_s16x4, vp));
+                    }
+                };
 #pragma unroll
                 for (int kb = 0; kb < WBN / 32; kb++) {
                     const int c0 = t0 + 32 * kb;   // first streamed row of this block
@@ -259,13 +324,13 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
                     for (int r = 0; r < 16; r++) { sacc[r] = 0.f; gacc[r] = 0.f; }
 #pragma unroll
                     for (int ds = 0; ds < D / 16; ds++) {
-                        const v8 f1 = *reinterpret_cast<const v8*>(t1 + (32 * kb + l32) * TS1 + 8 * g + 16 * ds);
+                        const v8 f1 = rd_row(t1, c1, TS1, kb, ds);
                         sacc = BMM<T>::mfma(f1, xf[ds], sacc);
                     }
                     if (TWO) {
 #pragma unroll
                         for (int ds = 0; ds < D / 16; ds++) {
-                            const v8 f2 = *reinterpret_cast<const v8*>(t2 + (32 * kb + l32) * TS2 + 8 * g + 16 * ds);
+                            const v8 f2 = rd_row(t2, c2, TS2, kb, ds);
                             gacc = BMM<T>::mfma(f2, yf[ds], gacc);
                         }
                     }
@@ -395,14 +460,14 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
                     }
                     // OUT^T += (tile)^T W: transposing LDS reads, 4 streamed rows of one head-dim column per lane
                     const T* tt = MODE == MODE_DV ? t2 : t1;
+                    const char* ct = MODE == MODE_DV ? c2 : c1;
                     constexpr int TT = MODE == MODE_DV ? TS2 : TS1;
 #pragma unroll
                     for (int db = 0; db < D / 32; db++) {
-                        const T* vp = tt + (32 * kb + 4 * g + ((lane & 15) >> 2)) * TT + 16 * (l32 >> 4) + 4 * (lane & 3) + 32 * db;
-                        const b_s16x4 a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(BWD_LDS_PTR(b_s16x4, vp));
-                        const b_s16x4 a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(BWD_LDS_PTR(b_s16x4, vp + 8 * TT));
-                        const b_s16x4 a2 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(BWD_LDS_PTR(b_s16x4, vp + 16 * TT));
-                        const b_s16x4 a3 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(BWD_LDS_PTR(b_s16x4, vp + 24 * TT));
+                        const b_s16x4 a0 = rd_tr(tt, ct, TT, kb, db, 0);
+                        const b_s16x4 a1 = rd_tr(tt, ct, TT, kb, db, 1);
+                        const b_s16x4 a2 = rd_tr(tt, ct, TT, kb, db, 2);
+                        const b_s16x4 a3 = rd_tr(tt, ct, TT, kb, db, 3);
                         const b_s16x8 lo = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
                         const b_s16x8 hi = {a2[0], a2[1], a2[2], a2[3], a3[0], a3[1], a3[2], a3[3]};
                         oacc[db] = BMM<T>::mfma(__builtin_bit_cast(v8, lo), __builtin_bit_cast(v8, pk0), oacc[db]);
@@ -412,11 +477,10 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
                         // dV^T += dO^T P from the other tile
 #pragma unroll
                         for (int db = 0; db < D / 32; db++) {
-                            const T* vp = t2 + (32 * kb + 4 * g + ((lane & 15) >> 2)) * TS2 + 16 * (l32 >> 4) + 4 * (lane & 3) + 32 * db;
-                            const b_s16x4 a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(BWD_LDS_PTR(b_s16x4, vp));
-                            const b_s16x4 a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(BWD_LDS_PTR(b_s16x4, vp + 8 * TS2));
-                            const b_s16x4 a2 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(BWD_LDS_PTR(b_s16x4, vp + 16 * TS2));
-                            const b_s16x4 a3 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(BWD_LDS_PTR(b_s16x4, vp + 24 * TS2));
+                            const b_s16x4 a0 = rd_tr(t2, c2, TS2, kb, db, 0);
+                            const b_s16x4 a1 = rd_tr(t2, c2, TS2, kb, db, 1);
+                            const b_s16x4 a2 = rd_tr(t2, c2, TS2, kb, db, 2);
+                            const b_s16x4 a3 = rd_tr(t2, c2, TS2, kb, db, 3);
                             const b_s16x8 lo = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
                             const b_s16x8 hi = {a2[0], a2[1], a2[2], a2[3], a3[0], a3[1], a3[2], a3[3]};
                             oacc2[db] = BMM<T>::mfma(__builtin_bit_cast(v8, lo), __builtin_bit_cast(v8, qk0), oacc2[db]);
@@ -424,7 +488,11 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
                         }
                     }
                 }
-                if (more) stash(t0 + WBN, stage ^ 1);
+                if constexpr (BDMA) {
+                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wave's part of the next tile has arrived
+                } else {
+                    if (more) stash(t0 + WBN, stage ^ 1);
+                }
                 __syncthreads();
             }
         }
