@@ -104,7 +104,8 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
     // row-wise fragment read then start on 16 different multiples of 4 banks and the 4 rows of a transposing read lie 16
     // banks apart, so one layout serves the tile that is read both ways.  Two stages in separate arrays: the compiler
     // then does not make the reads of one stage wait for the copy in flight into the other.
-    constexpr bool BDMA = D == 128;
+    // (not the dV kernel, which has half the matrix work per tile to hide the copies behind and measured 20 % slower with them)
+    constexpr bool BDMA = D == 128 && MODE != MODE_DV;
     constexpr int DBLK = 1040, DTILE = (WBN / 4) * DBLK;
     __shared__ __attribute__((aligned(16))) char d1a[BDMA ? DTILE : 16];
     __shared__ __attribute__((aligned(16))) char d1b[BDMA ? DTILE : 16];
