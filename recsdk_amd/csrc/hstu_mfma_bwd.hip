@@ -83,7 +83,10 @@ template <> __device__ __forceinline__ float bwd_half<_Float16>(unsigned w, int 
 
 template <typename T, int D, int MODE, bool BIAS>
 // (head dim 256 keeps 32 operand fragments and a 32 x 256 accumulator per wave: one wave per SIMD)
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 256 ? 1 : (D == 32 ? 3 : 2), D == 256 ? 1 : (D == 32 ? 3 : 2))))
+// waves per SIMD: one at head dim 256 (see above), three where the registers allow it (head dim 32; at head dim 64 the
+// kernels with one accumulator, since their tiles are copied straight into LDS), else two
+#define BWD_WAVES(D, MODE) ((D) == 256 ? 1 : ((D) == 32 || ((D) == 64 && (MODE) != MODE_DKV)) ? 3 : 2)
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BWD_WAVES(D, MODE), BWD_WAVES(D, MODE))))
 void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
     typedef typename BMM<T>::v8 v8;
     const hstu_fwd_params& p = a.f.p;
@@ -98,15 +101,19 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
     constexpr bool TWO = MODE != MODE_DV;   // a second score-shaped GEMM (dO V^T)
     // two stages: the tiles of the next step are fetched into registers while this step computes, and written to the
     // other stage afterwards (one barrier per step)
-    // Head dim 128: the streamed tiles are copied global -> LDS by buffer loads with the LDS destination (no registers in
-    // between).  One wave instruction fills 1024 contiguous bytes = 4 rows, so a tile is 16 blocks of 4 rows, 16 bytes of
-    // padding behind each; inside a block row rho keeps its 16-byte chunk c in slot (c + 4 rho) % 16.  The 16 rows of a
-    // row-wise fragment read then start on 16 different multiples of 4 banks and the 4 rows of a transposing read lie 16
-    // banks apart, so one layout serves the tile that is read both ways.  Two stages in separate arrays: the compiler
-    // then does not make the reads of one stage wait for the copy in flight into the other.
+    // Head dims 64 and 128: the streamed tiles are copied global -> LDS by buffer loads with the LDS destination (no
+    // registers in between).  One wave instruction fills 1024 contiguous bytes = 4 rows of head dim 128 (8 of 64), so a tile
+    // is a sequence of such blocks, 16 bytes of padding behind each; inside a block row rho keeps its 16-byte chunk c in slot
+    // (c + 4 rho) % 16 (head dim 64: (c + 2 (rho / 2)) % 8).  The 16 rows of a row-wise fragment read then start on 16
+    // different multiples of 4 banks and the rows of a transposing read do not meet, so one layout serves the tile that is
+    // read both ways.  Two stages in separate arrays: the compiler then does not make the reads of one stage wait for the
+    // copy in flight into the other.
     // (not the dV kernel, which has half the matrix work per tile to hide the copies behind and measured 20 % slower with them)
-    constexpr bool BDMA = D == 128 && MODE != MODE_DV;
-    constexpr int DBLK = 1040, DTILE = (WBN / 4) * DBLK;
+    constexpr bool BDMA = (D == 128 || D == 64) && MODE != MODE_DV;
+    constexpr int RPB = D == 128 ? 4 : 8;            // rows per block
+    constexpr int CPR = D / 8;                       // 16-byte chunks per row
+    constexpr int DBLK = 1040, DTILE = (WBN / RPB) * DBLK;
+    auto slot_of = [](int c, int rho) __attribute__((always_inline)) -> int { return D == 128 ? ((c + 4 * rho) & 15) : ((c + 2 * (rho >> 1)) & 7); };
     __shared__ __attribute__((aligned(16))) char d1a[BDMA ? DTILE : 16];
     __shared__ __attribute__((aligned(16))) char d1b[BDMA ? DTILE : 16];
     __shared__ __attribute__((aligned(16))) char d2a[BDMA ? DTILE : 16];
@@ -200,12 +207,13 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
                     const int64_t first = ((MODE == MODE_DQ ? s.k_start : s.q_start) * (int64_t)sheads + shead) * D;
                     __amdgpu_buffer_rsrc_t r1 = __builtin_amdgcn_make_buffer_rsrc((void*)((MODE == MODE_DQ ? kb_ : qb) + first), 0, 0x7fffffff, 0x00020000);
                     __amdgpu_buffer_rsrc_t r2 = __builtin_amdgcn_make_buffer_rsrc((void*)((MODE == MODE_DQ ? vb : gb) + first), 0, 0x7fffffff, 0x00020000);
-                    const int rho = lane >> 4;
-                    const unsigned chunk = (unsigned)(((lane & 15) - 4 * rho) & 15) << 4;
+                    const int rho = lane / CPR;
+                    const unsigned chunk = (unsigned)(D == 128 ? ((lane % CPR) - 4 * rho) & 15 : ((lane % CPR) - 2 * (rho >> 1)) & 7) << 4;
+                    constexpr int BPW = WBN / RPB / 4;   // blocks per wave and tile
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        const int blk = 4 * w + i;
-                        const int row = t0 + 4 * blk + rho;
+                    for (int i = 0; i < BPW; i++) {
+                        const int blk = BPW * w + i;
+                        const int row = t0 + RPB * blk + rho;
                         const unsigned off = row < t_end ? (unsigned)row * rowstride + chunk : 0x80000000u;
                         __builtin_amdgcn_raw_ptr_buffer_load_lds(r1, BWD_LDS_PTR(void, d1 + blk * DBLK), 16, off, 0, 0, 0);
                         __builtin_amdgcn_raw_ptr_buffer_load_lds(r2, BWD_LDS_PTR(void, d2 + blk * DBLK), 16, off, 0, 0, 0);
@@ -263,7 +271,7 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
                 // 32 kb + 8 j + 4 g .. + 3 of head-dim column 32 db + l32 per lane)
                 auto rd_row = [&](const T* tp, const char* tc, int ts, int kb, int ds) __attribute__((always_inline)) -> v8 {
                     if constexpr (BDMA)
-                        return *reinterpret_cast<const v8*>(tc + (8 * kb + (l32 >> 2)) * DBLK + (l32 & 3) * 256 + (((g + 2 * ds + 4 * (l32 & 3)) & 15) << 4));
+                        return *reinterpret_cast<const v8*>(tc + ((32 / RPB) * kb + l32 / RPB) * DBLK + (l32 % RPB) * (2 * D) + (slot_of(g + 2 * ds, l32 % RPB) << 4));
                     else
                         return *reinterpret_cast<const v8*>(tp + (32 * kb + l32) * ts + 8 * g + 16 * ds);
                 };
@@ -271,7 +279,8 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
                     const int trho = (lane & 15) >> 2;
                     if constexpr (BDMA) {
                         const int chunk = 4 * db + 2 * (l32 >> 4) + ((lane & 3) >> 1);
-                        const char* at = tc + (8 * kb + g + 2 * j) * DBLK + trho * 256 + (((chunk + 4 * trho) & 15) << 4) + 8 * (lane & 1);
+                        const int r = 8 * j + 4 * g + trho;     // row of the 32-row block
+                        const char* at = tc + ((32 / RPB) * kb + r / RPB) * DBLK + (r % RPB) * (2 * D) + (slot_of(chunk, r % RPB) << 4) + 8 * (lane & 1);
                         return __builtin_amdgcn_ds_read_tr16_b64_v4i16(BWD_LDS_PTR(b_s16x4, at));
                     } else {
                         const T* vp = tp + (32 * kb + 4 * g + trho + 8 * j) * ts + 16 * (l32 >> 4) + 4 * (lane & 3) + 32 * db;
