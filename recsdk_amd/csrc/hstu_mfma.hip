@@ -417,8 +417,10 @@ template <int D, int EXTRA, bool PAGED> struct Shape {
     static constexpr bool RDMA = DMA && REV;
     static constexpr int BNT = (LEAN || XDMA) ? 32 : 64;     // K columns per step
     // waves per SIMD; head dim 256 needs the registers of a whole SIMD lane for its 32 x 256 accumulator and Q fragments
-    // (the variants with a bias or a mask copied by DMA fit three at the price of 7 spilled registers: 2 % faster than two)
-    static constexpr int WAVES = D == 256 ? 1 : ((LEAN || (D <= 64 && EXTRA != 1) || (XDMA && EXTRA != 7)) ? 3 : 2);
+    // (the variants with a bias or a mask copied by DMA fit three at the price of 7 spilled registers: 2 % faster than two;
+    // the plain variant at head dim 32 needs 88 registers and 26.6 KB of LDS and runs four: 5 % faster than three, while
+    // head dim 64 would have to move accumulators through AGPR copies for a fourth wave and loses 5 %)
+    static constexpr int WAVES = D == 256 ? 1 : ((D == 32 && EXTRA == 0 && !PAGED) ? 4 : ((LEAN || (D <= 64 && EXTRA != 1) || (XDMA && EXTRA != 7)) ? 3 : 2));
 };
 
 template <typename T, int D, int EXTRA, bool PAGED>
@@ -427,7 +429,7 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
     typedef Tile<D> TL;
     typedef Shape<D, EXTRA, PAGED> SH;
     constexpr int BNT = SH::BNT;
-    constexpr bool LEAN = SH::WAVES == 3;          // register-tight variants read V fragments right before use
+    constexpr bool LEAN = SH::WAVES >= 3;          // register-tight variants read V fragments right before use
     constexpr bool PARK_OUT = LEAN;                // output tiles leave through LDS as whole rows
     constexpr int NBLK4 = BNT / 4;                 // 4-row blocks per tile
     typedef typename MM<T>::v8 v8;
