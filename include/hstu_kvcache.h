@@ -67,8 +67,9 @@ int hstu_hip_kv_token_positions(int32_t batch, const int32_t* append_indptr, con
  *   s = max(s before, absmax(new rows) / 448)   if the page already held rows below its first new slot,
  *   s = absmax(new rows) / 448 (1 if that is 0)  otherwise;
  * rows already there are requantised from q * (s before) when s grew, and untouched when it did not.  Pages fill from
- * slot 0 upwards (what the reference's manager does).  The workspace needs no initialisation; the work of a call grows
- * with the new tokens, not with the size of the table. */
+ * slot 0 upwards (what the reference's manager does).  The workspace (16-byte aligned) needs no initialisation; the
+ * work of a call grows with the new tokens, not with the size of the table.  Tokens may come in any order; in the order
+ * of hstu_hip_kv_token_positions (consecutive positions of a user side by side) every source row is read once. */
 typedef struct hstu_kv_append_fp8_params {
     uint32_t struct_size;
     int32_t src_dtype;        /* HSTU_F16 / HSTU_BF16: append_key, append_value */

@@ -221,6 +221,6 @@ def test_fp8_append_abi_validation():
     rc, msg, p = call(ws_bytes=16)
     assert rc == -3 and "workspace" in msg
     need = C.c_uint64(0)
-    assert L.hstu_hip_kv_append_fp8_get_workspace_size(C.byref(p), C.byref(need)) == 0 and need.value == (10 * (2 * 2 + 1) + 1 + 8) * 4   # maxima and first slots of all pages, then the list of (at most nnz_max) touched pages
+    assert L.hstu_hip_kv_append_fp8_get_workspace_size(C.byref(p), C.byref(need)) == 0 and need.value == (72 + 8 * 8) * 4   # maxima, first slots and run counts of all pages (60 words), the count and list of (at most nnz_max) scattered pages (9), the count of runs, padding to 16 bytes (72), 8-word records of (at most nnz_max) runs
     rc, _, _ = call(nnz_max=0)
     assert rc == 0

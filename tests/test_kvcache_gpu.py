@@ -166,12 +166,33 @@ def _fp8_scenario(seed, users, heads, dim, page, dtype):
     return dict(pages=pages, kv_indices=perm, kv_indptr=indptr, steps=steps, users=users)
 
 
-@pytest.mark.parametrize("dim,heads,page,dtype", [(128, 4, 64, torch.bfloat16), (64, 2, 32, torch.float16), (256, 1, 16, torch.bfloat16),
-                                                  (8, 3, 8, torch.bfloat16)])
-def test_fp8_append_matches_oracle_bit_for_bit(dim, heads, page, dtype):
+def _token_order(bi, nnz, order, seed):
+    """A permutation of the new tokens: 'runs' keeps them as they come; 'mixed' shuffles the tokens of every third user,
+    reverses those of the next and keeps the rest (pages with one run and pages with many in one call)."""
+    perm = np.arange(nnz)
+    if order == "runs":
+        return perm
+    rng = np.random.default_rng(seed)
+    for b in np.unique(bi[:nnz]):
+        idx = np.nonzero(bi[:nnz] == b)[0]
+        if b % 3 == 0:
+            perm[idx] = rng.permutation(idx)
+        elif b % 3 == 1:
+            perm[idx] = idx[::-1]
+    return perm
+
+
+@pytest.mark.parametrize("dim,heads,page,dtype,order", [(128, 4, 64, torch.bfloat16, "runs"), (64, 2, 32, torch.float16, "runs"),
+                                                        (256, 1, 16, torch.bfloat16, "runs"), (8, 3, 8, torch.bfloat16, "runs"),
+                                                        (128, 4, 64, torch.bfloat16, "mixed"), (32, 2, 24, torch.float16, "mixed"),
+                                                        (512, 1, 64, torch.bfloat16, "runs"), (512, 2, 48, torch.float16, "mixed"),
+                                                        (256, 2, 64, torch.bfloat16, "mixed"), (16, 1, 200, torch.bfloat16, "runs")])
+def test_fp8_append_matches_oracle_bit_for_bit(dim, heads, page, dtype, order):
     """Bytes and scales after a prefill and after an extension of partly filled pages, against the oracle's restatement
-    of this library's own definition (no reference counterpart: parity with the reference unpinned by construction)."""
-    say("kv append fp8", dim, heads, page, dtype)
+    of this library's own definition (no reference counterpart: parity with the reference unpinned by construction).
+    'runs': tokens in the order of hstu_hip_kv_token_positions (every page finished by the one-pass kernel, or, for pages
+    of more than 2048 cells of 8 elements, by the kernels for scattered pages); 'mixed': tokens of some users out of order."""
+    say("kv append fp8", dim, heads, page, dtype, order)
     s = _fp8_scenario(5, 9, heads, dim, page, dtype)
     cache = torch.zeros(s["pages"], 2, page, heads, dim, dtype=torch.uint8)
     scales = torch.ones(s["pages"], 2, heads)
@@ -180,12 +201,20 @@ def test_fp8_append_matches_oracle_bit_for_bit(dim, heads, page, dtype):
     zeros = torch.zeros(s["users"], dtype=torch.int32)
     for n, st in enumerate(s["steps"]):
         bi, pos = KO.paged_batch_indices_positions(st["append_indptr"].numpy(), st["seq_lens"].numpy())
-        KO.append_paged_kvcache_fp8(cache, scales, st["key"], st["value"], bi, pos, zeros.numpy(), st["nnz"], s["kv_indices"].numpy(),
+        perm = _token_order(bi, st["nnz"], order, 100 + n)
+        bi, pos = bi.copy(), pos.copy()
+        bi[: st["nnz"]], pos[: st["nnz"]] = bi[perm], pos[perm]
+        key, value = st["key"][torch.from_numpy(perm)], st["value"][torch.from_numpy(perm)]     # row of token i = i (offsets are zero)
+        KO.append_paged_kvcache_fp8(cache, scales, key, value, bi, pos, zeros.numpy(), st["nnz"], s["kv_indices"].numpy(),
                                     s["kv_indptr"].numpy())
         dbi = torch.empty(max(st["nnz"], 1), dtype=torch.int32, device="cuda")
         dpos = torch.empty_like(dbi)
-        kvcache.get_paged_batch_indices_positions(st["append_indptr"].cuda(), st["seq_lens"].cuda(), dbi, dpos)
-        ws = kvcache.append_kvcache_fp8(st["key"].cuda(), st["value"].cuda(), dbi, dpos, zeros.cuda(),
+        if order == "runs":
+            kvcache.get_paged_batch_indices_positions(st["append_indptr"].cuda(), st["seq_lens"].cuda(), dbi, dpos)
+        else:
+            dbi[: st["nnz"]] = torch.from_numpy(bi[: st["nnz"]].astype(np.int32)).cuda()
+            dpos[: st["nnz"]] = torch.from_numpy(pos[: st["nnz"]].astype(np.int32)).cuda()
+        ws = kvcache.append_kvcache_fp8(key.cuda(), value.cuda(), dbi, dpos, zeros.cuda(),
                                         torch.tensor([st["nnz"]], dtype=torch.int32, device="cuda"), st["nnz"], dc, ds,
                                         s["kv_indices"].cuda(), s["kv_indptr"].cuda(), workspace=ws)
         torch.cuda.synchronize()
@@ -216,7 +245,7 @@ def test_fp8_append_of_a_few_tokens_into_a_large_table_with_a_dirty_workspace():
     dbi = torch.empty(11, dtype=torch.int32, device="cuda")
     dpos = torch.empty_like(dbi)
     kvcache.get_paged_batch_indices_positions(append_indptr.cuda(), seq_lens.cuda(), dbi, dpos)
-    ws = torch.full((pages * (2 * heads + 1) * 4 + 4096,), 0xA5, dtype=torch.uint8, device="cuda")
+    ws = torch.full((pages * (2 * heads + 2) * 4 + 4096,), 0xA5, dtype=torch.uint8, device="cuda")
     kvcache.append_kvcache_fp8(key.cuda(), value.cuda(), dbi, dpos, zeros.cuda(), torch.tensor([11], dtype=torch.int32, device="cuda"), 11,
                                dc, ds, kv_indices.cuda(), kv_indptr.cuda(), workspace=ws)
     torch.cuda.synchronize()
@@ -251,12 +280,23 @@ def test_fp8_prefill_equals_whole_page_quantisation_and_feeds_paged_fp8():
     assert torch.equal(cache8.cpu()[touched], want8.view(torch.uint8)[touched])
 
 
-def test_fp8_prefill_at_the_bench_shape_against_torch_on_the_gpu():
+@pytest.mark.parametrize("dtype,spread", [(torch.bfloat16, False), (torch.float16, True), (torch.bfloat16, True)])
+def test_fp8_prefill_at_the_bench_shape_against_torch_on_the_gpu(dtype, spread):
     """Config 5's history (32 users x U[1024, 4096] tokens, 4 heads x 128, 64-token pages) is too long for the token loop
     of the oracle; the prefill is checked through what it must equal: the 2-byte table written by the 2-byte append
-    (bit-exact against the oracle at smaller sizes), quantised page by page with torch's own GPU routines."""
-    say("kv append fp8 at the bench shape")
-    c = W.kv_append_config(0, users=32, heads=4, dim=128, prev_lo=0, prev_hi=0, new_lo=1024, new_hi=4096, page_size=64)
+    (bit-exact against the oracle at smaller sizes), quantised page by page with torch's own GPU routines (a true
+    division per element: 87 million quotients against the kernel's shared-reciprocal division).  `spread`: every token's
+    rows scaled by a power of two or a random factor over 18 octaves, so that the scales cover many binades and, for the
+    powers of two, most quotients are exact and sit on e4m3 ties."""
+    say("kv append fp8 at the bench shape", dtype, spread)
+    c = W.kv_append_config(0, users=32, heads=4, dim=128, prev_lo=0, prev_hi=0, new_lo=1024, new_hi=4096, page_size=64, dtype=dtype)
+    if spread:
+        g = torch.Generator().manual_seed(9)
+        rows = c["append_key"].shape[0]
+        e = torch.randint(-12, 7, (rows, 1, 1), generator=g).float()
+        amp = torch.where(torch.rand(rows, 1, 1, generator=g) < 0.5, torch.exp2(e), torch.exp2(e + torch.rand(rows, 1, 1, generator=g)))
+        c["append_key"] = (c["append_key"].float() * amp).to(dtype)
+        c["append_value"] = (c["append_value"].float() * amp * 0.75).to(dtype)
     d = W.to_device(c)
     n = c["nnz"]
     bi = torch.empty(n, dtype=torch.int32, device="cuda")
