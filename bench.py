@@ -80,6 +80,19 @@ def build_workload(name, torch, W):
     raise SystemExit(f"unknown workload {name}")
 
 
+def bench_kind(workload):
+    """Which leg of this file measures a workload (the names of several legs end alike)."""
+    if workload in ("copy", "rates", "kv_append", "kv_append_fp8", "in_linear_silu", "in_linear_silu_bwd"):
+        return workload
+    if workload in ("rab_time", "rab_time_bwd", "rab_pos"):
+        return "bias"
+    if workload in ("nmd_fwd", "nmd_bwd"):
+        return "nmd"
+    if workload == "config2_bwd" or (workload.startswith("ref_") and workload.endswith("_bwd")):
+        return "attention_backward"
+    return "attention_forward"
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -100,23 +113,24 @@ def main():
     from recsdk_amd import _capi, workloads as W
 
     assert torch.cuda.is_available(), "bench.py needs the MI355X"
-    if args.workload == "copy":
+    kind = bench_kind(args.workload)
+    if kind == "copy":
         return copy_calibration(args, torch)
-    if args.workload == "rates":
+    if kind == "rates":
         return issue_rates(args, torch, _capi)
-    if args.workload.endswith("_bwd"):
+    if kind == "attention_backward":
         return backward_bench(args, torch, W, _capi)
-    if args.workload == "kv_append":
+    if kind == "kv_append":
         return kv_append_bench(args, torch, W)
-    if args.workload == "kv_append_fp8":
+    if kind == "kv_append_fp8":
         return kv_append_fp8_bench(args, torch, W)
-    if args.workload in ("rab_time", "rab_time_bwd", "rab_pos"):
+    if kind == "bias":
         return bias_bench(args, torch)
-    if args.workload in ("nmd_fwd", "nmd_bwd"):
+    if kind == "nmd":
         return nmd_bench(args, torch)
-    if args.workload == "in_linear_silu":
+    if kind == "in_linear_silu":
         return in_linear_silu_bench(args, torch)
-    if args.workload == "in_linear_silu_bwd":
+    if kind == "in_linear_silu_bwd":
         return in_linear_silu_bwd_bench(args, torch)
     cfg, op, flops, alg_bytes, desc = build_workload(args.workload, torch, W)
     dev = W.to_device(cfg)

@@ -361,3 +361,15 @@ def test_rate_diagnostics_reject_bad_arguments():
     for mode, waves in [(1, 4), (2, 4), (3, 3), (0, 5), (0, 0), (9, 1)]:
         assert lib.hstu_hip_measure_block_rates(mode, waves, 10, 0x1000, 0x1000, 0x1000, None) == -1, (mode, waves)
     assert lib.hstu_hip_measure_block_rates(0, 1, 0, 0x1000, 0x1000, 0x1000, None) == -1      # no iterations
+
+
+def test_bench_routes_every_workload_to_its_own_leg():
+    """The workload names of several legs end alike (`*_bwd`): each must reach the leg that measures it."""
+    import bench
+    want = {"config2": "attention_forward", "config5": "attention_forward", "ref_bias": "attention_forward", "config2_fp8": "attention_forward",
+            "config2_bwd": "attention_backward", "ref_bias_bwd": "attention_backward", "ref_nobias_d32_bwd": "attention_backward",
+            "rab_time": "bias", "rab_time_bwd": "bias", "rab_pos": "bias", "nmd_fwd": "nmd", "nmd_bwd": "nmd",
+            "in_linear_silu": "in_linear_silu", "in_linear_silu_bwd": "in_linear_silu_bwd", "kv_append": "kv_append",
+            "kv_append_fp8": "kv_append_fp8", "copy": "copy", "rates": "rates"}
+    for name, kind in want.items():
+        assert bench.bench_kind(name) == kind, name
