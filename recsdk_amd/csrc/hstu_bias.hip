@@ -112,13 +112,15 @@ __device__ __forceinline__ float wave_sum(float x) {
     return x;
 }
 
-// grid: x = column groups of 64 * RAB_JPT, y = row groups of RAB_ROWS rows i, z = n * batch + b; wave w takes rows
-// w, w + 4, ...  Neighbouring columns mostly share a bucket, so equal neighbours are first merged inside a lane and the
-// lanes of a wave that hold one id are then summed across the wave (one LDS atomic per distinct id and wave instead of
-// 64 colliding ones).  A workgroup per layer re-reads the ids for every layer (a third of the gradient's bytes again
-// at fp16) but measured fastest at 8 layers: 480 us, against 620-720 us with 4 layers per workgroup and 630-940 us
-// with all of them -- the reduction leaves a wave's loads idle, and more workgroups hide that better than fewer
-// bytes do.
+// A workgroup = one tile (64 * RAB_JPT columns x RAB_ROWS rows i) of one (layer, user); wave w takes rows w, w + 4, ...
+// Neighbouring columns mostly share a bucket, so equal neighbours are first merged inside a lane and the lanes of a wave
+// that hold one id are then summed across the wave (one LDS atomic per distinct id and wave instead of 64 colliding
+// ones).  A workgroup per layer reads the ids again for every layer (a third of the gradient's bytes at fp16 with
+// 4-byte ids), so the layers of one tile are numbered to run side by side on one XCD and all but the first find the ids
+// in its L2 (484 -> 424 us at 8 layers); a lane's four ids are one 16-byte read (424 -> 337 us: four 4-byte reads
+// per lane asked the memory pipeline for every cache line four times).  Several layers per workgroup measured slower
+// (620-940 us): the reduction leaves a wave's loads idle, and more workgroups hide that better.  8 / 12 / 16 rows per
+// workgroup measure the same, 32 and 64 are 8 % and 30 % slower.
 constexpr int RAB_ROWS = 16;
 template <typename T, typename I>
 __global__ __launch_bounds__(RAB_NT) void hstu_rab_time_bwd_kernel(const hstu_rab_time_bwd_params p) {
@@ -126,15 +128,24 @@ __global__ __launch_bounds__(RAB_NT) void hstu_rab_time_bwd_kernel(const hstu_ra
     const int nb = p.num_buckets, s = p.seq_len;
     for (int k = threadIdx.x; k < nb; k += RAB_NT) hist[k] = 0.f;
     __syncthreads();
-    const int n = blockIdx.z / p.batch, b = blockIdx.z % p.batch;
+    // workgroup L runs on XCD L % 8: the layers of one tile of ids are the workgroups L = (hi * layers + n) * 8 + lo of tile
+    // hi * 8 + lo, so that they meet in one L2 within a few dispatches and the ids come from HBM once
+    const unsigned L = blockIdx.x, nl = (unsigned)p.num_layers;
+    const unsigned tile = (L / (8 * nl)) * 8 + L % 8;
+    const int n = (int)((L / 8) % nl);
+    const unsigned gx = (unsigned)(s + 64 * RAB_JPT - 1) / (64 * RAB_JPT), gy = (unsigned)(s + RAB_ROWS - 1) / RAB_ROWS;
+    if (tile >= gx * gy * (unsigned)p.batch) return;   // (the whole workgroup: the padding of the last group of 8 tiles)
+    const int b = (int)(tile / (gx * gy));
+    const unsigned bx = tile % gx, by = tile / gx % gy;
     const int lane = threadIdx.x & 63;
-    const int j0 = (blockIdx.x * 64 + lane) * RAB_JPT;
+    const int j0 = (bx * 64 + lane) * RAB_JPT;
     const int64_t s2 = 2 * (int64_t)s;
     const T* g = reinterpret_cast<const T*>(p.grad) + ((int64_t)n * p.batch + b) * s2 * s2;
     const I* bt = reinterpret_cast<const I*>(p.bucket_ts) + (int64_t)b * s * s;
     const bool wide = j0 + RAB_JPT <= s && (s2 * sizeof(T)) % 16 == 0;
-    const int i_end = min((int)(blockIdx.y + 1) * RAB_ROWS, s);
-    for (int i = blockIdx.y * RAB_ROWS + (threadIdx.x >> 6); i < i_end; i += RAB_NT / 64) {   // wave-uniform
+    const bool wide_id = j0 + RAB_JPT <= s && ((int64_t)s * sizeof(I)) % 16 == 0 && (reinterpret_cast<uintptr_t>(p.bucket_ts) & 15) == 0;
+    const int i_end = min((int)(by + 1) * RAB_ROWS, s);
+    for (int i = by * RAB_ROWS + (threadIdx.x >> 6); i < i_end; i += RAB_NT / 64) {   // wave-uniform
         float sum[RAB_JPT];
         int id[RAB_JPT];
 #pragma unroll
@@ -159,11 +170,25 @@ __global__ __launch_bounds__(RAB_NT) void hstu_rab_time_bwd_kernel(const hstu_ra
                     if (j0 + k < s)
                         sum[k] = (to_float(row[2 * k]) + to_float(row[2 * k + 1])) + (to_float(row[s2 + 2 * k]) + to_float(row[s2 + 2 * k + 1]));
             }
+            if (wide_id) {
+                // the lane's ids as 16-byte reads (rows of ids start on 16-byte boundaries)
+                typedef __attribute__((ext_vector_type(4))) unsigned int u4;
+                constexpr int NI = RAB_JPT * sizeof(I) / 16;
+                I raw[RAB_JPT];
 #pragma unroll
-            for (int k = 0; k < RAB_JPT; k++) {
-                if (j0 + k >= s) break;
-                const int64_t v = (int64_t)bt[(int64_t)i * s + j0 + k];
-                id[k] = (v >= 0 && v < nb) ? (int)v : -1;
+                for (int q = 0; q < NI; q++) reinterpret_cast<u4*>(raw)[q] = reinterpret_cast<const u4*>(bt + (int64_t)i * s + j0)[q];
+#pragma unroll
+                for (int k = 0; k < RAB_JPT; k++) {
+                    const int64_t v = (int64_t)raw[k];
+                    id[k] = (v >= 0 && v < nb) ? (int)v : -1;
+                }
+            } else {
+#pragma unroll
+                for (int k = 0; k < RAB_JPT; k++) {
+                    if (j0 + k >= s) break;
+                    const int64_t v = (int64_t)bt[(int64_t)i * s + j0 + k];
+                    id[k] = (v >= 0 && v < nb) ? (int)v : -1;
+                }
             }
             // equal neighbours inside the lane first
 #pragma unroll
@@ -265,7 +290,8 @@ template <typename T, typename I>
 static void launch_rab_time_bwd(const hstu_rab_time_bwd_params& p, hipStream_t st) {
     const unsigned gx = (unsigned)((p.seq_len + 64 * RAB_JPT - 1) / (64 * RAB_JPT));
     const unsigned gy = (unsigned)((p.seq_len + RAB_ROWS - 1) / RAB_ROWS);
-    hipLaunchKernelGGL((hstu_rab_time_bwd_kernel<T, I>), dim3(gx, gy, (unsigned)(p.num_layers * p.batch)), dim3(RAB_NT), 0, st, p);
+    const unsigned tiles = gx * gy * (unsigned)p.batch;
+    hipLaunchKernelGGL((hstu_rab_time_bwd_kernel<T, I>), dim3((tiles + 7) / 8 * 8 * (unsigned)p.num_layers), dim3(RAB_NT), 0, st, p);
 }
 
 template <typename T>
