@@ -59,16 +59,33 @@ __global__ __launch_bounds__(RAB_NT) void hstu_rab_time_kernel(const hstu_rab_ti
     const I* ts = reinterpret_cast<const I*>(p.timestamps) + (int64_t)b * s;
     const I ti = ts[i];
     int bucket[RAB_JPT];
+    // a lane's four timestamps and ids as 16-byte accesses when the rows start on 16-byte boundaries (four accesses of one
+    // element per lane would each ask for every cache line of the wave's stretch)
+    constexpr int NI = RAB_JPT * sizeof(I) / 16;
+    const bool whole = j0 + RAB_JPT <= s && ((int64_t)s * sizeof(I)) % 16 == 0;
+    I tj[RAB_JPT];
+    if (whole && (reinterpret_cast<uintptr_t>(p.timestamps) & 15) == 0) {
 #pragma unroll
-    for (int k = 0; k < RAB_JPT; k++) {
-        const int j = min(j0 + k, s - 1);
-        bucket[k] = bucket_of(bounds, W - 1, abs_diff_f32<I>(ti, ts[j]), inv);
+        for (int q = 0; q < NI; q++) reinterpret_cast<u4*>(tj)[q] = reinterpret_cast<const u4*>(ts + j0)[q];
+    } else {
+#pragma unroll
+        for (int k = 0; k < RAB_JPT; k++) tj[k] = ts[min(j0 + k, s - 1)];
     }
+#pragma unroll
+    for (int k = 0; k < RAB_JPT; k++) bucket[k] = bucket_of(bounds, W - 1, abs_diff_f32<I>(ti, tj[k]), inv);
     if (p.bucket_ts_out) {
         I* bo = reinterpret_cast<I*>(p.bucket_ts_out) + ((int64_t)b * s + i) * s;
+        if (whole && (reinterpret_cast<uintptr_t>(p.bucket_ts_out) & 15) == 0) {
+            I bi[RAB_JPT];
 #pragma unroll
-        for (int k = 0; k < RAB_JPT; k++)
-            if (j0 + k < s) bo[j0 + k] = (I)bucket[k];
+            for (int k = 0; k < RAB_JPT; k++) bi[k] = (I)bucket[k];
+#pragma unroll
+            for (int q = 0; q < NI; q++) reinterpret_cast<u4*>(bo + j0)[q] = reinterpret_cast<const u4*>(bi)[q];
+        } else {
+#pragma unroll
+            for (int k = 0; k < RAB_JPT; k++)
+                if (j0 + k < s) bo[j0 + k] = (I)bucket[k];
+        }
     }
     T* out = reinterpret_cast<T*>(p.rab_time_out);
     const int64_t s2 = 2 * (int64_t)s;
