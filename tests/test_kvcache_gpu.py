@@ -224,6 +224,43 @@ def test_fp8_append_matches_oracle_bit_for_bit(dim, heads, page, dtype, order):
     assert int((cache != 0).sum()) > 0
 
 
+def test_fp8_append_skips_invalid_tokens_and_tokens_past_the_device_count():
+    """Tokens with a user index or a position outside what the host described are skipped (the reference's kernel checks
+    nothing: append_paged_kvcache_kernel.h:42-76; this library does, so that a bad index cannot write outside the table),
+    and so are the tokens behind the count in device memory.  A skipped token in the middle of a run cuts the run in two:
+    its page then goes through the kernels for scattered pages.  Expected: the oracle on the valid tokens alone."""
+    say("kv append fp8, invalid tokens")
+    heads, dim, page, dtype = 2, 64, 32, torch.bfloat16
+    s = _fp8_scenario(11, 7, heads, dim, page, dtype)
+    cache = torch.zeros(s["pages"], 2, page, heads, dim, dtype=torch.uint8)
+    scales = torch.ones(s["pages"], 2, heads)
+    dc, ds = cache.cuda(), scales.cuda()
+    zeros = torch.zeros(s["users"], dtype=torch.int32)
+    g = torch.Generator().manual_seed(3)
+    for n, st in enumerate(s["steps"]):
+        nnz = st["nnz"]
+        bi, pos = KO.paged_batch_indices_positions(st["append_indptr"].numpy(), st["seq_lens"].numpy())
+        bi, pos = bi.copy(), pos.copy()
+        bad = torch.randperm(nnz, generator=g)[:9].numpy()
+        bi[bad[:3]] = -1
+        bi[bad[3:5]] = s["users"]
+        pos[bad[5:7]] = -2
+        pos[bad[7:9]] = 10 ** 6                       # far behind the user's pages
+        count = nnz - 4                                 # the last four tokens are padding
+        ok = np.ones(nnz, dtype=bool)
+        ok[bad] = False
+        ok[count:] = False
+        keep = np.nonzero(ok)[0]
+        KO.append_paged_kvcache_fp8(cache, scales, st["key"][torch.from_numpy(keep)], st["value"][torch.from_numpy(keep)], bi[keep], pos[keep],
+                                    zeros.numpy(), len(keep), s["kv_indices"].numpy(), s["kv_indptr"].numpy())
+        kvcache.append_kvcache_fp8(st["key"].cuda(), st["value"].cuda(), torch.from_numpy(bi.astype(np.int32)).cuda(),
+                                   torch.from_numpy(pos.astype(np.int32)).cuda(), zeros.cuda(),
+                                   torch.tensor([count], dtype=torch.int32, device="cuda"), nnz, dc, ds, s["kv_indices"].cuda(), s["kv_indptr"].cuda())
+        torch.cuda.synchronize()
+        assert torch.equal(ds.cpu(), scales), f"scales after step {n}"
+        assert torch.equal(dc.cpu(), cache), f"bytes after step {n}"
+
+
 def test_fp8_append_of_a_few_tokens_into_a_large_table_with_a_dirty_workspace():
     """The work of a call follows the new tokens: a 20000-page table, 11 new tokens of two users, a workspace full of
     arbitrary bytes.  Only the touched pages and their scales change."""
