@@ -122,6 +122,96 @@ __global__ __launch_bounds__(RAB_NT) void hstu_rab_time_kernel(const hstu_rab_ti
     }
 }
 
+// The same for rows whose length is a multiple of 4 (rows of the outputs then start on 16-byte boundaries, but in general
+// not on cache lines: 2s = 4600 two-byte columns are 71.9 lines).  A wave's store of 64 x 16 bytes that starts inside a
+// line leaves two lines half written for the neighbouring wave to finish, and those partial writes cost the memory 40 %
+// of its rate (s = 2304 ran at 5.6 TB/s where s = 2300 ran at 3.9).  So the lanes of a wave are made to cover whole lines
+// of every row: a "unit" is what a lane stores (4 columns j = 8 output columns), a workgroup computes the buckets of 256
+// units, parks them in LDS (4 ids of one byte), and stores 248 of them per output row, starting `a` units further right,
+// where a < 8 is what brings lane 0 of each wave onto a line boundary of THAT row (rows 2i and 2i+1 differ); the
+// first `a` units of a row go to the eight spare lanes of the row's first workgroup.
+constexpr int RAB_UPW = 248;   // units a workgroup stores per row: a multiple of the units per line
+template <typename T, typename I>
+__global__ __launch_bounds__(RAB_NT) void hstu_rab_time_lines_kernel(const hstu_rab_time_params p) {
+    constexpr int LPV = 16 / sizeof(T);
+    constexpr int MAXL = (HSTU_RAB_MAX_LAYERS + LPV - 1) / LPV * LPV;
+    typedef __attribute__((ext_vector_type(4))) unsigned int u4;
+    __shared__ float bounds[HSTU_RAB_MAX_BUCKETS + 1];
+    __shared__ __attribute__((aligned(16))) T wtab[HSTU_RAB_MAX_BUCKETS * MAXL];
+    __shared__ unsigned ids[RAB_NT];
+    const int W = p.weight_cols, s = p.seq_len, nl = p.num_layers;
+    const int lpad = (nl + LPV - 1) / LPV * LPV;
+    for (int k = threadIdx.x; k <= W; k += RAB_NT) bounds[k] = p.bucket_bounds[k];
+    for (int k = threadIdx.x; k < nl * W; k += RAB_NT) wtab[(k % W) * lpad + k / W] = reinterpret_cast<const T*>(p.weights)[k];
+    __syncthreads();
+    const int units = s / RAB_JPT;
+    const unsigned groups = (unsigned)(units + RAB_UPW - 1) / RAB_UPW;
+    const unsigned row = blockIdx.x / groups, grp = blockIdx.x % groups;
+    const int b = row / s, i = row % s, tid = threadIdx.x;
+    const float inv = p.bucket_divisor > 0.f ? 0.69314718f / p.bucket_divisor : 0.f;
+    const I* ts = reinterpret_cast<const I*>(p.timestamps) + (int64_t)b * s;
+    {
+        const int j0 = (RAB_UPW * (int)grp + tid) * RAB_JPT;
+        unsigned packed = 0;
+        if (j0 < s) {
+            const I ti = ts[i];
+#pragma unroll
+            for (int k = 0; k < RAB_JPT; k++) packed |= (unsigned)bucket_of(bounds, W - 1, abs_diff_f32<I>(ti, ts[j0 + k]), inv) << (8 * k);
+        }
+        ids[tid] = packed;
+    }
+    __syncthreads();
+    // which unit this lane stores for a row that starts at address `rowp`, chunks of CB bytes per lane; -1: none
+    auto unit_of = [&](uintptr_t rowp, int cb, int& src) __attribute__((always_inline)) -> int {
+        const int cpl = 128 / cb;
+        const int a = (cpl - (int)((rowp / (unsigned)cb) % (unsigned)cpl)) % cpl;
+        int v;
+        if (tid < RAB_UPW) { src = tid + a; v = RAB_UPW * (int)grp + src; }
+        else { src = tid - RAB_UPW; v = (grp == 0 && src < a) ? src : units; }
+        return v < units ? v : -1;
+    };
+    if (p.bucket_ts_out) {
+        I* bo = reinterpret_cast<I*>(p.bucket_ts_out) + ((int64_t)b * s + i) * s;
+        int src;
+        const int v = unit_of(reinterpret_cast<uintptr_t>(bo), RAB_JPT * sizeof(I), src);
+        if (v >= 0) {
+            const unsigned pk = ids[src];
+            I bi[RAB_JPT];
+#pragma unroll
+            for (int k = 0; k < RAB_JPT; k++) bi[k] = (I)((pk >> (8 * k)) & 0xffu);
+#pragma unroll
+            for (int q = 0; q < (int)(RAB_JPT * sizeof(I) / 16); q++) reinterpret_cast<u4*>(bo + (int64_t)v * RAB_JPT)[q] = reinterpret_cast<const u4*>(bi)[q];
+        }
+    }
+    T* out = reinterpret_cast<T*>(p.rab_time_out);
+    const int64_t s2 = 2 * (int64_t)s;
+#pragma unroll
+    for (int rsel = 0; rsel < 2; rsel++) {
+        // row 2i + rsel of layer 0; the planes of the other layers are a whole number of lines further on
+        T* rowp = out + ((int64_t)b * s2 + 2 * i + rsel) * s2;
+        int src;
+        const int v = unit_of(reinterpret_cast<uintptr_t>(rowp), 2 * RAB_JPT * sizeof(T), src);
+        if (v < 0) continue;
+        const unsigned pk = ids[src];
+        for (int n0 = 0; n0 < nl; n0 += LPV) {
+            T val[RAB_JPT][LPV];
+#pragma unroll
+            for (int k = 0; k < RAB_JPT; k++) *reinterpret_cast<u4*>(val[k]) = *reinterpret_cast<const u4*>(wtab + ((pk >> (8 * k)) & 0xffu) * lpad + n0);
+#pragma unroll
+            for (int l = 0; l < LPV; l++) {
+                const int n = n0 + l;
+                if (n >= nl) break;
+                T two[2 * RAB_JPT];
+#pragma unroll
+                for (int k = 0; k < RAB_JPT; k++) two[2 * k] = two[2 * k + 1] = val[k][l];
+                T* dst = rowp + (int64_t)n * p.batch * s2 * s2 + (int64_t)v * (2 * RAB_JPT);
+#pragma unroll
+                for (int q = 0; q < (int)(2 * RAB_JPT * sizeof(T) / 16); q++) __builtin_nontemporal_store(reinterpret_cast<const u4*>(two)[q], reinterpret_cast<u4*>(dst) + q);
+            }
+        }
+    }
+}
+
 // sum of x over the 64 lanes
 __device__ __forceinline__ float wave_sum(float x) {
 #pragma unroll
@@ -299,6 +389,13 @@ __global__ __launch_bounds__(RAB_NT) void hstu_rab_pos_kernel(const T* rel, cons
 
 template <typename T, typename I>
 static void launch_rab_time(const hstu_rab_time_params& p, hipStream_t st) {
+    // rows of whole 16-byte chunks on chunk boundaries: the variant whose waves store whole cache lines
+    const uintptr_t ob = reinterpret_cast<uintptr_t>(p.rab_time_out), ib = reinterpret_cast<uintptr_t>(p.bucket_ts_out);
+    if (p.seq_len % RAB_JPT == 0 && ob % (2 * RAB_JPT * sizeof(T)) == 0 && ib % (RAB_JPT * sizeof(I)) == 0) {
+        const unsigned groups = (unsigned)((p.seq_len / RAB_JPT + RAB_UPW - 1) / RAB_UPW);
+        hipLaunchKernelGGL((hstu_rab_time_lines_kernel<T, I>), dim3(groups * (unsigned)(p.batch * p.seq_len)), dim3(RAB_NT), 0, st, p);
+        return;
+    }
     const unsigned gx = (unsigned)((p.seq_len + RAB_NT * RAB_JPT - 1) / (RAB_NT * RAB_JPT));
     hipLaunchKernelGGL((hstu_rab_time_kernel<T, I>), dim3(gx * (unsigned)(p.batch * p.seq_len)), dim3(RAB_NT), 0, st, p);
 }

@@ -33,7 +33,11 @@ def _timestamps(train_len, candidate_len, valid_lens, dtype):
 
 @pytest.mark.parametrize("num_layers,train_len,candidate_len,bs,dtype,tsdtype", [
     (1, 500, 600, 2, torch.float16, torch.int32), (8, 300, 0, 3, torch.float32, torch.int32), (3, 257, 90, 2, torch.bfloat16, torch.int64),
-    (2, 31, 0, 1, torch.float16, torch.int32)])
+    (2, 31, 0, 1, torch.float16, torch.int32),
+    # rows of whole 16-byte chunks (s a multiple of 4) take the variant that stores whole cache lines: 8-byte ids, more
+    # layers than one table read holds, more than one workgroup per row (s / 4 > 248), fp32 chunks of 32 bytes
+    (3, 256, 96, 2, torch.bfloat16, torch.int64), (20, 36, 0, 2, torch.float16, torch.int64), (2, 1000, 200, 1, torch.float16, torch.int32),
+    (5, 1020, 0, 1, torch.float32, torch.int64)])
 def test_rab_time_with_index(num_layers, train_len, candidate_len, bs, dtype, tsdtype):
     say("rab_time", num_layers, train_len, candidate_len, bs, dtype, tsdtype)
     g = torch.Generator().manual_seed(7)
