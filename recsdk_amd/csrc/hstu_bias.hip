@@ -351,8 +351,16 @@ __global__ __launch_bounds__(RAB_NT) void hstu_rab_pos_kernel(const T* rel, cons
         return from_float<T>(__fadd_rn(keep, fill));
     };
     const int base = blockIdx.x * RAB_NT * 8;
-    const int j0 = base + threadIdx.x * 8;
     if (seq2 % 8 == 0) {
+        // rows of whole chunks of 8 columns: the lanes of a wave cover whole cache lines of output row i (the planes of the
+        // users are a whole number of lines apart).  A workgroup takes RAB_UPW chunks, starting `a` chunks further right,
+        // where a is what brings lane 0 of each wave onto a line boundary of this row; the first `a` chunks of the row go
+        // to the spare lanes of its first workgroup.
+        constexpr int cb = 8 * sizeof(T), cpl = 128 / cb;
+        const int a = (cpl - (int)((reinterpret_cast<uintptr_t>(out + (int64_t)i * seq2) / cb) % cpl)) % cpl;
+        const int tid = threadIdx.x;
+        int chunk = tid < RAB_UPW ? RAB_UPW * (int)blockIdx.x + tid + a : ((blockIdx.x == 0 && tid - RAB_UPW < a) ? tid - RAB_UPW : seq2);
+        const int j0 = chunk * 8;
         if (j0 >= seq2) return;
         typedef __attribute__((ext_vector_type(4))) unsigned int u4;
         constexpr int NV = 8 * sizeof(T) / 16;
@@ -410,7 +418,8 @@ static void launch_rab_time_bwd(const hstu_rab_time_bwd_params& p, hipStream_t s
 
 template <typename T>
 static void launch_rab_pos(int seq2, const void* rel, const void* identity, const int64_t* lens, int batch, void* out, hipStream_t st) {
-    const unsigned gx = (unsigned)((seq2 + RAB_NT * 8 - 1) / (RAB_NT * 8));
+    // (rows of whole 8-column chunks: RAB_UPW chunks per workgroup, see the kernel)
+    const unsigned gx = seq2 % 8 == 0 ? (unsigned)((seq2 / 8 + RAB_UPW - 1) / RAB_UPW) : (unsigned)((seq2 + RAB_NT * 8 - 1) / (RAB_NT * 8));
     for (int u0 = 0; u0 < batch; u0 += RAB_POS_USERS) {
         RabPosLens l;
         const int nu = batch - u0 < RAB_POS_USERS ? batch - u0 : RAB_POS_USERS;
