@@ -409,6 +409,8 @@ template <int D, int EXTRA, bool PAGED> struct Shape {
     static constexpr bool DMA = (!PAGED && D == 128) || PDMA;
     // head dim 64, rows straight from k / v, no dense bias or custom mask: direct copies too, 8 rows per instruction
     static constexpr bool DMA64 = !PAGED && D == 64 && (EXTRA == 0 || (EXTRA >= 2 && EXTRA <= 4));
+    // head dim 32, plain variant: 16 rows of 64 bytes per instruction
+    static constexpr bool DMA32 = !PAGED && D == 32 && EXTRA == 0;
     static constexpr bool LEAN = DMA && (EXTRA == 0 || EXTRA == 8 || EXTRA == 9 || EXTRA == 10);
     // EXTRA 10: the plain variant on sequences whose rows are taken in reverse order (row i of q / k / v / out is row
     // L - 1 - i of its sequence in memory).  With K in the place of q, Q in the place of k and dO in the place of v the
@@ -420,10 +422,10 @@ template <int D, int EXTRA, bool PAGED> struct Shape {
     static constexpr int BNT = (LEAN || XDMA) ? 32 : 64;     // K columns per step
     // waves per SIMD; head dim 256 needs the registers of a whole SIMD lane for its 32 x 256 accumulator and Q fragments
     // (the variants with a bias or a mask copied by DMA fit three at the price of 7 spilled registers: 2 % faster than two;
-    // the plain variants at head dims 32 and 64 need 88 / 113 registers and 26.6 / 34 KB of LDS and run four: 5 % / 1 % faster
+    // the plain variants at head dims 32 and 64 need 81 / 113 registers and 16 / 34 KB of LDS and run four: 5 % / 1 % faster
     // than three -- at head dim 64 only since its tiles are copied straight into LDS; with the register loader it took 135
-    // registers and lost 5 % to AGPR copies under the cap of 128)
-    static constexpr int WAVES = D == 256 ? 1 : ((D <= 64 && EXTRA == 0 && !PAGED) ? 4 : ((LEAN || (D <= 64 && EXTRA != 1) || (XDMA && EXTRA != 7)) ? 3 : 2));
+    // registers and lost 5 % to AGPR copies under the cap of 128.  Five and six at head dim 32: no faster, 1.5 % slower)
+        static constexpr int WAVES = D == 256 ? 1 : ((D <= 64 && EXTRA == 0 && !PAGED) ? 4 : ((LEAN || (D <= 64 && EXTRA != 1) || (XDMA && EXTRA != 7)) ? 3 : 2));
 };
 
 template <typename T, int D, int EXTRA, bool PAGED>
@@ -449,7 +451,12 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
     // read start on 16 different multiples of 4 banks, the 4 rows of a transposing read lie 16 banks apart.
     constexpr bool DMA64 = SH::DMA64;
     constexpr int B64 = 1040, NBLK8 = BNT / 8;
-    constexpr int STAGE_BYTES = DMA ? NBLK4 * (KBLK + VBLK) : (DMA64 ? 2 * NBLK8 * B64 : (TL::K_ELEMS + TL::V_ELEMS) * 2);
+    // Head dim 32: blocks of 16 rows = 1024 bytes, row rho keeping its chunk c in slot (c + rho / 4) % 4: the 16 rows of a
+    // row-wise read then fall on 16 different groups of 4 banks, and a transposing read covers 4 whole consecutive rows.
+    constexpr bool DMA32 = SH::DMA32;
+    constexpr int NBLK16 = BNT / 16;
+    constexpr int STAGE_BYTES = DMA ? NBLK4 * (KBLK + VBLK) : (DMA64 ? 2 * NBLK8 * B64 : (DMA32 ? 2 * NBLK16 * 1024 : (TL::K_ELEMS + TL::V_ELEMS) * 2));
+    constexpr bool ANY_DMA = DMA || DMA64 || DMA32;
     // two separate arrays: reads of one tile are then independent of the copy in flight into the other
     __shared__ __attribute__((aligned(1024))) char lds0[STAGE_BYTES];
     __shared__ __attribute__((aligned(1024))) char lds1[STAGE_BYTES];
@@ -615,7 +622,7 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
         // visible row and zeroed when written to LDS) so that they stay in straight-line code and only the LDS
         // write waits for them.  Direct path: a buffer view of this (sequence, kv head) that ends with the last
         // visible row, so rows past it read as zeros.
-        u32x4 kreg[(DMA || DMA64) ? 1 : TL::NCH], vreg[(DMA || DMA64) ? 1 : TL::NCH];
+        u32x4 kreg[ANY_DMA ? 1 : TL::NCH], vreg[ANY_DMA ? 1 : TL::NCH];
         const char* kview = reinterpret_cast<const char*>(p.k) + ((int64_t)s.k_start * p.heads_k + hk) * D * 2;
         const char* vview = reinterpret_cast<const char*>(p.v) + ((int64_t)s.k_start * p.heads_k + hk) * D * 2;
         const unsigned view_bytes = kend > 0 ? (unsigned)(kend - 1) * rowstride + D * 2 : 0;
@@ -718,6 +725,16 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                     __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, LDS_PTR(void, dst + blk * B64), 16, lo + so, 0, 0, 0);
                     __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, LDS_PTR(void, dst + (NBLK8 + blk) * B64), 16, lo + so, 0, 0, 0);
                 }
+            } else if constexpr (DMA32) {
+                const unsigned tile_off = (unsigned)k0 * rowstride;
+                __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc((void*)(kview + tile_off), 0, (int)(view_bytes - tile_off), 0x00020000);
+                __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc((void*)(vview + tile_off), 0, (int)(view_bytes - tile_off), 0x00020000);
+                const int rho = lane >> 2;
+                const unsigned lo = (unsigned)rho * rowstride + ((((lane & 3) - (rho >> 2)) & 3) << 4);   // lane L fills slot L % 4 of row L / 4
+                static_assert(!DMA32 || NBLK16 == 4, "one block of K and one of V per wave");
+                const unsigned so = (unsigned)(16 * w) * rowstride;
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, LDS_PTR(void, dst + w * 1024), 16, lo + so, 0, 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, LDS_PTR(void, dst + (NBLK16 + w) * 1024), 16, lo + so, 0, 0, 0);
             } else if (PAGED && p.page_size % BNT == 0 && k0 + BNT <= s.hist_k) {
                 // the whole tile lies in one page of the history (pages hold a multiple of the tile's columns and the
                 // history starts at column 0): one page lookup for the tile, rows at a fixed stride
@@ -799,7 +816,7 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
         auto stash = [&](int kt, char* dst) __attribute__((always_inline)) {
             const int k0 = kt * BNT;
             const int buf = kt & 1;
-            if (!DMA && !DMA64 && k0 < kend) {
+            if (!ANY_DMA && k0 < kend) {
                 T* dk = reinterpret_cast<T*>(dst);
                 T* dv = dk + TL::K_ELEMS;
 #pragma unroll
@@ -821,7 +838,7 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                 if (tab_pos && tid < PW - 1) lds_pos[buf * PW + tid] = pw_reg;
                 if (tab_ts && tid < BN) lds_tk[buf * BN + tid] = tk_reg;
             }
-            if constexpr (DMA || DMA64) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            if constexpr (ANY_DMA) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             if constexpr (SH::PDMA8) {
                 // widen this wave's staged history rows (e4m3 x the page's scale, rounded once to the I/O dtype) into the tile:
                 // lane L holds 16 elements of key k0 + 8w + L / 8 = chunks 2 (L % 8) and + 1 of row rho = that key % 4
@@ -850,6 +867,9 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
             } else if constexpr (DMA64) {
                 const int rho = l32 & 7;   // row l32 of the 32-key block: block l32 / 8, chunk g + 2 ds
                 return *reinterpret_cast<const v8*>(cur + (4 * kb + (l32 >> 3)) * B64 + rho * 128 + (((g + 2 * ds + 2 * (rho >> 1)) & 7) << 4));
+            } else if constexpr (DMA32) {
+                const int rho = l32 & 15;   // row l32 of the 32-key block: block l32 / 16, chunk g + 2 ds
+                return *reinterpret_cast<const v8*>(cur + (2 * kb + (l32 >> 4)) * 1024 + rho * 64 + (((g + 2 * ds + (rho >> 2)) & 3) << 4));
             } else {
                 return *reinterpret_cast<const v8*>(reinterpret_cast<const T*>(cur) + (32 * kb + l32) * TL::KS + 8 * g + 16 * ds);
             }
@@ -864,6 +884,11 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                 const int rho = 4 * g + ((lane & 15) >> 2), chunk = 4 * db + 2 * (l32 >> 4) + ((lane & 3) >> 1);
                 return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
                     LDS_PTR(s16x4, cur + (NBLK8 + 4 * kb + part) * B64 + rho * 128 + (((chunk + 2 * (rho >> 1)) & 7) << 4) + 8 * (lane & 1)));
+            } else if constexpr (DMA32) {
+                // row 8 part + 4 g + (lane % 16) / 4 of the 32-key block; 8 bytes of chunk 2 (l32 / 16) + (lane % 4) / 2
+                const int r = 8 * part + 4 * g + ((lane & 15) >> 2), rho = r & 15, chunk = 2 * (l32 >> 4) + ((lane & 3) >> 1);
+                return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    LDS_PTR(s16x4, cur + (NBLK16 + 2 * kb + (r >> 4)) * 1024 + rho * 64 + (((chunk + (rho >> 2)) & 3) << 4) + 8 * (lane & 1)));
             } else {
                 const T* vp = reinterpret_cast<const T*>(cur) + TL::K_ELEMS + (32 * kb + 8 * part + 4 * g + ((lane & 15) >> 2)) * TL::VS + 16 * (l32 >> 4) + 4 * (lane & 3);
                 return __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, vp + 32 * db));
