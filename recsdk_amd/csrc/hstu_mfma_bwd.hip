@@ -84,8 +84,9 @@ template <> __device__ __forceinline__ float bwd_half<_Float16>(unsigned w, int 
 template <typename T, int D, int MODE, bool BIAS>
 // (head dim 256 keeps 32 operand fragments and a 32 x 256 accumulator per wave: one wave per SIMD)
 // waves per SIMD: one at head dim 256 (see above), three where the registers allow it (head dim 32; at head dim 64 the
-// kernels with one accumulator, since their tiles are copied straight into LDS), else two
-#define BWD_WAVES(D, MODE) ((D) == 256 ? 1 : ((D) == 32 || ((D) == 64 && (MODE) != MODE_DKV)) ? 3 : 2)
+// kernels with one accumulator, since their tiles are copied straight into LDS), four for the dQ kernel at head dim 32
+// (108 registers), else two
+#define BWD_WAVES(D, MODE) ((D) == 256 ? 1 : ((D) == 32 && (MODE) == MODE_DQ) ? 4 : ((D) == 32 || ((D) == 64 && (MODE) != MODE_DKV)) ? 3 : 2)
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BWD_WAVES(D, MODE), BWD_WAVES(D, MODE))))
 void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
     typedef typename BMM<T>::v8 v8;
@@ -109,11 +110,11 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
     // read both ways.  Two stages in separate arrays: the compiler then does not make the reads of one stage wait for the
     // copy in flight into the other.
     // (not the dV kernel, which has half the matrix work per tile to hide the copies behind and measured 20 % slower with them)
-    constexpr bool BDMA = (D == 128 || D == 64) && MODE != MODE_DV;
-    constexpr int RPB = D == 128 ? 4 : 8;            // rows per block
+    constexpr bool BDMA = (D == 128 || D == 64 || D == 32) && MODE != MODE_DV;
+    constexpr int RPB = 512 / D;                     // rows per block: what one copy instruction (1 KB) brings
     constexpr int CPR = D / 8;                       // 16-byte chunks per row
     constexpr int DBLK = 1040, DTILE = (WBN / RPB) * DBLK;
-    auto slot_of = [](int c, int rho) __attribute__((always_inline)) -> int { return D == 128 ? ((c + 4 * rho) & 15) : ((c + 2 * (rho >> 1)) & 7); };
+    auto slot_of = [](int c, int rho) __attribute__((always_inline)) -> int { return D == 128 ? ((c + 4 * rho) & 15) : (D == 64 ? ((c + 2 * (rho >> 1)) & 7) : ((c + (rho >> 2)) & 3)); };
     __shared__ __attribute__((aligned(16))) char d1a[BDMA ? DTILE : 16];
     __shared__ __attribute__((aligned(16))) char d1b[BDMA ? DTILE : 16];
     __shared__ __attribute__((aligned(16))) char d2a[BDMA ? DTILE : 16];
@@ -208,7 +209,7 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
                     __amdgpu_buffer_rsrc_t r1 = __builtin_amdgcn_make_buffer_rsrc((void*)((MODE == MODE_DQ ? kb_ : qb) + first), 0, 0x7fffffff, 0x00020000);
                     __amdgpu_buffer_rsrc_t r2 = __builtin_amdgcn_make_buffer_rsrc((void*)((MODE == MODE_DQ ? vb : gb) + first), 0, 0x7fffffff, 0x00020000);
                     const int rho = lane / CPR;
-                    const unsigned chunk = (unsigned)(D == 128 ? ((lane % CPR) - 4 * rho) & 15 : ((lane % CPR) - 2 * (rho >> 1)) & 7) << 4;
+                    const unsigned chunk = (unsigned)(D == 128 ? ((lane % CPR) - 4 * rho) & 15 : (D == 64 ? ((lane % CPR) - 2 * (rho >> 1)) & 7 : ((lane % CPR) - (rho >> 2)) & 3)) << 4;
                     constexpr int BPW = WBN / RPB / 4;   // blocks per wave and tile
 #pragma unroll
                     for (int i = 0; i < BPW; i++) {
