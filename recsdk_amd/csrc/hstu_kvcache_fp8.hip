@@ -47,10 +47,11 @@ __device__ __forceinline__ unsigned kf_quant2(float a, float b, float s) {
     return (unsigned)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false) & 0xffffu;
 }
 
-// x / s rounded to nearest like the division above, for a divisor shared by many elements: r = 1.0f / s (rounded to
-// nearest), the product x * r is corrected twice by its remainder (each fma is exact in the remainder).  For s in
-// [2^-100, 2^100] only (r and the remainders stay normal numbers); quotients below the fp32 normal range are far below
-// half of the smallest e4m3 number and round to the same zero either way.
+// x / s for a divisor shared by many elements: r = 1.0f / s (rounded to nearest), the product x * r is corrected twice by
+// its remainder (each fma is exact in the remainder).  The result is the IEEE quotient unless x / s lies within 2^-48
+// (relative) of an fp32 rounding boundary, and the e4m3 byte differs only if that boundary is also next to an e4m3 tie.
+// For s in [2^-100, 2^100] only (r and the remainders stay normal numbers); quotients below the fp32 normal range are far
+// below half of the smallest e4m3 number and round to the same zero either way.
 __device__ __forceinline__ float kf_div_by(float x, float s, float r) {
     float q = x * r;
     q = __builtin_fmaf(__builtin_fmaf(-s, q, x), r, q);
