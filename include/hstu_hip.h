@@ -196,6 +196,10 @@ typedef struct hstu_bwd_params {
                              * written completely (zeros outside the sequences and where the mask is 0) */
 } hstu_bwd_params;
 
+/* To the caller the backward is one piece of work on `stream`, also under stream capture.  Large calls (3000 and more
+ * (Q tile, head) items) run their dQ and K-side kernels side by side on two streams of the library's own per device, forked
+ * from and joined to `stream` by events (default priority; created at the first such call on a device: make that call
+ * outside a capture).  HSTU_HIP_SERIAL_BACKWARD=1 in the environment (read once per device) keeps everything on `stream`. */
 int hstu_hip_jagged_backward_get_workspace_size(const hstu_bwd_params* p, uint64_t* workspace_bytes);
 int hstu_hip_jagged_backward(const hstu_bwd_params* p, void* workspace, uint64_t workspace_bytes, void* stream);
 

@@ -17,6 +17,8 @@
 // With a dense attn_bias (BIAS) the scores are S + bias, read from [batch, heads, max_q, max_k] next to every block, and
 // the dQ kernel, which owns whole Q rows, also writes dBias = dS (hstu_jagged.cpp:69-138: the only case that produces it)
 // into a buffer that a fill kernel has zeroed: blocks the mask hides are never visited.
+#include <cstdlib>
+#include <mutex>
 #include "hstu_device.h"
 
 namespace hstu {
@@ -597,6 +599,39 @@ uint64_t mfma_backward_workspace_bytes(const BArgs& a) {
     return one_list(a.f.p) ? q : q + work_list_shape(swapped_roles(a.f).p).bytes;
 }
 
+// The dQ kernel and the K-side kernels are independent of each other (they read q, k, v, dO and the work lists and write
+// different gradients), and each ends with a tail in which a few long items run while most of the chip idles.  They are
+// therefore launched on three streams -- the caller's and two of the library's own per device, forked from and joined to
+// the caller's stream by events -- so that the next kernel's workgroups fill the slots the previous one's tail leaves
+// empty.  To the caller the call still is one piece of work on its stream (also under stream capture, where the events
+// become edges of the graph).  Streams of default priority, events without timing, created on the first call on a device;
+// if that fails everything runs on the caller's stream.
+struct BwdFork {
+    hipStream_t side[2];
+    hipEvent_t ev[3];
+    bool ok;
+};
+static BwdFork* bwd_fork() {
+    constexpr int MAXDEV = 64;
+    static std::mutex mu;
+    static BwdFork forks[MAXDEV];
+    static bool tried[MAXDEV];
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAXDEV) return nullptr;
+    std::lock_guard<std::mutex> lock(mu);
+    BwdFork& f = forks[dev];
+    if (!tried[dev]) {
+        tried[dev] = true;
+        const char* serial = getenv("HSTU_HIP_SERIAL_BACKWARD");   // read once per device: "1" keeps the backward on the caller's stream
+        bool ok = !(serial && serial[0] == '1');
+        for (int i = 0; i < 2; i++) ok = ok && hipStreamCreateWithFlags(&f.side[i], hipStreamNonBlocking) == hipSuccess;
+        for (int i = 0; i < 3; i++) ok = ok && hipEventCreateWithFlags(&f.ev[i], hipEventDisableTiming) == hipSuccess;
+        if (!ok) (void)hipGetLastError();
+        f.ok = ok;
+    }
+    return f.ok ? &f : nullptr;
+}
+
 template <typename T, int D>
 static hipError_t launch_bwd_td(const BArgs& a, unsigned* ws, hipStream_t stream) {
     const KArgs kside = swapped_roles(a.f);
@@ -610,47 +645,70 @@ static hipError_t launch_bwd_td(const BArgs& a, unsigned* ws, hipStream_t stream
         e = launch_work_list(kside, wsk, false, stream);   // tile costs are only roughly those of the K tiles: no pairs
         if (e != hipSuccess) return e;
     }
+    // fork: the K-side kernels wait for the work lists only.  Worth it when the kernels are long against the few microseconds
+    // the events cost: at 3840 items per kernel (B = 32, h = 8, S = 2048) -2 .. -7 %, at 1440 (the headline batch) +2 %
+    BwdFork* fk = lq.grid >= 3000 ? bwd_fork() : nullptr;
+    hipStream_t sk = stream, sv = stream;
+    if (fk) {
+        if (hipEventRecord(fk->ev[0], stream) == hipSuccess && hipStreamWaitEvent(fk->side[0], fk->ev[0], 0) == hipSuccess &&
+            hipStreamWaitEvent(fk->side[1], fk->ev[0], 0) == hipSuccess) {
+            sk = fk->side[0];
+            sv = fk->side[1];
+        } else {
+            (void)hipGetLastError();
+            fk = nullptr;
+        }
+    }
+    auto join = [&](hipError_t err) -> hipError_t {
+        if (fk) {
+            // (also after a failed launch: the caller's stream must not run ahead of what did get launched)
+            const bool ok = hipEventRecord(fk->ev[1], sk) == hipSuccess && hipEventRecord(fk->ev[2], sv) == hipSuccess &&
+                            hipStreamWaitEvent(stream, fk->ev[1], 0) == hipSuccess && hipStreamWaitEvent(stream, fk->ev[2], 0) == hipSuccess;
+            if (!ok && err == hipSuccess) err = hipGetLastError();
+        }
+        return err;
+    };
     if (a.f.p.attn_bias) {
         // dBias: zero everywhere, then the dQ kernel writes the blocks the mask lets it visit
         const hstu_fwd_params& p = a.f.p;
         const unsigned zrows = (unsigned)(p.max_seq_len_q < 512 ? p.max_seq_len_q : 512);   // max_seq_len_k % 8 == 0
         hipLaunchKernelGGL(hstu_bwd_zero_bias_kernel<T>, dim3(zrows, (unsigned)(p.batch * p.heads_q)), dim3(256), 0, stream, a);
         e = hipGetLastError();
-        if (e != hipSuccess) return e;
+        if (e != hipSuccess) return join(e);
         hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DQ, true>), dim3(lq.grid), dim3(256), 0, stream, a, wsq);
         e = hipGetLastError();
-        if (e != hipSuccess) return e;
+        if (e != hipSuccess) return join(e);
         if constexpr (D <= 64) {
-            hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DKV, true>), dim3(lk.grid), dim3(256), 0, stream, a, wsk);
-            return hipGetLastError();
+            hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DKV, true>), dim3(lk.grid), dim3(256), 0, sk, a, wsk);
+            return join(hipGetLastError());
         }
-        hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DK, true>), dim3(lk.grid), dim3(256), 0, stream, a, wsk);
+        hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DK, true>), dim3(lk.grid), dim3(256), 0, sk, a, wsk);
         e = hipGetLastError();
-        if (e != hipSuccess) return e;
-        hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DV, true>), dim3(lk.grid), dim3(256), 0, stream, a, wsk);
-        return hipGetLastError();
+        if (e != hipSuccess) return join(e);
+        hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DV, true>), dim3(lk.grid), dim3(256), 0, sv, a, wsk);
+        return join(hipGetLastError());
     }
     hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DQ, false>), dim3(lq.grid), dim3(256), 0, stream, a, wsq);
     e = hipGetLastError();
-    if (e != hipSuccess) return e;
+    if (e != hipSuccess) return join(e);
     if constexpr (D <= 64) {
         // both K-side accumulators fit: S, G, dS and P once per block
-        hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DKV, false>), dim3(lk.grid), dim3(256), 0, stream, a, wsk);
-        return hipGetLastError();
+        hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DKV, false>), dim3(lk.grid), dim3(256), 0, sk, a, wsk);
+        return join(hipGetLastError());
     }
-    hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DK, false>), dim3(lk.grid), dim3(256), 0, stream, a, wsk);
+    hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DK, false>), dim3(lk.grid), dim3(256), 0, sk, a, wsk);
     e = hipGetLastError();
-    if (e != hipSuccess) return e;
+    if (e != hipSuccess) return join(e);
     if (D == 128 && shared && reversed_forward_supported(a.f.p)) {
         // plain causal self-attention: dV[j] = sum over i >= j of P[i][j] dO[i] is the forward with K as q, Q as k and
         // dO as v on rows taken in reverse order, and the forward's kernel for this head dim (direct copies into LDS,
         // 32-row tiles, three workgroups per CU) is the faster one
         KArgs r = a.f;
         r.p.q = a.f.p.k; r.p.k = a.f.p.q; r.p.v = a.grad_out; r.p.out = a.grad_v;
-        return launch_reversed_forward(r, wsq, stream);
+        return join(launch_reversed_forward(r, wsq, sv));
     }
-    hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DV, false>), dim3(lk.grid), dim3(256), 0, stream, a, wsk);
-    return hipGetLastError();
+    hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DV, false>), dim3(lk.grid), dim3(256), 0, sv, a, wsk);
+    return join(hipGetLastError());
 }
 
 hipError_t launch_backward_mfma(const BArgs& a, void* workspace, hipStream_t stream) {

@@ -12,9 +12,13 @@ from tests.test_parity_gpu import say
 pytestmark = pytest.mark.gpu
 
 
-def test_forward_and_backward_replayed_from_a_graph():
-    say("graph capture of forward + backward")
-    cfg = W.jagged_config(3, 6, 4, 128, 100, 700, torch.bfloat16, max_seq_len=700)
+@pytest.mark.parametrize("batch,heads,lo,hi", [(6, 4, 100, 700), (32, 8, 1200, 2048)])
+def test_forward_and_backward_replayed_from_a_graph(batch, heads, lo, hi):
+    """The second geometry has more than 3000 items per backward kernel: the library then launches its dQ and K-side kernels
+    on three streams forked from and joined to the caller's by events, which the capture must turn into edges of the graph;
+    that case is also compared with the plain kernels, which run on the caller's stream alone."""
+    say("graph capture of forward + backward", batch, heads, lo, hi)
+    cfg = W.jagged_config(3, batch, heads, 128, lo, hi, torch.bfloat16, max_seq_len=hi)
     dev = W.to_device(cfg)
     q, k, v = dev["q"], dev["k"], dev["v"]
     grad = torch.randn_like(q)
@@ -38,7 +42,20 @@ def test_forward_and_backward_replayed_from_a_graph():
         torch.cuda.synchronize()
         return [t.clone() for t in (out, dq, dk, dv)]
 
-    eager()   # everything the first call sets up lazily happens outside the capture
+    first = eager()   # everything the first call sets up lazily happens outside the capture
+    if batch * heads > 64:
+        # the same gradients from the plain fp32-FMA kernels (one stream), to the tolerance of two 16-bit implementations
+        bwd.fwd.flags |= _capi.FLAG_FORCE_GENERIC
+        ng = C.c_uint64(0)
+        assert L.hstu_hip_jagged_backward_get_workspace_size(C.byref(bwd), C.byref(ng)) == 0
+        wsg = torch.empty(max(ng.value, 16), dtype=torch.uint8, device="cuda")
+        s0 = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+        assert L.hstu_hip_jagged_backward(C.byref(bwd), wsg.data_ptr(), ng.value, s0) == 0, L.hstu_hip_last_error()
+        torch.cuda.synchronize()
+        for name, got, ref in zip(("dq", "dk", "dv"), first[1:], (dq, dk, dv)):
+            scale = float(ref.float().abs().max())
+            assert float((got.float() - ref.float()).abs().max()) <= 2e-2 * scale, name
+        bwd.fwd.flags &= ~_capi.FLAG_FORCE_GENERIC
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
         step(torch.cuda.current_stream())
