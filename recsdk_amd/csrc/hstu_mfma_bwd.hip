@@ -611,9 +611,13 @@ struct BwdFork {
     hipEvent_t ev[3];
     bool ok;
 };
+static std::mutex& bwd_fork_mutex() {
+    static std::mutex mu;
+    return mu;
+}
 static BwdFork* bwd_fork() {
     constexpr int MAXDEV = 64;
-    static std::mutex mu;
+    std::mutex& mu = bwd_fork_mutex();
     static BwdFork forks[MAXDEV];
     static bool tried[MAXDEV];
     int dev = -1;
@@ -649,6 +653,10 @@ static hipError_t launch_bwd_td(const BArgs& a, unsigned* ws, hipStream_t stream
     // the events cost: at 3840 items per kernel (B = 32, h = 8, S = 2048) -2 .. -7 %, at 1440 (the headline batch) +2 %
     BwdFork* fk = lq.grid >= 3000 ? bwd_fork() : nullptr;
     hipStream_t sk = stream, sv = stream;
+    // the events and side streams of a device are shared by all callers: from the first record to the last wait of this call
+    // no other host thread may record them (the calls below only enqueue work, so the lock is held for microseconds)
+    std::unique_lock<std::mutex> fork_lock(bwd_fork_mutex(), std::defer_lock);
+    if (fk) fork_lock.lock();
     if (fk) {
         if (hipEventRecord(fk->ev[0], stream) == hipSuccess && hipStreamWaitEvent(fk->side[0], fk->ev[0], 0) == hipSuccess &&
             hipStreamWaitEvent(fk->side[1], fk->ev[0], 0) == hipSuccess) {

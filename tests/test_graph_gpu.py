@@ -71,3 +71,48 @@ def test_forward_and_backward_replayed_from_a_graph(batch, heads, lo, hi):
         torch.cuda.synchronize()
         for name, got, ref in zip(("out", "dq", "dk", "dv"), (out, dq, dk, dv), want):
             assert torch.equal(got, ref), f"replay {replay}: {name} differs from the eager call"
+
+
+def test_large_backward_from_two_host_threads_on_two_streams():
+    """The streams and events that a large backward forks onto are shared by all callers of a device: two host threads that
+    call at the same time on streams of their own must each get what they get alone, bit for bit."""
+    import threading
+    say("large backward from two host threads")
+    L = _capi.lib()
+    jobs = []
+    for seed in (11, 12):
+        cfg = W.jagged_config(seed, 32, 8, 128, 1200, 2048, torch.bfloat16, max_seq_len=2048)
+        dev = W.to_device(cfg)
+        q, k, v = dev["q"], dev["k"], dev["v"]
+        grad = torch.randn_like(q)
+        out, dq, dk, dv = (torch.empty_like(q) for _ in range(4))
+        fwd, keep = _capi.make_params(q, k, v, out, seq_offset_q=dev["seq_offset"], max_seq_len_q=cfg["max_seq_len"], alpha=cfg["alpha"])
+        bwd = _capi.make_backward_params(fwd, grad, dq, dk, dv, None)
+        nb = C.c_uint64(0)
+        assert L.hstu_hip_jagged_backward_get_workspace_size(C.byref(bwd), C.byref(nb)) == 0
+        ws = torch.empty(max(nb.value, 16), dtype=torch.uint8, device="cuda")
+        jobs.append(dict(bwd=bwd, nb=nb.value, ws=ws, outs=(dq, dk, dv), keep=(dev, keep, grad, out), stream=torch.cuda.Stream()))
+    torch.cuda.synchronize()
+
+    def run(job, times):
+        s = C.c_void_p(job["stream"].cuda_stream)
+        for _ in range(times):
+            assert L.hstu_hip_jagged_backward(C.byref(job["bwd"]), job["ws"].data_ptr(), job["nb"], s) == 0, L.hstu_hip_last_error()
+
+    want = []
+    for job in jobs:   # alone
+        run(job, 1)
+        torch.cuda.synchronize()
+        want.append([t.clone() for t in job["outs"]])
+        for t in job["outs"]:
+            t.fill_(float("nan"))
+    torch.cuda.synchronize()
+    threads = [threading.Thread(target=run, args=(job, 6)) for job in jobs]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    for job, ref in zip(jobs, want):
+        for name, got, r in zip(("dq", "dk", "dv"), job["outs"], ref):
+            assert torch.equal(got, r), name
