@@ -606,24 +606,19 @@ uint64_t mfma_backward_workspace_bytes(const BArgs& a) {
 // empty.  To the caller the call still is one piece of work on its stream (also under stream capture, where the events
 // become edges of the graph).  Streams of default priority, events without timing, created on the first call on a device;
 // if that fails everything runs on the caller's stream.
-struct BwdFork {
-    hipStream_t side[2];
-    hipEvent_t ev[3];
-    bool ok;
-};
-static std::mutex& bwd_fork_mutex() {
+std::mutex& side_streams_mutex() {
     static std::mutex mu;
     return mu;
 }
-static BwdFork* bwd_fork() {
+SideStreams* side_streams() {
     constexpr int MAXDEV = 64;
-    std::mutex& mu = bwd_fork_mutex();
-    static BwdFork forks[MAXDEV];
+    std::mutex& mu = side_streams_mutex();
+    static SideStreams forks[MAXDEV];
     static bool tried[MAXDEV];
     int dev = -1;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAXDEV) return nullptr;
     std::lock_guard<std::mutex> lock(mu);
-    BwdFork& f = forks[dev];
+    SideStreams& f = forks[dev];
     if (!tried[dev]) {
         tried[dev] = true;
         const char* serial = getenv("HSTU_HIP_SERIAL_BACKWARD");   // read once per device: "1" keeps the backward on the caller's stream
@@ -651,11 +646,11 @@ static hipError_t launch_bwd_td(const BArgs& a, unsigned* ws, hipStream_t stream
     }
     // fork: the K-side kernels wait for the work lists only.  Worth it when the kernels are long against the few microseconds
     // the events cost: at 3840 items per kernel (B = 32, h = 8, S = 2048) -2 .. -7 %, at 1440 (the headline batch) +2 %
-    BwdFork* fk = lq.grid >= 3000 ? bwd_fork() : nullptr;
+    SideStreams* fk = lq.grid >= 3000 ? side_streams() : nullptr;
     hipStream_t sk = stream, sv = stream;
     // the events and side streams of a device are shared by all callers: from the first record to the last wait of this call
     // no other host thread may record them (the calls below only enqueue work, so the lock is held for microseconds)
-    std::unique_lock<std::mutex> fork_lock(bwd_fork_mutex(), std::defer_lock);
+    std::unique_lock<std::mutex> fork_lock(side_streams_mutex(), std::defer_lock);
     if (fk) fork_lock.lock();
     if (fk) {
         if (hipEventRecord(fk->ev[0], stream) == hipSuccess && hipStreamWaitEvent(fk->side[0], fk->ev[0], 0) == hipSuccess &&
