@@ -30,7 +30,7 @@ TRAFFIC_SOURCE = {"config2": "profiles/hstu_mfma_kernel_configs2-5.md", "config2
                   "in_linear_silu": "profiles/hstu_in_linear_silu_kernel.md", "in_linear_silu_bwd": "profiles/hstu_in_linear_silu_backward_kernels.md",
                   "kv_append_fp8": "profiles/hstu_kv_append_fp8_kernels.md"}
 MEASURED_TRAFFIC_BYTES = {"config2": 184.5e6, "config2_fp8": 116.5e6, "ref_bias": 1553.7e6, "kv_append": 351.9e6, "rab_time": 1443.4e6, "rab_time_bwd": 1589.7e6, "rab_pos": 297.7e6,
-                          "nmd_fwd": 826.4e6, "nmd_bwd": 1380.0e6, "in_linear_silu": 1092.8e6, "in_linear_silu_bwd": 2405.4e6, "kv_append_fp8": 268.4e6}
+                          "nmd_fwd": 826.4e6, "nmd_bwd": 1380.0e6, "in_linear_silu": 1092.8e6, "in_linear_silu_bwd": 1458.3e6, "kv_append_fp8": 268.4e6}
 
 
 def build_workload(name, torch, W):
@@ -656,8 +656,8 @@ def in_linear_silu_bwd_bench(args, torch):
         "dtype": "bf16", "data": "synthetic", "us_per_call": round(ms * 1e3, 2), "tflops": round(flops / (ms * 1e-3) / 1e12, 1),
         "config": {"workload": "in_linear_silu_bwd: x [16384, 64], W [16384, 64], gradients 4 x [16384, 4096], linear_output [16384, 16384] bf16, seed 13",
                    "algorithmic_bytes_per_call": alg, "flops_per_call": flops, "workspace_bytes": need.value,
-                   "entry": "hstu_hip_in_linear_silu_backward (include/hstu_layer.h): two operand packs, hstu_ilb_xgrad_kernel, hstu_ilb_wgrad_kernel, three reductions"},
-        "roofline": {"bound": "hbm", "kernel": "hstu_ilb_xgrad_kernel + hstu_ilb_wgrad_kernel (+ 4 small kernels; all inside the events)",
+                   "entry": "hstu_hip_in_linear_silu_backward (include/hstu_layer.h): two operand packs, hstu_ilb_wgrad_kernel (one pass: weight_grad, bias_grad and x_grad slabs), three reductions"},
+        "roofline": {"bound": "hbm", "kernel": "hstu_ilb_wgrad_kernel, one pass (+ 5 small kernels; all inside the events)",
                      "achieved": round(alg / (kern_ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS,
                      "unit": "GB/s", "frac": round(alg / (kern_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
                      "kernel_us": round(kern_ms * 1e3, 2)},

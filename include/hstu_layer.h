@@ -118,10 +118,10 @@ typedef struct hstu_in_linear_silu_bwd_params {
     int32_t n;
     int32_t split[4];
     int32_t grad_dtype;       /* HSTU_F32 or dtype */
-    int32_t algorithm;        /* 0: the library chooses (today: 1); 1: two product kernels that each stream the inputs;
-                                 2: one pass over the inputs, k <= 64 only: x_grad as fp32 partial slabs per 256
-                                 columns of n in the workspace (ceil(n / 256) * m * k * 4 bytes); half the HBM traffic,
-                                 measured no faster */
+    int32_t algorithm;        /* 0: the library chooses (today: 2 for k <= 64, else 1); 1: two product kernels that each
+                                 stream the inputs; 2: one pass over the inputs, k <= 64 only: x_grad as fp32 partial slabs
+                                 per 512 columns of n in the workspace (ceil(n / 512) * m * k * 4 bytes); half the HBM
+                                 traffic, a third less time at m = n = 16384 */
     const void* x;            /* [m, k] */
     const void* weight;       /* [n, k] */
     const void* grad[4];      /* user_grad [m, split[0]], value_grad, query_grad, key_grad */

@@ -8,16 +8,20 @@
 // cust_op/ascendc_op/ai_core_op/in_linear_silu_backward/v220/op_kernel/in_linear_silu_backward.h:267-332).
 //
 // n is at least 4 k, so both products are skinny: every element of dlin meets only k multiply-adds per product and the
-// op is bounded by reading grad and linear_output from HBM.  dlin is therefore never written to memory: each of the two
-// product kernels streams grad and linear_output once and rebuilds dlin in registers.
-//   * hstu_ilb_xgrad_kernel: a workgroup owns 32 rows m; its four waves take every fourth 64-column piece of n, build
-//     dlin in the layout the loads arrive in (eight lanes = 128 contiguous bytes of one row), park it in LDS, read it
-//     back as an MFMA operand (a lane = one row, 8 consecutive n: one 16-byte read) and multiply by rows of W^T; the
-//     four partial results meet in LDS.
-//   * hstu_ilb_wgrad_kernel: a wave owns 64 columns n and walks down m in tiles of 32 rows; dlin is built in the layout
-//     the loads arrive in (a lane = 8 consecutive n of one row), parked in LDS and read back transposed (a lane = one
-//     column n, 8 consecutive m) against rows of x^T.  m is cut into S ranges to fill the chip; the S partial results
-//     are added in a fixed order by hstu_ilb_reduce_kernel, so the result is reproducible.
+// op is bounded by reading grad and linear_output from HBM.  dlin is therefore never written to memory: it is rebuilt in
+// registers from grad and linear_output.
+//   * k <= 64 (the library's choice there): ONE pass over the inputs.  hstu_ilb_wgrad_kernel<.., FUSED, 8 waves>: a wave
+//     owns 64 columns n and walks down a range of m in tiles of 32 rows; dlin is built in the layout the loads arrive in
+//     (a lane = 8 consecutive n of one row), parked in LDS and read back transposed (a lane = one column n, 8 consecutive
+//     m) against rows of x^T for weight_grad, and row-wise against the wave's 64 rows of W (held in registers) for the
+//     tile's x_grad; the eight waves' x_grad pieces meet in LDS and leave as the workgroup's partial slab (one slab per
+//     512 columns of n).  The partial sums over the ranges of m (weight_grad, bias_grad) and over the slabs (x_grad) are
+//     added in a fixed order by hstu_ilb_reduce_kernel, so the result is reproducible.
+//   * k > 64, or on request: two product kernels that each stream the inputs once.
+//     hstu_ilb_xgrad_kernel: a workgroup owns 32 rows m; its four waves take every fourth 64-column piece of n, build
+//     dlin, park it in LDS, read it back as an MFMA operand (a lane = one row, 8 consecutive n: one 16-byte read) and
+//     multiply by rows of W^T; the four partial results meet in LDS.
+//     hstu_ilb_wgrad_kernel<.., not FUSED>: the weight_grad half of the one-pass kernel, four waves per workgroup.
 // Both products want their small operand with the summed index contiguous per lane: W^T and x^T are written to the
 // workspace first, already cut into MFMA operand fragments (hstu_ilb_pack_kernel: one fragment = 32 columns k x 16
 // summed indices = 1 KiB that a wave loads with one fully contiguous instruction; together at most half of what grad
@@ -43,6 +47,7 @@ template <> struct IlbMM<_Float16> {
 };
 
 constexpr int ILB_NT = 256;
+constexpr int ILB_FUSED_NW = 8, ILB_FUSED_COLS = 64 * ILB_FUSED_NW;   // the one-pass variant: waves per workgroup, columns of n per workgroup and slab
 constexpr int ILB_PARK = 64 * 2 + 16;   // bytes of one parked row of 64 columns: 8 rows further down is 32 banks away
 
 struct IlbArgs {
@@ -222,22 +227,25 @@ __global__ __launch_bounds__(ILB_NT) void hstu_ilb_xgrad_kernel(const IlbArgs a)
     }
 }
 
-// weight_grad and bias_grad partial sums.  grid = (ceil(n / 256), ceil(k / KC), S), 4 waves of 64 columns n each.
-// FUSED (k <= 64 only, on request: it halves the HBM traffic but measured no faster, the two workgroup barriers per
-// tile and 171 registers cost what the second pass over the inputs costs): the parked tile is also multiplied by the wave's 64 rows of W, which stay in registers; the
-// four waves' products meet in LDS and leave as this workgroup's partial x_grad of the tile (one slab per 256 columns
-// of n, added up by hstu_ilb_reduce_kernel), so that the gradients and linear_output are streamed once instead of twice.
-template <typename T, int KC, bool FUSED>
-__global__ __launch_bounds__(ILB_NT) void hstu_ilb_wgrad_kernel(const IlbArgs a) {
+// weight_grad and bias_grad partial sums.  grid = (ceil(n / (64 NW)), ceil(k / KC), S), NW waves of 64 columns n each.
+// FUSED (k <= 64): the parked tile is also multiplied by the wave's 64 rows of W, which stay in registers; the waves'
+// products meet in LDS and leave as this workgroup's partial x_grad of the tile (one slab per 64 NW columns of n, added up
+// by hstu_ilb_reduce_kernel), so that the gradients and linear_output are streamed once instead of twice.  With four
+// waves (64 slabs of 256 columns: as much partial-sum traffic again as half the inputs, two workgroup barriers per 16 KB
+// of input) it measured no faster than the two product kernels (458 us at m = n = 16384); with eight waves (32 slabs,
+// half the barriers per byte) and one workgroup per CU it takes 292 us.
+template <typename T, int KC, bool FUSED, int NW = 4>
+__global__ __launch_bounds__(64 * NW) void hstu_ilb_wgrad_kernel(const IlbArgs a) {
     typedef typename IlbMM<T>::v8 v8;
     constexpr int KB = KC / 32;
-    __shared__ __attribute__((aligned(16))) char park_all[(ILB_NT / 64) * 32 * ILB_PARK];
-    __shared__ float red[FUSED ? 4 : 1][FUSED ? 32 : 1][KC + 1];
+    constexpr int NT = 64 * NW;   // NW waves of 64 columns each
+    __shared__ __attribute__((aligned(16))) char park_all[NW * 32 * ILB_PARK];
+    __shared__ float red[FUSED ? NW : 1][FUSED ? 32 : 1][KC + 1];
     const hstu_in_linear_silu_bwd_params& p = a.p;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int g = lane >> 5, l32 = lane & 31;
     const int N = p.n, K = p.k;
-    const int nw = blockIdx.x * 256 + 64 * w;     // first column of this wave
+    const int nw = blockIdx.x * NT + 64 * w;      // first column of this wave
     const bool wave_on = nw < N;
     if (!FUSED && !wave_on) return;               // whole wave; without FUSED nothing below synchronises across waves
     const int k0 = blockIdx.y * KC;
@@ -349,9 +357,12 @@ __global__ __launch_bounds__(ILB_NT) void hstu_ilb_wgrad_kernel(const IlbArgs a)
                 for (int r = 0; r < 16; r++) red[w][l32][32 * kb + 8 * (r / 4) + 4 * g + (r % 4)] = ax[kb][r];
             __syncthreads();
             float* xp = a.xpart + ((int64_t)blockIdx.x * p.m + m0) * K;
-            for (int i = threadIdx.x; i < 32 * KC; i += ILB_NT) {
+            for (int i = threadIdx.x; i < 32 * KC; i += NT) {
                 const int r = i / KC, c = i % KC;
-                if (m0 + r < mend && c < K) xp[(int64_t)r * K + c] = ((red[0][r][c] + red[1][r][c]) + red[2][r][c]) + red[3][r][c];
+                float sum = red[0][r][c];
+#pragma unroll
+                for (int ww = 1; ww < NW; ww++) sum += red[ww][r][c];   // in the order of the waves: reproducible
+                if (m0 + r < mend && c < K) xp[(int64_t)r * K + c] = sum;
             }
             __syncthreads();
         }
@@ -422,8 +433,13 @@ static IlbPlan ilb_plan(const hstu_in_linear_silu_bwd_params* p) {
     IlbPlan pl;
     pl.kc = p->k > 64 ? 128 : 64;
     const int64_t tiles = (p->m + 31) / 32;
-    const int64_t blocks = (int64_t)((p->n + 255) / 256) * ((p->k + pl.kc - 1) / pl.kc);
-    int64_t parts = (1024 + blocks - 1) / blocks;
+    // one pass over the inputs (k <= 64): the library's choice unless the caller asks for the two product kernels
+    pl.fused = p->algorithm == 2 || (p->algorithm == 0 && p->k <= 64);
+    // ranges of m: about 1024 workgroups for the two product kernels; the one-pass kernel holds one workgroup of 8 waves per
+    // CU, and one round of them (256) measured fastest: 292 us at m = n = 16384 against 310 / 353 us with 512 / 1024
+    const int64_t blocks = pl.fused ? (int64_t)((p->n + ILB_FUSED_COLS - 1) / ILB_FUSED_COLS)
+                                    : (int64_t)((p->n + 255) / 256) * ((p->k + pl.kc - 1) / pl.kc);
+    int64_t parts = ((pl.fused ? 256 : 1024) + blocks - 1) / blocks;
     if (parts > tiles) parts = tiles;
     if (parts < 1) parts = 1;
     pl.rows_per_part = ((tiles + parts - 1) / parts) * 32;
@@ -447,12 +463,10 @@ static IlbPlan ilb_plan(const hstu_in_linear_silu_bwd_params* p) {
     if (nparts < 1) nparts = 1;
     pl.cols_per_part = (int)((rounds + nparts - 1) / nparts) * 256;
     pl.nparts = (p->n + pl.cols_per_part - 1) / pl.cols_per_part;
-    // on request (k <= 64): one pass over the inputs, x_grad as one partial slab per 256 columns of n
-    const uint64_t slabs = (uint64_t)rounds;
-    pl.fused = p->algorithm == 2;
+    // one pass over the inputs: x_grad as one partial slab per 512 columns of n
     if (pl.fused) {
-        pl.nparts = (int)slabs;
-        pl.cols_per_part = 256;
+        pl.nparts = (int)((p->n + ILB_FUSED_COLS - 1) / ILB_FUSED_COLS);
+        pl.cols_per_part = ILB_FUSED_COLS;
     }
     pl.off_xpart = o;
     if (pl.nparts > 1 || pl.fused) o = ilb_align(o + (uint64_t)pl.nparts * p->m * p->k * 4);
@@ -506,7 +520,8 @@ static void ilb_launch(const IlbArgs& a, const IlbPlan& pl, hipStream_t st) {
     const unsigned kchunks = (unsigned)((p.k + pl.kc - 1) / pl.kc);
     const dim3 gx((unsigned)(pl.mpad / 32), kchunks, (unsigned)pl.nparts), gw((unsigned)((p.n + 255) / 256), kchunks, (unsigned)pl.parts);
     if (pl.fused) {
-        hipLaunchKernelGGL((hstu_ilb_wgrad_kernel<T, 64, true>), gw, dim3(ILB_NT), 0, st, a);
+        const dim3 gf((unsigned)((p.n + ILB_FUSED_COLS - 1) / ILB_FUSED_COLS), kchunks, (unsigned)pl.parts);
+        hipLaunchKernelGGL((hstu_ilb_wgrad_kernel<T, 64, true, ILB_FUSED_NW>), gf, dim3(64 * ILB_FUSED_NW), 0, st, a);
     } else if (pl.kc == 64) {
         hipLaunchKernelGGL((hstu_ilb_xgrad_kernel<T, 64>), gx, dim3(ILB_NT), 0, st, a);
         hipLaunchKernelGGL((hstu_ilb_wgrad_kernel<T, 64, false>), gw, dim3(ILB_NT), 0, st, a);

@@ -136,14 +136,20 @@ def test_in_linear_silu_backward_validation_and_workspace():
     assert L.hstu_hip_in_linear_silu_backward_get_workspace_size(C.byref(p), C.byref(need)) == 0
     parts = 4
     al = lambda v: (v + 255) // 256 * 256
+    # (the library's choice at k <= 64 is the one-pass kernel: its x_grad leaves as one partial slab per 512 columns of n)
+    assert need.value == al(128 // 16 * 1024) + al(64 // 16 * 1024) + al(parts * 64 * 16 * 4) + al(parts * 64 * 4) + al(1 * 100 * 16 * 4)
+    p.algorithm = 1
+    assert L.hstu_hip_in_linear_silu_backward_get_workspace_size(C.byref(p), C.byref(need)) == 0
     assert need.value == al(128 // 16 * 1024) + al(64 // 16 * 1024) + al(parts * 64 * 16 * 4) + al(parts * 64 * 4)
-    big = mk(m=16384, k=64, n=16384, split=[4096] * 4)
+    big = mk(m=16384, k=64, n=16384, split=[4096] * 4, algorithm=1)
     assert L.hstu_hip_in_linear_silu_backward_get_workspace_size(C.byref(big), C.byref(need)) == 0
-    # 16 ranges of m for weight_grad; x_grad: 2 ranges of n with the two product kernels, 64 slabs in one pass
+    # the two product kernels: 16 ranges of m for weight_grad, 2 ranges of n for x_grad
     assert need.value == al(64 * 16384 * 2) * 2 + al(16 * 16384 * 64 * 4) + al(16 * 16384 * 4) + al(2 * 16384 * 64 * 4)
-    big.algorithm = 2
-    assert L.hstu_hip_in_linear_silu_backward_get_workspace_size(C.byref(big), C.byref(need)) == 0
-    assert need.value == al(64 * 16384 * 2) * 2 + al(16 * 16384 * 64 * 4) + al(16 * 16384 * 4) + al(64 * 16384 * 64 * 4)
+    for algorithm in (0, 2):
+        # one pass: 8 ranges of m (one workgroup per CU), 32 slabs of x_grad
+        big.algorithm = algorithm
+        assert L.hstu_hip_in_linear_silu_backward_get_workspace_size(C.byref(big), C.byref(need)) == 0
+        assert need.value == al(64 * 16384 * 2) * 2 + al(8 * 16384 * 64 * 4) + al(8 * 16384 * 4) + al(32 * 16384 * 64 * 4)
     m = torch.ops.mxrec
     assert str(m.in_linear_silu.default._schema) == "mxrec::in_linear_silu(Tensor x, Tensor weight, Tensor bias, int[] attr_dict) -> Tensor[]"
     assert str(m.in_linear_silu_backward.default._schema) == ("mxrec::in_linear_silu_backward(Tensor x, Tensor weight, Tensor? bias, Tensor user_grad, "
