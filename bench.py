@@ -82,7 +82,7 @@ def build_workload(name, torch, W):
 
 def bench_kind(workload):
     """Which leg of this file measures a workload (the names of several legs end alike)."""
-    if workload in ("copy", "rates", "kv_append", "kv_append_fp8", "in_linear_silu", "in_linear_silu_bwd"):
+    if workload in ("copy", "kv_append", "kv_append_fp8", "in_linear_silu", "in_linear_silu_bwd"):
         return workload
     if workload in ("rab_time", "rab_time_bwd", "rab_pos"):
         return "bias"
@@ -98,7 +98,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=1000)
-    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "ref_bias", "ref_nobias", "ref_nobias_d32", "ref_nobias_d64", "ref_nobias_d256", "config2_fp8", "ref_nobias_fp8", "config2_bwd", "ref_bias_bwd", "ref_nobias_bwd", "ref_nobias_d32_bwd", "ref_nobias_d64_bwd", "ref_nobias_d256_bwd", "kv_append", "kv_append_fp8", "rab_time", "rab_time_bwd", "rab_pos", "nmd_fwd", "nmd_bwd", "in_linear_silu", "in_linear_silu_bwd", "copy", "rates"],
+    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "ref_bias", "ref_nobias", "ref_nobias_d32", "ref_nobias_d64", "ref_nobias_d256", "config2_fp8", "ref_nobias_fp8", "config2_bwd", "ref_bias_bwd", "ref_nobias_bwd", "ref_nobias_d32_bwd", "ref_nobias_d64_bwd", "ref_nobias_d256_bwd", "kv_append", "kv_append_fp8", "rab_time", "rab_time_bwd", "rab_pos", "nmd_fwd", "nmd_bwd", "in_linear_silu", "in_linear_silu_bwd", "copy"],
                     help="'copy' runs a plain 256 MiB device copy: the known-size kernel the FETCH_SIZE/WRITE_SIZE counters are scaled by")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--settle-ms", type=float, default=80.0,
@@ -116,8 +116,6 @@ def main():
     kind = bench_kind(args.workload)
     if kind == "copy":
         return copy_calibration(args, torch)
-    if kind == "rates":
-        return issue_rates(args, torch, _capi)
     if kind == "attention_backward":
         return backward_bench(args, torch, W, _capi)
     if kind == "kv_append":
@@ -671,55 +669,6 @@ def in_linear_silu_bwd_bench(args, torch):
         out["cpu_baseline"] = {"value": round(alg * rows / m_ / dt / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
                                "sample": f"the first {rows} rows once (oracle in torch, fp64), {dt:.2f} s"}
     print(json.dumps(out), flush=True)
-
-
-def issue_rates(args, torch, _capi):
-    """What the matrix cores and the vector unit of this GPU sustain on the pieces of one 32 x 32 score block, alone and
-    together, at 1-4 waves per SIMD, on zero and on random operands (hstu_hip_measure_block_rates, include/hstu_diag.h).
-    One JSON line; times are per iteration of one wave on its SIMD (all SIMDs of the chip busy), from HIP events."""
-    import ctypes as C
-    L = _capi.lib()
-    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
-    g = torch.Generator(device="cuda").manual_seed(3)
-    rnd = (torch.rand(65536 * 8, generator=g, device="cuda") - 0.5).to(torch.bfloat16)     # 1 MiB
-    # for the fp8 instruction: e4m3 values in (-2, 2)
-    rnd8 = ((torch.rand(65536 * 16, generator=g, device="cuda") - 0.5) * 4).to(torch.float8_e4m3fn)
-    zero = torch.zeros(65536 * 8, device="cuda", dtype=torch.bfloat16)
-    sink = torch.empty(256 * 256 * 4, device="cuda", dtype=torch.float32)
-    ticks = torch.zeros(2 * 1024, device="cuda", dtype=torch.int64)
-    iters = 4000
-    modes = [("silu_x16", 0, (1, 2, 3, 4), 16), ("mfma_x16", 1, (1, 2, 3), 16), ("block", 2, (1, 2, 3), 16),
-             ("pipelined_block", 3, (1, 2), 16), ("mfma_fp8_x4", 4, (1, 2, 3, 4), 4)]
-    rows = []
-    for name, mode, waves_list, units in modes:
-        for data_name in ("zeros", "random"):
-            for waves in waves_list:
-                ops = zero if data_name == "zeros" else (rnd8 if mode == 4 else rnd)
-
-                def run():
-                    if L.hstu_hip_measure_block_rates(mode, waves, iters, ops.data_ptr(), sink.data_ptr(), ticks.data_ptr(), stream) != 0:
-                        raise RuntimeError("hstu_hip_measure_block_rates rejected its arguments")
-                for _ in range(3):
-                    run()
-                torch.cuda.synchronize()
-                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                e0.record()
-                run()
-                e1.record()
-                torch.cuda.synchronize()
-                ms = e0.elapsed_time(e1)
-                t = ticks[: 2 * 256 * waves].view(-1, 2).double().sum(0)
-                ns = ms * 1e6 / (iters * waves)          # per iteration of one wave while `waves` waves share the SIMD
-                # core clocks per tick of the 100 MHz constant clock -> the core clock during the run
-                ghz = float(t[0] / t[1]) * 0.1
-                flops = 16 * 2 * 32 * 32 * 16 if mode != 0 else 0     # per iteration of one wave (fp8: 4 x 32x32x64, the same)
-                rows.append({"piece": name, "operands": data_name, "waves_per_simd": waves, "ns_per_iteration": round(ns, 1),
-                             "core_clock_ghz": round(ghz, 3), "clk_per_unit": round(ns * ghz / units, 1),
-                             "chip_tflops": round(flops * 1024 / ns / 1e3, 1) if flops else None})
-    print(json.dumps({"metric": "issue_rates", "n_gpus": 1, "iterations_per_wave": iters, "unit": "ns per iteration of one wave on its SIMD",
-                      "note": "clk_per_unit = core clocks per SiLU element (silu), per 32x32x16 MFMA (mfma, block, pipelined) or per 32x32x64 fp8 MFMA; "
-                              "core_clock_ghz from s_memtime / s_memrealtime inside the kernel; chip_tflops = MFMA FLOPs of all 1024 SIMDs",
-                      "rows": rows}), flush=True)
 
 
 def copy_calibration(args, torch):

@@ -18,7 +18,7 @@ LIB = os.path.join(HERE, "lib")
 OBJ = os.path.join(HERE, "lib", "obj")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
-HIP_SOURCES = ["hstu_abi.hip", "hstu_generic.hip", "hstu_mfma.hip", "hstu_mfma_fp8.hip", "hstu_backward.hip", "hstu_mfma_bwd.hip", "hstu_kvcache.hip", "hstu_kvcache_fp8.hip", "hstu_bias.hip", "hstu_layer.hip", "hstu_linear.hip", "hstu_linear_bwd.hip", "hstu_rates.hip"]
+HIP_SOURCES = ["hstu_abi.hip", "hstu_generic.hip", "hstu_mfma.hip", "hstu_mfma_fp8.hip", "hstu_backward.hip", "hstu_mfma_bwd.hip", "hstu_kvcache.hip", "hstu_kvcache_fp8.hip", "hstu_bias.hip", "hstu_layer.hip", "hstu_linear.hip", "hstu_linear_bwd.hip"]
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
              # packed fp32 VALU forms are kept out of every kernel in this library
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
@@ -70,7 +70,7 @@ def build_ops(verbose=False):
            "-DUSE_ROCM", "-D__HIP_PLATFORM_AMD__", *inc, "-I", os.path.join(HERE, "..", "include"),
            os.path.join(CSRC, "mxrec_hstu_ops.cpp"), "-o", ops_lib_path(),
            "-L", LIB, "-lhstu_hip", "-Wl,-rpath,$ORIGIN",
-           "-L", tlib, "-ltorch", "-ltorch_cpu", "-lc10", "-ltorch_hip", "-lc10_hip"]
+           "-L", tlib, "-ltorch", "-ltorch_cpu", "-lc10", "-ltorch_hip", "-lc10_hip", "-lamdhip64"]
     out = _run(cmd)
     if verbose and out.strip():
         print(out)

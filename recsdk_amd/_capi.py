@@ -32,7 +32,6 @@ EXPORTS = [
     "hstu_hip_norm_multiply_dropout", "hstu_hip_norm_multiply_dropout_backward",
     "hstu_hip_norm_multiply_dropout_backward_get_workspace_size", "hstu_hip_in_linear_silu",
     "hstu_hip_in_linear_silu_backward", "hstu_hip_in_linear_silu_backward_get_workspace_size",
-    "hstu_hip_measure_block_rates",
 ]
 
 
@@ -181,7 +180,6 @@ def lib() -> C.CDLL:
         _lib.hstu_hip_rab_time_backward.argtypes = [C.POINTER(HstuRabTimeBwdParams), C.c_void_p]
         _lib.hstu_hip_rab_pos.argtypes = [C.c_int32, C.c_int32, C.c_void_p, C.c_void_p, C.POINTER(C.c_int64), C.c_int32, C.c_void_p, C.c_void_p]
         _lib.hstu_hip_kv_token_positions.argtypes = [C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]
-        _lib.hstu_hip_measure_block_rates.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
     return _lib
 
 

@@ -106,6 +106,7 @@ struct ListCacheEntry {
     hstu_fwd_params shape;                  // the scalar fields of the call that built it (pointers zeroed)
     void* stream = nullptr;
     int device = -1;
+    unsigned long long capture = 0;         // id of the stream capture the list was built in (0: built by an eager call)
 };
 
 static hstu_fwd_params scalar_fields(hstu_fwd_params p) {
@@ -117,9 +118,32 @@ static hstu_fwd_params scalar_fields(hstu_fwd_params p) {
     return p;
 }
 
+// Id of the capture `stream` is recording into, 0 when it is not capturing.
+static unsigned long long capture_id_of(hipStream_t stream) {
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    unsigned long long id = 0;
+    if (hipStreamGetCaptureInfo(stream, &status, &id) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    return status == hipStreamCaptureStatusActive ? (id ? id : ~0ull) : 0;
+}
+
+// A list is reused only where it is known to be current when the kernel runs:
+//   * eager calls reuse the list of the last eager call on their (device, stream) -- the tensors' version counters show
+//     in-place writes made through torch (writes that bypass them -- `.data`, a foreign kernel on the raw pointer -- do not);
+//   * a call recorded into a stream capture reuses only a list that was built inside the same capture (its schedule
+//     kernel then precedes it in the graph, so every replay rebuilds the list from the offsets of that replay), and its
+//     workspace is allocated inside the capture, so it belongs to the graph's memory pool; eager calls never see it;
+//   * tensors without a version counter (created under torch.inference_mode()) are not cached at all.
 static void run_abi_cached(const hstu_fwd_params& p0, const at::Tensor& q, const std::vector<at::Tensor>& geo, const char* op) {
     static std::mutex mu;
-    static std::vector<ListCacheEntry> cache;   // a handful of (device, stream) pairs
+    static std::vector<ListCacheEntry> cache;   // a handful of (device, stream) pairs, eager and capturing apart
+    for (const auto& t : geo)
+        if (t.defined() && t.is_inference()) {
+            run_abi(hstu_hip_jagged_forward_get_workspace_size, hstu_hip_jagged_forward, p0, q, op);
+            return;
+        }
     hstu_fwd_params p = p0;
     uint64_t ws_bytes = 0;
     int rc = hstu_hip_jagged_forward_get_workspace_size(&p, &ws_bytes);
@@ -132,6 +156,7 @@ static void run_abi_cached(const hstu_fwd_params& p0, const at::Tensor& q, const
         TORCH_CHECK(rc == HSTU_OK, "mxrec::", op, ": ", hstu_hip_last_error());
         return;
     }
+    const unsigned long long capture = capture_id_of(stream.stream());
     // what the list depends on besides the offsets: every scalar field, and which optional inputs are there
     hstu_fwd_params shape = scalar_fields(p);
     shape.flags = (p.attn_bias ? 1u : 0u) | (p.mask ? 2u : 0u) | (p.pos_table ? 4u : 0u) | (p.ts_table ? 8u : 0u);
@@ -139,8 +164,9 @@ static void run_abi_cached(const hstu_fwd_params& p0, const at::Tensor& q, const
     ListCacheEntry* hit = nullptr;
     ListCacheEntry* slot = nullptr;
     for (auto& e : cache)
-        if (e.device == q.device().index() && e.stream == (void*)stream.stream()) slot = &e;
-    if (slot && slot->ws.defined() && (uint64_t)slot->ws.numel() >= ws_bytes && std::memcmp(&slot->shape, &shape, sizeof(shape)) == 0) {
+        if (e.device == q.device().index() && e.stream == (void*)stream.stream() && (e.capture != 0) == (capture != 0)) slot = &e;
+    if (slot && slot->capture == capture && slot->ws.defined() && (uint64_t)slot->ws.numel() >= ws_bytes &&
+        std::memcmp(&slot->shape, &shape, sizeof(shape)) == 0) {
         bool same = true;
         for (size_t i = 0; i < geo.size(); i++) {
             const at::Tensor& a = slot->geo[i];
@@ -156,10 +182,11 @@ static void run_abi_cached(const hstu_fwd_params& p0, const at::Tensor& q, const
         return;
     }
     if (!slot) {
-        if (cache.size() >= 8) cache.erase(cache.begin());
+        if (cache.size() >= 16) cache.erase(cache.begin());
         cache.emplace_back();
         slot = &cache.back();
     }
+    // (a workspace of an earlier capture that is released here goes back to that graph's pool, which keeps it for the replays)
     slot->ws = at::empty({(int64_t)ws_bytes}, q.options().dtype(at::kByte));
     slot->geo = geo;
     slot->versions.clear();
@@ -167,6 +194,7 @@ static void run_abi_cached(const hstu_fwd_params& p0, const at::Tensor& q, const
     slot->shape = shape;
     slot->stream = (void*)stream.stream();
     slot->device = q.device().index();
+    slot->capture = capture;
     rc = hstu_hip_jagged_forward(&p, slot->ws.data_ptr(), ws_bytes, (void*)stream.stream());
     if (rc != HSTU_OK) slot->ws = at::Tensor();
     TORCH_CHECK(rc == HSTU_OK, "mxrec::", op, ": ", hstu_hip_last_error());

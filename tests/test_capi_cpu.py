@@ -354,15 +354,6 @@ def test_dense_backward_validation():
     assert rc == -3 and "workspace" in _capi.lib().hstu_hip_last_error().decode()
 
 
-def test_rate_diagnostics_reject_bad_arguments():
-    # host checks only: nothing is launched
-    lib = _capi.lib()
-    assert lib.hstu_hip_measure_block_rates(0, 1, 10, None, None, None, None) == -1          # no buffers
-    for mode, waves in [(1, 4), (2, 4), (3, 3), (0, 5), (0, 0), (9, 1)]:
-        assert lib.hstu_hip_measure_block_rates(mode, waves, 10, 0x1000, 0x1000, 0x1000, None) == -1, (mode, waves)
-    assert lib.hstu_hip_measure_block_rates(0, 1, 0, 0x1000, 0x1000, 0x1000, None) == -1      # no iterations
-
-
 def test_bench_routes_every_workload_to_its_own_leg():
     """The workload names of several legs end alike (`*_bwd`): each must reach the leg that measures it."""
     import bench
@@ -370,6 +361,6 @@ def test_bench_routes_every_workload_to_its_own_leg():
             "config2_bwd": "attention_backward", "ref_bias_bwd": "attention_backward", "ref_nobias_d32_bwd": "attention_backward",
             "rab_time": "bias", "rab_time_bwd": "bias", "rab_pos": "bias", "nmd_fwd": "nmd", "nmd_bwd": "nmd",
             "in_linear_silu": "in_linear_silu", "in_linear_silu_bwd": "in_linear_silu_bwd", "kv_append": "kv_append",
-            "kv_append_fp8": "kv_append_fp8", "copy": "copy", "rates": "rates"}
+            "kv_append_fp8": "kv_append_fp8", "copy": "copy"}
     for name, kind in want.items():
         assert bench.bench_kind(name) == kind, name

@@ -116,3 +116,97 @@ def test_large_backward_from_two_host_threads_on_two_streams():
     for job, ref in zip(jobs, want):
         for name, got, r in zip(("dq", "dk", "dv"), job["outs"], ref):
             assert torch.equal(got, r), name
+
+
+def _torch_op(q, k, v, off, max_len, alpha):
+    return torch.ops.mxrec.hstu_jagged(q, k, v, None, None, 0, max_len, 0.0, off, None, None, 0, alpha)
+
+
+def _capi_forward(q, k, v, off, max_len, alpha):
+    """The same call through the C ABI with a workspace of its own (no list reuse)."""
+    out = torch.empty_like(q)
+    L = _capi.lib()
+    fwd, keep = _capi.make_params(q, k, v, out, seq_offset_q=off, max_seq_len_q=max_len, alpha=alpha)
+    n = C.c_uint64(0)
+    assert L.hstu_hip_jagged_forward_get_workspace_size(C.byref(fwd), C.byref(n)) == 0
+    ws = torch.empty(max(n.value, 16), dtype=torch.uint8, device="cuda")
+    s = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    assert L.hstu_hip_jagged_forward(C.byref(fwd), ws.data_ptr(), n.value, s) == 0, L.hstu_hip_last_error()
+    torch.cuda.synchronize()
+    return out
+
+
+def _two_geometries(total, batch, seed):
+    """Two offset vectors of `batch` sequences over the same number of rows."""
+    g = torch.Generator().manual_seed(seed)
+    offs = []
+    for _ in range(2):
+        cuts = torch.sort(torch.randperm(total - 1, generator=g)[: batch - 1] + 1).values
+        offs.append(torch.cat([torch.zeros(1, dtype=torch.int64), cuts, torch.tensor([total])]).to(torch.int32))
+    return offs
+
+
+def test_torch_op_work_list_cache_under_stream_capture():
+    """mxrec::hstu_jagged keeps the work list of its last call per (device, stream).  A capture must not record a call that
+    reuses a list built outside the capture: the replay after the offsets tensor was rewritten in place has to follow the
+    new offsets.  Two layers inside one capture still share one list, and a second graph captured afterwards on the same
+    stream replays correctly by itself."""
+    say("torch op: work-list cache under stream capture")
+    total, batch, heads, d, max_len = 3000, 7, 4, 128, 3000
+    off_a, off_b = (o.cuda() for o in _two_geometries(total, batch, 11))
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    q, k, v = ((torch.randn(total, heads, d, generator=gen, device="cuda") * 0.5).to(torch.bfloat16) for _ in range(3))
+    off = off_a.clone()
+    alpha = d ** -0.5
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):   # eager warm-up on the capture stream: the second call reuses the first one's list
+            warm = _torch_op(q, k, v, off, max_len, alpha)
+    side.synchronize()
+    assert torch.equal(warm, _capi_forward(q, k, v, off_a, max_len, alpha))
+    g1 = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g1, stream=side):
+        out1 = _torch_op(q, k, v, off, max_len, alpha)          # builds its list inside the capture
+        out2 = _torch_op(out1, k, v, off, max_len, alpha)       # second layer: reuses it
+    g2 = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g2, stream=side):
+        out3 = _torch_op(q, k, v, off, max_len, alpha)
+    for name, geometry in (("first", off_a), ("second", off_b), ("first again", off_a)):
+        off.copy_(geometry)
+        want1 = _capi_forward(q, k, v, geometry, max_len, alpha)
+        want2 = _capi_forward(want1, k, v, geometry, max_len, alpha)
+        for t in (out1, out2, out3):
+            t.fill_(float("nan"))
+        g1.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out1, want1), f"{name} geometry: layer 1 of the replay differs from the eager call"
+        assert torch.equal(out2, want2), f"{name} geometry: layer 2 of the replay differs from the eager call"
+        # an eager call on the capture stream in between must neither use nor disturb the graphs' lists
+        with torch.cuda.stream(side):
+            eager = _torch_op(q, k, v, off, max_len, alpha)
+        side.synchronize()
+        assert torch.equal(eager, want1), f"{name} geometry: eager call after the capture"
+        g2.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out3, want1), f"{name} geometry: the second graph alone"
+
+
+def test_torch_op_under_inference_mode():
+    """Tensors created under torch.inference_mode() have no version counter: the op must run (without list reuse) and
+    follow an in-place change of the offsets."""
+    say("torch op under inference_mode")
+    total, batch, heads, d, max_len = 2500, 5, 2, 128, 2500
+    with torch.inference_mode():
+        off_a, off_b = (o.cuda() for o in _two_geometries(total, batch, 5))
+        gen = torch.Generator(device="cuda").manual_seed(9)
+        q, k, v = ((torch.randn(total, heads, d, generator=gen, device="cuda") * 0.5).to(torch.bfloat16) for _ in range(3))
+        off = off_a.clone()
+        assert off.is_inference()
+        got = [_torch_op(q, k, v, off, max_len, d ** -0.5) for _ in range(2)]
+        off.copy_(off_b)
+        got.append(_torch_op(q, k, v, off, max_len, d ** -0.5))
+        torch.cuda.synchronize()
+        want_a = _capi_forward(q, k, v, off_a, max_len, d ** -0.5)
+        want_b = _capi_forward(q, k, v, off_b, max_len, d ** -0.5)
+    assert torch.equal(got[0], want_a) and torch.equal(got[1], want_a) and torch.equal(got[2], want_b)
