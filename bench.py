@@ -101,6 +101,10 @@ def main():
     ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "ref_bias", "ref_nobias", "ref_nobias_d32", "ref_nobias_d64", "ref_nobias_d256", "config2_fp8", "ref_nobias_fp8", "config2_bwd", "ref_bias_bwd", "ref_nobias_bwd", "ref_nobias_d32_bwd", "ref_nobias_d64_bwd", "ref_nobias_d256_bwd", "kv_append", "kv_append_fp8", "rab_time", "rab_time_bwd", "rab_pos", "nmd_fwd", "nmd_bwd", "in_linear_silu", "in_linear_silu_bwd", "copy"],
                     help="'copy' runs a plain 256 MiB device copy: the known-size kernel the FETCH_SIZE/WRITE_SIZE counters are scaled by")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--timeline", action="store_true",
+                    help="forward workloads: instead of timing the call, run it on the diagnostics flavour of the library "
+                         "(lib/libhstu_hip_timeline.so, built by recsdk_amd/_build.py) and print where the workgroups of the main "
+                         "kernel spend their time, from the stamps they leave")
     ap.add_argument("--settle-ms", type=float, default=80.0,
                     help="untimed calls before the warm-up until the GPU has been busy this long: its clocks need about 50 ms of load to "
                          "settle (reported as clock_settle; 0 switches it off)")
@@ -165,6 +169,8 @@ def main():
         if rc != 0:
             raise RuntimeError(L.hstu_hip_last_error().decode())
 
+    if args.timeline:
+        return item_timeline(args, torch, _capi, op, params, ws, nws.value, desc, kernel)
     settle = settle_clocks(step, args.settle_ms, torch)
     for _ in range(args.warmup):
         step()
@@ -215,6 +221,93 @@ def main():
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(cfg, op, flops, torch, args.workload, W)
     print(json.dumps(result), flush=True)
+
+
+def item_timeline(args, torch, _capi, op, params, ws, ws_bytes, desc, kernel):
+    """Per-workgroup timeline of the main forward kernel.  The diagnostics library is the product's sources with the
+    kernel compiled under -DHSTU_ITEM_TIMING: thread 0 of every workgroup stamps (constant 100 MHz clock) its start, the
+    moment it knows its item, its first K/V tile in LDS, the end of its last K loop and its end.  One JSON line per
+    flavour of the call: as the C ABI runs it, and with the work list reused (HSTU_FLAG_REUSE_WORKSPACE)."""
+    import ctypes as C
+    import numpy as np
+    from recsdk_amd import _build
+    path = _build.timeline_lib_path()
+    if not os.path.exists(path):
+        raise SystemExit(f"{path} is missing: build it with `python recsdk_amd/_build.py timeline`")
+    # a second copy of the library in this process: its own symbols first, none of them exported to later loads
+    TL = C.CDLL(path, mode=os.RTLD_LOCAL | os.RTLD_DEEPBIND)
+    fn = getattr(TL, f"hstu_hip_{op}_forward")
+    fn.argtypes = [C.POINTER(_capi.HstuFwdParams), C.c_void_p, C.c_uint64, C.c_void_p]
+    TL.hstu_hip_timeline_read.argtypes = [C.c_void_p, C.c_size_t]
+    TL.hstu_hip_last_error.restype = C.c_char_p
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for reuse in (False, True):
+        if reuse:
+            params.flags |= _capi.FLAG_REUSE_WORKSPACE
+
+        def step():
+            if fn(C.byref(params), C.c_void_p(ws.data_ptr()), ws_bytes, stream) != 0:
+                raise RuntimeError(TL.hstu_hip_last_error().decode())
+        if not reuse:
+            step()
+        settle_clocks(step, args.settle_ms, torch)
+        for _ in range(max(args.warmup, 50)):
+            step()
+        torch.cuda.synchronize()
+        buf = np.zeros(8 * 32768, dtype=np.uint32)
+        if TL.hstu_hip_timeline_read(buf.ctypes.data_as(C.c_void_p), C.c_size_t(buf.nbytes)) != 0:
+            raise RuntimeError("reading the stamps failed")
+        r = buf.reshape(-1, 8)
+        r = r[r[:, 0] != 0]
+        us = lambda ticks: ticks / 100.0
+        t0 = r[:, 0].astype(np.int64)
+        t0 -= t0.min()
+        pro, dur, ntk = r[:, 1].astype(np.int64), r[:, 2].astype(np.int64), r[:, 4].astype(np.int64)
+        rec, loop = r[:, 6].astype(np.int64), r[:, 7].astype(np.int64)
+        act = r[:, 5] != 0xffffffff
+        end = t0 + dur
+        span = int(end.max())
+        T = span + 1
+        resident, inloop, rate = np.zeros(T + 1), np.zeros(T + 1), np.zeros(T + 1)
+        for s_, p_, l_, n_, d_ in zip(t0[act], pro[act], loop[act], ntk[act], dur[act]):
+            resident[s_:s_ + d_] += 1
+            if l_ > p_:
+                inloop[s_ + p_:s_ + l_] += 1
+                rate[s_ + p_:s_ + l_] += n_ / (l_ - p_)
+        slots = int(resident.max())
+        total = slots * span
+        first = act & (t0 < 100)          # resident from the start: the first round of workgroups
+        later = act & ~first
+        st, en = np.sort(t0[act]), np.sort(end[act])
+        lag = st[slots:] - en[:len(st) - slots] if len(st) > slots else np.zeros(1)
+        step_t = 400
+        longest = np.argsort(-dur * act)[:20]
+        last = np.argsort(-end * act)[:20]
+        row = lambda i: {"start_us": us(t0[i]), "k_tiles": int(ntk[i]), "to_first_tile_us": us(pro[i]), "k_loops_us": us(loop[i] - pro[i]),
+                         "after_loops_us": us(dur[i] - loop[i]), "end_us": us(end[i])}
+        out = {
+            "metric": "hstu_item_timeline", "workload": desc, "kernel": kernel, "work_list_reused": reuse, "n_gpus": 1,
+            "unit": "us (10 ns ticks of the constant clock, thread 0 of every workgroup)",
+            "kernel_span_us": us(span), "workgroups": int(len(r)), "items": int(act.sum()), "slots": slots, "k_tiles": int(ntk[act].sum()),
+            "slot_time_share": {"to_record": round(float(rec[act].sum()) / total, 3), "record_to_first_tile": round(float((pro - rec)[act].sum()) / total, 3),
+                                "k_loops": round(float((loop - pro)[act].sum()) / total, 3), "after_loops": round(float((dur - loop)[act].sum()) / total, 3),
+                                "empty": round(float(total - dur[act].sum()) / total, 3)},
+            "first_round": {"items": int(first.sum()), "to_record_us": round(us(rec[first].mean()), 2), "to_first_tile_us": round(us(pro[first].mean()), 2),
+                            "end_us_min_median_max": [us(x) for x in (end[first].min(), int(np.median(end[first])), end[first].max())] if first.any() else None},
+            "later_items": {"items": int(later.sum()), "to_record_us": round(us(rec[later].mean()), 2) if later.any() else None,
+                            "to_first_tile_us": round(us(pro[later].mean()), 2) if later.any() else None,
+                            "start_us_min_max": [us(t0[later].min()), us(t0[later].max())] if later.any() else None,
+                            "k_tiles_mean": round(float(ntk[later].mean()), 1) if later.any() else None},
+            "us_per_k_tile_in_loop": round(us(float((loop - pro)[act].sum())) / max(int(ntk[act].sum()), 1), 3),
+            "after_loops_us_mean": round(us(float((dur - loop)[act].mean())), 2),
+            "slot_refill_lag_us_mean_p90": [round(us(float(lag.mean())), 2), round(us(float(np.percentile(lag, 90))), 2)],
+            "every_4us": [{"t_us": us(i), "resident": int(resident[i:i + step_t].mean()), "in_k_loop": int(inloop[i:i + step_t].mean()),
+                           "k_tiles_per_us": int(rate[i:i + step_t].mean() * 100)} for i in range(0, T, step_t)],
+            "longest_items": [row(i) for i in longest],
+            "last_ending_items": [row(i) for i in last],
+        }
+        print(json.dumps(out), flush=True)
+    params.flags &= ~_capi.FLAG_REUSE_WORKSPACE
 
 
 def backward_bench(args, torch, W, _capi):

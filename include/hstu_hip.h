@@ -51,7 +51,9 @@ enum { HSTU_MASK_TRIL = 0, HSTU_MASK_TRIU = 1, HSTU_MASK_NONE = 2, HSTU_MASK_CUS
 #define HSTU_FLAG_FORCE_GENERIC 2u /* run the plain fp32-FMA kernel even where an MFMA kernel exists (testing) */
 /* The workspace still holds the work list an earlier call built for the same sequence offsets, num_context,
  * num_target, page offsets, shapes and attributes (e.g. the other layers of one model on one batch): do not
- * rebuild it.  Only q/k/v/out/bias/table contents may differ between such calls. */
+ * rebuild it.  Only q/k/v/out/bias/table contents may differ between such calls.  (Every call without the flag leaves
+ * the list in the workspace, also the calls that need no schedule kernel of their own: plain causal self-attention at head
+ * dim 128 on at most 64 sequences, whose workgroups derive their items from the offsets and write them down as they go.) */
 #define HSTU_FLAG_REUSE_WORKSPACE 4u
 
 /*

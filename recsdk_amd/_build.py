@@ -58,6 +58,23 @@ def build_hip(verbose=False, extra_flags=()):
     return hip_lib_path()
 
 
+def timeline_lib_path():
+    return os.path.join(LIB, "libhstu_hip_timeline.so")
+
+
+def build_timeline(verbose=False):
+    """Diagnostics flavour of the library: the same sources with the main forward kernel compiled under
+    ``-DHSTU_ITEM_TIMING`` (every workgroup stamps its start, first tile, last K loop and end), as a library of its own next
+    to the product's, which stays free of it.  ``bench.py --timeline`` loads it.  Needs the objects of ``build_hip``."""
+    o = os.path.join(OBJ, "hstu_mfma_timeline.o")
+    out = _run([HIPCC, *HIP_FLAGS, "-DHSTU_ITEM_TIMING", "-c", os.path.join(CSRC, "hstu_mfma.hip"), "-o", o])
+    if verbose and out.strip():
+        print(out)
+    objs = [os.path.join(OBJ, s.replace(".hip", ".o")) for s in HIP_SOURCES if s != "hstu_mfma.hip"]
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", timeline_lib_path(), o, *objs])
+    return timeline_lib_path()
+
+
 def build_ops(verbose=False):
     import torch
     from torch.utils import cpp_extension as ce
@@ -79,10 +96,11 @@ def build_ops(verbose=False):
 
 def build_all(verbose=False):
     build_hip(verbose)
+    build_timeline(verbose)
     build_ops(verbose)
 
 
 if __name__ == "__main__":
     what = sys.argv[1] if len(sys.argv) > 1 else "all"
-    {"hip": build_hip, "ops": build_ops, "all": build_all}[what](verbose=True)
+    {"hip": build_hip, "timeline": build_timeline, "ops": build_ops, "all": build_all}[what](verbose=True)
     print("built", what)

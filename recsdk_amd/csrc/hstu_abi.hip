@@ -271,10 +271,9 @@ int hstu_hip_describe_kernel(const hstu_fwd_params* p, char* buf, size_t n) {
     int rc = validate(p, op, &a);
     if (rc != HSTU_OK) return rc;
     const char* name = nullptr;
-    if ((p->flags & HSTU_FLAG_FORCE_GENERIC) || !mfma_supported(a, &name)) {
-        name = p->dtype == HSTU_F32 ? "generic_f32" : (p->dtype == HSTU_F16 ? "generic_f16" : (p->dtype == HSTU_BF16 ? "generic_bf16" : "generic_fp8"));
-    }
-    snprintf(buf, n, "%s", name);
+    const bool mfma = !(p->flags & HSTU_FLAG_FORCE_GENERIC) && mfma_supported(a, &name);
+    if (!mfma) name = p->dtype == HSTU_F32 ? "generic_f32" : (p->dtype == HSTU_F16 ? "generic_f16" : (p->dtype == HSTU_BF16 ? "generic_bf16" : "generic_fp8"));
+    snprintf(buf, n, "%s%s", name, mfma && mfma_self_scheduled(a) ? "_selfsched" : "");
     return HSTU_OK;
 }
 

@@ -32,6 +32,8 @@ bool mfma_supported(const KArgs& a, const char** name);
 // bytes of device workspace the MFMA path needs for its work list; the buffer needs no initialisation
 uint64_t mfma_workspace_bytes(const KArgs& a);
 hipError_t launch_mfma(const KArgs& a, void* workspace, hipStream_t stream);
+// the call runs without a schedule kernel: the workgroups of the main kernel derive their items from the offsets
+bool mfma_self_scheduled(const KArgs& a);
 // the same three for float8_e4m3fn q / k / v (reached through the three above)
 bool mfma_fp8_supported(const KArgs& a, const char** name);
 uint64_t mfma_fp8_workspace_bytes(const KArgs& a);

@@ -392,6 +392,86 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
 }
 
 
+#ifdef HSTU_ITEM_TIMING
+// Diagnostics build only (lib/libhstu_hip_timeline.so; the product library is built without it): every workgroup of the
+// main kernel leaves {start, time to its first K/V tile in LDS, time to its end, hardware id, K tiles, item word, time to
+// its record, time to the end of its last K loop} in 10 ns ticks of the constant clock.
+__device__ unsigned g_item_times[8 * 32768];
+}  // namespace hstu
+extern "C" int hstu_hip_timeline_read(void* dst, size_t bytes) {
+    return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(hstu::g_item_times), bytes);
+}
+namespace hstu {
+#endif
+
+// The record of workgroup blockIdx.x without a work list, computed by one wave (lane b holds sequence b; the caller
+// guarantees batch <= 64, one set of offsets for q and k, no context or target rows, the plain causal mask).  The order is
+// the schedule kernel's with a coarser key: sequences by their number of Q tiles (longest first, then by batch index),
+// (sequence, head) groups r = rank * heads + head dealt to the XCDs in snake order (XCD x owns r = 16 u + x and
+// 16 u + 15 - x), a group's tiles last tile first, the first two tiles of a sequence of five or more tiles as one item.
+// Everything after the offsets have arrived is wave-uniform: one ballot per tile count and scalar arithmetic, so it costs
+// the vector unit (which the other workgroups of the CU keep busy) next to nothing.  No list can exceed the grid: with
+// entries per group falling along r, the lists differ by at most one group's entries.
+__device__ __forceinline__ void self_record(const KArgs& a, int ntiles_attr, int lane, unsigned* out) {
+    const hstu_fwd_params& p = a.p;
+    const int B = p.batch, H = p.heads_q;
+    const int is64 = p.index_type == HSTU_I64;
+    const bool mine = lane < B;
+    const int64_t o0 = ld_idx(p.seq_offset_q, mine ? lane : 0, is64), o1 = ld_idx(p.seq_offset_q, mine ? lane + 1 : 0, is64);
+    const int len = (int)(o1 - o0);
+    const int t = (len + BM - 1) / BM;
+    // class of a sequence = its tile count; sequences longer than the attribute covers form the class above
+    const int cls = mine ? min(t, ntiles_attr + 1) : 0;
+    const int x = blockIdx.x & 7;
+    const unsigned pos = blockIdx.x >> 3;
+    // r's of XCD x below n
+    auto below = [&](unsigned n) -> unsigned { return 2u * (n >> 4) + ((n & 15u) > (unsigned)x ? 1u : 0u) + ((n & 15u) > (unsigned)(15 - x) ? 1u : 0u); };
+    unsigned seqs_before = 0, entries_before = 0;
+    unsigned found_cls = 0, found_g = 0, found_i = 0, found_first = 0, found_e = 0;
+    for (int c = ntiles_attr + 1; c >= 1; c--) {
+        const unsigned long long m = __ballot(cls == c);
+        const unsigned n = (unsigned)__builtin_popcountll(m);
+        if (n == 0) continue;
+        const unsigned nt = (unsigned)min(c, ntiles_attr);
+        const unsigned e = nt - ((c <= ntiles_attr && c >= 5) ? 1u : 0u);       // entries of a group of this class
+        const unsigned g0 = below(seqs_before * (unsigned)H), g1 = below((seqs_before + n) * (unsigned)H);
+        const unsigned span = (g1 - g0) * e;
+        if (found_cls == 0 && pos < entries_before + span) {
+            found_cls = (unsigned)c;
+            found_g = g0 + (pos - entries_before) / e;
+            found_i = (pos - entries_before) % e;
+            found_first = seqs_before;
+            found_e = e;
+        }
+        seqs_before += n;
+        entries_before += span;
+    }
+    if (found_cls == 0) {
+        if (lane == 0) {
+            out[0] = ITEM_EMPTY;
+#pragma unroll
+            for (int i = 1; i < REC; i++) out[i] = 0u;
+        }
+        return;
+    }
+    // group found_g of this XCD's list: r = 16 (g / 2) + (x or 15 - x); its sequence is the (rank - found_first)-th of its class
+    const unsigned r = 16u * (found_g >> 1) + ((found_g & 1u) ? (unsigned)(15 - x) : (unsigned)x);
+    const unsigned rank = r / (unsigned)H, h = r - rank * (unsigned)H;
+    const unsigned long long m = __ballot(cls == (int)found_cls);
+    const unsigned nth = rank - found_first;
+    const unsigned before_me = __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)m, 0u));
+    const unsigned long long pick = __ballot(cls == (int)found_cls && before_me == nth);
+    const int fb = pick ? __builtin_ctzll(pick) : 0;
+    const unsigned q0 = (unsigned)__builtin_amdgcn_readlane((int)o0, fb), lq = (unsigned)__builtin_amdgcn_readlane(len, fb);
+    if (lane == 0) {
+        const bool sw = found_cls > (unsigned)ntiles_attr, pr = !sw && found_cls >= 5;
+        const bool both = pr && found_i == found_e - 1;
+        const unsigned tile = both ? 0u : (found_e - 1 - found_i) + (pr ? 1u : 0u), part = both ? 1u : 0u;
+        out[0] = (unsigned)fb | h << 12 | tile << 16 | ((found_i == 0 && sw) ? 1u << 24 : 0u) | part << 25 | 1u << 28;
+        out[1] = q0; out[2] = lq; out[3] = q0; out[4] = lq; out[5] = 0u; out[6] = 0u; out[7] = 0u;
+    }
+}
+
 // EXTRA: 5 / 6 / 7 = a dense bias / a custom mask / both, rows on 16-byte boundaries, and nothing else: the general
 // variant's per-score code carries every option as a run-time test and runs 2.7 x slower than these on the same input;
 // 0 = no bias / built-in mask only, 1 = dense bias and/or custom mask (tables, if any, gathered from
@@ -428,7 +508,10 @@ template <int D, int EXTRA, bool PAGED> struct Shape {
         static constexpr int WAVES = D == 256 ? 1 : ((D <= 64 && EXTRA == 0 && !PAGED) ? 4 : ((LEAN || (D <= 64 && EXTRA != 1) || (XDMA && EXTRA != 7)) ? 3 : 2));
 };
 
-template <typename T, int D, int EXTRA, bool PAGED>
+// SELF: no schedule kernel.  For small batches of plain causal self-attention (at most 64 sequences, one set of offsets
+// for q and k) the first wave of every workgroup derives its record from the offsets themselves (self_record), which
+// costs a workgroup a few hundred nanoseconds and saves the call a kernel and the gap between two kernels.
+template <typename T, int D, int EXTRA, bool PAGED, bool SELF = false>
 __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(Shape<D, EXTRA, PAGED>::WAVES, Shape<D, EXTRA, PAGED>::WAVES)))
 void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const float* part_base) {
     typedef Tile<D> TL;
@@ -501,17 +584,45 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave index, kept in a scalar register
     const int g = lane >> 5, l32 = lane & 31;
 
+#ifdef HSTU_ITEM_TIMING
+    const unsigned long long it0 = __builtin_amdgcn_s_memrealtime();
+    unsigned long long it1 = it0, it_loop = it0, it_rec = it0;
+    int it_ntk = 0;
+#endif
     // blockIdx -> record of the work list (see above)
     unsigned rw[REC];
-    {
+    int64_t owned_rows;
+    if constexpr (SELF) {
+        __shared__ unsigned lds_rec[REC];
+        if (tid < 64) self_record(a, (p.max_seq_len_q + BM - 1) / BM, lane, lds_rec);
+        {
+            const int64_t rows = ld_idx(p.seq_offset_q, p.batch, p.index_type == HSTU_I64);
+            owned_rows = (int64_t)(((uint64_t)(unsigned)__builtin_amdgcn_readfirstlane((int)(rows >> 32)) << 32) |
+                                   (unsigned)__builtin_amdgcn_readfirstlane((int)rows));
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < REC; i++) rw[i] = __builtin_amdgcn_readfirstlane(lds_rec[i]);
+        // the record also goes where the schedule kernel would have put it, so that the caller's workspace holds the list
+        // afterwards and later calls on this geometry can pass HSTU_FLAG_REUSE_WORKSPACE
+        if (tid < REC) const_cast<unsigned*>(ws)[WS_HEADER + REC * (size_t)blockIdx.x + tid] = lds_rec[tid];
+        if (blockIdx.x == 0 && tid == 0) {
+            const_cast<unsigned*>(ws)[0] = 0u;
+            *reinterpret_cast<int64_t*>(const_cast<unsigned*>(ws) + 2) = owned_rows;
+        }
+    } else {
         const unsigned* rec = ws + WS_HEADER + REC * (size_t)blockIdx.x;
 #pragma unroll
         for (int i = 0; i < REC; i++) rw[i] = rec[i];
+        // rows the sequences own, for the zero fill at the end: requested here so that nothing waits for it there
+        owned_rows = *reinterpret_cast<const int64_t*>(ws + 2);
     }
-    // rows the sequences own, for the zero fill at the end: requested here so that nothing waits for it there
-    int64_t owned_rows = *reinterpret_cast<const int64_t*>(ws + 2);
     asm volatile("" : "+s"(owned_rows));
     const unsigned item = rw[0];
+#ifdef HSTU_ITEM_TIMING
+    asm volatile("" :: "s"(item));
+    it_rec = __builtin_amdgcn_s_memrealtime();
+#endif
     const bool active = item != ITEM_EMPTY;
     const int b = active ? (int)(item & 0xfff) : 0, h = active ? (int)((item >> 12) & 0xf) : 0;
     const int tile0 = (int)((item >> 16) & 0xff);
@@ -901,6 +1012,10 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
         if (kt0 < kt1) fetch(kt0, lds0);
         if (XDMA && kt0 < kt1) fetch_x(kt0, lds_xd0);
         stash(kt0, lds0);
+#ifdef HSTU_ITEM_TIMING
+        if (it1 == it0) it1 = __builtin_amdgcn_s_memrealtime();
+        it_ntk += kt1 - kt0;
+#endif
 
         auto iteration = [&](int kt, const char* cur, char* nxt, const char* xcur, char* xnxt) __attribute__((always_inline)) {
             const int buf = kt & 1;
@@ -1156,6 +1271,9 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
             if (kt + 1 < kt1) iteration(kt + 1, lds1, lds0, lds_xd1, lds_xd0);
         }
 
+#ifdef HSTU_ITEM_TIMING
+        it_loop = __builtin_amdgcn_s_memrealtime();
+#endif
         // ---- epilogue: O^T accumulator register r of block db holds d = 32*db + 8*(r/4) + 4*g + r%4 for row qi
         if (PARK_OUT && nsplit == 1) {
             // Through LDS, so that the stores are whole rows: each wave parks its 32 x D tile in the K/V stage that
@@ -1222,6 +1340,17 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
         __syncthreads();   // the next tile's loads overwrite the stages the output tiles were parked in
     }
 
+#ifdef HSTU_ITEM_TIMING
+    if (tid == 0 && blockIdx.x < 32768) {
+        const unsigned long long it2 = __builtin_amdgcn_s_memrealtime();
+        unsigned* o = g_item_times + 8 * blockIdx.x;
+        o[0] = (unsigned)it0; o[1] = (unsigned)(it1 - it0); o[2] = (unsigned)(it2 - it0);
+        o[3] = __builtin_amdgcn_s_getreg((31 << 11) | 4);     // HW_ID: wave 3:0, SIMD 5:4, CU 11:8, SH 12, SE 15:13
+        o[4] = (unsigned)it_ntk; o[5] = item;
+        o[6] = (unsigned)(it_rec - it0);                      // time to the record
+        o[7] = (unsigned)(it_loop - it0);
+    }
+#endif
     // rows past the last offset are zero (the reference zero-fills its output: hstu_jagged.cpp:56-59)
     if (owned_rows < p.total_q) {
         const int64_t n = (p.total_q - owned_rows) * p.heads_q * (int64_t)D;
@@ -1273,6 +1402,18 @@ bool mfma_supported(const KArgs& a, const char** name) {
     return true;
 }
 
+// The plain head-dim-128 variant without a schedule kernel (see SELF): one lane per sequence, at most 64 tile-count classes,
+// and lists that cannot overflow (q and k share their offsets, so entries per group fall along the order).  A caller that
+// already holds a list (HSTU_FLAG_REUSE_WORKSPACE) keeps using it: reading a record is cheaper than deriving it.
+bool mfma_self_scheduled(const KArgs& a) {
+    const hstu_fwd_params& p = a.p;
+    return a.op == OP_JAGGED && (p.dtype == HSTU_BF16 || p.dtype == HSTU_F16) && p.dim_qk == 128 && p.dim_v == 128 &&
+           p.batch <= 64 && p.seq_offset_q && p.seq_offset_q == p.seq_offset_k && !p.num_context && !p.num_target &&
+           p.mask_type == HSTU_MASK_TRIL && !p.attn_bias && !p.pos_table && !p.ts_table &&
+           p.max_seq_len_q == p.max_seq_len_k && p.max_seq_len_q <= 64 * BM &&
+           !(p.flags & HSTU_FLAG_REUSE_WORKSPACE) && sched_dims(p).nsplit == 1;
+}
+
 hipError_t launch_work_list(const KArgs& a, unsigned* ws, bool pair, hipStream_t stream) {
     SchedDims d = sched_dims(a.p, true);
     d.pair = pair ? 1 : 0;
@@ -1305,13 +1446,20 @@ static hipError_t launch_td(const KArgs& a, unsigned* ws, hipStream_t stream) {
     const int groups = p.batch * p.heads_q;
     const int sched_threads = groups <= 128 ? 256 : (groups <= 512 ? 512 : SCHED_NT);   // spare threads write a group's records side by side
     hipError_t e = hipSuccess;
+    dim3 grid(8 * d.cap), block(NT);   // the overflow list starts at entry gridDim.x of the lists
+    const float* part = reinterpret_cast<const float*>(reinterpret_cast<const char*>(ws) + list_bytes(d));
+    if constexpr (D == 128) {
+        // small batches: the workgroups of the plain variant find their items themselves, no schedule kernel
+        if (extra == 0 && !paged && mfma_self_scheduled(a)) {
+            hipLaunchKernelGGL((hstu_mfma_kernel<T, D, 0, false, true>), grid, block, 0, stream, a, ws, part);
+            return hipGetLastError();
+        }
+    }
     if (!(p.flags & HSTU_FLAG_REUSE_WORKSPACE)) {
         hipLaunchKernelGGL(hstu_schedule_kernel, dim3(1), dim3(sched_threads), 0, stream, a, d, ws);
         e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
-    dim3 grid(8 * d.cap), block(NT);   // the overflow list starts at entry gridDim.x of the lists
-    const float* part = reinterpret_cast<const float*>(reinterpret_cast<const char*>(ws) + list_bytes(d));
 #define HSTU_LAUNCH(E, P) hipLaunchKernelGGL((hstu_mfma_kernel<T, D, E, P>), grid, block, 0, stream, a, ws, part)
     if constexpr (D == 32 || D == 256) {
         // the head dims at the ends of the reference's sweep: plain and general variants only (bias tables are gathered

@@ -128,7 +128,8 @@ def test_paged_and_dense_validation():
 def test_describe_kernel_selection():
     buf = C.create_string_buffer(64)
     lib = _capi.lib()
-    for over, want in [(dict(), "mfma_bf16_d128"), (dict(dim_qk=64, dim_v=64, dtype=_capi.HSTU_F16), "mfma_f16_d64"),
+    for over, want in [(dict(), "mfma_bf16_d128_selfsched"), (dict(flags=_capi.FLAG_REUSE_WORKSPACE), "mfma_bf16_d128"), (dict(batch=65), "mfma_bf16_d128"),
+                       (dict(dim_qk=64, dim_v=64, dtype=_capi.HSTU_F16), "mfma_f16_d64"),
                        (dict(dtype=_capi.HSTU_F32), "generic_f32"), (dict(dim_v=64), "generic_bf16"),
                        (dict(dim_qk=32, dim_v=32), "mfma_bf16_d32"), (dict(dim_qk=256, dim_v=256, dtype=_capi.HSTU_F16), "mfma_f16_d256"),
                        (dict(dim_qk=96, dim_v=96), "generic_bf16"),

@@ -214,7 +214,7 @@ def test_config2_headline_full_size():
     say("config2", sum(cfg["lens"]))
     ref = T.oracle_jagged(cfg)
     out, name = T.run_capi(cfg)
-    assert name == "mfma_bf16_d128"
+    assert name == "mfma_bf16_d128_selfsched"
     T.assert_parity(out, ref, torch.bfloat16, what="config2")
     lowp = T.oracle_jagged(cfg, mode="lowp")
     assert O.mismatch_ratio_close(out, lowp, 5e-3, 5e-3)
@@ -327,7 +327,7 @@ def test_reference_user_shape_long_sequences():
     dtype = torch.bfloat16
     cfg = W.reference_benchmark_config(batch=32, heads=4, dim=128, max_seq_len=7621, has_rab=False)
     out, name = T.run_capi(cfg)
-    assert name == "mfma_bf16_d128", name
+    assert name == "mfma_bf16_d128_selfsched", name
     gen, _ = T.run_capi(cfg, flags=FORCE_GENERIC)
     T.assert_parity(out, gen.float(), dtype, what="reference user shape vs generic kernel")
 
@@ -430,3 +430,40 @@ def test_limits_longest_sequence_and_most_groups():
     assert name.startswith("mfma_"), name
     gen, _ = T.run_capi(cfg, flags=FORCE_GENERIC)
     T.assert_parity(out, gen.float(), dtype, what="2048 x 16 groups vs generic kernel")
+
+
+@pytest.mark.parametrize("index_dtype", [torch.int32, torch.int64])
+@pytest.mark.parametrize("lens,heads,max_len", [
+    ([1], 1, 1), ([129], 3, 129), ([300, 0, 17, 0, 640], 4, 640), ([1000, 513, 512, 511, 129, 128, 127], 16, 1000),
+    (list(range(0, 64 * 17, 17)), 2, 1071), ([700] * 64, 8, 700), ([900, 140, 400], 5, 256),
+    ([2000, 64, 8000, 1], 16, 8192)])
+def test_self_scheduled_small_batches(lens, heads, max_len, index_dtype):
+    """Plain causal self-attention at head dim 128 on at most 64 sequences runs without the schedule kernel: every
+    workgroup derives its item from the offsets.  Every row must be produced exactly as by the list-driven grid (the call
+    also leaves the list in the workspace: the second call reuses it), empty sequences, one-row sequences, 64 sequences,
+    a max_seq_len attribute below the longest sequence and both offset dtypes included."""
+    say("self_scheduled", lens[:6], heads, max_len, index_dtype)
+    dtype = torch.bfloat16
+    cfg, _ = _jag(81, lens, heads, heads, 128, 128, dtype, index_dtype=index_dtype)
+    cfg["max_seq_len"] = max_len
+    out, name = T.run_capi(cfg)
+    assert name.endswith("_selfsched"), name
+    again, _ = T.run_capi(cfg, reuse_from=cfg)      # the list the first call left behind, read by the second
+    assert torch.equal(out, again)
+    gen, _ = T.run_capi(cfg, flags=FORCE_GENERIC)
+    T.assert_parity(out, gen.float(), dtype, what="self-scheduled vs generic kernel")
+    if sum(lens) <= 3000:
+        T.assert_parity(out, T.oracle_jagged(cfg), dtype, what="self-scheduled vs oracle")
+
+
+def test_self_scheduling_is_left_to_the_work_list_where_it_does_not_apply():
+    say("self_scheduled: not taken")
+    dtype = torch.bfloat16
+    cfg, _ = _jag(82, [200] * 65, 2, 2, 128, 128, dtype)                       # more than 64 sequences
+    assert not T.run_capi(cfg)[1].endswith("_selfsched")
+    cfg, _ = _jag(83, [200, 100], 2, 2, 128, 128, dtype, lens_k=[300, 100])    # K longer than Q
+    assert not T.run_capi(cfg)[1].endswith("_selfsched")
+    cfg, _ = _jag(84, [200, 100], 2, 2, 128, 128, dtype)
+    cfg["num_target"] = torch.tensor([5, 5])
+    cfg["target_group_size"] = 1
+    assert not T.run_capi(cfg)[1].endswith("_selfsched")
