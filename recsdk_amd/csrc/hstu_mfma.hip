@@ -13,6 +13,8 @@
 // Element-wise order follows the reference (vector_score_inter.h:299-323): x = alpha*(S+bias), SiLU,
 // then scale*mask; P is rounded to the I/O dtype before PV as there (vector_score_inter.h:177-184),
 // S itself stays in fp32.
+#include <type_traits>
+
 #include "hstu_device.h"
 
 namespace hstu {
@@ -551,13 +553,18 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
     constexpr bool DENSE_ONLY = EXTRA >= 5 && EXTRA <= 7, XB = EXTRA == 5 || EXTRA == 7, XM = EXTRA == 6 || EXTRA == 7;
     __shared__ float lds_pos[tab_pos ? 2 * PW : 1];
     __shared__ __attribute__((aligned(8))) double lds_tk[tab_ts ? 2 * BN : 1];
+    __shared__ __attribute__((aligned(16))) double lds_tkr[tab_ts ? 2 * (BN / 32) * 2 : 2];   // per stage and 32-key block: earliest, latest key time
+    __shared__ __attribute__((aligned(16))) float lds_tkf[tab_ts ? 2 * BN : 4];   // key times relative to the earliest one of their block
 
     // The time table, indexed by the top bits of (float)|dt| itself (exponent and three mantissa bits, counted from 1.0f):
     // cell c covers the values whose bits start with 0x3f8 + c, a range no wider than a factor 1.125, so at most one
     // bucket bound falls inside it (host-checked through the spacing the hint promises).  Entry {that bound or the next
-    // one above the cell, table[bucket below it], table[bucket from it on]}: one read and one comparison give the bias.
+    // one above the cell, table[bucket below it], table[bucket from it on], the bound after that one}: one read and one
+    // comparison give the bias.
     constexpr int TS_CELLS = 512;
     __shared__ __attribute__((aligned(16))) float lds_tsq[tab_ts ? 4 * TS_CELLS : 4];
+    // per cell: the smallest integer |dt| whose fp32 rounding reaches the cell's bound (see the block-wise path below)
+    __shared__ __attribute__((aligned(8))) double lds_tsx[tab_ts ? TS_CELLS : 1];
     // paged: page ids of this user and, for an fp8 cache, the (K, V) scales of this kv head
     // fp8 pages by direct copies: raw rows of the next tile (32 keys x 128 bytes of K, then of V; wave w owns keys 8w..8w+7)
     __shared__ __attribute__((aligned(1024))) char lds_raw[SH::PDMA8 ? 2 * 4096 : 16];
@@ -707,8 +714,14 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                 const float lo = __builtin_bit_cast(float, 0x3f800000u + ((unsigned)c << 20));
                 const int f = min((int)(__builtin_amdgcn_logf(lo) * p.ts_log2_scale + 0.5f), p.num_buckets + 1);
                 const int bk = max(min(lo >= p.ts_bounds[f] ? f : f - 1, p.num_buckets), 0);
-                const f32x4 entry = {p.ts_bounds[bk + 1], p.ts_table[bk], p.ts_table[min(bk + 1, p.num_buckets)], 0.f};
+                const f32x4 entry = {p.ts_bounds[bk + 1], p.ts_table[bk], p.ts_table[min(bk + 1, p.num_buckets)], p.ts_bounds[min(bk + 2, p.num_buckets + 1)]};
                 *reinterpret_cast<f32x4*>(lds_tsq + 4 * c) = entry;
+                // integers x with RN_f32(x) >= b are those from the midpoint m of b and its predecessor on -- from m itself if it
+                // is an integer and b's mantissa is even (the tie goes to b), else from the next integer
+                const unsigned bb = __builtin_bit_cast(unsigned, entry[0]);
+                const double m = 0.5 * ((double)__builtin_bit_cast(float, bb - 1u) + (double)entry[0]);
+                const double cm = __builtin_ceil(m);
+                lds_tsx[c] = cm + ((cm == m && (bb & 1u)) ? 1.0 : 0.0);
             }
         }
         float pw_reg = 0.f;
@@ -947,7 +960,24 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
             }
             if (TAB) {
                 if (tab_pos && tid < PW - 1) lds_pos[buf * PW + tid] = pw_reg;
-                if (tab_ts && tid < BN) lds_tk[buf * BN + tid] = tk_reg;
+                if (tab_ts && tid < BN) {
+                    lds_tk[buf * BN + tid] = tk_reg;
+                    // earliest and latest key time of each 32-key block (lane t of the first wave holds key t)
+                    double lo = tk_reg, hi = tk_reg;
+#pragma unroll
+                    for (int off = 1; off < 32; off <<= 1) {
+                        const double a = __shfl_xor(lo, off, 64), b = __shfl_xor(hi, off, 64);
+                        lo = a < lo ? a : lo;
+                        hi = b > hi ? b : hi;
+                    }
+                    // relative to the earliest one the key times of a block are small integers: exact in fp32 below 2^24 (a block
+                    // that spans more reports a latest time of +inf, which sends it down the general path)
+                    lds_tkf[buf * BN + tid] = (float)(tk_reg - lo);
+                    if ((tid & 31) == 0) {
+                        lds_tkr[(buf * (BN / 32) + (tid >> 5)) * 2] = lo;
+                        lds_tkr[(buf * (BN / 32) + (tid >> 5)) * 2 + 1] = hi - lo < 16777216.0 ? hi : __builtin_inf();
+                    }
+                }
             }
             if constexpr (ANY_DMA) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             if constexpr (SH::PDMA8) {
@@ -1109,7 +1139,38 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
 #pragma unroll
                     for (int r = 0; r < 16; r++) sacc[r] += posv[r];
                 }
-                if (tab_ts && D > 64) {
+                // Time-bucket bias of a block whose scores lie in at most two neighbouring buckets.  The rows of a wave and the keys
+                // of a block are 32 positions each; away from the diagonal |dt| varies by less than the factor between two bucket
+                // bounds over the block, so one table cell -- that of the lane's smallest |dt|, row time minus the latest key
+                // time -- names the only bound b that can fall into the lane's range, the values on either side of it and the
+                // bound after it.  When every lane's largest |dt| stays below that next bound (and no key is later than the
+                // row), a score's bias is `dt >= b ? above : below`, and since fp32 rounding is monotone that comparison is
+                // `key time <= row time - X` with X the smallest integer that rounds to at least b.  With key times relative
+                // to the block's earliest one (integers below 2^24, exact in fp32) that is four 16-byte reads per block and
+                // three instructions per score instead of two reads and seven instructions per score, with the same bucket
+                // ids bit for bit.
+                bool ts_fast = false;
+                if constexpr (tab_ts) {
+                    const double kmin = lds_tkr[(buf * (BN / 32) + kb) * 2], kmax = lds_tkr[(buf * (BN / 32) + kb) * 2 + 1];
+                    const double dlo_d = tqd - kmax;
+                    const float dlo = __builtin_amdgcn_fmed3f((float)dlo_d, 1.0f, ts_top), dhi = (float)(tqd - kmin);
+                    const unsigned cell16 = ((__builtin_bit_cast(unsigned, dlo) >> 16) & 0xfff0u) - 0x3f80u;
+                    const f32x4 ent = *reinterpret_cast<const f32x4*>(reinterpret_cast<const char*>(lds_tsq) + cell16);
+                    const bool lane_ok = (dlo_d >= 0.0 && dhi < ent[3]) || !qvalid;
+                    ts_fast = __all(lane_ok);
+                    if (ts_fast) {
+                            // key time <= row time - X, both relative to the block's earliest key: an integer; clamped to what the
+                            // relative key times can be, fp32 holds it exactly (beyond 2^24 the rounded value still clamps right)
+                            const double xmin = *reinterpret_cast<const double*>(reinterpret_cast<const char*>(lds_tsx) + (cell16 >> 1));
+                            const float thr = __builtin_amdgcn_fmed3f((float)((tqd - xmin) - kmin), -1.0f, 16777216.0f);
+                            f32x4 kt[4];
+#pragma unroll
+                            for (int q = 0; q < 4; q++) kt[q] = *reinterpret_cast<const f32x4*>(lds_tkf + buf * BN + 32 * kb + 8 * q + 4 * g);
+#pragma unroll
+                            for (int r = 0; r < 16; r++) sacc[r] += kt[r >> 2][r & 3] <= thr ? ent[2] : ent[1];
+                    }
+                }
+                if (tab_ts && D > 64 && !ts_fast) {
                     // time-bucket bias, a batch of scores at a time: all table reads of a batch are in flight before the first is
                     // used (one read right before its use leaves its whole latency exposed, sixteen times per block)
                     constexpr int TSB = 4;
@@ -1133,6 +1194,8 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                     }
                 }
                 float pf[16];
+                // (two copies of this loop where the time table is read score by score: with and without those reads)
+                auto silu_pass = [&](auto inline_ts) __attribute__((always_inline)) {
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
                     float x = sacc[r];
@@ -1161,8 +1224,9 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                     if (TAB) {
                         const int jj = 32 * kb + 8 * (r >> 2) + 4 * g + (r & 3);        // j - k0
                         if (tab_pos && !POS_AHEAD) x += lds_pos[buf * PW + jj - (32 * w + l32) + (BM - 1)];
-                        if (tab_ts && D <= 64) {
-                            // (three waves per SIMD leave no registers for reads in flight: one score at a time)
+                        if constexpr (decltype(inline_ts)::value) {
+                            // (three waves per SIMD leave no registers for reads in flight: one score at a time, between the
+                            // transcendental instructions of its neighbours)
                             const float dt = (float)__builtin_fabs(tqd - lds_tk[buf * BN + jj]);
                             const float dc = __builtin_amdgcn_fmed3f(dt, 1.0f, ts_top);
                             const unsigned cell16 = ((__builtin_bit_cast(unsigned, dc) >> 16) & 0xfff0u) - 0x3f80u;
@@ -1175,6 +1239,9 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                     if (EXTRA == 1 || XM) pv *= mval;
                     pf[r] = pv;
                 }
+                };
+                if (tab_ts && D <= 64 && !ts_fast) silu_pass(std::true_type{});
+                else silu_pass(std::false_type{});
                 // The built-in mask: the two-per-CU variants zero the fp32 values; the register-tight ones mask the packed
                 // pairs instead (fewer operations, and a fully visible block then needs no copies at the join)
                 if (!LEAN) {

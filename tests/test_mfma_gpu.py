@@ -467,3 +467,30 @@ def test_self_scheduling_is_left_to_the_work_list_where_it_does_not_apply():
     cfg["num_target"] = torch.tensor([5, 5])
     cfg["target_group_size"] = 1
     assert not T.run_capi(cfg)[1].endswith("_selfsched")
+
+
+@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("gap", [600.0, 20.0, 4e4])
+def test_mfma_time_table_blockwise_path(d, gap):
+    """Blocks away from the diagonal take the time-bucket bias block-wise (one table cell per lane, key times compared with
+    a threshold); the bucket ids must stay those of the formula.  Sequences long enough for such blocks, a table whose
+    neighbouring buckets differ by 8 (one wrong id moves an output far beyond the tolerance), and the cases that must
+    leave the block-wise path: timestamps out of order, a jump of more than 2^24 seconds inside a block, runs of equal
+    timestamps, keys later than their rows (context rows)."""
+    say("mfma_time_table_blockwise", d, gap)
+    rng = np.random.default_rng(41)
+    lens = [900, 517, 700, 333, 640]
+    cfg, _ = _jag(41, lens, 2, 2, d, d, torch.bfloat16)
+    nb = 128
+    cfg["ts_table"] = torch.tensor([4.0 if b % 2 else -4.0 for b in range(nb + 1)], dtype=torch.float32)
+    ts = [1_700_000_000 + np.cumsum(rng.exponential(gap, l).astype(np.int64)) for l in lens]
+    ts[1] = ts[1][rng.permutation(len(ts[1]))]                 # out of order
+    ts[2][400:] += 1 << 25                                      # a jump inside a block
+    ts[3][100:140] = ts[3][100]                                 # equal timestamps
+    cfg["timestamps"] = torch.from_numpy(np.concatenate(ts))
+    cfg["num_context"] = torch.tensor([0, 0, 0, 0, 37])        # rows that see later keys
+    out, name = T.run_capi(cfg)
+    assert name == f"mfma_bf16_d{d}", name
+    T.assert_parity(out, T.oracle_jagged(cfg), torch.bfloat16, what="block-wise time table vs oracle")
+    gen, _ = T.run_capi(cfg, flags=FORCE_GENERIC)
+    T.assert_parity(out, gen.float(), torch.bfloat16, what="block-wise time table vs generic kernel")
