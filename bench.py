@@ -66,16 +66,18 @@ def build_workload(name, torch, W):
         kv = sum(c["hist"]) * 2 * 4 * 128
         qo = 2 * 32 * 256 * 4 * 128 * 2
         return c, "paged", flops, kv + 2 * qo, "config5 paged fp8-KV: 32 users x 256 candidates, hist~U[1024,4096], 64-token pages"
-    if name in ("ref_bias", "ref_nobias", "ref_nobias_d32", "ref_nobias_d64", "ref_nobias_d256"):
-        dim = int(name.split("_d")[1]) if "_d" in name else 128   # the ends and the middle of the reference's head-dim sweep
-        c = W.reference_benchmark_config(has_rab=name == "ref_bias", dim=dim)
-        flops = W.headline_flops(c["lens"], 8, dim)
+    if name in ("ref_bias", "ref_nobias", "ref_nobias_d32", "ref_nobias_d64", "ref_nobias_d256", "ref_nobias_d64v32", "ref_nobias_d128v48"):
+        dims = name.split("_d")[1] if "_d" in name else "128"     # the ends and the middle of the reference's head-dim sweep,
+        dim = int(dims.split("v")[0])                             # and the (dim_qk, dim_v) pairs of its user cases
+        dim_v = int(dims.split("v")[1]) if "v" in dims else dim   # (test_forward_op_benchmark.py:192-193)
+        c = W.reference_benchmark_config(has_rab=name == "ref_bias", dim=dim, dim_v=dim_v)
+        flops = W.headline_flops(c["lens"], 8, (dim + dim_v) / 2)
         t = sum(c["lens"])
-        b = 4 * t * 8 * dim * 2
+        b = 2 * t * 8 * (dim + dim_v) * 2
         # of the dense bias only the causal half is needed: sum over sequences and heads of L (L + 1) / 2 two-byte values
         if name == "ref_bias":
             b += sum(8 * l * (l + 1) // 2 * 2 for l in c["lens"])
-        return c, "jagged", flops, b, ("reference benchmark shape (test_forward_op_benchmark.py:246-259): B=32 h=8 d=" + str(dim) + " S=2048, every length "
+        return c, "jagged", flops, b, ("reference benchmark shape (test_forward_op_benchmark.py:246-259): B=32 h=8 d=" + (str(dim) if dim_v == dim else f"({dim}, {dim_v})") + " S=2048, every length "
                                       "0.9 S, alpha=0.5, silu_scale=1/1024, bf16, causal, " + ("dense attn_bias [B,h,S,S]" if name == "ref_bias" else "no bias"))
     raise SystemExit(f"unknown workload {name}")
 
@@ -98,7 +100,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=1000)
-    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "ref_bias", "ref_nobias", "ref_nobias_d32", "ref_nobias_d64", "ref_nobias_d256", "config2_fp8", "ref_nobias_fp8", "config2_bwd", "ref_bias_bwd", "ref_nobias_bwd", "ref_nobias_d32_bwd", "ref_nobias_d64_bwd", "ref_nobias_d256_bwd", "kv_append", "kv_append_fp8", "rab_time", "rab_time_bwd", "rab_pos", "nmd_fwd", "nmd_bwd", "in_linear_silu", "in_linear_silu_bwd", "copy"],
+    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "ref_bias", "ref_nobias", "ref_nobias_d32", "ref_nobias_d64", "ref_nobias_d256", "ref_nobias_d64v32", "ref_nobias_d128v48", "config2_fp8", "ref_nobias_fp8", "config2_bwd", "ref_bias_bwd", "ref_nobias_bwd", "ref_nobias_d32_bwd", "ref_nobias_d64_bwd", "ref_nobias_d256_bwd", "kv_append", "kv_append_fp8", "rab_time", "rab_time_bwd", "rab_pos", "nmd_fwd", "nmd_bwd", "in_linear_silu", "in_linear_silu_bwd", "copy"],
                     help="'copy' runs a plain 256 MiB device copy: the known-size kernel the FETCH_SIZE/WRITE_SIZE counters are scaled by")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--timeline", action="store_true",

@@ -87,6 +87,7 @@ __device__ __forceinline__ RowRef<T, PAGED> kv_row_ref(const KArgs& a, const Seq
     r.scale = 1.f;
     r.fp8 = false;
     if (!PAGED) {
+        // (D is the row width in elements: dim_qk for k, dim_v for v -- the same for all variants but the uneven one)
         r.ptr = reinterpret_cast<const T*>(which ? p.v : p.k) + ((s.k_start + j) * p.heads_k + hk) * (int64_t)D;
         return r;
     }
@@ -181,6 +182,17 @@ struct SchedDims {
     int pair;          // 1: the first two Q tiles of a long sequence may become one item
 };
 
+// head dims the matrix-core kernels take through the padded variant (EXTRA 11): multiples of 16 up to 256 that are not one
+// of 32 / 64 / 128 / 256 for both q.k and v
+static bool uneven_dims(const hstu_fwd_params& p) {
+    const int d = p.dim_qk;
+    return d != p.dim_v || (d != 32 && d != 64 && d != 128 && d != 256);
+}
+static int padded_dim(const hstu_fwd_params& p) {
+    const int d = p.dim_qk > p.dim_v ? p.dim_qk : p.dim_v;
+    return d <= 32 ? 32 : (d <= 64 ? 64 : (d <= 128 ? 128 : 256));
+}
+
 static SchedDims sched_dims(const hstu_fwd_params& p, bool whole_tiles = false) {
     SchedDims d;
     d.pair = 1;
@@ -193,7 +205,7 @@ static SchedDims sched_dims(const hstu_fwd_params& p, bool whole_tiles = false) 
     // they simply add up) go through the workspace and a small reduction kernel.
     d.nsplit = 1;
     const int ktiles = (p.max_seq_len_k + BN - 1) / BN;
-    if (!whole_tiles && !(p.flags & FLAG_WHOLE_TILES) && d.bound < 384 && ktiles >= 16) {
+    if (!whole_tiles && !(p.flags & FLAG_WHOLE_TILES) && !uneven_dims(p) && d.bound < 384 && ktiles >= 16) {
         int s = 768 / (int)(d.bound ? d.bound : 1);
         if (s > 4) s = 4;
         if (s > ktiles / 4) s = ktiles / 4;
@@ -488,7 +500,11 @@ __device__ __forceinline__ void self_record(const KArgs& a, int ntiles_attr, int
 template <int D, int EXTRA, bool PAGED> struct Shape {
     static constexpr bool PDMA8 = PAGED && EXTRA == 9 && D == 128;
     static constexpr bool PDMA = PAGED && (EXTRA == 8 || EXTRA == 9) && D == 128;
-    static constexpr bool DMA = (!PAGED && D == 128) || PDMA;
+    // EXTRA 11: the plain variant (built-in mask, no bias) for head dims that are multiples of 16 other than D, and for
+    // dim_qk != dim_v: D is the next of 32 / 64 / 128 / 256 above both, rows come in through registers and the columns
+    // past the real dims are zeros in the fragments and in LDS, the output keeps its dim_v columns.
+    static constexpr bool UNEVEN = EXTRA == 11;
+    static constexpr bool DMA = (!PAGED && D == 128 && !UNEVEN) || PDMA;
     // head dim 64, rows straight from k / v, no dense bias or custom mask: direct copies too, 8 rows per instruction
     static constexpr bool DMA64 = !PAGED && D == 64 && (EXTRA == 0 || (EXTRA >= 2 && EXTRA <= 4));
     // head dim 32, plain variant: 16 rows of 64 bytes per instruction
@@ -507,7 +523,7 @@ template <int D, int EXTRA, bool PAGED> struct Shape {
     // the plain variants at head dims 32 and 64 need 81 / 113 registers and 16 / 34 KB of LDS and run four: 5 % / 1 % faster
     // than three -- at head dim 64 only since its tiles are copied straight into LDS; with the register loader it took 135
     // registers and lost 5 % to AGPR copies under the cap of 128.  Five and six at head dim 32: no faster, 1.5 % slower)
-        static constexpr int WAVES = D == 256 ? 1 : ((D <= 64 && EXTRA == 0 && !PAGED) ? 4 : ((LEAN || (D <= 64 && EXTRA != 1) || (XDMA && EXTRA != 7)) ? 3 : 2));
+        static constexpr int WAVES = D == 256 ? 1 : (UNEVEN && D == 128) ? 2 : ((D <= 64 && EXTRA == 0 && !PAGED) ? 4 : ((LEAN || (D <= 64 && EXTRA != 1) || (XDMA && EXTRA != 7)) ? 3 : 2));
 };
 
 // SELF: no schedule kernel.  For small batches of plain causal self-attention (at most 64 sequences, one set of offsets
@@ -683,12 +699,14 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
         v8 qf[D / 16];
         {
             const int qrow = SH::REV ? s.lq - 1 - min(qi, s.lq - 1) : min(qi, s.lq - 1);
-            const T* qp = qbase + ((s.q_start + qrow) * p.heads_q + h) * (int64_t)D + 8 * g;
+            const int dq_real = SH::UNEVEN ? p.dim_qk : D;
+            const T* qp = qbase + ((s.q_start + qrow) * p.heads_q + h) * (int64_t)dq_real + 8 * g;
 #pragma unroll
             for (int ds = 0; ds < D / 16; ds++) {
                 const u32x4 z = {0, 0, 0, 0};
-                const u32x4 x = *reinterpret_cast<const u32x4*>(qp + 16 * ds);
-                qf[ds] = __builtin_bit_cast(v8, qvalid ? x : z);
+                const bool have = !SH::UNEVEN || 16 * ds < dq_real;
+                const u32x4 x = *reinterpret_cast<const u32x4*>(qp + (have ? 16 * ds : 0));
+                qf[ds] = __builtin_bit_cast(v8, qvalid && have ? x : z);
             }
         }
         f32x16 oacc[D / 32];
@@ -896,10 +914,11 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                     const int row = c / (D / 8), cc = c % (D / 8);
                     const int jl = min(k0 + row, kend - 1);
                     const int j = SH::REV ? s.lk - 1 - jl : jl;
-                    RowRef<T, PAGED> rk = kv_row_ref<T, PAGED>(a, s, 0, j, hk, D, lds_pid, lds_psc);
-                    RowRef<T, PAGED> rv = kv_row_ref<T, PAGED>(a, s, 1, j, hk, D, lds_pid, lds_psc);
-                    kreg[i] = load_chunk<T, PAGED>(rk, cc);
-                    vreg[i] = load_chunk<T, PAGED>(rv, cc);
+                    RowRef<T, PAGED> rk = kv_row_ref<T, PAGED>(a, s, 0, j, hk, SH::UNEVEN ? p.dim_qk : D, lds_pid, lds_psc);
+                    RowRef<T, PAGED> rv = kv_row_ref<T, PAGED>(a, s, 1, j, hk, SH::UNEVEN ? p.dim_v : D, lds_pid, lds_psc);
+                    // (uneven dims: chunks past the real row width are read from chunk 0 and zeroed when written to LDS)
+                    kreg[i] = load_chunk<T, PAGED>(rk, SH::UNEVEN && cc * 8 >= p.dim_qk ? 0 : cc);
+                    vreg[i] = load_chunk<T, PAGED>(rv, SH::UNEVEN && cc * 8 >= p.dim_v ? 0 : cc);
                     if (PAGED) {
                         kscale[i] = rk.scale;
                         vscale[i] = rv.scale;
@@ -954,8 +973,8 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                         kx = dequant_chunk<T>(kx, kscale[i]);
                         vx = dequant_chunk<T>(vx, vscale[i]);
                     }
-                    *reinterpret_cast<u32x4*>(dk + row * TL::KS + cc * 8) = ok ? kx : z;
-                    *reinterpret_cast<u32x4*>(dv + row * TL::VS + cc * 8) = ok ? vx : z;
+                    *reinterpret_cast<u32x4*>(dk + row * TL::KS + cc * 8) = ok && (!SH::UNEVEN || cc * 8 < p.dim_qk) ? kx : z;
+                    *reinterpret_cast<u32x4*>(dv + row * TL::VS + cc * 8) = ok && (!SH::UNEVEN || cc * 8 < p.dim_v) ? vx : z;
                 }
             }
             if (TAB) {
@@ -1368,16 +1387,18 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
             for (int i = 0; i < 32 / RPI; i++) {
                 const int row = RPI * i + orow;
                 const u32x4 x = *reinterpret_cast<const u32x4*>(park + row * ORS + ochunk * 16);
-                if (r0 + row < s.lq) {
+                const int dv_real = SH::UNEVEN ? p.dim_v : D;
+                if (r0 + row < s.lq && (!SH::UNEVEN || ochunk * 8 < dv_real)) {
                     const int out_row = SH::REV ? s.lq - 1 - (r0 + row) : r0 + row;
-                    *reinterpret_cast<u32x4*>(obase + ((s.q_start + out_row) * p.heads_q + h) * (int64_t)D + ochunk * 8) = x;
+                    *reinterpret_cast<u32x4*>(obase + ((s.q_start + out_row) * p.heads_q + h) * (int64_t)dv_real + ochunk * 8) = x;
                 }
             }
         } else if (nsplit == 1) {
             // the two lanes of a row hold alternating 8-byte pieces of it: they exchange halves (v_permlane32_swap: upper half of
             // one register with the lower half of another) and store 16 bytes each
             const int orow = qvalid ? (SH::REV ? s.lq - 1 - qi : qi) : 0;
-            T* op = obase + ((s.q_start + orow) * p.heads_q + h) * (int64_t)D + 8 * g;
+            const int dv_real = SH::UNEVEN ? p.dim_v : D;
+            T* op = obase + ((s.q_start + orow) * p.heads_q + h) * (int64_t)dv_real + 8 * g;
 #pragma unroll
             for (int db = 0; db < D / 32; db++) {
 #pragma unroll
@@ -1388,7 +1409,7 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                     const u32x2 s0 = __builtin_amdgcn_permlane32_swap(o[0], o[2], false, false);
                     const u32x2 s1 = __builtin_amdgcn_permlane32_swap(o[1], o[3], false, false);
                     const u32x4 out4 = {s0[0], s1[0], s0[1], s1[1]};
-                    if (qvalid) *reinterpret_cast<u32x4*>(op + 32 * db + 16 * pr) = out4;
+                    if (qvalid && (!SH::UNEVEN || 32 * db + 16 * pr < dv_real)) *reinterpret_cast<u32x4*>(op + 32 * db + 16 * pr) = out4;
                 }
             }
         } else if (qvalid) {
@@ -1420,8 +1441,8 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
 #endif
     // rows past the last offset are zero (the reference zero-fills its output: hstu_jagged.cpp:56-59)
     if (owned_rows < p.total_q) {
-        const int64_t n = (p.total_q - owned_rows) * p.heads_q * (int64_t)D;
-        T* o = obase + owned_rows * p.heads_q * (int64_t)D;
+        const int64_t n = (p.total_q - owned_rows) * p.heads_q * (int64_t)(SH::UNEVEN ? p.dim_v : D);
+        T* o = obase + owned_rows * p.heads_q * (int64_t)(SH::UNEVEN ? p.dim_v : D);
         for (int64_t e = (int64_t)blockIdx.x * NT + tid; e < n; e += (int64_t)gridDim.x * NT) o[e] = (T)0.f;
     }
 }
@@ -1454,8 +1475,16 @@ bool mfma_supported(const KArgs& a, const char** name) {
     *name = nullptr;
     if (p.dtype == HSTU_FP8_E4M3) return mfma_fp8_supported(a, name);
     if (p.dtype != HSTU_BF16 && p.dtype != HSTU_F16) return false;
-    const int d = p.dim_qk;
-    if (d != p.dim_v || (d != 32 && d != 64 && d != 128 && d != 256)) return false;
+    int d = p.dim_qk;
+    const bool uneven = uneven_dims(p);
+    if (uneven) {
+        // other multiples of 16 up to 256, and dim_qk != dim_v (the reference's own benchmark list has (64, 32) and (128, 48),
+        // cust_op/test/hstu_v2/test_forward_op_benchmark.py:192-193): the padded plain variant -- built-in mask or none, no
+        // bias, no tables, rows straight from k / v
+        if (p.dim_qk % 16 || p.dim_v % 16 || p.dim_qk > 256 || p.dim_v > 256) return false;
+        if (a.op == OP_PAGED || p.attn_bias || p.mask_type == HSTU_MASK_CUSTOM || p.pos_table || p.ts_table) return false;
+        d = padded_dim(p);
+    }
     if (a.op == OP_PAGED && (d == 32 || d == 256)) return false;   // paged K/V: head dims 64 and 128 only
     // rows are read and written 16 bytes at a time (vector loads, direct copies into LDS): buffers that do not start on
     // such a boundary take the plain kernel
@@ -1464,6 +1493,11 @@ bool mfma_supported(const KArgs& a, const char** name) {
     if (all & 15) return false;
     if (a.op == OP_PAGED && (p.max_seq_len_k + p.page_size - 1) / p.page_size > MAXP) return false;  // page ids of a user must fit the LDS copy
     const bool bf = p.dtype == HSTU_BF16;
+    if (uneven) {
+        *name = d == 32 ? (bf ? "mfma_bf16_d32_padded" : "mfma_f16_d32_padded") : d == 64 ? (bf ? "mfma_bf16_d64_padded" : "mfma_f16_d64_padded")
+              : d == 128 ? (bf ? "mfma_bf16_d128_padded" : "mfma_f16_d128_padded") : (bf ? "mfma_bf16_d256_padded" : "mfma_f16_d256_padded");
+        return true;
+    }
     *name = d == 32 ? (bf ? "mfma_bf16_d32" : "mfma_f16_d32") : d == 64 ? (bf ? "mfma_bf16_d64" : "mfma_f16_d64")
           : d == 128 ? (bf ? "mfma_bf16_d128" : "mfma_f16_d128") : (bf ? "mfma_bf16_d256" : "mfma_f16_d256");
     return true;
@@ -1528,7 +1562,9 @@ static hipError_t launch_td(const KArgs& a, unsigned* ws, hipStream_t stream) {
         if (e != hipSuccess) return e;
     }
 #define HSTU_LAUNCH(E, P) hipLaunchKernelGGL((hstu_mfma_kernel<T, D, E, P>), grid, block, 0, stream, a, ws, part)
-    if constexpr (D == 32 || D == 256) {
+    if (uneven_dims(p)) {
+        HSTU_LAUNCH(11, false);
+    } else if constexpr (D == 32 || D == 256) {
         // the head dims at the ends of the reference's sweep: plain and general variants only (bias tables are gathered
         // from global memory by the general one)
         if (extra == 0) HSTU_LAUNCH(0, false);
@@ -1582,15 +1618,16 @@ hipError_t launch_mfma(const KArgs& a, void* workspace, hipStream_t stream) {
     const hstu_fwd_params& p = a.p;
     unsigned* ws = reinterpret_cast<unsigned*>(workspace);
     if (p.dtype == HSTU_FP8_E4M3) return launch_mfma_fp8(a, workspace, stream);
+    const int d = uneven_dims(p) ? padded_dim(p) : p.dim_qk;
     if (p.dtype == HSTU_BF16) {
-        switch (p.dim_qk) {
+        switch (d) {
             case 32: return launch_td<__bf16, 32>(a, ws, stream);
             case 64: return launch_td<__bf16, 64>(a, ws, stream);
             case 128: return launch_td<__bf16, 128>(a, ws, stream);
             default: return launch_td<__bf16, 256>(a, ws, stream);
         }
     }
-    switch (p.dim_qk) {
+    switch (d) {
         case 32: return launch_td<_Float16, 32>(a, ws, stream);
         case 64: return launch_td<_Float16, 64>(a, ws, stream);
         case 128: return launch_td<_Float16, 128>(a, ws, stream);

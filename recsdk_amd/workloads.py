@@ -100,7 +100,7 @@ def config4(seed=0, dtype=torch.bfloat16, batch=128):
 
 
 def reference_benchmark_config(seed=123, batch=32, heads=8, dim=128, max_seq_len=2048, has_rab=True, dtype=torch.bfloat16,
-                               ratio=0.9) -> Dict:
+                               ratio=0.9, dim_v=None) -> Dict:
     """The shape of the reference's own forward benchmark (cust_op/test/hstu_v2/test_forward_op_benchmark.py:246-259 with
     the generator of utils/data.py:85-143): every sequence has int(0.9 * max_seq_len) rows, q/k/v and the dense bias
     ("rab", [batch, heads, max_seq_len, max_seq_len]) are uniform in (-1, 1), built-in causal mask, alpha = 0.5,
@@ -113,7 +113,7 @@ def reference_benchmark_config(seed=123, batch=32, heads=8, dim=128, max_seq_len
     def uni(shape):
         return torch.from_numpy(rng.uniform(-1.0, 1.0, shape).astype(np.float32)).to(dtype)
 
-    c = dict(q=uni((t, heads, dim)), k=uni((t, heads, dim)), v=uni((t, heads, dim)), seq_offset=offsets(lens), lens=lens,
+    c = dict(q=uni((t, heads, dim)), k=uni((t, heads, dim)), v=uni((t, heads, dim_v or dim)), seq_offset=offsets(lens), lens=lens,
              max_seq_len=max_seq_len, alpha=0.5, silu_scale=1.0 / 1024, mask_type=0)
     if has_rab:
         c["attn_bias"] = torch.cat([uni((1, heads, max_seq_len, max_seq_len)) for _ in range(batch)])

@@ -494,3 +494,23 @@ def test_mfma_time_table_blockwise_path(d, gap):
     T.assert_parity(out, T.oracle_jagged(cfg), torch.bfloat16, what="block-wise time table vs oracle")
     gen, _ = T.run_capi(cfg, flags=FORCE_GENERIC)
     T.assert_parity(out, gen.float(), torch.bfloat16, what="block-wise time table vs generic kernel")
+
+
+@pytest.mark.parametrize("dtype", LOWP)
+@pytest.mark.parametrize("dqk,dv", [(64, 32), (128, 48), (48, 48), (80, 16), (16, 16), (96, 96), (144, 256), (256, 16), (32, 64), (112, 80)])
+def test_mfma_uneven_head_dims(dqk, dv, dtype):
+    """Head dims that are multiples of 16 other than 32 / 64 / 128 / 256, and dim_qk != dim_v (the reference's benchmark list
+    has (64, 32) and (128, 48), cust_op/test/hstu_v2/test_forward_op_benchmark.py:192-193; its sweeps draw dim_v from
+    range(16, 513, 16)): the padded matrix-core variant, with GQA, longer K than Q, an empty sequence, rows past the last
+    offset, and without a mask."""
+    say("mfma_uneven", dtype, dqk, dv)
+    cfg, _ = _jag(51, [70, 0, 200, 33, 257], 4, 2, dqk, dv, dtype, lens_k=[130, 0, 200, 97, 300], index_dtype=torch.int32, extra_rows=5)
+    out, name = T.run_capi(cfg)
+    assert name.endswith("_padded"), name
+    out = _check(cfg, dtype, f"uneven dims ({dqk}, {dv})")
+    assert out.shape[2] == dv and torch.equal(out[-5:], torch.zeros_like(out[-5:]))
+    cfg["mask_type"] = 2
+    _check(cfg, dtype, f"uneven dims ({dqk}, {dv}), no mask")
+    # the reference's own cases: every sequence 0.9 of the attribute, q shorter than k and q longer than its attribute share
+    cfg2, _ = _jag(52, [28] * 6, 4, 4, dqk, dv, dtype, lens_k=[449] * 6)
+    _check(cfg2, dtype, f"uneven dims ({dqk}, {dv}), short q against long k")
