@@ -77,11 +77,14 @@ struct RowRef {
     bool fp8;
 };
 
-constexpr int MAXP = 320;  // pages of one user whose ids (and fp8 scales) are kept in LDS; later pages are looked up in global memory
+// pages of one user whose ids (and fp8 scales) are kept in LDS: the reference's longest sequence (20480) in its smallest pages
+// (32 rows, tiling_policy_paged.cpp:218-221); half of that in the head-dim-128 variants whose tiles go through registers
+// (64-key tiles: the larger copy would leave one workgroup per CU)
+constexpr int MAXP_ALL = 640, MAXP_HALF = 320;
 
 template <typename T, bool PAGED>
 __device__ __forceinline__ RowRef<T, PAGED> kv_row_ref(const KArgs& a, const Seq& s, int which, int j, int hk, int D,
-                                                       const int* lds_pid, const float* lds_psc) {
+                                                       const int* lds_pid, const float* lds_psc, int MAXP = MAXP_ALL) {
     const hstu_fwd_params& p = a.p;
     RowRef<T, PAGED> r;
     r.scale = 1.f;
@@ -504,6 +507,7 @@ template <int D, int EXTRA, bool PAGED> struct Shape {
     // dim_qk != dim_v: D is the next of 32 / 64 / 128 / 256 above both, rows come in through registers and the columns
     // past the real dims are zeros in the fragments and in LDS, the output keeps its dim_v columns.
     static constexpr bool UNEVEN = EXTRA == 11;
+    static constexpr int MAXP = (PAGED && D == 128 && EXTRA != 8 && EXTRA != 9) ? MAXP_HALF : MAXP_ALL;
     static constexpr bool DMA = (!PAGED && D == 128 && !UNEVEN) || PDMA;
     // head dim 64, rows straight from k / v, no dense bias or custom mask: direct copies too, 8 rows per instruction
     static constexpr bool DMA64 = !PAGED && D == 64 && (EXTRA == 0 || (EXTRA >= 2 && EXTRA <= 4));
@@ -534,6 +538,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(Shape<D, EXT
 void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const float* part_base) {
     typedef Tile<D> TL;
     typedef Shape<D, EXTRA, PAGED> SH;
+    constexpr int MAXP = SH::MAXP;
     constexpr int BNT = SH::BNT;
     constexpr bool LEAN = SH::WAVES >= 3;          // register-tight variants read V fragments right before use
     constexpr bool PARK_OUT = LEAN;                // output tiles leave through LDS as whole rows
@@ -914,8 +919,8 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                     const int row = c / (D / 8), cc = c % (D / 8);
                     const int jl = min(k0 + row, kend - 1);
                     const int j = SH::REV ? s.lk - 1 - jl : jl;
-                    RowRef<T, PAGED> rk = kv_row_ref<T, PAGED>(a, s, 0, j, hk, SH::UNEVEN ? p.dim_qk : D, lds_pid, lds_psc);
-                    RowRef<T, PAGED> rv = kv_row_ref<T, PAGED>(a, s, 1, j, hk, SH::UNEVEN ? p.dim_v : D, lds_pid, lds_psc);
+                    RowRef<T, PAGED> rk = kv_row_ref<T, PAGED>(a, s, 0, j, hk, SH::UNEVEN ? p.dim_qk : D, lds_pid, lds_psc, MAXP);
+                    RowRef<T, PAGED> rv = kv_row_ref<T, PAGED>(a, s, 1, j, hk, SH::UNEVEN ? p.dim_v : D, lds_pid, lds_psc, MAXP);
                     // (uneven dims: chunks past the real row width are read from chunk 0 and zeroed when written to LDS)
                     kreg[i] = load_chunk<T, PAGED>(rk, SH::UNEVEN && cc * 8 >= p.dim_qk ? 0 : cc);
                     vreg[i] = load_chunk<T, PAGED>(rv, SH::UNEVEN && cc * 8 >= p.dim_v ? 0 : cc);
@@ -1491,7 +1496,11 @@ bool mfma_supported(const KArgs& a, const char** name) {
     const uintptr_t all = reinterpret_cast<uintptr_t>(p.q) | reinterpret_cast<uintptr_t>(p.k) | reinterpret_cast<uintptr_t>(p.v) |
                           reinterpret_cast<uintptr_t>(p.out) | reinterpret_cast<uintptr_t>(p.kv_cache);
     if (all & 15) return false;
-    if (a.op == OP_PAGED && (p.max_seq_len_k + p.page_size - 1) / p.page_size > MAXP) return false;  // page ids of a user must fit the LDS copy
+    if (a.op == OP_PAGED) {   // page ids of a user must fit the LDS copy of the variant the call takes
+        const bool copies = d == 128 && !p.attn_bias && p.mask_type != HSTU_MASK_CUSTOM && !p.pos_table && !p.ts_table &&
+                            ((p.cache_dtype == p.dtype && p.page_size % 4 == 0) || (p.cache_dtype == HSTU_FP8_E4M3 && p.page_size % 8 == 0));
+        if ((p.max_seq_len_k + p.page_size - 1) / p.page_size > ((d == 128 && !copies) ? MAXP_HALF : MAXP_ALL)) return false;
+    }
     const bool bf = p.dtype == HSTU_BF16;
     if (uneven) {
         *name = d == 32 ? (bf ? "mfma_bf16_d32_padded" : "mfma_f16_d32_padded") : d == 64 ? (bf ? "mfma_bf16_d64_padded" : "mfma_f16_d64_padded")

@@ -514,3 +514,24 @@ def test_mfma_uneven_head_dims(dqk, dv, dtype):
     # the reference's own cases: every sequence 0.9 of the attribute, q shorter than k and q longer than its attribute share
     cfg2, _ = _jag(52, [28] * 6, 4, 4, dqk, dv, dtype, lens_k=[449] * 6)
     _check(cfg2, dtype, f"uneven dims ({dqk}, {dv}), short q against long k")
+
+
+@pytest.mark.parametrize("d,page_size,fp8,want_mfma", [(128, 32, False, True), (128, 32, True, True), (64, 32, False, True),
+                                                        (128, 34, False, False)])
+def test_mfma_paged_long_page_lists(d, page_size, fp8, want_mfma):
+    """A user whose history fills more than 320 pages (the reference allows sequences of 20480 in 32-row pages = 640 pages,
+    tiling_policy_paged.cpp:218-221) stays on the matrix cores; only the head-dim-128 variant that takes its tiles through
+    registers (page sizes that are no multiple of 4) keeps the shorter list and hands such a user to the plain kernel."""
+    say("mfma_paged_long", d, page_size, fp8)
+    dtype = torch.bfloat16
+    cfg = W.paged_config(61, 2, 2, d, 13000, 20000, 24, page_size, dtype)
+    assert max(cfg["hist"]) > 320 * page_size
+    kw = {}
+    if fp8:
+        cfg["kv_cache_fp8"], cfg["kv_scales"] = W.quantize_pages_fp8(cfg["kv_cache"])
+        kw["use_fp8"] = True
+    out, name = T.run_capi(cfg, op="paged", **kw)
+    assert name.startswith("mfma_") == want_mfma, name
+    gen, gname = T.run_capi(cfg, op="paged", flags=FORCE_GENERIC, **kw)
+    assert gname.startswith("generic")
+    T.assert_parity(out, gen.float(), dtype, what="long page list vs generic kernel")
