@@ -55,6 +55,8 @@ enum { HSTU_MASK_TRIL = 0, HSTU_MASK_TRIU = 1, HSTU_MASK_NONE = 2, HSTU_MASK_CUS
  * the list in the workspace, also the calls that need no schedule kernel of their own: plain causal self-attention at head
  * dim 128 on at most 64 sequences, whose workgroups derive their items from the offsets and write them down as they go.) */
 #define HSTU_FLAG_REUSE_WORKSPACE 4u
+/* backward only: run all kernels of this call on `stream` itself (see hstu_hip_jagged_backward) */
+#define HSTU_FLAG_SERIAL_BACKWARD 8u
 
 /*
  * One argument block for the three forward ops.  Pointers are device pointers unless stated.
@@ -199,9 +201,12 @@ typedef struct hstu_bwd_params {
 } hstu_bwd_params;
 
 /* To the caller the backward is one piece of work on `stream`, also under stream capture.  Large calls (3000 and more
- * (Q tile, head) items) run their dQ and K-side kernels side by side on two streams of the library's own per device, forked
- * from and joined to `stream` by events (default priority; created at the first such call on a device: make that call
- * outside a capture).  HSTU_HIP_SERIAL_BACKWARD=1 in the environment (read once per device) keeps everything on `stream`. */
+ * (Q tile, head) items) run their dQ and K-side kernels side by side on two streams of the library's own, forked from and
+ * joined to `stream` by events (default priority; one pair per caller stream, up to 8 per device, created at that stream's
+ * first such call outside a capture -- a capture that comes first runs on `stream` alone).  While such a call is being
+ * captured its side streams capture too: another host thread's large backward on the same caller stream must not overlap
+ * the capture.  HSTU_FLAG_SERIAL_BACKWARD in fwd.flags keeps the call on `stream`; HSTU_HIP_SERIAL_BACKWARD=1 in the
+ * environment (read once) does so for every call. */
 int hstu_hip_jagged_backward_get_workspace_size(const hstu_bwd_params* p, uint64_t* workspace_bytes);
 int hstu_hip_jagged_backward(const hstu_bwd_params* p, void* workspace, uint64_t workspace_bytes, void* stream);
 

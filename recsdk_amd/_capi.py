@@ -18,7 +18,7 @@ from . import _build
 HSTU_F32, HSTU_F16, HSTU_BF16, HSTU_FP8_E4M3 = 0, 1, 2, 3
 HSTU_I32, HSTU_I64 = 0, 1
 MASK_TRIL, MASK_TRIU, MASK_NONE, MASK_CUSTOM = 0, 1, 2, 3
-FLAG_DETERMINISTIC, FLAG_FORCE_GENERIC, FLAG_REUSE_WORKSPACE = 1, 2, 4
+FLAG_DETERMINISTIC, FLAG_FORCE_GENERIC, FLAG_REUSE_WORKSPACE, FLAG_SERIAL_BACKWARD = 1, 2, 4, 8
 
 EXPORTS = [
     "hstu_hip_jagged_forward_get_workspace_size", "hstu_hip_jagged_forward", "hstu_hip_jagged_forward_noalloc",

@@ -123,7 +123,7 @@ static int validate(const hstu_fwd_params* p, int op, KArgs* out, bool need_out 
     }
 
     out->p = *p;
-    out->p.flags &= HSTU_FLAG_DETERMINISTIC | HSTU_FLAG_FORCE_GENERIC | HSTU_FLAG_REUSE_WORKSPACE;   // the rest is the library's own
+    out->p.flags &= HSTU_FLAG_DETERMINISTIC | HSTU_FLAG_FORCE_GENERIC | HSTU_FLAG_REUSE_WORKSPACE | HSTU_FLAG_SERIAL_BACKWARD;   // the rest is the library's own
     out->op = op;
     out->head_ratio = p->heads_q / p->heads_k;
     out->out_scale = p->alpha * p->silu_scale;
@@ -284,7 +284,7 @@ int hstu_hip_describe_backward_kernel(const hstu_bwd_params* p, char* buf, size_
     if (rc != HSTU_OK) return rc;
     const bool mfma = !(p->fwd.flags & HSTU_FLAG_FORCE_GENERIC) && mfma_backward_supported(a);
     const char* dt = p->fwd.dtype == HSTU_F32 ? "f32" : (p->fwd.dtype == HSTU_F16 ? "f16" : "bf16");
-    if (mfma) snprintf(buf, n, "mfma_bwd_%s_d%d%s", dt, p->fwd.dim_qk, p->fwd.attn_bias ? "_bias" : "");
+    if (mfma) snprintf(buf, n, "mfma_bwd_%s_d%d%s", dt, p->fwd.dim_qk, p->fwd.attn_bias ? "_bias" : (p->fwd.mask_type == HSTU_MASK_CUSTOM ? "_mask" : ""));
     else snprintf(buf, n, "generic_bwd_%s", dt);
     return HSTU_OK;
 }

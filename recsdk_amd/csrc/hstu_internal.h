@@ -54,18 +54,20 @@ WorkList work_list_shape(const hstu_fwd_params& p);
 hipError_t launch_work_list(const KArgs& a, unsigned* ws, bool pair, hipStream_t stream);
 // dV of the backward as a forward pass over reversed rows (head dim 128, plain causal self-attention without GQA):
 // `a` carries K as q, Q as k, dO as v and dV as out; `ws` is a list launch_work_list() built for the same geometry.
-// Two streams and three events of the library's own per device, for entry points that run independent kernels side by side:
-// forked from and joined to the caller's stream by the events, so that the call stays one piece of work on that stream
-// (also under stream capture).  Default priority, events without timing, created at the first use on a device; nullptr if
-// that failed or HSTU_HIP_SERIAL_BACKWARD=1 is set (read once per device).  They are shared by all callers of a device: a
-// call holds side_streams_mutex() from its first event record to its last wait (these only enqueue work).
+// Two streams and three events of the library's own for entry points that run independent kernels side by side: forked from
+// and joined to the caller's stream by the events, so that the call stays one piece of work on that stream (also under stream
+// capture).  Default priority, events without timing.  Every caller stream gets a set of its own (up to 8 per device, made
+// at the stream's first such call; further streams share the last set), so that host threads on streams of their own do
+// not queue up behind one pair of side streams.  A call holds the set's mutex from its first event record to its last
+// wait (these only enqueue work).  nullptr: run on the caller's stream -- HSTU_HIP_SERIAL_BACKWARD=1 is set, or the set
+// could not be made (tried again at the next call, three times per set; never while the caller's stream is capturing,
+// since creating streams may not be legal then).
 struct SideStreams {
     hipStream_t side[2];
     hipEvent_t ev[3];
-    bool ok;
+    std::mutex mu;
 };
-SideStreams* side_streams();
-std::mutex& side_streams_mutex();
+SideStreams* side_streams(hipStream_t caller);
 bool reversed_forward_supported(const hstu_fwd_params& p);
 hipError_t launch_reversed_forward(const KArgs& a, const unsigned* ws, hipStream_t stream);
 

@@ -584,8 +584,6 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
     // comparison give the bias.
     constexpr int TS_CELLS = 512;
     __shared__ __attribute__((aligned(16))) float lds_tsq[tab_ts ? 4 * TS_CELLS : 4];
-    // per cell: the smallest integer |dt| whose fp32 rounding reaches the cell's bound (see the block-wise path below)
-    __shared__ __attribute__((aligned(8))) double lds_tsx[tab_ts ? TS_CELLS : 1];
     // paged: page ids of this user and, for an fp8 cache, the (K, V) scales of this kv head
     // fp8 pages by direct copies: raw rows of the next tile (32 keys x 128 bytes of K, then of V; wave w owns keys 8w..8w+7)
     __shared__ __attribute__((aligned(1024))) char lds_raw[SH::PDMA8 ? 2 * 4096 : 16];
@@ -739,12 +737,6 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                 const int bk = max(min(lo >= p.ts_bounds[f] ? f : f - 1, p.num_buckets), 0);
                 const f32x4 entry = {p.ts_bounds[bk + 1], p.ts_table[bk], p.ts_table[min(bk + 1, p.num_buckets)], p.ts_bounds[min(bk + 2, p.num_buckets + 1)]};
                 *reinterpret_cast<f32x4*>(lds_tsq + 4 * c) = entry;
-                // integers x with RN_f32(x) >= b are those from the midpoint m of b and its predecessor on -- from m itself if it
-                // is an integer and b's mantissa is even (the tie goes to b), else from the next integer
-                const unsigned bb = __builtin_bit_cast(unsigned, entry[0]);
-                const double m = 0.5 * ((double)__builtin_bit_cast(float, bb - 1u) + (double)entry[0]);
-                const double cm = __builtin_ceil(m);
-                lds_tsx[c] = cm + ((cm == m && (bb & 1u)) ? 1.0 : 0.0);
             }
         }
         float pw_reg = 0.f;
@@ -1185,7 +1177,12 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                     if (ts_fast) {
                             // key time <= row time - X, both relative to the block's earliest key: an integer; clamped to what the
                             // relative key times can be, fp32 holds it exactly (beyond 2^24 the rounded value still clamps right)
-                            const double xmin = *reinterpret_cast<const double*>(reinterpret_cast<const char*>(lds_tsx) + (cell16 >> 1));
+                            // X: integers x with RN_f32(x) >= b are those from the midpoint m of b and its predecessor on -- from
+                            // m itself if it is an integer and b's mantissa is even (the tie goes to b), else from the next integer
+                            const unsigned bb = __builtin_bit_cast(unsigned, ent[0]);
+                            const double m = 0.5 * ((double)__builtin_bit_cast(float, bb - 1u) + (double)ent[0]);
+                            const double cm = __builtin_ceil(m);
+                            const double xmin = cm + ((cm == m && (bb & 1u)) ? 1.0 : 0.0);
                             const float thr = __builtin_amdgcn_fmed3f((float)((tqd - xmin) - kmin), -1.0f, 16777216.0f);
                             f32x4 kt[4];
 #pragma unroll

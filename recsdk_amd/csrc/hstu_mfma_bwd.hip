@@ -83,7 +83,7 @@ template <typename T> __device__ __forceinline__ float bwd_half(unsigned w, int 
 template <> __device__ __forceinline__ float bwd_half<__bf16>(unsigned w, int hi) { return __builtin_bit_cast(float, hi ? (w & 0xffff0000u) : (w << 16)); }
 template <> __device__ __forceinline__ float bwd_half<_Float16>(unsigned w, int hi) { return (float)__builtin_bit_cast(b_f16x2, w)[hi]; }
 
-template <typename T, int D, int MODE, bool BIAS>
+template <typename T, int D, int MODE, int XK>
 // (head dim 256 keeps 32 operand fragments and a 32 x 256 accumulator per wave: one wave per SIMD)
 // waves per SIMD: one at head dim 256 (see above), three where the registers allow it (head dim 32; at head dim 64 the
 // kernels with one accumulator, since their tiles are copied straight into LDS), four for the dQ kernel at head dim 32
@@ -93,6 +93,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BWD_WAVES(D
 void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
     typedef typename BMM<T>::v8 v8;
     const hstu_fwd_params& p = a.f.p;
+    // XK: 0 = scores as they are, 1 = a dense attn_bias is added (and its gradient written), 2 = a custom mask multiplies P and
+    // dS (mask_type 3: [batch, heads, max_q, max_k] like the bias and read the same way; the built-in mask is then off)
+    constexpr bool BIAS = XK == 1, XMASK = XK == 2, XLOAD = XK != 0;
     // row strides of the LDS tiles in elements: +16 bytes keeps the 16-byte row-wise reads of 16 rows on distinct banks,
     // +64 bytes does the same for the 4-row transposing reads; a tile that is read both ways (K for dQ, Q for dK) takes a
     // stride of 12 banks modulo 64 (52 at head dim 64), under which the 16 rows of a row-wise read start on 16 different
@@ -125,7 +128,7 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
     // K-side kernels with a bias: per wave 16 rows x 32 columns of the bias, parked as they lie in memory and read back
     // transposed (row stride 72 bytes)
     constexpr int BTS = 72;
-    constexpr bool BIAS_T = BIAS && MODE != MODE_DQ;
+    constexpr bool BIAS_T = XLOAD && MODE != MODE_DQ;
     __shared__ __attribute__((aligned(16))) char bias_tile[BIAS_T ? 4 * 16 * BTS : 16];
     __shared__ __attribute__((aligned(16))) T t2s[BDMA ? 1 : 2][BDMA ? 8 : WBN * TS2];
 
@@ -308,10 +311,10 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
                     // [max_q, max_k] square reads offset 0 and becomes 0).  The dQ kernel owns rows: four 8-byte pieces of
                     // its row.  The K-side kernels own columns: the block comes in as it lies in memory, two times 16 rows of
                     // 64 bytes (lane L: row L / 4, 16-byte piece L % 4), and is turned in LDS further down.
-                    const T* bias_bh = reinterpret_cast<const T*>(p.attn_bias) + ((int64_t)b * p.heads_q + h) * p.max_seq_len_q * (int64_t)p.max_seq_len_k;
-                    b_u32x4 braw_q[(BIAS && MODE == MODE_DQ) ? 2 : 1];
+                    const T* bias_bh = reinterpret_cast<const T*>(XMASK ? p.mask : p.attn_bias) + ((int64_t)b * p.heads_q + h) * p.max_seq_len_q * (int64_t)p.max_seq_len_k;
+                    b_u32x4 braw_q[(XLOAD && MODE == MODE_DQ) ? 2 : 1];
                     b_u32x4 braw_k[BIAS_T ? 2 : 1];
-                    if (BIAS && MODE == MODE_DQ) {
+                    if (XLOAD && MODE == MODE_DQ) {
                         // 16 bytes per lane: columns c0 + 16 pr + 8 g .. + 7 of its row (the two lanes of a row then cover 32
                         // contiguous bytes per load); the halves are exchanged between the lanes further down
 #pragma unroll
@@ -350,8 +353,8 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
                     // accumulator register r holds streamed row c0 + 8*(r/4) + 4*g + r%4 for the owned row of this lane
                     // the bias of this lane's 16 elements as 8 words of two 16-bit values (pair x = elements 2x, 2x + 1), widened
                     // where they are used
-                    unsigned bias_w[BIAS ? 8 : 1];
-                    if (BIAS && MODE == MODE_DQ) {
+                    unsigned bias_w[XLOAD ? 8 : 1];
+                    if (XLOAD && MODE == MODE_DQ) {
                         // score registers 4 q .. 4 q + 3 are columns 8 q + 4 g .. + 3: of the 8 columns a lane loaded for q = 2 pr
                         // and 2 pr + 1, the lane with g = 0 keeps the first four and takes the first four of its partner
                         // (lane + 32), the lane with g = 1 takes the partner's last four and keeps its own: v_permlane32_swap
@@ -401,6 +404,13 @@ void hstu_bwd_mfma_kernel(const BArgs a, const unsigned* __restrict__ ws) {
                             if constexpr (MODE == MODE_DKV) pv[r] = sv * sg;
                         } else {
                             wv[r] = sv * sg;
+                        }
+                        if constexpr (XMASK) {
+                            // P = silu(x) * scale * mask, so the mask value multiplies P and, through it, dS (elements outside the
+                            // [max_q, max_k] square were read as 0: masked, as in the forward)
+                            const float mv = bwd_half<T>(bias_w[r >> 1], r & 1);
+                            wv[r] *= mv;
+                            if constexpr (MODE == MODE_DKV) pv[r] *= mv;
                         }
                     }
                     b_u32x4 pk0, pk1, qk0, qk1;   // dS (or, in the dV kernel, P); P of the fused kernel
@@ -560,7 +570,9 @@ bool mfma_backward_supported(const BArgs& a) {
     const hstu_fwd_params& p = a.f.p;
     if (p.dtype != HSTU_BF16 && p.dtype != HSTU_F16) return false;
     if (p.dim_qk != p.dim_v || (p.dim_qk != 32 && p.dim_qk != 64 && p.dim_qk != 128 && p.dim_qk != 256)) return false;
-    if (p.mask_type == HSTU_MASK_CUSTOM) return false;
+    // a custom mask is read like a dense bias (8 bytes at a time along its rows); with a bias next to it: the plain kernels
+    if (p.mask_type == HSTU_MASK_CUSTOM &&
+        (p.attn_bias || !p.mask || p.max_seq_len_k % 8 != 0 || (reinterpret_cast<uintptr_t>(p.mask) & 15))) return false;
     // a dense bias is read 8 bytes at a time along its rows, its gradient written the same way
     if (p.attn_bias && (p.max_seq_len_k % 8 != 0 || ((reinterpret_cast<uintptr_t>(p.attn_bias) | reinterpret_cast<uintptr_t>(a.grad_bias)) & 15)))
         return false;
@@ -606,29 +618,53 @@ uint64_t mfma_backward_workspace_bytes(const BArgs& a) {
 // empty.  To the caller the call still is one piece of work on its stream (also under stream capture, where the events
 // become edges of the graph).  Streams of default priority, events without timing, created on the first call on a device;
 // if that fails everything runs on the caller's stream.
-std::mutex& side_streams_mutex() {
+SideStreams* side_streams(hipStream_t caller) {
+    constexpr int MAXDEV = 64, SETS = 8;
+    struct Slot {
+        SideStreams set;
+        hipStream_t owner = nullptr;
+        int state = 0;        // 0 = free, 1 = made, -1 = given up
+        int failures = 0;
+    };
     static std::mutex mu;
-    return mu;
-}
-SideStreams* side_streams() {
-    constexpr int MAXDEV = 64;
-    std::mutex& mu = side_streams_mutex();
-    static SideStreams forks[MAXDEV];
-    static bool tried[MAXDEV];
+    static Slot slots[MAXDEV][SETS];
+    static int serial = -1;
     int dev = -1;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAXDEV) return nullptr;
     std::lock_guard<std::mutex> lock(mu);
-    SideStreams& f = forks[dev];
-    if (!tried[dev]) {
-        tried[dev] = true;
-        const char* serial = getenv("HSTU_HIP_SERIAL_BACKWARD");   // read once per device: "1" keeps the backward on the caller's stream
-        bool ok = !(serial && serial[0] == '1');
-        for (int i = 0; i < 2; i++) ok = ok && hipStreamCreateWithFlags(&f.side[i], hipStreamNonBlocking) == hipSuccess;
-        for (int i = 0; i < 3; i++) ok = ok && hipEventCreateWithFlags(&f.ev[i], hipEventDisableTiming) == hipSuccess;
-        if (!ok) (void)hipGetLastError();
-        f.ok = ok;
+    if (serial < 0) {
+        const char* e = getenv("HSTU_HIP_SERIAL_BACKWARD");   // "1" keeps every backward on the caller's stream
+        serial = (e && e[0] == '1') ? 1 : 0;
     }
-    return f.ok ? &f : nullptr;
+    if (serial) return nullptr;
+    Slot* slot = nullptr;
+    for (int i = 0; i < SETS && !slot; i++)
+        if (slots[dev][i].state == 1 && slots[dev][i].owner == caller) slot = &slots[dev][i];
+    for (int i = 0; i < SETS && !slot; i++)
+        if (slots[dev][i].state == 0) slot = &slots[dev][i];
+    if (!slot) return slots[dev][SETS - 1].state == 1 ? &slots[dev][SETS - 1].set : nullptr;   // more caller streams than sets: share
+    if (slot->state == 1) return &slot->set;
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(caller, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
+        (void)hipGetLastError();
+        return nullptr;    // not now: the next call outside a capture makes the set
+    }
+    SideStreams& f = slot->set;
+    int ns = 0, ne = 0;
+    bool ok = true;
+    for (; ns < 2 && ok; ns++) ok = hipStreamCreateWithFlags(&f.side[ns], hipStreamNonBlocking) == hipSuccess;
+    for (; ne < 3 && ok; ne++) ok = hipEventCreateWithFlags(&f.ev[ne], hipEventDisableTiming) == hipSuccess;
+    if (!ok) {
+        (void)hipGetLastError();
+        // (the loops count the failed attempt too)
+        for (int i = 0; i + 1 < ns; i++) (void)hipStreamDestroy(f.side[i]);
+        for (int i = 0; i + 1 < ne; i++) (void)hipEventDestroy(f.ev[i]);
+        if (++slot->failures >= 3) slot->state = -1;
+        return nullptr;
+    }
+    slot->owner = caller;
+    slot->state = 1;
+    return &f;
 }
 
 template <typename T, int D>
@@ -646,12 +682,13 @@ static hipError_t launch_bwd_td(const BArgs& a, unsigned* ws, hipStream_t stream
     }
     // fork: the K-side kernels wait for the work lists only.  Worth it when the kernels are long against the few microseconds
     // the events cost: at 3840 items per kernel (B = 32, h = 8, S = 2048) -2 .. -7 %, at 1440 (the headline batch) +2 %
-    SideStreams* fk = lq.grid >= 3000 ? side_streams() : nullptr;
+    SideStreams* fk = (lq.grid >= 3000 && !(a.f.p.flags & HSTU_FLAG_SERIAL_BACKWARD)) ? side_streams(stream) : nullptr;
     hipStream_t sk = stream, sv = stream;
-    // the events and side streams of a device are shared by all callers: from the first record to the last wait of this call
-    // no other host thread may record them (the calls below only enqueue work, so the lock is held for microseconds)
-    std::unique_lock<std::mutex> fork_lock(side_streams_mutex(), std::defer_lock);
-    if (fk) fork_lock.lock();
+    // a set can be shared (two host threads on one stream, or more caller streams than sets): from the first record to the
+    // last wait of this call no other host thread may record its events (the calls below only enqueue work, so the lock is
+    // held for microseconds)
+    std::unique_lock<std::mutex> fork_lock;
+    if (fk) fork_lock = std::unique_lock<std::mutex>(fk->mu);
     if (fk) {
         if (hipEventRecord(fk->ev[0], stream) == hipSuccess && hipStreamWaitEvent(fk->side[0], fk->ev[0], 0) == hipSuccess &&
             hipStreamWaitEvent(fk->side[1], fk->ev[0], 0) == hipSuccess) {
@@ -678,28 +715,42 @@ static hipError_t launch_bwd_td(const BArgs& a, unsigned* ws, hipStream_t stream
         hipLaunchKernelGGL(hstu_bwd_zero_bias_kernel<T>, dim3(zrows, (unsigned)(p.batch * p.heads_q)), dim3(256), 0, stream, a);
         e = hipGetLastError();
         if (e != hipSuccess) return join(e);
-        hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DQ, true>), dim3(lq.grid), dim3(256), 0, stream, a, wsq);
+        hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DQ, 1>), dim3(lq.grid), dim3(256), 0, stream, a, wsq);
         e = hipGetLastError();
         if (e != hipSuccess) return join(e);
         if constexpr (D <= 64) {
-            hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DKV, true>), dim3(lk.grid), dim3(256), 0, sk, a, wsk);
+            hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DKV, 1>), dim3(lk.grid), dim3(256), 0, sk, a, wsk);
             return join(hipGetLastError());
         }
-        hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DK, true>), dim3(lk.grid), dim3(256), 0, sk, a, wsk);
+        hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DK, 1>), dim3(lk.grid), dim3(256), 0, sk, a, wsk);
         e = hipGetLastError();
         if (e != hipSuccess) return join(e);
-        hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DV, true>), dim3(lk.grid), dim3(256), 0, sv, a, wsk);
+        hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DV, 1>), dim3(lk.grid), dim3(256), 0, sv, a, wsk);
         return join(hipGetLastError());
     }
-    hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DQ, false>), dim3(lq.grid), dim3(256), 0, stream, a, wsq);
+    if (a.f.p.mask_type == HSTU_MASK_CUSTOM) {
+        hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DQ, 2>), dim3(lq.grid), dim3(256), 0, stream, a, wsq);
+        e = hipGetLastError();
+        if (e != hipSuccess) return join(e);
+        if constexpr (D <= 64) {
+            hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DKV, 2>), dim3(lk.grid), dim3(256), 0, sk, a, wsk);
+            return join(hipGetLastError());
+        }
+        hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DK, 2>), dim3(lk.grid), dim3(256), 0, sk, a, wsk);
+        e = hipGetLastError();
+        if (e != hipSuccess) return join(e);
+        hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DV, 2>), dim3(lk.grid), dim3(256), 0, sv, a, wsk);
+        return join(hipGetLastError());
+    }
+    hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DQ, 0>), dim3(lq.grid), dim3(256), 0, stream, a, wsq);
     e = hipGetLastError();
     if (e != hipSuccess) return join(e);
     if constexpr (D <= 64) {
         // both K-side accumulators fit: S, G, dS and P once per block
-        hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DKV, false>), dim3(lk.grid), dim3(256), 0, sk, a, wsk);
+        hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DKV, 0>), dim3(lk.grid), dim3(256), 0, sk, a, wsk);
         return join(hipGetLastError());
     }
-    hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DK, false>), dim3(lk.grid), dim3(256), 0, sk, a, wsk);
+    hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DK, 0>), dim3(lk.grid), dim3(256), 0, sk, a, wsk);
     e = hipGetLastError();
     if (e != hipSuccess) return join(e);
     if (D == 128 && shared && reversed_forward_supported(a.f.p)) {
@@ -710,7 +761,7 @@ static hipError_t launch_bwd_td(const BArgs& a, unsigned* ws, hipStream_t stream
         r.p.q = a.f.p.k; r.p.k = a.f.p.q; r.p.v = a.grad_out; r.p.out = a.grad_v;
         return join(launch_reversed_forward(r, wsq, sv));
     }
-    hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DV, false>), dim3(lk.grid), dim3(256), 0, sv, a, wsk);
+    hipLaunchKernelGGL((hstu_bwd_mfma_kernel<T, D, MODE_DV, 0>), dim3(lk.grid), dim3(256), 0, sv, a, wsk);
     return join(hipGetLastError());
 }
 

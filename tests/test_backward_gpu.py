@@ -157,6 +157,12 @@ MFMA_CASES = [
     dict(lens_q=[300, 129, 64, 1, 0, 257], nq=2, nk=2, d=256, dtype=torch.bfloat16),
     dict(lens_q=[130, 40], nq=2, nk=1, d=256, dtype=torch.float16, lens_k=[333, 40]),
     dict(lens_q=[200, 72], nq=2, nk=2, d=256, dtype=torch.bfloat16, bias=True),
+    # custom mask (mask_type 3, rows of max_seq_len_k % 8 == 0 elements): read like a bias, multiplies P and dS
+    dict(lens_q=[296, 129, 64, 1, 0, 257], nq=2, nk=2, d=128, dtype=torch.bfloat16, mask="custom"),
+    dict(lens_q=[200, 77], nq=4, nk=2, d=64, dtype=torch.float16, mask="custom"),                      # GQA
+    dict(lens_q=[130, 40], nq=2, nk=1, d=128, dtype=torch.float16, lens_k=[336, 40], mask="custom"),   # delta-q + GQA
+    dict(lens_q=[264, 150], nq=2, nk=2, d=32, dtype=torch.bfloat16, mask="custom"),
+    dict(lens_q=[136, 72], nq=2, nk=2, d=256, dtype=torch.bfloat16, mask="custom"),
 ]
 
 
@@ -293,3 +299,16 @@ def test_hstu_dense_backward_op_and_autograd():
         assert torch.equal(q.grad.cpu(), want[0]) and torch.equal(k.grad.cpu(), want[1]) and torch.equal(v.grad.cpu(), want[2])
         if b is not None:
             assert torch.equal(b.grad.cpu(), want[3])
+
+
+def test_backward_serial_flag_gives_the_same_bits():
+    """HSTU_FLAG_SERIAL_BACKWARD keeps a large backward (more than 3000 items per kernel: normally three streams) on the
+    caller's stream: same sums in the same order, so the same bits."""
+    say("backward serial flag")
+    from recsdk_amd import _capi
+    cfg, grad = _case(31, [1300] * 36, 8, 8, 128, 128, torch.bfloat16)
+    forked = T.run_capi_backward(cfg, grad)
+    assert T.last_backward_kernel.startswith("mfma_bwd_")
+    serial = T.run_capi_backward(cfg, grad, flags=_capi.FLAG_SERIAL_BACKWARD)
+    for a, b in zip(forked[:3], serial[:3]):
+        assert torch.equal(a, b)
