@@ -139,11 +139,15 @@ def test_describe_kernel_selection():
         p = _params(**over)
         assert lib.hstu_hip_describe_kernel(C.byref(p), buf, 64) == 0
         assert buf.value.decode() == want
-    # paged: the MFMA kernel keeps one user's page ids in LDS (320 entries); longer page lists take the generic kernel
+    # paged: the MFMA kernel keeps one user's page ids in LDS (640 entries; 320 in the head-dim-128 variant that takes its
+    # tiles through registers: page sizes that are no multiple of 4); longer page lists take the generic kernel
     paged = dict(kv_cache=0x1000, page_offsets=0x1000, page_ids=0x1000, last_page_len=0x1000, cache_dtype=_capi.HSTU_BF16)
     for over, want in [(dict(page_size=64, max_seq_len_k=20480), "mfma_bf16_d128"),
-                       (dict(page_size=8, max_seq_len_k=2560), "mfma_bf16_d128"),
-                       (dict(page_size=8, max_seq_len_k=2561), "generic_bf16"),
+                       (dict(page_size=32, max_seq_len_k=20480), "mfma_bf16_d128"),
+                       (dict(page_size=8, max_seq_len_k=5120), "mfma_bf16_d128"),
+                       (dict(page_size=8, max_seq_len_k=5121), "generic_bf16"),
+                       (dict(page_size=10, max_seq_len_k=3200), "mfma_bf16_d128"),
+                       (dict(page_size=10, max_seq_len_k=3201), "generic_bf16"),
                        (dict(page_size=64, dim_qk=256, dim_v=256), "generic_bf16")]:
         p = _params(**paged, **over)
         assert lib.hstu_hip_describe_kernel(C.byref(p), buf, 64) == 0
