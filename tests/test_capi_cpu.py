@@ -328,7 +328,11 @@ def test_backward_validation_and_workspace():
     rc, n, msg = _bwd_ws(_bwd_params(attn_bias=0x1000, grad_bias=0x1000, max_seq_len_q=60, max_seq_len_k=60))
     assert rc == 0 and n == 0, msg                           # rows of 60 elements -> plain kernels
     rc, n, msg = _bwd_ws(_bwd_params(mask=0x1000, mask_type=3))
-    assert rc == 0 and n == 0, msg                           # custom mask -> plain kernels
+    assert rc == 0 and n == 1024, msg                        # custom mask on aligned rows: MFMA kernels too
+    rc, n, msg = _bwd_ws(_bwd_params(mask=0x1000, mask_type=3, attn_bias=0x1000, grad_bias=0x1000))
+    assert rc == 0 and n == 0, msg                           # custom mask next to a bias -> plain kernels
+    rc, n, msg = _bwd_ws(_bwd_params(mask=0x1000, mask_type=3, max_seq_len_q=60, max_seq_len_k=60))
+    assert rc == 0 and n == 0, msg                           # rows of 60 elements -> plain kernels
     for d, want in ((32, True), (256, True), (96, False), (512, False)):
         rc, n, msg = _bwd_ws(_bwd_params(dim_qk=d, dim_v=d))
         assert rc == 0 and (n > 0) == want, (d, n, msg)      # head dims 32 / 64 / 128 / 256 have matrix-core kernels
