@@ -1516,7 +1516,7 @@ bool mfma_self_scheduled(const KArgs& a) {
     const hstu_fwd_params& p = a.p;
     return a.op == OP_JAGGED && (p.dtype == HSTU_BF16 || p.dtype == HSTU_F16) && p.dim_qk == 128 && p.dim_v == 128 &&
            p.batch <= 64 && p.seq_offset_q && p.seq_offset_q == p.seq_offset_k && !p.num_context && !p.num_target &&
-           p.mask_type == HSTU_MASK_TRIL && !p.attn_bias && !p.pos_table && !p.ts_table &&
+           p.mask_type == HSTU_MASK_TRIL && !p.attn_bias && !p.ts_table &&
            p.max_seq_len_q == p.max_seq_len_k && p.max_seq_len_q <= 64 * BM &&
            !(p.flags & HSTU_FLAG_REUSE_WORKSPACE) && sched_dims(p).nsplit == 1;
 }
@@ -1556,9 +1556,11 @@ static hipError_t launch_td(const KArgs& a, unsigned* ws, hipStream_t stream) {
     dim3 grid(8 * d.cap), block(NT);   // the overflow list starts at entry gridDim.x of the lists
     const float* part = reinterpret_cast<const float*>(reinterpret_cast<const char*>(ws) + list_bytes(d));
     if constexpr (D == 128) {
-        // small batches: the workgroups of the plain variant find their items themselves, no schedule kernel
-        if (extra == 0 && !paged && mfma_self_scheduled(a)) {
-            hipLaunchKernelGGL((hstu_mfma_kernel<T, D, 0, false, true>), grid, block, 0, stream, a, ws, part);
+        // small batches: the workgroups of the plain variant (and of the one with a position table) find their items themselves,
+        // no schedule kernel
+        if ((extra == 0 || extra == 2) && !paged && mfma_self_scheduled(a)) {
+            if (extra == 0) hipLaunchKernelGGL((hstu_mfma_kernel<T, D, 0, false, true>), grid, block, 0, stream, a, ws, part);
+            else hipLaunchKernelGGL((hstu_mfma_kernel<T, D, 2, false, true>), grid, block, 0, stream, a, ws, part);
             return hipGetLastError();
         }
     }

@@ -237,7 +237,7 @@ def test_config3_skewed_with_pos_table():
     say("config3", cfg["lens"])
     ref = T.oracle_jagged(cfg)
     out, name = T.run_capi(cfg)
-    assert name == "mfma_bf16_d128"
+    assert name == "mfma_bf16_d128_selfsched"
     T.assert_parity(out, ref, torch.bfloat16, what="config3")
 
 
@@ -454,6 +454,13 @@ def test_self_scheduled_small_batches(lens, heads, max_len, index_dtype):
     T.assert_parity(out, gen.float(), dtype, what="self-scheduled vs generic kernel")
     if sum(lens) <= 3000:
         T.assert_parity(out, T.oracle_jagged(cfg), dtype, what="self-scheduled vs oracle")
+        # the variant with a relative-position table derives its items the same way
+        rng = np.random.default_rng(7)
+        cfg["pos_table"] = torch.from_numpy(rng.normal(0, 0.5, 2 * max_len - 1).astype(np.float32))
+        if max(lens) <= max_len:
+            out, name = T.run_capi(cfg)
+            assert name.endswith("_selfsched"), name
+            T.assert_parity(out, T.oracle_jagged(cfg), dtype, what="self-scheduled with a position table vs oracle")
 
 
 def test_self_scheduling_is_left_to_the_work_list_where_it_does_not_apply():
