@@ -48,10 +48,14 @@ __device__ __forceinline__ int fp8_classify(const Seq& s, int tgs, int r0, int c
 // from 2 to 3 at head dim 64 and 11 % at 128, 4 % from 3 to 4 at 64); head dim 256 needs a whole SIMD lane's registers.
 template <int D> struct Fp8Shape { static constexpr int WAVES = D == 64 ? 4 : (D == 128 ? 3 : 1); };
 
-template <int D>
+// UNEVEN: head dims that are other multiples of 16 up to D, and dim_qk != dim_v (the reference's fp8 sweep draws dim_v from
+// 16 .. 80, test_hstu_jagged_forward.py): rows have their real widths in memory, the chunks past them are zeros in the
+// fragments and in LDS, the output keeps its dim_v columns.
+template <int D, bool UNEVEN = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(Fp8Shape<D>::WAVES, Fp8Shape<D>::WAVES)))
 void hstu_mfma_fp8_kernel(const KArgs a, const unsigned* __restrict__ ws) {
     const hstu_fwd_params& p = a.p;
+    const int dq_real = UNEVEN ? p.dim_qk : D, dv_real = UNEVEN ? p.dim_v : D;
     // row strides in bytes: +16 keeps the 16-byte row-wise reads of 16 K rows on distinct banks, +32 does the same for
     // the 8-row transposing reads of V
     constexpr int KS = D + 16, VS = D + 32;
@@ -110,14 +114,15 @@ void hstu_mfma_fp8_kernel(const KArgs a, const unsigned* __restrict__ ws) {
         // Q fragments (B operand of S^T = K Q^T): column = Q row, lane half g holds head-dim bytes 64t + 32g .. + 31
         q_i32x8 qf[D / 64];
         {
-            const unsigned char* qp = qbase + ((s.q_start + min(qi, s.lq - 1)) * p.heads_q + h) * (int64_t)D + 32 * g;
+            const unsigned char* qp = qbase + ((s.q_start + min(qi, s.lq - 1)) * p.heads_q + h) * (int64_t)dq_real + 32 * g;
 #pragma unroll
             for (int t = 0; t < D / 64; t++) {
                 const q_u32x4 z = {0, 0, 0, 0};
-                q_u32x4 x0 = *reinterpret_cast<const q_u32x4*>(qp + 64 * t);
-                q_u32x4 x1 = *reinterpret_cast<const q_u32x4*>(qp + 64 * t + 16);
-                x0 = qvalid ? x0 : z;
-                x1 = qvalid ? x1 : z;
+                const bool have0 = !UNEVEN || 64 * t + 32 * g < dq_real, have1 = !UNEVEN || 64 * t + 32 * g + 16 < dq_real;
+                q_u32x4 x0 = *reinterpret_cast<const q_u32x4*>(have0 ? qp + 64 * t : qp - 32 * g);
+                q_u32x4 x1 = *reinterpret_cast<const q_u32x4*>(have1 ? qp + 64 * t + 16 : qp - 32 * g);
+                x0 = qvalid && have0 ? x0 : z;
+                x1 = qvalid && have1 ? x1 : z;
                 qf[t] = (q_i32x8){(int)x0[0], (int)x0[1], (int)x0[2], (int)x0[3], (int)x1[0], (int)x1[1], (int)x1[2], (int)x1[3]};
             }
         }
@@ -130,25 +135,26 @@ void hstu_mfma_fp8_kernel(const KArgs a, const unsigned* __restrict__ ws) {
         // tile loader: thread t copies 16-byte chunk t % CPR of rows t / CPR (+ 256 / CPR per further chunk) of K and of V.
         // Offsets are 32-bit, relative to the first row of this sequence and kv head (a sequence spans at most
         // 20480 * 16 * 256 bytes)
-        const unsigned rowstride = (unsigned)p.heads_k * D;
-        const unsigned char* kseq = kbase + (s.k_start * p.heads_k + hk) * (int64_t)D;
-        const unsigned char* vseq = vbase + (s.k_start * p.heads_k + hk) * (int64_t)D;
+        const unsigned rowstride = (unsigned)p.heads_k * dq_real, rowstride_v = (unsigned)p.heads_k * dv_real;
+        const unsigned char* kseq = kbase + (s.k_start * p.heads_k + hk) * (int64_t)dq_real;
+        const unsigned char* vseq = vbase + (s.k_start * p.heads_k + hk) * (int64_t)dv_real;
         const int lrow = tid / CPR, lcc = tid % CPR;
+        // (uneven dims: a chunk past the real row width is read from chunk 0 and zeroed when written to LDS)
+        const bool kchunk = !UNEVEN || 16 * lcc < dq_real, vchunk = !UNEVEN || 16 * lcc < dv_real;
         q_u32x4 nk[NCH], nv[NCH];
         auto fetch = [&](int kt) __attribute__((always_inline)) {
 #pragma unroll
             for (int i = 0; i < NCH; i++) {
                 // nothing here waits for the data; rows past the end are read from the last row and zeroed in stash()
                 const int row = min(kt * FBN + lrow + (256 / CPR) * i, kend - 1);
-                const unsigned e = __umul24((unsigned)row, rowstride) + 16u * lcc;
-                nk[i] = *reinterpret_cast<const q_u32x4*>(kseq + e);
-                nv[i] = *reinterpret_cast<const q_u32x4*>(vseq + e);
+                nk[i] = *reinterpret_cast<const q_u32x4*>(kseq + __umul24((unsigned)row, rowstride) + (kchunk ? 16u * lcc : 0u));
+                nv[i] = *reinterpret_cast<const q_u32x4*>(vseq + __umul24((unsigned)row, rowstride_v) + (vchunk ? 16u * lcc : 0u));
             }
         };
         auto stash = [&](int kt, int stage) __attribute__((always_inline)) {
             unsigned char* kd = kst[stage] + lrow * KS + 16 * lcc;
             unsigned char* vd = vst[stage] + lrow * VS + 16 * lcc;
-            if ((kt + 1) * FBN <= kend) {   // wave-uniform: every row of the tile exists
+            if (!UNEVEN && (kt + 1) * FBN <= kend) {   // wave-uniform: every row of the tile exists
 #pragma unroll
                 for (int i = 0; i < NCH; i++) {
                     *reinterpret_cast<q_u32x4*>(kd + (256 / CPR) * i * KS) = nk[i];
@@ -160,8 +166,8 @@ void hstu_mfma_fp8_kernel(const KArgs a, const unsigned* __restrict__ ws) {
                 for (int i = 0; i < NCH; i++) {
                     const bool ok = kt * FBN + lrow + (256 / CPR) * i < kend;
                     const q_u32x4 z = {0, 0, 0, 0};
-                    *reinterpret_cast<q_u32x4*>(kd + (256 / CPR) * i * KS) = ok ? nk[i] : z;
-                    *reinterpret_cast<q_u32x4*>(vd + (256 / CPR) * i * VS) = ok ? nv[i] : z;
+                    *reinterpret_cast<q_u32x4*>(kd + (256 / CPR) * i * KS) = ok && kchunk ? nk[i] : z;
+                    *reinterpret_cast<q_u32x4*>(vd + (256 / CPR) * i * VS) = ok && vchunk ? nv[i] : z;
                 }
             }
         };
@@ -286,7 +292,7 @@ void hstu_mfma_fp8_kernel(const KArgs a, const unsigned* __restrict__ ws) {
 
         // epilogue: O^T accumulator register r of block db holds d = 32 * db + 8 * (r / 4) + 4g + r % 4 of row qi
         if (qvalid) {
-            _Float16* op = obase + ((s.q_start + qi) * p.heads_q + h) * (int64_t)D + 4 * g;
+            _Float16* op = obase + ((s.q_start + qi) * p.heads_q + h) * (int64_t)dv_real + 4 * g;
 #pragma unroll
             for (int db = 0; db < D / 32; db++) {
 #pragma unroll
@@ -295,7 +301,7 @@ void hstu_mfma_fp8_kernel(const KArgs a, const unsigned* __restrict__ ws) {
                     lo[0] = (_Float16)oacc[db][4 * rr]; lo[1] = (_Float16)oacc[db][4 * rr + 1];
                     hi[0] = (_Float16)oacc[db][4 * rr + 2]; hi[1] = (_Float16)oacc[db][4 * rr + 3];
                     const q_u32x2 o = {__builtin_bit_cast(unsigned, lo), __builtin_bit_cast(unsigned, hi)};
-                    *reinterpret_cast<q_u32x2*>(op + 32 * db + 8 * rr) = o;
+                    if (!UNEVEN || 32 * db + 8 * rr + 4 * g < dv_real) *reinterpret_cast<q_u32x2*>(op + 32 * db + 8 * rr) = o;
                 }
             }
         }
@@ -303,23 +309,37 @@ void hstu_mfma_fp8_kernel(const KArgs a, const unsigned* __restrict__ ws) {
 
     // rows past the last offset are zero (the reference zero-fills its output: hstu_jagged.cpp:56-59)
     if (owned_rows < p.total_q) {
-        const int64_t n = (p.total_q - owned_rows) * p.heads_q * (int64_t)D;
-        _Float16* o = obase + owned_rows * p.heads_q * (int64_t)D;
+        const int64_t n = (p.total_q - owned_rows) * p.heads_q * (int64_t)dv_real;
+        _Float16* o = obase + owned_rows * p.heads_q * (int64_t)dv_real;
         for (int64_t e = (int64_t)blockIdx.x * 256 + tid; e < n; e += (int64_t)gridDim.x * 256) o[e] = (_Float16)0.f;
     }
+}
+
+// head dims the padded variant takes: multiples of 16 up to 256 other than 64 / 128 / 256 for both q.k and v
+static bool fp8_uneven(const hstu_fwd_params& p) {
+    return p.dim_qk != p.dim_v || (p.dim_qk != 64 && p.dim_qk != 128 && p.dim_qk != 256);
+}
+static int fp8_padded_dim(const hstu_fwd_params& p) {
+    const int d = p.dim_qk > p.dim_v ? p.dim_qk : p.dim_v;
+    return d <= 64 ? 64 : (d <= 128 ? 128 : 256);
 }
 
 bool mfma_fp8_supported(const KArgs& a, const char** name) {
     const hstu_fwd_params& p = a.p;
     *name = nullptr;
     if (p.dtype != HSTU_FP8_E4M3 || a.op == OP_PAGED) return false;
-    const int d = p.dim_qk;
-    if (d != p.dim_v || (d != 64 && d != 128 && d != 256)) return false;
+    int d = p.dim_qk;
+    const bool uneven = fp8_uneven(p);
+    if (uneven) {
+        if (p.dim_qk % 16 || p.dim_v % 16 || p.dim_qk > 256 || p.dim_v > 256) return false;
+        d = fp8_padded_dim(p);
+    }
     if (p.attn_bias || p.pos_table || p.ts_table || p.mask_type == HSTU_MASK_CUSTOM) return false;   // the plain kernel's
     const uintptr_t all = reinterpret_cast<uintptr_t>(p.q) | reinterpret_cast<uintptr_t>(p.k) | reinterpret_cast<uintptr_t>(p.v) |
                           reinterpret_cast<uintptr_t>(p.out);
     if (all & 15) return false;   // rows are read 16 bytes at a time
-    *name = d == 64 ? "mfma_fp8_d64" : (d == 128 ? "mfma_fp8_d128" : "mfma_fp8_d256");
+    *name = uneven ? (d == 64 ? "mfma_fp8_d64_padded" : (d == 128 ? "mfma_fp8_d128_padded" : "mfma_fp8_d256_padded"))
+                   : (d == 64 ? "mfma_fp8_d64" : (d == 128 ? "mfma_fp8_d128" : "mfma_fp8_d256"));
     return true;
 }
 
@@ -333,10 +353,18 @@ hipError_t launch_mfma_fp8(const KArgs& a, void* workspace, hipStream_t stream) 
         if (e != hipSuccess) return e;
     }
     const dim3 grid(work_list_shape(p).grid), block(256);
+    if (fp8_uneven(p)) {
+        switch (fp8_padded_dim(p)) {
+            case 64: hipLaunchKernelGGL((hstu_mfma_fp8_kernel<64, true>), grid, block, 0, stream, a, ws); break;
+            case 128: hipLaunchKernelGGL((hstu_mfma_fp8_kernel<128, true>), grid, block, 0, stream, a, ws); break;
+            default: hipLaunchKernelGGL((hstu_mfma_fp8_kernel<256, true>), grid, block, 0, stream, a, ws); break;
+        }
+        return hipGetLastError();
+    }
     switch (p.dim_qk) {
-        case 64: hipLaunchKernelGGL(hstu_mfma_fp8_kernel<64>, grid, block, 0, stream, a, ws); break;
-        case 128: hipLaunchKernelGGL(hstu_mfma_fp8_kernel<128>, grid, block, 0, stream, a, ws); break;
-        default: hipLaunchKernelGGL(hstu_mfma_fp8_kernel<256>, grid, block, 0, stream, a, ws); break;
+        case 64: hipLaunchKernelGGL((hstu_mfma_fp8_kernel<64, false>), grid, block, 0, stream, a, ws); break;
+        case 128: hipLaunchKernelGGL((hstu_mfma_fp8_kernel<128, false>), grid, block, 0, stream, a, ws); break;
+        default: hipLaunchKernelGGL((hstu_mfma_fp8_kernel<256, false>), grid, block, 0, stream, a, ws); break;
     }
     return hipGetLastError();
 }

@@ -98,8 +98,9 @@ def test_fp8_mfma_builtin_masks(ctx, tgt, tgs):
 ])
 @pytest.mark.parametrize("bias", [False, True])
 def test_fp8_plain_kernel_reference_sweep(case, bias):
-    """Shapes of the reference's (switched-off) fp8 tests that have no matrix-core variant: Dqk != Dv, attn_bias and custom
-    mask in float8_e4m3fn (its op definition makes both follow the dtype of q: hstu_jagged_forward.cpp:79-86)."""
+    """Shapes of the reference's (switched-off) fp8 tests: Dqk != Dv (the padded matrix-core variant where both are
+    multiples of 16 and there is no bias), attn_bias and custom mask in float8_e4m3fn (its op definition makes both follow
+    the dtype of q: hstu_jagged_forward.cpp:79-86; the plain kernel)."""
     c = dict(case)
     say("fp8_plain", c, bias)
     lens = c.pop("lens")
@@ -109,7 +110,11 @@ def test_fp8_plain_kernel_reference_sweep(case, bias):
     b, n, mq, mk = len(lens), c["nq"], cfg["max_seq_len"], cfg.get("max_seq_len_k") or cfg["max_seq_len"]
     if bias:
         cfg["attn_bias"] = torch.from_numpy(rng.random((b, n, mq, mk)).astype(np.float32)).to(FP8)
-    _check(cfg, "fp8 plain kernel", False)
+    # without a bias, head dims that are multiples of 16 run on the matrix cores (the padded variant); 72 does not
+    padded = not bias and c["dqk"] % 16 == 0
+    out = _check(cfg, "fp8 sweep shape", padded)
+    if padded:
+        assert T.run_capi(cfg)[1].endswith("_padded") and out.shape[2] == c["dv"]
     cfg["mask"] = torch.from_numpy(rng.integers(0, 2, (b, n, mq, mk)).astype(np.float32)).to(FP8)
     cfg["mask_type"] = 3
     _check(cfg, "fp8 plain kernel, custom mask", False)
