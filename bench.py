@@ -23,13 +23,15 @@ PEAK_FP8_TFLOPS = 5000.0    # MI355X dense fp8 MFMA
 PEAK_HBM_GBS = 8000.0
 # HBM-side bytes per launch from rocprofv3 FETCH_SIZE/WRITE_SIZE, each scaled by what the same counter reads for the
 # plain 256 MiB copy of `--workload copy` (factors 2.000 and 1.000); see profiles/*.md
-TRAFFIC_SOURCE = {"config2": "profiles/hstu_mfma_kernel_configs2-5.md", "config2_fp8": "profiles/hstu_mfma_fp8_kernel.md",
+TRAFFIC_SOURCE = {"config2": "profiles/hstu_mfma_kernel_configs2-5.md", "config3": "profiles/hstu_mfma_kernel_configs2-5.md",
+                  "config4": "profiles/hstu_mfma_kernel_configs2-5.md", "config5": "profiles/hstu_mfma_kernel_configs2-5.md",
+                  "config2_bwd": "profiles/hstu_mfma_kernel_configs2-5.md", "config2_fp8": "profiles/hstu_mfma_fp8_kernel.md",
                   "ref_bias": "profiles/hstu_mfma_kernel_reference_benchmark_shape.md", "kv_append": "profiles/hstu_kv_append_kernel.md",
                   "rab_time": "profiles/hstu_rab_kernels.md", "rab_time_bwd": "profiles/hstu_rab_kernels.md", "rab_pos": "profiles/hstu_rab_kernels.md",
                   "nmd_fwd": "profiles/hstu_nmd_kernels.md", "nmd_bwd": "profiles/hstu_nmd_kernels.md",
                   "in_linear_silu": "profiles/hstu_in_linear_silu_kernel.md", "in_linear_silu_bwd": "profiles/hstu_in_linear_silu_backward_kernels.md",
                   "kv_append_fp8": "profiles/hstu_kv_append_fp8_kernels.md"}
-MEASURED_TRAFFIC_BYTES = {"config2": 184.5e6, "config2_fp8": 116.5e6, "ref_bias": 1553.7e6, "kv_append": 351.9e6, "rab_time": 1443.4e6, "rab_time_bwd": 1589.7e6, "rab_pos": 297.7e6,
+MEASURED_TRAFFIC_BYTES = {"config2": 182.5e6, "config3": 112.6e6, "config4": 145.6e6, "config5": 205.9e6, "config2_bwd": 659.2e6, "config2_fp8": 116.5e6, "ref_bias": 1553.7e6, "kv_append": 351.9e6, "rab_time": 1443.4e6, "rab_time_bwd": 1589.7e6, "rab_pos": 297.7e6,
                           "nmd_fwd": 826.4e6, "nmd_bwd": 1380.0e6, "in_linear_silu": 1092.8e6, "in_linear_silu_bwd": 1458.3e6, "kv_append_fp8": 268.4e6}
 
 
@@ -381,7 +383,8 @@ def backward_bench(args, torch, W, _capi):
         "config": {"workload": desc, "kernel": kernel,
                    "flops_per_call": flops, "algorithmic_bytes_per_call": alg_bytes, "entry": "hstu_hip_jagged_backward (C ABI)"},
         "roofline": {"bound": "mfma", "achieved": round(flops / (kern_ms * 1e-3) / 1e12, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(flops / (kern_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "frac": round(flops / (kern_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                     "traffic_source": TRAFFIC_SOURCE.get(args.workload),
                      "kernel_us": round(kern_ms * 1e3, 2)},
     }), flush=True)
 

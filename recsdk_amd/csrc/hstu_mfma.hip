@@ -421,72 +421,99 @@ extern "C" int hstu_hip_timeline_read(void* dst, size_t bytes) {
 namespace hstu {
 #endif
 
-// The record of workgroup blockIdx.x without a work list, computed by one wave (lane b holds sequence b; the caller
-// guarantees batch <= 64, one set of offsets for q and k, no context or target rows, the plain causal mask).  The order is
-// the schedule kernel's with a coarser key: sequences by their number of Q tiles (longest first, then by batch index),
-// (sequence, head) groups r = rank * heads + head dealt to the XCDs in snake order (XCD x owns r = 16 u + x and
-// 16 u + 15 - x), a group's tiles last tile first, the first two tiles of a sequence of five or more tiles as one item.
-// Everything after the offsets have arrived is wave-uniform: one ballot per tile count and scalar arithmetic, so it costs
-// the vector unit (which the other workgroups of the CU keep busy) next to nothing.  No list can exceed the grid: with
-// entries per group falling along r, the lists differ by at most one group's entries.
-__device__ __forceinline__ void self_record(const KArgs& a, int ntiles_attr, int lane, unsigned* out) {
+// Inclusive prefix sum over the 64 lanes of a wave by data-parallel-primitive moves: four shifts inside each row of 16
+// lanes, then lane 15 of rows 0 / 2 into rows 1 / 3 and lane 31 into rows 2 and 3.
+__device__ __forceinline__ unsigned wave_inclusive_sum(unsigned v) {
+    v += (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0x111, 0xf, 0xf, false);   // row_shr:1
+    v += (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0x112, 0xf, 0xf, false);   // row_shr:2
+    v += (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0x114, 0xf, 0xf, false);   // row_shr:4
+    v += (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0x118, 0xf, 0xf, false);   // row_shr:8
+    v += (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0x142, 0xa, 0xf, false);   // row_bcast:15, rows 1 and 3
+    v += (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0x143, 0xc, 0xf, false);   // row_bcast:31, rows 2 and 3
+    return v;
+}
+
+// x / y for x < 2^20 / y: exact, because (x + 0.5) / y lies at least 0.5 / y away from every integer
+__device__ __forceinline__ unsigned small_div(unsigned x, unsigned y) {
+    return (unsigned)(((float)x + 0.5f) * __builtin_amdgcn_rcpf((float)y));
+}
+
+// The record of workgroup blockIdx.x without a work list, computed by one wave on its own (the caller guarantees
+// batch <= 64, at most 63 Q tiles per sequence under the attribute, one set of offsets for q and k, no context or target
+// rows, the plain causal mask).  The order is the schedule kernel's with a coarser key: sequences by their number of Q
+// tiles (longest first, then by batch index), (sequence, head) groups r = rank * heads + head dealt to the XCDs in snake
+// order (XCD x owns r = 16 u + x and 16 u + 15 - x), a group's tiles last tile first, the first two tiles of a sequence
+// of five or more tiles as one item.  Lane b first holds sequence b, then lane k holds the class of the sequences with
+// cmax - k tiles (a histogram in `hist`, 64 words of LDS private to the wave): the sequences and the list entries ahead
+// of a class are two prefix sums over the lanes, so the cost does not grow with the number of classes.  No list can
+// exceed the grid: with entries per group falling along r, the lists differ by at most one group's entries.
+__device__ __forceinline__ void self_record(const KArgs& a, int ntiles_attr, int lane, unsigned* hist, unsigned (&rec)[REC], int64_t& rows) {
     const hstu_fwd_params& p = a.p;
     const int B = p.batch, H = p.heads_q;
     const int is64 = p.index_type == HSTU_I64;
     const bool mine = lane < B;
-    const int64_t o0 = ld_idx(p.seq_offset_q, mine ? lane : 0, is64), o1 = ld_idx(p.seq_offset_q, mine ? lane + 1 : 0, is64);
+    // offsets b and b + 1 of lane b's sequence in one load (two dependent loads would double the wait)
+    struct __attribute__((aligned(8))) I64x2 { int64_t lo, hi; };
+    struct __attribute__((aligned(4))) I32x2 { int lo, hi; };
+    const int mb = mine ? lane : 0;
+    int64_t o0, o1;
+    if (is64) {
+        const I64x2 v = *reinterpret_cast<const I64x2*>(static_cast<const int64_t*>(p.seq_offset_q) + mb);
+        o0 = v.lo; o1 = v.hi;
+    } else {
+        const I32x2 v = *reinterpret_cast<const I32x2*>(static_cast<const int*>(p.seq_offset_q) + mb);
+        o0 = v.lo; o1 = v.hi;
+    }
     const int len = (int)(o1 - o0);
+    // rows the sequences own = the last offset, which lane batch - 1 holds (a scalar load of its own would make every later
+    // wait for a kernel argument wait for a round trip to the L2 as well)
+    rows = (int64_t)(((uint64_t)(unsigned)__builtin_amdgcn_readlane((int)(o1 >> 32), B - 1) << 32) | (unsigned)__builtin_amdgcn_readlane((int)o1, B - 1));
     const int t = (len + BM - 1) / BM;
     // class of a sequence = its tile count; sequences longer than the attribute covers form the class above
-    const int cls = mine ? min(t, ntiles_attr + 1) : 0;
-    const int x = blockIdx.x & 7;
-    const unsigned pos = blockIdx.x >> 3;
-    // r's of XCD x below n
-    auto below = [&](unsigned n) -> unsigned { return 2u * (n >> 4) + ((n & 15u) > (unsigned)x ? 1u : 0u) + ((n & 15u) > (unsigned)(15 - x) ? 1u : 0u); };
-    unsigned seqs_before = 0, entries_before = 0;
-    unsigned found_cls = 0, found_g = 0, found_i = 0, found_first = 0, found_e = 0;
-    for (int c = ntiles_attr + 1; c >= 1; c--) {
-        const unsigned long long m = __ballot(cls == c);
-        const unsigned n = (unsigned)__builtin_popcountll(m);
-        if (n == 0) continue;
-        const unsigned nt = (unsigned)min(c, ntiles_attr);
-        const unsigned e = nt - ((c <= ntiles_attr && c >= 5) ? 1u : 0u);       // entries of a group of this class
-        const unsigned g0 = below(seqs_before * (unsigned)H), g1 = below((seqs_before + n) * (unsigned)H);
-        const unsigned span = (g1 - g0) * e;
-        if (found_cls == 0 && pos < entries_before + span) {
-            found_cls = (unsigned)c;
-            found_g = g0 + (pos - entries_before) / e;
-            found_i = (pos - entries_before) % e;
-            found_first = seqs_before;
-            found_e = e;
-        }
-        seqs_before += n;
-        entries_before += span;
-    }
-    if (found_cls == 0) {
-        if (lane == 0) {
-            out[0] = ITEM_EMPTY;
+    const int cmax = ntiles_attr + 1;
+    const int cls = mine ? min(t, cmax) : 0;
+    hist[lane] = 0u;
+    __builtin_amdgcn_wave_barrier();
+    if (cls > 0) atomicAdd(&hist[cmax - cls], 1u);
+    __builtin_amdgcn_wave_barrier();
+    const unsigned n = hist[lane];                       // sequences of class c
+    const int c = cmax - lane;                           // (lanes from cmax on: n = 0)
+    const unsigned x = blockIdx.x & 7u, pos = blockIdx.x >> 3;
+    // r's of XCD x below m
+    auto below = [&](unsigned m) -> unsigned { return 2u * (m >> 4) + ((m & 15u) > x ? 1u : 0u) + ((m & 15u) > 15u - x ? 1u : 0u); };
+    auto entries = [&](int cc) -> unsigned { return (unsigned)min(cc, ntiles_attr) - ((cc <= ntiles_attr && cc >= 5) ? 1u : 0u); };
+    const unsigned seqs_incl = wave_inclusive_sum(n), seqs_before = seqs_incl - n;
+    const unsigned g0 = below(seqs_before * (unsigned)H), g1 = below(seqs_incl * (unsigned)H);
+    const unsigned span = n ? (g1 - g0) * entries(c) : 0u;
+    const unsigned ent_incl = wave_inclusive_sum(span), ent_before = ent_incl - span;
+    const unsigned long long hit = __ballot(pos >= ent_before && pos < ent_incl);
+    if (hit == 0) {
+        rec[0] = ITEM_EMPTY;
 #pragma unroll
-            for (int i = 1; i < REC; i++) out[i] = 0u;
-        }
+        for (int i = 1; i < REC; i++) rec[i] = 0u;
         return;
     }
+    const int fk = __builtin_ctzll(hit);
+    const int found_cls = cmax - fk;
+    const unsigned found_first = (unsigned)__builtin_amdgcn_readlane((int)seqs_before, fk);
+    const unsigned d = pos - (unsigned)__builtin_amdgcn_readlane((int)ent_before, fk);
+    const unsigned found_e = entries(found_cls);
+    const unsigned gi = small_div(d, found_e);
+    const unsigned found_g = (unsigned)__builtin_amdgcn_readlane((int)g0, fk) + gi, found_i = d - gi * found_e;
     // group found_g of this XCD's list: r = 16 (g / 2) + (x or 15 - x); its sequence is the (rank - found_first)-th of its class
-    const unsigned r = 16u * (found_g >> 1) + ((found_g & 1u) ? (unsigned)(15 - x) : (unsigned)x);
-    const unsigned rank = r / (unsigned)H, h = r - rank * (unsigned)H;
-    const unsigned long long m = __ballot(cls == (int)found_cls);
+    const unsigned r = 16u * (found_g >> 1) + ((found_g & 1u) ? 15u - x : x);
+    const unsigned rank = small_div(r, (unsigned)H), h = r - rank * (unsigned)H;
+    const unsigned long long m = __ballot(cls == found_cls);
     const unsigned nth = rank - found_first;
     const unsigned before_me = __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)m, 0u));
-    const unsigned long long pick = __ballot(cls == (int)found_cls && before_me == nth);
+    const unsigned long long pick = __ballot(cls == found_cls && before_me == nth);
     const int fb = pick ? __builtin_ctzll(pick) : 0;
     const unsigned q0 = (unsigned)__builtin_amdgcn_readlane((int)o0, fb), lq = (unsigned)__builtin_amdgcn_readlane(len, fb);
-    if (lane == 0) {
-        const bool sw = found_cls > (unsigned)ntiles_attr, pr = !sw && found_cls >= 5;
-        const bool both = pr && found_i == found_e - 1;
-        const unsigned tile = both ? 0u : (found_e - 1 - found_i) + (pr ? 1u : 0u), part = both ? 1u : 0u;
-        out[0] = (unsigned)fb | h << 12 | tile << 16 | ((found_i == 0 && sw) ? 1u << 24 : 0u) | part << 25 | 1u << 28;
-        out[1] = q0; out[2] = lq; out[3] = q0; out[4] = lq; out[5] = 0u; out[6] = 0u; out[7] = 0u;
-    }
+    const bool sw = found_cls > ntiles_attr, pr = !sw && found_cls >= 5;
+    const bool both = pr && found_i == found_e - 1;
+    const unsigned tile = both ? 0u : (found_e - 1 - found_i) + (pr ? 1u : 0u), part = both ? 1u : 0u;
+    rec[0] = (unsigned)fb | h << 12 | tile << 16 | ((found_i == 0 && sw) ? 1u << 24 : 0u) | part << 25 | 1u << 28;
+    rec[1] = q0; rec[2] = lq; rec[3] = q0; rec[4] = lq; rec[5] = 0u; rec[6] = 0u; rec[7] = 0u;
 }
 
 // EXTRA: 5 / 6 / 7 = a dense bias / a custom mask / both, rows on 16-byte boundaries, and nothing else: the general
@@ -531,8 +558,8 @@ template <int D, int EXTRA, bool PAGED> struct Shape {
 };
 
 // SELF: no schedule kernel.  For small batches of plain causal self-attention (at most 64 sequences, one set of offsets
-// for q and k) the first wave of every workgroup derives its record from the offsets themselves (self_record), which
-// costs a workgroup a few hundred nanoseconds and saves the call a kernel and the gap between two kernels.
+// for q and k) every wave of a workgroup derives the workgroup's record from the offsets themselves (self_record), which
+// costs a workgroup about a microsecond and saves the call a kernel and the gap between two kernels.
 template <typename T, int D, int EXTRA, bool PAGED, bool SELF = false>
 __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(Shape<D, EXTRA, PAGED>::WAVES, Shape<D, EXTRA, PAGED>::WAVES)))
 void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const float* part_base) {
@@ -619,19 +646,18 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
     unsigned rw[REC];
     int64_t owned_rows;
     if constexpr (SELF) {
-        __shared__ unsigned lds_rec[REC];
-        if (tid < 64) self_record(a, (p.max_seq_len_q + BM - 1) / BM, lane, lds_rec);
-        {
-            const int64_t rows = ld_idx(p.seq_offset_q, p.batch, p.index_type == HSTU_I64);
-            owned_rows = (int64_t)(((uint64_t)(unsigned)__builtin_amdgcn_readfirstlane((int)(rows >> 32)) << 32) |
-                                   (unsigned)__builtin_amdgcn_readfirstlane((int)rows));
-        }
-        __syncthreads();
+        // every wave derives the record by itself: no exchange through LDS, no barrier
+        __shared__ unsigned lds_hist[4 * 64];
+        unsigned rv[REC];
+        self_record(a, (p.max_seq_len_q + BM - 1) / BM, lane, lds_hist + 64 * w, rv, owned_rows);
 #pragma unroll
-        for (int i = 0; i < REC; i++) rw[i] = __builtin_amdgcn_readfirstlane(lds_rec[i]);
+        for (int i = 0; i < REC; i++) rw[i] = __builtin_amdgcn_readfirstlane(rv[i]);
         // the record also goes where the schedule kernel would have put it, so that the caller's workspace holds the list
         // afterwards and later calls on this geometry can pass HSTU_FLAG_REUSE_WORKSPACE
-        if (tid < REC) const_cast<unsigned*>(ws)[WS_HEADER + REC * (size_t)blockIdx.x + tid] = lds_rec[tid];
+        if (tid < REC) {
+            const unsigned val = tid == 0 ? rw[0] : ((tid == 1 || tid == 3) ? rw[1] : ((tid == 2 || tid == 4) ? rw[2] : 0u));
+            const_cast<unsigned*>(ws)[WS_HEADER + REC * (size_t)blockIdx.x + tid] = val;
+        }
         if (blockIdx.x == 0 && tid == 0) {
             const_cast<unsigned*>(ws)[0] = 0u;
             *reinterpret_cast<int64_t*>(const_cast<unsigned*>(ws) + 2) = owned_rows;
@@ -1509,7 +1535,7 @@ bool mfma_supported(const KArgs& a, const char** name) {
     return true;
 }
 
-// The plain head-dim-128 variant without a schedule kernel (see SELF): one lane per sequence, at most 64 tile-count classes,
+// The plain head-dim-128 variant without a schedule kernel (see SELF): one lane per sequence, at most 64 tile-count classes (63 tile counts and the class of longer sequences),
 // and lists that cannot overflow (q and k share their offsets, so entries per group fall along the order).  A caller that
 // already holds a list (HSTU_FLAG_REUSE_WORKSPACE) keeps using it: reading a record is cheaper than deriving it.
 bool mfma_self_scheduled(const KArgs& a) {
@@ -1517,7 +1543,7 @@ bool mfma_self_scheduled(const KArgs& a) {
     return a.op == OP_JAGGED && (p.dtype == HSTU_BF16 || p.dtype == HSTU_F16) && p.dim_qk == 128 && p.dim_v == 128 &&
            p.batch <= 64 && p.seq_offset_q && p.seq_offset_q == p.seq_offset_k && !p.num_context && !p.num_target &&
            p.mask_type == HSTU_MASK_TRIL && !p.attn_bias && !p.ts_table &&
-           p.max_seq_len_q == p.max_seq_len_k && p.max_seq_len_q <= 64 * BM &&
+           p.max_seq_len_q == p.max_seq_len_k && p.max_seq_len_q <= 63 * BM &&
            !(p.flags & HSTU_FLAG_REUSE_WORKSPACE) && sched_dims(p).nsplit == 1;
 }
 

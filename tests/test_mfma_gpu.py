@@ -436,7 +436,7 @@ def test_limits_longest_sequence_and_most_groups():
 @pytest.mark.parametrize("lens,heads,max_len", [
     ([1], 1, 1), ([129], 3, 129), ([300, 0, 17, 0, 640], 4, 640), ([1000, 513, 512, 511, 129, 128, 127], 16, 1000),
     (list(range(0, 64 * 17, 17)), 2, 1071), ([700] * 64, 8, 700), ([900, 140, 400], 5, 256),
-    ([2000, 64, 8000, 1], 16, 8192)])
+    ([2000, 64, 8000, 1], 16, 8064), ([40] * 33 + [5000], 8, 4100)])
 def test_self_scheduled_small_batches(lens, heads, max_len, index_dtype):
     """Plain causal self-attention at head dim 128 on at most 64 sequences runs without the schedule kernel: every
     workgroup derives its item from the offsets.  Every row must be produced exactly as by the list-driven grid (the call
@@ -473,6 +473,9 @@ def test_self_scheduling_is_left_to_the_work_list_where_it_does_not_apply():
     cfg, _ = _jag(84, [200, 100], 2, 2, 128, 128, dtype)
     cfg["num_target"] = torch.tensor([5, 5])
     cfg["target_group_size"] = 1
+    assert not T.run_capi(cfg)[1].endswith("_selfsched")
+    cfg, _ = _jag(85, [200, 100], 2, 2, 128, 128, dtype)                       # an attribute of 64 Q tiles: one class too many
+    cfg["max_seq_len"] = 8192
     assert not T.run_capi(cfg)[1].endswith("_selfsched")
 
 
