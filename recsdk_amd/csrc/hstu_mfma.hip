@@ -439,42 +439,55 @@ __device__ __forceinline__ unsigned small_div(unsigned x, unsigned y) {
 }
 
 // The record of workgroup blockIdx.x without a work list, computed by one wave on its own (the caller guarantees
-// batch <= 64, at most 63 Q tiles per sequence under the attribute, one set of offsets for q and k, no context or target
-// rows, the plain causal mask).  The order is the schedule kernel's with a coarser key: sequences by their number of Q
-// tiles (longest first, then by batch index), (sequence, head) groups r = rank * heads + head dealt to the XCDs in snake
-// order (XCD x owns r = 16 u + x and 16 u + 15 - x), a group's tiles last tile first, the first two tiles of a sequence
-// of five or more tiles as one item.  Lane b first holds sequence b, then lane k holds the class of the sequences with
-// cmax - k tiles (a histogram in `hist`, 64 words of LDS private to the wave): the sequences and the list entries ahead
-// of a class are two prefix sums over the lanes, so the cost does not grow with the number of classes.  No list can
-// exceed the grid: with entries per group falling along r, the lists differ by at most one group's entries.
+// batch <= 128, at most 63 Q tiles per sequence under the attribute, one set of offsets for q and k, no context rows, the
+// built-in causal mask; target rows are fine).  The order is the schedule kernel's with a coarser key: sequences by
+// their number of Q tiles (longest first, then by batch index), (sequence, head) groups r = rank * heads + head dealt to
+// the XCDs in snake order (XCD x owns r = 16 u + x and 16 u + 15 - x), a group's tiles last tile first, the first two
+// tiles of a sequence of five or more tiles as one item.  Lane b first holds sequences b and b + 64, then lane k holds the
+// class of the sequences with cmax - k tiles (a histogram in `hist`, 64 words of LDS private to the wave): the sequences
+// and the list entries ahead of a class are two prefix sums over the lanes, so the cost does not grow with the number of
+// classes.  No list can exceed the grid: with entries per group falling along r, the lists differ by at most one group's
+// entries.
 __device__ __forceinline__ void self_record(const KArgs& a, int ntiles_attr, int lane, unsigned* hist, unsigned (&rec)[REC], int64_t& rows) {
     const hstu_fwd_params& p = a.p;
     const int B = p.batch, H = p.heads_q;
     const int is64 = p.index_type == HSTU_I64;
-    const bool mine = lane < B;
-    // offsets b and b + 1 of lane b's sequence in one load (two dependent loads would double the wait)
+    // offsets b and b + 1 of a sequence in one load (two dependent loads would double the wait)
     struct __attribute__((aligned(8))) I64x2 { int64_t lo, hi; };
     struct __attribute__((aligned(4))) I32x2 { int lo, hi; };
-    const int mb = mine ? lane : 0;
-    int64_t o0, o1;
-    if (is64) {
-        const I64x2 v = *reinterpret_cast<const I64x2*>(static_cast<const int64_t*>(p.seq_offset_q) + mb);
-        o0 = v.lo; o1 = v.hi;
-    } else {
-        const I32x2 v = *reinterpret_cast<const I32x2*>(static_cast<const int*>(p.seq_offset_q) + mb);
-        o0 = v.lo; o1 = v.hi;
-    }
-    const int len = (int)(o1 - o0);
-    // rows the sequences own = the last offset, which lane batch - 1 holds (a scalar load of its own would make every later
-    // wait for a kernel argument wait for a round trip to the L2 as well)
-    rows = (int64_t)(((uint64_t)(unsigned)__builtin_amdgcn_readlane((int)(o1 >> 32), B - 1) << 32) | (unsigned)__builtin_amdgcn_readlane((int)o1, B - 1));
-    const int t = (len + BM - 1) / BM;
-    // class of a sequence = its tile count; sequences longer than the attribute covers form the class above
     const int cmax = ntiles_attr + 1;
-    const int cls = mine ? min(t, cmax) : 0;
+    int64_t o0[2], o1[2];
+    int len[2], cls[2], tgt[2];
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+        const bool mine = lane + 64 * u < B;
+        const int mb = mine ? lane + 64 * u : 0;
+        if (is64) {
+            const I64x2 v = *reinterpret_cast<const I64x2*>(static_cast<const int64_t*>(p.seq_offset_q) + mb);
+            o0[u] = v.lo; o1[u] = v.hi;
+        } else {
+            const I32x2 v = *reinterpret_cast<const I32x2*>(static_cast<const int*>(p.seq_offset_q) + mb);
+            o0[u] = v.lo; o1[u] = v.hi;
+        }
+        tgt[u] = p.num_target ? (int)ld_idx(p.num_target, mb, is64) : 0;
+    }
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+        len[u] = (int)(o1[u] - o0[u]);
+        // class of a sequence = its tile count; sequences longer than the attribute covers form the class above
+        cls[u] = lane + 64 * u < B ? min((len[u] + BM - 1) / BM, cmax) : 0;
+    }
+    // rows the sequences own = the last offset, which the lane of sequence batch - 1 holds (a scalar load of its own would make
+    // every later wait for a kernel argument wait for a round trip to the L2 as well)
+    {
+        const int64_t last = B > 64 ? o1[1] : o1[0];
+        const int ll = (B - 1) & 63;
+        rows = (int64_t)(((uint64_t)(unsigned)__builtin_amdgcn_readlane((int)(last >> 32), ll) << 32) | (unsigned)__builtin_amdgcn_readlane((int)last, ll));
+    }
     hist[lane] = 0u;
     __builtin_amdgcn_wave_barrier();
-    if (cls > 0) atomicAdd(&hist[cmax - cls], 1u);
+    if (cls[0] > 0) atomicAdd(&hist[cmax - cls[0]], 1u);
+    if (cls[1] > 0) atomicAdd(&hist[cmax - cls[1]], 1u);
     __builtin_amdgcn_wave_barrier();
     const unsigned n = hist[lane];                       // sequences of class c
     const int c = cmax - lane;                           // (lanes from cmax on: n = 0)
@@ -503,17 +516,25 @@ __device__ __forceinline__ void self_record(const KArgs& a, int ntiles_attr, int
     // group found_g of this XCD's list: r = 16 (g / 2) + (x or 15 - x); its sequence is the (rank - found_first)-th of its class
     const unsigned r = 16u * (found_g >> 1) + ((found_g & 1u) ? 15u - x : x);
     const unsigned rank = small_div(r, (unsigned)H), h = r - rank * (unsigned)H;
-    const unsigned long long m = __ballot(cls == found_cls);
-    const unsigned nth = rank - found_first;
+    // the nth sequence of the class in batch order: sequences 0..63 first, then 64..127
+    const unsigned long long m0 = __ballot(cls[0] == found_cls), m1 = __ballot(cls[1] == found_cls);
+    unsigned nth = rank - found_first;
+    const unsigned in0 = (unsigned)__builtin_popcountll(m0);
+    const bool second = nth >= in0;
+    const unsigned long long m = second ? m1 : m0;
+    if (second) nth -= in0;
     const unsigned before_me = __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)m, 0u));
-    const unsigned long long pick = __ballot(cls == found_cls && before_me == nth);
-    const int fb = pick ? __builtin_ctzll(pick) : 0;
-    const unsigned q0 = (unsigned)__builtin_amdgcn_readlane((int)o0, fb), lq = (unsigned)__builtin_amdgcn_readlane(len, fb);
+    const unsigned long long pick = __ballot(((m >> lane) & 1ull) && before_me == nth);
+    const int fl = pick ? __builtin_ctzll(pick) : 0;
+    const unsigned q0 = (unsigned)__builtin_amdgcn_readlane((int)(second ? o0[1] : o0[0]), fl);
+    const unsigned lq = (unsigned)__builtin_amdgcn_readlane(second ? len[1] : len[0], fl);
+    const unsigned tg = (unsigned)__builtin_amdgcn_readlane(second ? tgt[1] : tgt[0], fl);
+    const unsigned fb = (unsigned)fl + (second ? 64u : 0u);
     const bool sw = found_cls > ntiles_attr, pr = !sw && found_cls >= 5;
     const bool both = pr && found_i == found_e - 1;
     const unsigned tile = both ? 0u : (found_e - 1 - found_i) + (pr ? 1u : 0u), part = both ? 1u : 0u;
-    rec[0] = (unsigned)fb | h << 12 | tile << 16 | ((found_i == 0 && sw) ? 1u << 24 : 0u) | part << 25 | 1u << 28;
-    rec[1] = q0; rec[2] = lq; rec[3] = q0; rec[4] = lq; rec[5] = 0u; rec[6] = 0u; rec[7] = 0u;
+    rec[0] = fb | h << 12 | tile << 16 | ((found_i == 0 && sw) ? 1u << 24 : 0u) | part << 25 | 1u << 28;
+    rec[1] = q0; rec[2] = lq; rec[3] = q0; rec[4] = lq; rec[5] = 0u; rec[6] = tg; rec[7] = 0u;
 }
 
 // EXTRA: 5 / 6 / 7 = a dense bias / a custom mask / both, rows on 16-byte boundaries, and nothing else: the general
@@ -655,7 +676,7 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
         // the record also goes where the schedule kernel would have put it, so that the caller's workspace holds the list
         // afterwards and later calls on this geometry can pass HSTU_FLAG_REUSE_WORKSPACE
         if (tid < REC) {
-            const unsigned val = tid == 0 ? rw[0] : ((tid == 1 || tid == 3) ? rw[1] : ((tid == 2 || tid == 4) ? rw[2] : 0u));
+            const unsigned val = tid == 0 ? rw[0] : ((tid == 1 || tid == 3) ? rw[1] : ((tid == 2 || tid == 4) ? rw[2] : (tid == 6 ? rw[6] : 0u)));
             const_cast<unsigned*>(ws)[WS_HEADER + REC * (size_t)blockIdx.x + tid] = val;
         }
         if (blockIdx.x == 0 && tid == 0) {
@@ -1535,14 +1556,36 @@ bool mfma_supported(const KArgs& a, const char** name) {
     return true;
 }
 
-// The plain head-dim-128 variant without a schedule kernel (see SELF): one lane per sequence, at most 64 tile-count classes (63 tile counts and the class of longer sequences),
-// and lists that cannot overflow (q and k share their offsets, so entries per group fall along the order).  A caller that
-// already holds a list (HSTU_FLAG_REUSE_WORKSPACE) keeps using it: reading a record is cheaper than deriving it.
+// Which variant of the kernel (template argument EXTRA, before the paged / padded choices) the options of a call ask for.
+static int forward_extra(const KArgs& a) {
+    const hstu_fwd_params& p = a.p;
+    const bool dense_extra = p.attn_bias || p.mask_type == HSTU_MASK_CUSTOM;
+    // the time table is used from LDS when it fits and the search hint is there; else the general path searches the
+    // bounds in global memory
+    // the LDS time table: buckets at least a factor 2^(1/5) apart (wider than its cells) and the last bound below 2^62
+    const bool ts_in_lds = p.ts_table && p.ts_log2_scale > 0.f && p.ts_log2_scale <= 5.0f && p.num_buckets <= 62.f * p.ts_log2_scale;
+    // a dense bias and / or a custom mask alone, rows on 16-byte boundaries: the variants without the other options
+    const bool custom = p.mask_type == HSTU_MASK_CUSTOM;
+    const bool dense_only = dense_extra && !p.pos_table && !p.ts_table && a.op != OP_PAGED && p.max_seq_len_k % 8 == 0 &&
+                            ((reinterpret_cast<uintptr_t>(p.attn_bias) | (custom ? reinterpret_cast<uintptr_t>(p.mask) : 0)) & 15) == 0;
+    if (dense_only) return p.attn_bias ? (custom ? 7 : 5) : 6;
+    if (dense_extra || (p.ts_table && !ts_in_lds)) return 1;
+    if (p.pos_table && p.ts_table) return 4;
+    if (p.ts_table) return 3;
+    if (p.pos_table) return 2;
+    return 0;
+}
+
+// Launches without a schedule kernel (see SELF): the variants with the built-in mask and at most the bias tables at head
+// dims 64 and 128, one or two sequences per lane, at most 64 tile-count classes (63 tile counts and the class of longer
+// sequences), and lists that cannot overflow (q and k share their offsets, so entries per group fall along the order).
+// A caller that already holds a list (HSTU_FLAG_REUSE_WORKSPACE) keeps using it.
 bool mfma_self_scheduled(const KArgs& a) {
     const hstu_fwd_params& p = a.p;
-    return a.op == OP_JAGGED && (p.dtype == HSTU_BF16 || p.dtype == HSTU_F16) && p.dim_qk == 128 && p.dim_v == 128 &&
-           p.batch <= 64 && p.seq_offset_q && p.seq_offset_q == p.seq_offset_k && !p.num_context && !p.num_target &&
-           p.mask_type == HSTU_MASK_TRIL && !p.attn_bias && !p.ts_table &&
+    const int extra = forward_extra(a);
+    return a.op == OP_JAGGED && (p.dtype == HSTU_BF16 || p.dtype == HSTU_F16) && p.dim_qk == p.dim_v && (p.dim_qk == 128 || p.dim_qk == 64) &&
+           p.batch >= 1 && p.batch <= 128 && p.seq_offset_q && p.seq_offset_q == p.seq_offset_k && !p.num_context &&
+           p.mask_type == HSTU_MASK_TRIL && (extra == 0 || (extra >= 2 && extra <= 4)) &&
            p.max_seq_len_q == p.max_seq_len_k && p.max_seq_len_q <= 63 * BM &&
            !(p.flags & HSTU_FLAG_REUSE_WORKSPACE) && sched_dims(p).nsplit == 1;
 }
@@ -1560,33 +1603,20 @@ template <typename T, int D>
 static hipError_t launch_td(const KArgs& a, unsigned* ws, hipStream_t stream) {
     const hstu_fwd_params& p = a.p;
     const SchedDims d = sched_dims(p);
-    const bool dense_extra = p.attn_bias || p.mask_type == HSTU_MASK_CUSTOM;
-    // the time table is used from LDS when it fits and the search hint is there; else the general path searches the
-    // bounds in global memory
-    // the LDS time table: buckets at least a factor 2^(1/5) apart (wider than its cells) and the last bound below 2^62
-    const bool ts_in_lds = p.ts_table && p.ts_log2_scale > 0.f && p.ts_log2_scale <= 5.0f && p.num_buckets <= 62.f * p.ts_log2_scale;
-    // a dense bias and / or a custom mask alone, rows on 16-byte boundaries: the variants without the other options
-    const bool custom = p.mask_type == HSTU_MASK_CUSTOM;
-    const bool dense_only = dense_extra && !p.pos_table && !p.ts_table && a.op != OP_PAGED && p.max_seq_len_k % 8 == 0 &&
-                            ((reinterpret_cast<uintptr_t>(p.attn_bias) | (custom ? reinterpret_cast<uintptr_t>(p.mask) : 0)) & 15) == 0;
-    int extra = 0;
-    if (dense_only) extra = p.attn_bias ? (custom ? 7 : 5) : 6;
-    else if (dense_extra || (p.ts_table && !ts_in_lds)) extra = 1;
-    else if (p.pos_table && p.ts_table) extra = 4;
-    else if (p.ts_table) extra = 3;
-    else if (p.pos_table) extra = 2;
+    const int extra = forward_extra(a);
     const bool paged = a.op == OP_PAGED;
     const int groups = p.batch * p.heads_q;
     const int sched_threads = groups <= 128 ? 256 : (groups <= 512 ? 512 : SCHED_NT);   // spare threads write a group's records side by side
     hipError_t e = hipSuccess;
     dim3 grid(8 * d.cap), block(NT);   // the overflow list starts at entry gridDim.x of the lists
     const float* part = reinterpret_cast<const float*>(reinterpret_cast<const char*>(ws) + list_bytes(d));
-    if constexpr (D == 128) {
-        // small batches: the workgroups of the plain variant (and of the one with a position table) find their items themselves,
-        // no schedule kernel
-        if ((extra == 0 || extra == 2) && !paged && mfma_self_scheduled(a)) {
+    if constexpr (D == 128 || D == 64) {
+        // small batches: the workgroups find their items themselves, no schedule kernel
+        if (!paged && mfma_self_scheduled(a)) {
             if (extra == 0) hipLaunchKernelGGL((hstu_mfma_kernel<T, D, 0, false, true>), grid, block, 0, stream, a, ws, part);
-            else hipLaunchKernelGGL((hstu_mfma_kernel<T, D, 2, false, true>), grid, block, 0, stream, a, ws, part);
+            else if (extra == 2) hipLaunchKernelGGL((hstu_mfma_kernel<T, D, 2, false, true>), grid, block, 0, stream, a, ws, part);
+            else if (extra == 3) hipLaunchKernelGGL((hstu_mfma_kernel<T, D, 3, false, true>), grid, block, 0, stream, a, ws, part);
+            else hipLaunchKernelGGL((hstu_mfma_kernel<T, D, 4, false, true>), grid, block, 0, stream, a, ws, part);
             return hipGetLastError();
         }
     }

@@ -128,8 +128,9 @@ def test_paged_and_dense_validation():
 def test_describe_kernel_selection():
     buf = C.create_string_buffer(64)
     lib = _capi.lib()
-    for over, want in [(dict(), "mfma_bf16_d128_selfsched"), (dict(flags=_capi.FLAG_REUSE_WORKSPACE), "mfma_bf16_d128"), (dict(batch=65), "mfma_bf16_d128"),
-                       (dict(dim_qk=64, dim_v=64, dtype=_capi.HSTU_F16), "mfma_f16_d64"),
+    for over, want in [(dict(), "mfma_bf16_d128_selfsched"), (dict(flags=_capi.FLAG_REUSE_WORKSPACE), "mfma_bf16_d128"), (dict(batch=128), "mfma_bf16_d128_selfsched"), (dict(batch=129), "mfma_bf16_d128"),
+                       (dict(num_target=0x2000), "mfma_bf16_d128_selfsched"), (dict(num_context=0x2000), "mfma_bf16_d128"),
+                       (dict(dim_qk=64, dim_v=64, dtype=_capi.HSTU_F16), "mfma_f16_d64_selfsched"),
                        (dict(dtype=_capi.HSTU_F32), "generic_f32"), (dict(dim_v=64), "mfma_bf16_d128_padded"), (dict(dim_qk=64, dim_v=32), "mfma_bf16_d64_padded"),
                        (dict(dim_qk=72, dim_v=64), "generic_bf16"), (dict(dim_v=64, attn_bias=0x1000), "generic_bf16"),
                        (dict(dim_qk=32, dim_v=32), "mfma_bf16_d32"), (dict(dim_qk=256, dim_v=256, dtype=_capi.HSTU_F16), "mfma_f16_d256"),

@@ -164,7 +164,7 @@ def test_mfma_time_table_bucket_range(d, nb, divisor, gap):
     ts = [1_700_000_000 + np.cumsum(rng.exponential(gap, l).astype(np.int64)) for l in lens]
     cfg["timestamps"] = torch.from_numpy(np.concatenate(ts))
     out, name = T.run_capi(cfg)
-    assert name == f"mfma_bf16_d{d}", name
+    assert name == f"mfma_bf16_d{d}_selfsched", name
     T.assert_parity(out, T.oracle_jagged(cfg), torch.bfloat16, what="time table range")
     gen, _ = T.run_capi(cfg, flags=FORCE_GENERIC)
     T.assert_parity(out, gen.float(), torch.bfloat16, what="time table range vs generic kernel")
@@ -246,7 +246,7 @@ def test_config4_target_aware():
     say("config4", sum(cfg["lens"]))
     ref = T.oracle_jagged(cfg)
     out, name = T.run_capi(cfg)
-    assert name == "mfma_bf16_d64"
+    assert name == "mfma_bf16_d64_selfsched"
     T.assert_parity(out, ref, torch.bfloat16, what="config4")
 
 
@@ -268,7 +268,9 @@ def test_config4_full_size_properties():
     say("config4_full", sum(cfg["lens"]))
     dtype = torch.bfloat16
     out, name = T.run_capi(cfg)
-    assert name == "mfma_bf16_d64"
+    assert name == "mfma_bf16_d64_selfsched"
+    again, _ = T.run_capi(cfg, reuse_from=cfg)      # the same launch over the list that the first call left in the workspace
+    assert torch.equal(out, again)
     gen, _ = T.run_capi(cfg, flags=FORCE_GENERIC)
     T.assert_parity(out, gen.float(), dtype, what="config4 full size vs generic kernel")
     assert torch.equal(T.run_op(cfg, op="table"), out)
@@ -463,16 +465,47 @@ def test_self_scheduled_small_batches(lens, heads, max_len, index_dtype):
             T.assert_parity(out, T.oracle_jagged(cfg), dtype, what="self-scheduled with a position table vs oracle")
 
 
+@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("nseq,heads,tables", [(65, 2, "none"), (128, 4, "both"), (100, 1, "pos"), (128, 16, "time"), (7, 3, "both")])
+def test_self_scheduled_two_sequences_per_lane_targets_and_tables(d, nseq, heads, tables):
+    """Up to 128 sequences (a lane of the deriving wave then holds two), target rows, head dim 64 and the variants with
+    bias tables also run without the schedule kernel: same bits as over the list the call leaves behind, parity with the
+    plain kernel, and with the oracle where that takes seconds."""
+    say("self_scheduled_wide", d, nseq, heads, tables)
+    dtype = torch.bfloat16
+    rng = np.random.default_rng(90 + nseq)
+    lens = [int(x) for x in rng.integers(0, 700, nseq)]
+    lens[nseq // 2] = 0
+    lens[-1] = 900                                   # the last sequence (its offset is the row count) is the longest
+    cfg, _ = _jag(90 + nseq, lens, heads, heads, d, d, dtype)
+    cfg["num_target"] = torch.tensor([min(l, int(t)) for l, t in zip(lens, rng.integers(0, 40, nseq))])
+    cfg["target_group_size"] = 2
+    if tables in ("pos", "both"):
+        cfg["pos_table"] = torch.from_numpy(rng.normal(0, 0.5, 2 * cfg["max_seq_len"] - 1).astype(np.float32))
+    if tables in ("time", "both"):
+        cfg["ts_table"] = torch.from_numpy(rng.normal(0, 0.5, 129).astype(np.float32))
+        cfg["timestamps"] = torch.from_numpy(np.concatenate([1_700_000_000 + np.cumsum(rng.exponential(600.0, l).astype(np.int64)) for l in lens]))
+    out, name = T.run_capi(cfg)
+    assert name == f"mfma_bf16_d{d}_selfsched", name
+    again, _ = T.run_capi(cfg, reuse_from=cfg)
+    assert torch.equal(out, again)
+    gen, _ = T.run_capi(cfg, flags=FORCE_GENERIC)
+    T.assert_parity(out, gen.float(), dtype, what="self-scheduled (wide) vs generic kernel")
+    if sum(lens) * heads <= 12000:
+        T.assert_parity(out, T.oracle_jagged(cfg), dtype, what="self-scheduled (wide) vs oracle")
+
+
 def test_self_scheduling_is_left_to_the_work_list_where_it_does_not_apply():
     say("self_scheduled: not taken")
     dtype = torch.bfloat16
-    cfg, _ = _jag(82, [200] * 65, 2, 2, 128, 128, dtype)                       # more than 64 sequences
+    cfg, _ = _jag(82, [200] * 129, 2, 2, 128, 128, dtype)                      # more than 128 sequences
     assert not T.run_capi(cfg)[1].endswith("_selfsched")
     cfg, _ = _jag(83, [200, 100], 2, 2, 128, 128, dtype, lens_k=[300, 100])    # K longer than Q
     assert not T.run_capi(cfg)[1].endswith("_selfsched")
     cfg, _ = _jag(84, [200, 100], 2, 2, 128, 128, dtype)
-    cfg["num_target"] = torch.tensor([5, 5])
-    cfg["target_group_size"] = 1
+    cfg["num_context"] = torch.tensor([5, 5])                                  # context rows
+    assert not T.run_capi(cfg)[1].endswith("_selfsched")
+    cfg, _ = _jag(86, [200, 100], 2, 2, 32, 32, dtype)                         # head dim 32
     assert not T.run_capi(cfg)[1].endswith("_selfsched")
     cfg, _ = _jag(85, [200, 100], 2, 2, 128, 128, dtype)                       # an attribute of 64 Q tiles: one class too many
     cfg["max_seq_len"] = 8192
