@@ -38,6 +38,7 @@ bool mfma_self_scheduled(const KArgs& a);
 bool mfma_fp8_supported(const KArgs& a, const char** name);
 uint64_t mfma_fp8_workspace_bytes(const KArgs& a);
 hipError_t launch_mfma_fp8(const KArgs& a, void* workspace, hipStream_t stream);
+bool mfma_fp8_self_scheduled(const KArgs& a);
 
 // The device-built work list of the MFMA kernels, for kernels outside hstu_mfma.hip.  Layout (uint32 words): 16 header
 // words ([2..3] = rows the sequences own, int64), then `grid` records of 8 words, read by workgroup index:

@@ -17,6 +17,7 @@
 // then keys 16u + 8g .. + 7 of the block, 8 consecutive keys per transposing read.  alpha * silu_scale cannot move to the
 // epilogue here: it decides where P falls on the e4m3 grid.
 #include "hstu_device.h"
+#include "hstu_self_sched.h"
 
 namespace hstu {
 
@@ -51,7 +52,9 @@ template <int D> struct Fp8Shape { static constexpr int WAVES = D == 64 ? 4 : (D
 // UNEVEN: head dims that are other multiples of 16 up to D, and dim_qk != dim_v (the reference's fp8 sweep draws dim_v from
 // 16 .. 80, test_hstu_jagged_forward.py): rows have their real widths in memory, the chunks past them are zeros in the
 // fragments and in LDS, the output keeps its dim_v columns.
-template <int D, bool UNEVEN = false>
+// SELF: no schedule kernel; every wave derives the workgroup's record from the offsets (self_record) and wave 0 leaves it in
+// the workspace, where the schedule kernel would have put it.
+template <int D, bool UNEVEN = false, bool SELF = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(Fp8Shape<D>::WAVES, Fp8Shape<D>::WAVES)))
 void hstu_mfma_fp8_kernel(const KArgs a, const unsigned* __restrict__ ws) {
     const hstu_fwd_params& p = a.p;
@@ -70,12 +73,27 @@ void hstu_mfma_fp8_kernel(const KArgs a, const unsigned* __restrict__ ws) {
 
     // workgroup -> record of the device-built work list
     unsigned rw[WORK_RECORD_WORDS];
-    {
+    int64_t owned_rows;
+    if constexpr (SELF) {
+        __shared__ unsigned lds_hist[4 * 64];
+        unsigned rv[WORK_RECORD_WORDS];
+        self_record(a, (p.max_seq_len_q + FBM - 1) / FBM, lane, lds_hist + 64 * w, rv, owned_rows);
+#pragma unroll
+        for (int i = 0; i < WORK_RECORD_WORDS; i++) rw[i] = __builtin_amdgcn_readfirstlane(rv[i]);
+        if (tid < WORK_RECORD_WORDS) {
+            const unsigned val = tid == 0 ? rw[0] : ((tid == 1 || tid == 3) ? rw[1] : ((tid == 2 || tid == 4) ? rw[2] : (tid == 6 ? rw[6] : 0u)));
+            const_cast<unsigned*>(ws)[WORK_HEADER_WORDS + WORK_RECORD_WORDS * (size_t)blockIdx.x + tid] = val;
+        }
+        if (blockIdx.x == 0 && tid == 0) {
+            const_cast<unsigned*>(ws)[0] = 0u;
+            *reinterpret_cast<int64_t*>(const_cast<unsigned*>(ws) + 2) = owned_rows;
+        }
+    } else {
         const unsigned* rec = ws + WORK_HEADER_WORDS + WORK_RECORD_WORDS * (size_t)blockIdx.x;
 #pragma unroll
         for (int i = 0; i < WORK_RECORD_WORDS; i++) rw[i] = rec[i];
+        owned_rows = *reinterpret_cast<const int64_t*>(ws + 2);
     }
-    const int64_t owned_rows = *reinterpret_cast<const int64_t*>(ws + 2);
     const unsigned item = rw[0];
     const bool active = item != WORK_ITEM_EMPTY;
     const int b = active ? (int)(item & 0xfff) : 0, h = active ? (int)((item >> 12) & 0xf) : 0;
@@ -345,14 +363,30 @@ bool mfma_fp8_supported(const KArgs& a, const char** name) {
 
 uint64_t mfma_fp8_workspace_bytes(const KArgs& a) { return work_list_shape(a.p).bytes; }
 
+// launches without the schedule kernel: the conditions of the 16-bit kernels (mfma_self_scheduled)
+bool mfma_fp8_self_scheduled(const KArgs& a) {
+    const hstu_fwd_params& p = a.p;
+    return a.op == OP_JAGGED && p.batch >= 1 && p.batch <= 128 && p.seq_offset_q && p.seq_offset_q == p.seq_offset_k && !p.num_context &&
+           p.mask_type == HSTU_MASK_TRIL && p.max_seq_len_q == p.max_seq_len_k && p.max_seq_len_q <= 63 * FBM &&
+           !(p.flags & HSTU_FLAG_REUSE_WORKSPACE);
+}
+
 hipError_t launch_mfma_fp8(const KArgs& a, void* workspace, hipStream_t stream) {
     const hstu_fwd_params& p = a.p;
     unsigned* ws = reinterpret_cast<unsigned*>(workspace);
+    const dim3 grid(work_list_shape(p).grid), block(256);
+    if (!fp8_uneven(p) && mfma_fp8_self_scheduled(a)) {
+        switch (p.dim_qk) {
+            case 64: hipLaunchKernelGGL((hstu_mfma_fp8_kernel<64, false, true>), grid, block, 0, stream, a, ws); break;
+            case 128: hipLaunchKernelGGL((hstu_mfma_fp8_kernel<128, false, true>), grid, block, 0, stream, a, ws); break;
+            default: hipLaunchKernelGGL((hstu_mfma_fp8_kernel<256, false, true>), grid, block, 0, stream, a, ws); break;
+        }
+        return hipGetLastError();
+    }
     if (!(p.flags & HSTU_FLAG_REUSE_WORKSPACE)) {
         const hipError_t e = launch_work_list(a, ws, true, stream);
         if (e != hipSuccess) return e;
     }
-    const dim3 grid(work_list_shape(p).grid), block(256);
     if (fp8_uneven(p)) {
         switch (fp8_padded_dim(p)) {
             case 64: hipLaunchKernelGGL((hstu_mfma_fp8_kernel<64, true>), grid, block, 0, stream, a, ws); break;

@@ -161,7 +161,8 @@ def test_fp8_inputs_selection_and_rejections():
     buf = C.create_string_buffer(64)
     lib = _capi.lib()
     fp8 = dict(dtype=_capi.HSTU_FP8_E4M3)
-    for over, want in [(dict(), "mfma_fp8_d128"), (dict(dim_qk=64, dim_v=64), "mfma_fp8_d64"), (dict(dim_qk=256, dim_v=256), "mfma_fp8_d256"),
+    for over, want in [(dict(), "mfma_fp8_d128_selfsched"), (dict(dim_qk=64, dim_v=64), "mfma_fp8_d64_selfsched"), (dict(dim_qk=256, dim_v=256), "mfma_fp8_d256_selfsched"),
+                       (dict(batch=129), "mfma_fp8_d128"), (dict(flags=_capi.FLAG_REUSE_WORKSPACE), "mfma_fp8_d128"),
                        (dict(dim_qk=32, dim_v=32), "mfma_fp8_d64_padded"), (dict(dim_qk=96, dim_v=80), "mfma_fp8_d128_padded"),
                        (dict(dim_qk=72, dim_v=32), "generic_fp8"), (dict(dim_qk=96, dim_v=80, attn_bias=0x1000), "generic_fp8"),
                        (dict(attn_bias=0x1000), "generic_fp8"), (dict(mask_type=3, mask=0x1000), "generic_fp8"),

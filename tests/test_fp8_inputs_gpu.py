@@ -176,7 +176,9 @@ def test_fp8_full_size_training_batch():
         cfg[x] = (torch.rand(cfg[x].shape, generator=g) * 2 - 1).to(FP8)
     cfg["silu_scale"] = 1.0 / 64
     out, name = T.run_capi(cfg)
-    assert name == "mfma_fp8_d128", name
+    assert name == "mfma_fp8_d128_selfsched", name
+    again, _ = T.run_capi(cfg, reuse_from=cfg)      # the same launch over the list that the first call left in the workspace
+    assert torch.equal(out, again)
     gen, gname = T.run_capi(cfg, flags=FORCE_GENERIC)
     assert gname == "generic_fp8"
     _close(out, gen, "fp8 config 2, matrix-core vs plain kernel")
