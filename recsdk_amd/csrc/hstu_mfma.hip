@@ -685,14 +685,6 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
         float ts_top = 1.0f;
         if (tab_ts) {
             ts_top = fminf(p.ts_bounds[p.num_buckets], __builtin_bit_cast(float, 0x3f800000u + ((unsigned)(TS_CELLS - 1) << 20)));
-            for (int c = tid; c < TS_CELLS; c += NT) {
-                // bucket of the cell's lowest value: the rounded log estimate f or f - 1, the exact bound of f decides
-                const float lo = __builtin_bit_cast(float, 0x3f800000u + ((unsigned)c << 20));
-                const int f = min((int)(__builtin_amdgcn_logf(lo) * p.ts_log2_scale + 0.5f), p.num_buckets + 1);
-                const int bk = max(min(lo >= p.ts_bounds[f] ? f : f - 1, p.num_buckets), 0);
-                const f32x4 entry = {p.ts_bounds[bk + 1], p.ts_table[bk], p.ts_table[min(bk + 1, p.num_buckets)], p.ts_bounds[min(bk + 2, p.num_buckets + 1)]};
-                *reinterpret_cast<f32x4*>(lds_tsq + 4 * c) = entry;
-            }
         }
         float pw_reg = 0.f;
         double tk_reg = 0;
@@ -1012,6 +1004,18 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
         const int kt0 = part * per, kt1 = min(ntk, kt0 + per);
         if (kt0 < kt1) fetch(kt0, lds0);
         if (XDMA && kt0 < kt1) fetch_x(kt0, lds_xd0);
+        if (tab_ts) {
+            // the cells of the time table, built behind the request for the first K/V tile: the two dependent reads per cell
+            // (bound, then values) then run while that tile is on its way; the barrier in stash() publishes them
+            for (int c = tid; c < TS_CELLS; c += NT) {
+                // bucket of the cell's lowest value: the rounded log estimate f or f - 1, the exact bound of f decides
+                const float lo = __builtin_bit_cast(float, 0x3f800000u + ((unsigned)c << 20));
+                const int f = min((int)(__builtin_amdgcn_logf(lo) * p.ts_log2_scale + 0.5f), p.num_buckets + 1);
+                const int bk = max(min(lo >= p.ts_bounds[f] ? f : f - 1, p.num_buckets), 0);
+                const f32x4 entry = {p.ts_bounds[bk + 1], p.ts_table[bk], p.ts_table[min(bk + 1, p.num_buckets)], p.ts_bounds[min(bk + 2, p.num_buckets + 1)]};
+                *reinterpret_cast<f32x4*>(lds_tsq + 4 * c) = entry;
+            }
+        }
         stash(kt0, lds0);
 #ifdef HSTU_ITEM_TIMING
         if (it1 == it0) it1 = __builtin_amdgcn_s_memrealtime();
