@@ -31,7 +31,7 @@ TRAFFIC_SOURCE = {"config2": "profiles/hstu_mfma_kernel_configs2-5.md", "config3
                   "nmd_fwd": "profiles/hstu_nmd_kernels.md", "nmd_bwd": "profiles/hstu_nmd_kernels.md",
                   "in_linear_silu": "profiles/hstu_in_linear_silu_kernel.md", "in_linear_silu_bwd": "profiles/hstu_in_linear_silu_backward_kernels.md",
                   "kv_append_fp8": "profiles/hstu_kv_append_fp8_kernels.md"}
-MEASURED_TRAFFIC_BYTES = {"config2": 183.3e6, "config3": 113.4e6, "config4": 140.8e6, "config5": 205.8e6, "config2_bwd": 682.4e6, "config2_fp8": 116.5e6, "ref_bias": 1553.7e6, "kv_append": 351.9e6, "rab_time": 1443.4e6, "rab_time_bwd": 1589.7e6, "rab_pos": 297.7e6,
+MEASURED_TRAFFIC_BYTES = {"config2": 189.9e6, "config3": 112.5e6, "config4": 142.2e6, "config5": 205.6e6, "config2_bwd": 662.8e6, "config2_fp8": 116.5e6, "ref_bias": 1553.7e6, "kv_append": 351.9e6, "rab_time": 1443.4e6, "rab_time_bwd": 1589.7e6, "rab_pos": 297.7e6,
                           "nmd_fwd": 826.4e6, "nmd_bwd": 1380.0e6, "in_linear_silu": 1092.8e6, "in_linear_silu_bwd": 1458.3e6, "kv_append_fp8": 268.4e6}
 
 
