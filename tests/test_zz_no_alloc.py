@@ -56,6 +56,30 @@ def test_noalloc_with_fp8_inputs():
     assert torch.equal(want.view(torch.int16), got.view(torch.int16))
 
 
+def test_noalloc_on_the_plain_kernel():
+    """HSTU_FLAG_FORCE_GENERIC (and everything else the matrix-core kernels do not take) runs the plain kernel, which uses no
+    device memory beyond its arguments: same bits as through the entry point with a workspace."""
+    from recsdk_amd import _capi
+    cfg = W.jagged_config(6, 4, 2, 64, 20, 200, torch.bfloat16, max_seq_len=200)
+    q, k, v = cfg["q"].cuda(), cfg["k"].cuda(), cfg["v"].cuda()
+    outs = []
+    for noalloc in (False, True):
+        out = torch.full_like(q, float("nan"))
+        p, keep = _capi.make_params(q, k, v, out, seq_offset_q=cfg["seq_offset"].cuda(), max_seq_len_q=cfg["max_seq_len"],
+                                    alpha=cfg["alpha"], flags=_capi.FLAG_FORCE_GENERIC)
+        assert _capi.describe_kernel(p) == "generic_bf16"
+        if noalloc:
+            free_before = torch.cuda.mem_get_info()[0]
+            _capi.run_noalloc(p)
+            torch.cuda.synchronize()
+            assert torch.cuda.mem_get_info()[0] == free_before
+        else:
+            _capi.run("jagged", p)
+        torch.cuda.synchronize()
+        outs.append(out.cpu())
+    assert torch.isfinite(outs[0].float()).all() and torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
+
+
 def test_noalloc_rejects_a_batch_beyond_its_array():
     """More (Q tile, head) items than the fixed array holds: HSTU_ERR_WORKSPACE and a message, nothing launched."""
     from recsdk_amd import _capi
