@@ -468,6 +468,15 @@ def test_self_scheduled_small_batches(lens, heads, max_len, index_dtype):
 @pytest.mark.parametrize("d", [64, 128])
 @pytest.mark.parametrize("nseq,heads,tables", [(65, 2, "none"), (128, 4, "both"), (100, 1, "pos"), (128, 16, "time"), (7, 3, "both")])
 def test_self_scheduled_two_sequences_per_lane_targets_and_tables(d, nseq, heads, tables):
+    _self_scheduled_wide(d, nseq, heads, tables, torch.int64)
+
+
+def test_self_scheduled_two_sequences_per_lane_int32_offsets():
+    _self_scheduled_wide(128, 128, 2, "pos", torch.int32)
+    _self_scheduled_wide(64, 97, 4, "none", torch.int32)
+
+
+def _self_scheduled_wide(d, nseq, heads, tables, index_dtype):
     """Up to 128 sequences (a lane of the deriving wave then holds two), target rows, head dim 64 and the variants with
     bias tables also run without the schedule kernel: same bits as over the list the call leaves behind, parity with the
     plain kernel, and with the oracle where that takes seconds."""
@@ -477,8 +486,8 @@ def test_self_scheduled_two_sequences_per_lane_targets_and_tables(d, nseq, heads
     lens = [int(x) for x in rng.integers(0, 700, nseq)]
     lens[nseq // 2] = 0
     lens[-1] = 900                                   # the last sequence (its offset is the row count) is the longest
-    cfg, _ = _jag(90 + nseq, lens, heads, heads, d, d, dtype)
-    cfg["num_target"] = torch.tensor([min(l, int(t)) for l, t in zip(lens, rng.integers(0, 40, nseq))])
+    cfg, _ = _jag(90 + nseq, lens, heads, heads, d, d, dtype, index_dtype=index_dtype)
+    cfg["num_target"] = torch.tensor([min(l, int(t)) for l, t in zip(lens, rng.integers(0, 40, nseq))], dtype=index_dtype)
     cfg["target_group_size"] = 2
     if tables in ("pos", "both"):
         cfg["pos_table"] = torch.from_numpy(rng.normal(0, 0.5, 2 * cfg["max_seq_len"] - 1).astype(np.float32))
