@@ -471,14 +471,20 @@ def test_self_scheduled_two_sequences_per_lane_targets_and_tables(d, nseq, heads
     _self_scheduled_wide(d, nseq, heads, tables, torch.int64)
 
 
+@pytest.mark.parametrize("d", [32, 256])
+@pytest.mark.parametrize("nseq,heads", [(3, 8), (64, 2), (128, 3)])
+def test_self_scheduled_plain_variant_at_head_dims_32_and_256(d, nseq, heads):
+    _self_scheduled_wide(d, nseq, heads, "none", torch.int64)
+
+
 def test_self_scheduled_two_sequences_per_lane_int32_offsets():
     _self_scheduled_wide(128, 128, 2, "pos", torch.int32)
     _self_scheduled_wide(64, 97, 4, "none", torch.int32)
 
 
 def _self_scheduled_wide(d, nseq, heads, tables, index_dtype):
-    """Up to 128 sequences (a lane of the deriving wave then holds two), target rows, head dim 64 and the variants with
-    bias tables also run without the schedule kernel: same bits as over the list the call leaves behind, parity with the
+    """Up to 128 sequences (a lane of the deriving wave then holds two), target rows, the other head dims and the variants
+    with bias tables also run without the schedule kernel: same bits as over the list the call leaves behind, parity with the
     plain kernel, and with the oracle where that takes seconds."""
     say("self_scheduled_wide", d, nseq, heads, tables)
     dtype = torch.bfloat16
@@ -514,7 +520,8 @@ def test_self_scheduling_is_left_to_the_work_list_where_it_does_not_apply():
     cfg, _ = _jag(84, [200, 100], 2, 2, 128, 128, dtype)
     cfg["num_context"] = torch.tensor([5, 5])                                  # context rows
     assert not T.run_capi(cfg)[1].endswith("_selfsched")
-    cfg, _ = _jag(86, [200, 100], 2, 2, 32, 32, dtype)                         # head dim 32
+    cfg, _ = _jag(86, [200, 100], 2, 2, 32, 32, dtype)                         # head dim 32 has the plain variant only
+    cfg["pos_table"] = torch.zeros(2 * cfg["max_seq_len"] - 1)
     assert not T.run_capi(cfg)[1].endswith("_selfsched")
     cfg, _ = _jag(85, [200, 100], 2, 2, 128, 128, dtype)                       # an attribute of 64 Q tiles: one class too many
     cfg["max_seq_len"] = 8192
