@@ -1489,16 +1489,18 @@ static int forward_extra(const KArgs& a) {
 }
 
 // Launches without a schedule kernel (see SELF): the variants with the built-in mask and at most the bias tables at head
-// dims 64 and 128 (the plain variant also at 32 and 256), one or two sequences per lane, at most 64 tile-count classes (63 tile counts and the class of longer
+// dims 64 and 128 (the plain variant also at 32), one or two sequences per lane, at most 64 tile-count classes (63 tile counts and the class of longer
 // sequences), and lists that cannot overflow (q and k share their offsets, so entries per group fall along the order).
 // A caller that already holds a list (HSTU_FLAG_REUSE_WORKSPACE) keeps using it.
 bool mfma_self_scheduled(const KArgs& a) {
     const hstu_fwd_params& p = a.p;
     if (p.dtype == HSTU_FP8_E4M3) return p.dim_qk == p.dim_v && (p.dim_qk == 64 || p.dim_qk == 128 || p.dim_qk == 256) && mfma_fp8_self_scheduled(a);
     const int extra = forward_extra(a);
-    const bool tables_too = p.dim_qk == 128 || p.dim_qk == 64;   // head dims 32 and 256 have the plain variant only
+    // head dim 32 has the plain variant only; at head dim 256 a SIMD holds one wave and nothing hides the derivation
+    // (level with the schedule kernel on small batches, slower on large ones)
+    const bool tables_too = p.dim_qk == 128 || p.dim_qk == 64;
     return a.op == OP_JAGGED && (p.dtype == HSTU_BF16 || p.dtype == HSTU_F16) && p.dim_qk == p.dim_v &&
-           (p.dim_qk == 32 || p.dim_qk == 64 || p.dim_qk == 128 || p.dim_qk == 256) &&
+           (p.dim_qk == 32 || p.dim_qk == 64 || p.dim_qk == 128) &&
            p.batch >= 1 && p.batch <= 128 && p.seq_offset_q && p.seq_offset_q == p.seq_offset_k && !p.num_context &&
            p.mask_type == HSTU_MASK_TRIL && (extra == 0 || (tables_too && extra >= 2 && extra <= 4)) &&
            p.max_seq_len_q == p.max_seq_len_k && p.max_seq_len_q <= 63 * BM &&
@@ -1528,7 +1530,7 @@ static hipError_t launch_td(const KArgs& a, unsigned* ws, hipStream_t stream) {
     hipError_t e = hipSuccess;
     dim3 grid(8 * d.cap), block(NT);   // the overflow list starts at entry gridDim.x of the lists
     const float* part = reinterpret_cast<const float*>(reinterpret_cast<const char*>(ws) + list_bytes(d));
-    if constexpr (D == 32 || D == 256) {
+    if constexpr (D == 32) {
         if (!paged && !uneven_dims(p) && mfma_self_scheduled(a)) {
             hipLaunchKernelGGL((hstu_mfma_kernel<T, D, 0, false, true>), grid, block, 0, stream, a, ws, part);
             return hipGetLastError();
