@@ -192,3 +192,44 @@ def test_fp8_full_size_training_batch():
     same = torch.ones(out.shape[0], dtype=torch.bool)
     same[off[b]:off[b + 1]] = False
     assert torch.equal(out3[same], out[same]) and not torch.equal(out3[~same], out[~same])
+
+
+def test_fp8_self_derived_launches_match_the_list_driven_launch_on_random_batches():
+    """Random batches of up to 128 sequences at head dims 64 / 128 / 256 (uniform, heavy-tailed, half-empty, equal and
+    tile-aligned lengths, attributes below / at / above the longest sequence, both offset dtypes, target rows): the launch
+    that derives its items gives the same bits as the same call made ineligible by a num_context of zeros (which runs over
+    the schedule kernel's list), and as a second call over the list it left."""
+    rng = np.random.default_rng(6)
+    taken = 0
+    for it in range(50):
+        B = int(rng.choice([1, 2, 3, 7, 16, 33, 63, 64, 65, 100, 127, 128])) if rng.random() < 0.5 else int(rng.integers(1, 129))
+        H = int(rng.choice([1, 2, 3, 4, 5, 8, 16]))
+        d = int(rng.choice([64, 128, 256]))
+        kind = int(rng.integers(0, 5))
+        cap = max(1, min(8064, 40000 // B))
+        if kind == 0: lens = rng.integers(0, cap + 1, B)
+        elif kind == 1: lens = np.minimum((rng.pareto(1.1, B) * 64).astype(np.int64), cap)
+        elif kind == 2: lens = np.where(rng.random(B) < 0.5, 0, rng.integers(0, cap + 1, B))
+        elif kind == 3: lens = np.full(B, int(rng.integers(1, cap + 1)))
+        else: lens = (rng.integers(0, max(2, cap // 128 + 1), B) * 128 + rng.choice([-1, 0, 1], B)).clip(0, cap)
+        lens = [int(x) for x in lens]
+        if sum(lens) == 0: lens[0] = 5
+        idt = torch.int64 if rng.random() < 0.5 else torch.int32
+        cfg, _ = _jag8(6000 + it, lens, H, H, d, d, index_dtype=idt, silu_scale=1.0 / 64)
+        mx, r = max(lens), rng.random()
+        cfg["max_seq_len"] = mx if r < 0.6 else (max(1, mx // 2) if r < 0.8 else min(8064, mx + int(rng.integers(0, 700))))
+        if rng.random() < 0.4:
+            cfg["num_target"] = torch.tensor([min(l, int(t)) for l, t in zip(lens, rng.integers(0, 50, B))], dtype=idt)
+            cfg["target_group_size"] = int(rng.integers(1, 4))
+        say("fp8_self_derived_random", it, B, H, d, kind, sum(lens), mx, cfg["max_seq_len"])
+        out, name = T.run_capi(cfg)
+        if not name.endswith("_selfsched"):
+            continue
+        taken += 1
+        again, _ = T.run_capi(cfg, reuse_from=cfg)
+        assert torch.equal(out, again), "the list left behind gives other bits"
+        listed, name2 = T.run_capi(dict(cfg, num_context=torch.zeros(B, dtype=idt)))
+        assert name2.startswith("mfma_fp8_d") and not name2.endswith("_selfsched"), name2
+        assert torch.equal(torch.isnan(out), torch.isnan(listed)), "other rows produced"
+        assert torch.equal(torch.nan_to_num(out.float()), torch.nan_to_num(listed.float())), "other bits than over the schedule kernel's list"
+    assert taken >= 40, taken
