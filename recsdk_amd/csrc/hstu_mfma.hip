@@ -185,6 +185,7 @@ struct SchedDims {
     int nsplit;        // K ranges per Q tile (1 = none); each range is an item of its own
     int pair;          // 1: the first two Q tiles of a long sequence may become one item
     int interleave;    // 1: four neighbouring groups of a list with equal entry counts are written entry by entry in turn
+    int level_slots;   // > 0: workgroups a CU holds; lists of at most 32 times as many entries are levelled over the CUs (see hstu_schedule_kernel)
 };
 
 // head dims the matrix-core kernels take through the padded variant (EXTRA 11): multiples of 16 up to 256 that are not one
@@ -202,6 +203,7 @@ static SchedDims sched_dims(const hstu_fwd_params& p, bool whole_tiles = false) 
     SchedDims d;
     d.pair = 1;
     d.interleave = 0;
+    d.level_slots = 0;
     d.ntiles_attr = (p.max_seq_len_q + BM - 1) / BM;
     // sum over sequences of min(ceil(lq / BM), ntiles_attr) <= min(total_q / BM + batch, batch * ntiles_attr)
     const int64_t by_rows = p.total_q / BM + p.batch, by_attr = (int64_t)p.batch * d.ntiles_attr;
@@ -361,6 +363,7 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
         // the records of a group are written by `sub` threads side by side (a group has up to 160 * 4 of them)
         s_gpos[tid] = pos;
         s_val[tid] = v;
+        if (tid < 8) s_len[tid] = cb;   // entries of list x so far (all of them when the groups fit one chunk)
         __syncthreads();
         const unsigned gcount = min((unsigned)nthr, G - c0);
         unsigned sub = 1;
@@ -382,6 +385,11 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
             // which costs the kernels that lean on the L2 for a group's K/V rows more than it gives them: measured on one
             // box, -6 .. -7 % for the plain variants at head dims 32 and 256, +1 .. +3 % for the dense-bias variant, the paged
             // variant with split K ranges and the backward kernels; the host asks for it accordingly.
+            // When every workgroup of a launch is resident at once, the hardware places entries p, p + 32, p + 64 .. of an
+            // XCD's list on the same CU (32 CUs, taken in a fixed order).  With the list in falling order of cost all
+            // through, the CU of entry 0 then holds the dearest item of every round of 32 and ends last.  Writing the
+            // rounds after the first in rising order levels the CUs.
+            const unsigned level_n = (d.level_slots > 0 && G <= (unsigned)nthr && s_len[x] <= min(d.cap, 32u * (unsigned)d.level_slots)) ? s_len[x] : 0u;
             unsigned stride = 1, pos0 = gpos;
             if (d.interleave) {
                 const unsigned u0 = (gr >> 5) << 1, cx = (unsigned)x;
@@ -400,7 +408,11 @@ void hstu_schedule_kernel(const KArgs a, const SchedDims d, unsigned* __restrict
                 const bool both = pair && i == gv - 1;
                 const unsigned tile = both ? 0u : (gv - 1 - i) / ns + (pair ? 1u : 0u), part = both ? 1u : i % ns;
                 lo[0] = (unsigned)gb | gh << 12 | tile << 16 | ((i < ns && sw) ? 1u << 24 : 0u) | part << 25 | ns << 28;
-                const unsigned at = pos0 + stride * i;
+                unsigned at = pos0 + stride * i;
+                if (level_n && at >= 32u) {
+                    const unsigned r0 = at & ~31u;
+                    at = r0 + (min(32u, level_n - r0) - 1u - (at & 31u));
+                }
                 unsigned* rec = at < d.cap ? list + REC * (8 * (size_t)at + x) : ovf + REC * (size_t)atomicAdd(&s_ovf, 1u);
                 *reinterpret_cast<u32x4*>(rec) = lo;
                 *reinterpret_cast<u32x4*>(rec + 4) = hi;
@@ -1525,6 +1537,7 @@ static hipError_t launch_td(const KArgs& a, unsigned* ws, hipStream_t stream) {
     // (the order in which launch_td's schedule kernel writes four equal groups: see hstu_schedule_kernel)
     SchedDims dsched = d;
     dsched.interleave = (!paged && d.nsplit == 1 && (extra == 0 || (extra >= 2 && extra <= 4))) ? 1 : 0;
+    dsched.level_slots = (paged && d.nsplit > 1) ? 3 : 0;   // the paged variants hold two or three workgroups per CU
     const int groups = p.batch * p.heads_q;
     const int sched_threads = groups <= 128 ? 256 : (groups <= 512 ? 512 : SCHED_NT);   // spare threads write a group's records side by side
     hipError_t e = hipSuccess;
