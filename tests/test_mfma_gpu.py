@@ -321,6 +321,20 @@ def test_config5_full_size_properties():
     assert changed.min().item() >= 256 * u and changed.max().item() < 256 * (u + 1) and changed.numel() > 200
 
 
+@pytest.mark.parametrize("users", [11, 17, 23, 29])
+def test_paged_split_lists_with_part_rounds(users):
+    """Paged calls with split K ranges whose XCD lists end inside a round of 32 entries (the schedule kernel writes the
+    rounds after the first in rising order of cost, the last one over as many entries as it has): every row against the
+    plain-FMA kernel."""
+    cfg = W.config5(seed=users, users=users)
+    say("paged_split_part_rounds", users, cfg["hist"][:6])
+    out, name = T.run_capi(cfg, op="paged", use_fp8=True)
+    assert name == "mfma_bf16_d128"
+    gen, _ = T.run_capi(cfg, op="paged", use_fp8=True, flags=FORCE_GENERIC)
+    assert not torch.isnan(out.float()).any()
+    T.assert_parity(out, gen.float(), torch.bfloat16, what="paged, split K ranges, part rounds vs generic kernel")
+
+
 def test_reference_user_shape_long_sequences():
     """The reference benchmark's user case B=128, h=4, d=128, S=7621 with lengths int(0.9 S) = 6858
     (test_forward_op_benchmark.py:185-199), a quarter of its batch (the plain-FMA kernel it is checked against runs 10 x
