@@ -706,7 +706,8 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
             for (int i = tid; i < np; i += NT) {
                 const int64_t page = ld_idx(p.page_ids, s.page0 + i, is64);
                 lds_pid[i] = (int)page;
-                if (p.cache_dtype == HSTU_FP8_E4M3) {
+                // (the variant that copies raw fp8 rows reads the scales behind the request for its first tile, see below)
+                if (!SH::PDMA8 && p.cache_dtype == HSTU_FP8_E4M3) {
                     lds_psc[2 * i] = p.kv_scales[(page * 2 + 0) * p.heads_k + hk];
                     lds_psc[2 * i + 1] = p.kv_scales[(page * 2 + 1) * p.heads_k + hk];
                 }
@@ -1016,6 +1017,17 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
         const int kt0 = part * per, kt1 = min(ntk, kt0 + per);
         if (kt0 < kt1) fetch(kt0, lds0);
         if (XDMA && kt0 < kt1) fetch_x(kt0, lds_xd0);
+        if constexpr (SH::PDMA8) {
+            // the pages' scales, a read that depends on the page ids like the first tile's rows: requested behind them, the two
+            // round trips overlap; the widening in stash() is the first to need them
+            const int np = min((s.hist_k + p.page_size - 1) / p.page_size, MAXP);
+            for (int i = tid; i < np; i += NT) {
+                const int64_t page = lds_pid[i];
+                lds_psc[2 * i] = p.kv_scales[(page * 2 + 0) * p.heads_k + hk];
+                lds_psc[2 * i + 1] = p.kv_scales[(page * 2 + 1) * p.heads_k + hk];
+            }
+            __syncthreads();
+        }
         if (tab_ts) {
             // the cells of the time table, built behind the request for the first K/V tile: the two dependent reads per cell
             // (bound, then values) then run while that tile is on its way; the barrier in stash() publishes them
