@@ -68,6 +68,17 @@ def build_workload(name, torch, W):
         kv = sum(c["hist"]) * 2 * 4 * 128
         qo = 2 * 32 * 256 * 4 * 128 * 2
         return c, "paged", flops, kv + 2 * qo, "config5 paged fp8-KV: 32 users x 256 candidates, hist~U[1024,4096], 64-token pages"
+    if name in ("ref_bias_unmasked", "ref_nobias_unmasked"):
+        # The reference's benchmark calls its op with window_size = (-1, -1): no mask at all, every row of a sequence sees
+        # every column (test_forward_op_benchmark.py:201-205, 251-255; golden backend/pytorch_native_backend.py:74-81).
+        # Here that is mask_type NONE of the jagged op: twice the causal FLOPs, the whole bias plane of a sequence.
+        c = W.reference_benchmark_config(has_rab=name == "ref_bias_unmasked")
+        c["mask_type"] = 2
+        flops = 2.0 * W.headline_flops(c["lens"], 8, 128)
+        t = sum(c["lens"])
+        b = 4 * t * 8 * 128 * 2 + (sum(8 * l * l * 2 for l in c["lens"]) if "attn_bias" in c else 0)
+        return c, "jagged", flops, b, ("reference benchmark shape as the reference runs it (test_forward_op_benchmark.py:246-259, window_size (-1, -1)): B=32 h=8 d=128 "
+                                      "S=2048, every length 0.9 S, alpha=0.5, silu_scale=1/1024, bf16, no mask, " + ("dense attn_bias [B,h,S,S]" if "attn_bias" in c else "no bias"))
     if name in ("ref_bias", "ref_nobias", "ref_nobias_d32", "ref_nobias_d64", "ref_nobias_d256", "ref_nobias_d64v32", "ref_nobias_d128v48"):
         dims = name.split("_d")[1] if "_d" in name else "128"     # the ends and the middle of the reference's head-dim sweep,
         dim = int(dims.split("v")[0])                             # and the (dim_qk, dim_v) pairs of its user cases
@@ -102,7 +113,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=1000)
-    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "ref_bias", "ref_nobias", "ref_nobias_d32", "ref_nobias_d64", "ref_nobias_d256", "ref_nobias_d64v32", "ref_nobias_d128v48", "config2_fp8", "ref_nobias_fp8", "config2_bwd", "ref_bias_bwd", "ref_nobias_bwd", "ref_nobias_d32_bwd", "ref_nobias_d64_bwd", "ref_nobias_d256_bwd", "kv_append", "kv_append_fp8", "rab_time", "rab_time_bwd", "rab_pos", "nmd_fwd", "nmd_bwd", "in_linear_silu", "in_linear_silu_bwd", "copy"],
+    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "ref_bias", "ref_nobias", "ref_bias_unmasked", "ref_nobias_unmasked", "ref_nobias_d32", "ref_nobias_d64", "ref_nobias_d256", "ref_nobias_d64v32", "ref_nobias_d128v48", "config2_fp8", "ref_nobias_fp8", "config2_bwd", "ref_bias_bwd", "ref_nobias_bwd", "ref_nobias_d32_bwd", "ref_nobias_d64_bwd", "ref_nobias_d256_bwd", "kv_append", "kv_append_fp8", "rab_time", "rab_time_bwd", "rab_pos", "nmd_fwd", "nmd_bwd", "in_linear_silu", "in_linear_silu_bwd", "copy"],
                     help="'copy' runs a plain 256 MiB device copy: the known-size kernel the FETCH_SIZE/WRITE_SIZE counters are scaled by")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--timeline", action="store_true",
@@ -145,7 +156,7 @@ def main():
     fp8 = q.dtype == torch.float8_e4m3fn
     peak = PEAK_FP8_TFLOPS if fp8 else PEAK_BF16_TFLOPS
     kw = dict(seq_offset_q=dev["seq_offset"], seq_offset_k=dev.get("seq_offset_k"), max_seq_len_q=cfg["max_seq_len"],
-              max_seq_len_k=cfg.get("max_seq_len_k"), mask_type=0, alpha=cfg["alpha"], num_target=dev.get("num_target"),
+              max_seq_len_k=cfg.get("max_seq_len_k"), mask_type=cfg.get("mask_type", 0), alpha=cfg["alpha"], num_target=dev.get("num_target"),
               attn_bias=dev.get("attn_bias"), silu_scale=cfg.get("silu_scale", 0.0),
               target_group_size=cfg.get("target_group_size", 0), pos_table=dev.get("pos_table"),
               ts_table=dev.get("ts_table"), timestamps=dev.get("timestamps"))

@@ -103,8 +103,10 @@ def reference_benchmark_config(seed=123, batch=32, heads=8, dim=128, max_seq_len
                                ratio=0.9, dim_v=None) -> Dict:
     """The shape of the reference's own forward benchmark (cust_op/test/hstu_v2/test_forward_op_benchmark.py:246-259 with
     the generator of utils/data.py:85-143): every sequence has int(0.9 * max_seq_len) rows, q/k/v and the dense bias
-    ("rab", [batch, heads, max_seq_len, max_seq_len]) are uniform in (-1, 1), built-in causal mask, alpha = 0.5,
-    silu_scale = 1/1024 (test_forward_op_benchmark.py:108-109)."""
+    ("rab", [batch, heads, max_seq_len, max_seq_len]) are uniform in (-1, 1), alpha = 0.5, silu_scale = 1/1024
+    (test_forward_op_benchmark.py:108-109).  The reference's benchmark passes window_size (-1, -1), no mask at all
+    (utils/data.py:121-123); the configuration defaults to the built-in causal mask of the jagged op, and callers that
+    want the reference's own computation set ``mask_type`` to NONE (2)."""
     rng = np.random.default_rng(seed)
     l = int(ratio * max_seq_len)
     lens = [l] * batch
