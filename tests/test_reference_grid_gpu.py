@@ -1,8 +1,8 @@
 """The grids of the reference's own operator tests for the attention, judged by the reference's own rule.
 
 cust_op/test/hstu_v2/test_forward_op_precision.py (forward: batch sizes, head dims, head counts, dense bias, sequence
-lengths, the two lists of user shapes) and test_backward_op_precision_mask.py:331-351 (backward under the causal mask with
-context rows and target groups) draw their inputs with utils/data.py:85-143 -- q / k / v / bias / grad uniform in (-1, 1),
+lengths, the two lists of user shapes), test_backward_op_precision.py (the same grids for the gradients) and
+test_backward_op_precision_mask.py:331-351 (backward under the causal mask with context rows and target groups) draw their inputs with utils/data.py:85-143 -- q / k / v / bias / grad uniform in (-1, 1),
 alpha 0.5, silu_scale 1/1024, lengths either random in [1 + context + targets, S] with lq <= lk or all int(0.9 S) -- and
 accept a kernel when its largest error against the golden evaluated in fp32 is at most five times the largest error of
 the same golden evaluated in the I/O dtype (backend/pytorch_native_backend.py:138-220).  The same grids (the larger ones
@@ -151,9 +151,51 @@ def test_backward_has_mask_other_batches(batch, heads, mask, d, dtype):
     _backward_case(batch, heads, *mask, d, False, dtype, nseq=8)
 
 
-def _backward_case(batch, heads, s, ctx, tgt, tgs, d, rab, dtype, nseq=None):
-    say("reference_grid_backward", batch, heads, s, ctx, tgt, tgs, d, rab, dtype)
-    c, grad = _draw(123, batch, heads, d, d, s, s, rab, dtype, False, ctx=ctx or 0, tgt=tgt or 0, tgs=tgs or 0, causal=True)
+# test_backward_op_precision.py:228-240, 281-293, 334-346, 387-399, 440-451, 492-503, 552-563: the forward's grids again,
+# gradients under no mask (window_size (-1, -1))
+@pytest.mark.parametrize("dtype", [F16, BF16])
+@pytest.mark.parametrize("rab", [True, False])
+@pytest.mark.parametrize("batch", [1, 4, 16, 32])
+def test_backward_generic_batch_size(batch, rab, dtype):
+    _backward_case(batch, 1, 256, None, None, None, 32, rab, dtype, causal=False)
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16])
+@pytest.mark.parametrize("d", [32, 64, 128, 256])
+def test_backward_generic_head_dim(d, dtype):
+    _backward_case(1, 1, 256, None, None, None, d, False, dtype, causal=False)
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16])
+@pytest.mark.parametrize("heads", [1, 4, 8, 16])
+def test_backward_generic_head_num(heads, dtype):
+    _backward_case(1, heads, 256, None, None, None, 32, False, dtype, causal=False)
+
+
+@pytest.mark.parametrize("rab", [True, False])
+@pytest.mark.parametrize("d", [32, 128])
+@pytest.mark.parametrize("s", [512, 1024, 2048])
+@pytest.mark.parametrize("heads", [1, 4])
+def test_backward_generic_sequence(heads, s, d, rab):    # one seed of the ten, the dtypes in turn
+    _backward_case(8, heads, s, None, None, None, d, rab, BF16 if (s // 512 + d // 32 + heads) % 2 else F16, causal=False, seed=s + d, nseq=4)
+
+
+@pytest.mark.parametrize("batch,heads,dims,lens,dtype,nseq", [
+    (2048, 4, (64, 64), (52, 1000), F16, 16), (16, 4, (64, 64), (501, 1000), F16, 8), (2048, 2, (256, 256), (32, 32), F16, 64),
+    (96, 2, (256, 256), (512, 3072), F16, 2), (16, 4, (64, 32), (32, 499), F16, 16), (4, 4, (128, 48), (1001, 901), F16, 4),
+    (96, 3, (256, 256), (674, 674), BF16, 4)])
+def test_backward_user_case_1(batch, heads, dims, lens, dtype, nseq):
+    _backward_case(batch, heads, lens[0], None, None, None, dims[0], False, dtype, causal=False, nseq=nseq, dv=dims[1], sk=lens[1], all_equal=True)
+
+
+@pytest.mark.parametrize("s,dtype,d", [(512, F16, 32), (512, BF16, 64), (512, F16, 128), (512, BF16, 256), (2048, BF16, 128)])
+def test_backward_user_case_2(s, dtype, d):              # B = 32, h = 8, every sequence 0.9 S; thinned
+    _backward_case(32, 8, s, None, None, None, d, False, dtype, causal=False, nseq=2, all_equal=True)
+
+
+def _backward_case(batch, heads, s, ctx, tgt, tgs, d, rab, dtype, nseq=None, causal=True, seed=123, dv=None, sk=None, all_equal=False):
+    say("reference_grid_backward", batch, heads, s, ctx, tgt, tgs, d, rab, dtype, causal, dv, sk)
+    c, grad = _draw(seed, batch, heads, d, dv or d, s, sk or s, rab, dtype, all_equal, ctx=ctx or 0, tgt=tgt or 0, tgs=tgs or 0, causal=causal)
     n = min(nseq or batch, batch)
     rows_q, rows_k = int(c["seq_offset"][n]), int(c["seq_offset_k"][n])
     out, name = T.run_capi(c)
