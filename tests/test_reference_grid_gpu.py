@@ -7,8 +7,8 @@ alpha 0.5, silu_scale 1/1024, lengths either random in [1 + context + targets, S
 accept a kernel when its largest error against the golden evaluated in fp32 is at most five times the largest error of
 the same golden evaluated in the I/O dtype (backend/pytorch_native_backend.py:138-220).  The same grids (the larger ones
 thinned: one seed, goldens over the first sequences of the big batches) run here through the C ABI; the goldens are
-plain torch on the CPU in one dtype throughout, as the reference's are.  window_size (-1, -1) of the forward tests is no
-mask at all (mask_type NONE); (-1, 0) of the backward tests is the built-in causal mask.
+plain torch on the CPU in one dtype throughout, as the reference's are.  Their window_size (-1, -1) is no mask at all
+(mask_type NONE here); (-1, 0), which only the masked backward tests use, is the built-in causal mask.
 """
 import numpy as np
 import pytest
