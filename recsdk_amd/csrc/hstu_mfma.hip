@@ -1470,7 +1470,6 @@ bool mfma_supported(const KArgs& a, const char** name) {
         if (a.op == OP_PAGED || p.attn_bias || p.mask_type == HSTU_MASK_CUSTOM || p.pos_table || p.ts_table) return false;
         d = padded_dim(p);
     }
-    if (a.op == OP_PAGED && (d == 32 || d == 256)) return false;   // paged K/V: head dims 64 and 128 only
     // rows are read and written 16 bytes at a time (vector loads, direct copies into LDS): buffers that do not start on
     // such a boundary take the plain kernel
     const uintptr_t all = reinterpret_cast<uintptr_t>(p.q) | reinterpret_cast<uintptr_t>(p.k) | reinterpret_cast<uintptr_t>(p.v) |
@@ -1582,7 +1581,9 @@ static hipError_t launch_td(const KArgs& a, unsigned* ws, hipStream_t stream) {
     } else if constexpr (D == 32 || D == 256) {
         // the head dims at the ends of the reference's sweep: plain and general variants only (bias tables are gathered
         // from global memory by the general one)
-        if (extra == 0) HSTU_LAUNCH(0, false);
+        if (paged && extra == 0) HSTU_LAUNCH(0, true);
+        else if (paged) HSTU_LAUNCH(1, true);
+        else if (extra == 0) HSTU_LAUNCH(0, false);
         else if (extra == 5) HSTU_LAUNCH(5, false);
         else if (extra == 6) HSTU_LAUNCH(6, false);
         else if (extra == 7) HSTU_LAUNCH(7, false);

@@ -150,7 +150,7 @@ def test_describe_kernel_selection():
                        (dict(page_size=8, max_seq_len_k=5121), "generic_bf16"),
                        (dict(page_size=10, max_seq_len_k=3200), "mfma_bf16_d128"),
                        (dict(page_size=10, max_seq_len_k=3201), "generic_bf16"),
-                       (dict(page_size=64, dim_qk=256, dim_v=256), "generic_bf16")]:
+                       (dict(page_size=64, dim_qk=256, dim_v=256), "mfma_bf16_d256"), (dict(page_size=16, dim_qk=32, dim_v=32), "mfma_bf16_d32")]:
         p = _params(**paged, **over)
         assert lib.hstu_hip_describe_kernel(C.byref(p), buf, 64) == 0
         assert buf.value.decode() == want, over

@@ -203,7 +203,8 @@ def test_mfma_time_table_bucket_range(d, nb, divisor, gap):
 
 
 @pytest.mark.parametrize("dtype", LOWP)
-@pytest.mark.parametrize("d,page_size,new_hist", [(64, 32, 0), (128, 64, 7), (128, 16, 130), (128, 12, 5), (128, 10, 3)])
+@pytest.mark.parametrize("d,page_size,new_hist", [(64, 32, 0), (128, 64, 7), (128, 16, 130), (128, 12, 5), (128, 10, 3),
+                                                   (32, 32, 0), (32, 12, 5), (256, 64, 7), (256, 10, 3)])
 def test_mfma_paged(d, page_size, new_hist, dtype):
     say("mfma_paged", dtype, d, page_size, new_hist)
     cfg = W.paged_config(28, 5, 2, d, new_hist + 1, 400, 40, page_size, dtype, new_hist=new_hist)
@@ -211,7 +212,7 @@ def test_mfma_paged(d, page_size, new_hist, dtype):
     assert torch.equal(T.run_op(cfg, op="paged"), out)
 
 
-@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("d", [32, 64, 128, 256])
 def test_mfma_paged_fp8(d):
     """fp8 cache == the same kernel on the dequantised cache (bit for bit), <= 5e-2 from the unquantised oracle."""
     say("mfma_paged_fp8", d)
@@ -224,6 +225,22 @@ def test_mfma_paged_fp8(d):
     assert torch.equal(out8, out16)
     T.assert_parity(out8, T.oracle_paged(cfg), torch.bfloat16, tol=5e-2, what="fp8 vs unquantised oracle")
     assert torch.equal(T.run_op(cfg, op="paged_fp8"), out8)
+
+
+@pytest.mark.parametrize("d", [32, 256])
+def test_mfma_paged_with_dense_bias_at_head_dims_32_and_256(d):
+    """Paged K/V with a dense bias takes the general variant; head dims 32 and 256 have it too: every row against the
+    plain-FMA kernel."""
+    say("mfma_paged_bias", d)
+    dtype = torch.bfloat16
+    cfg = W.paged_config(31, 3, 2, d, 40, 500, 33, 16, dtype)
+    rng = np.random.default_rng(31)
+    cfg["attn_bias"] = torch.from_numpy(rng.normal(0, 0.3, (3, 2, cfg["max_seq_len"], cfg["max_seq_len_k"])).astype(np.float32)).to(dtype)
+    out, name = T.run_capi(cfg, op="paged")
+    assert name == f"mfma_bf16_d{d}", name
+    gen, gname = T.run_capi(cfg, op="paged", flags=FORCE_GENERIC)
+    assert gname.startswith("generic")
+    T.assert_parity(out, gen.float(), dtype, what="paged with a dense bias vs generic kernel")
 
 
 def test_mfma_dense_layout():
