@@ -498,7 +498,7 @@ template <int D, int EXTRA, bool PAGED> struct Shape {
         static constexpr int WAVES = D == 256 ? 1 : (UNEVEN && D == 128) ? 2 : ((D <= 64 && EXTRA == 0 && !PAGED) ? 4 : ((LEAN || (D <= 64 && EXTRA != 1) || (XDMA && EXTRA != 7)) ? 3 : 2));
 };
 
-// SELF: no schedule kernel.  For small batches of plain causal self-attention (at most 64 sequences, one set of offsets
+// SELF: no schedule kernel.  For small batches of plain causal self-attention (at most 128 sequences, one set of offsets
 // for q and k) every wave of a workgroup derives the workgroup's record from the offsets themselves (self_record), which
 // costs a workgroup about a microsecond and saves the call a kernel and the gap between two kernels.
 template <typename T, int D, int EXTRA, bool PAGED, bool SELF = false>

@@ -503,7 +503,7 @@ def test_limits_longest_sequence_and_most_groups():
     (list(range(0, 64 * 17, 17)), 2, 1071), ([700] * 64, 8, 700), ([900, 140, 400], 5, 256),
     ([2000, 64, 8000, 1], 16, 8064), ([40] * 33 + [5000], 8, 4100)])
 def test_self_scheduled_small_batches(lens, heads, max_len, index_dtype):
-    """Plain causal self-attention at head dim 128 on at most 64 sequences runs without the schedule kernel: every
+    """Plain causal self-attention at head dim 128 on small batches runs without the schedule kernel: every
     workgroup derives its item from the offsets.  Every row must be produced exactly as by the list-driven grid (the call
     also leaves the list in the workspace: the second call reuses it), empty sequences, one-row sequences, 64 sequences,
     a max_seq_len attribute below the longest sequence and both offset dtypes included."""
