@@ -68,6 +68,14 @@ def build_workload(name, torch, W):
         kv = sum(c["hist"]) * 2 * 4 * 128
         qo = 2 * 32 * 256 * 4 * 128 * 2
         return c, "paged", flops, kv + 2 * qo, "config5 paged fp8-KV: 32 users x 256 candidates, hist~U[1024,4096], 64-token pages"
+    if name in ("config5_d32", "config5_d256"):
+        # config 5's users and pages at the ends of the reference's head-dim sweep (paged rows through registers)
+        d = int(name.split("_d")[1])
+        c = W.paged_config(0, 32, 4, d, 1024, 4096, 256, 64, torch.bfloat16)
+        c["kv_cache_fp8"], c["kv_scales"] = W.quantize_pages_fp8(c["kv_cache"])
+        c["use_fp8"] = True
+        flops = float(sum(4.0 * 256 * (h + 1) * 4 * d for h in c["hist"]))
+        return c, "paged", flops, sum(c["hist"]) * 2 * 4 * d + 2 * 2 * 32 * 256 * 4 * d * 2, f"config5's geometry at head dim {d}: 32 users x 256 candidates, hist~U[1024,4096], fp8 KV in 64-token pages"
     if name in ("ref_bias_unmasked", "ref_nobias_unmasked"):
         # The reference's benchmark calls its op with window_size = (-1, -1): no mask at all, every row of a sequence sees
         # every column (test_forward_op_benchmark.py:201-205, 251-255; golden backend/pytorch_native_backend.py:74-81).
@@ -113,7 +121,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=1000)
-    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "ref_bias", "ref_nobias", "ref_bias_unmasked", "ref_nobias_unmasked", "ref_nobias_d32", "ref_nobias_d64", "ref_nobias_d256", "ref_nobias_d64v32", "ref_nobias_d128v48", "config2_fp8", "ref_nobias_fp8", "config2_bwd", "ref_bias_bwd", "ref_nobias_bwd", "ref_nobias_d32_bwd", "ref_nobias_d64_bwd", "ref_nobias_d256_bwd", "kv_append", "kv_append_fp8", "rab_time", "rab_time_bwd", "rab_pos", "nmd_fwd", "nmd_bwd", "in_linear_silu", "in_linear_silu_bwd", "copy"],
+    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "config5_d32", "config5_d256", "ref_bias", "ref_nobias", "ref_bias_unmasked", "ref_nobias_unmasked", "ref_nobias_d32", "ref_nobias_d64", "ref_nobias_d256", "ref_nobias_d64v32", "ref_nobias_d128v48", "config2_fp8", "ref_nobias_fp8", "config2_bwd", "ref_bias_bwd", "ref_nobias_bwd", "ref_nobias_d32_bwd", "ref_nobias_d64_bwd", "ref_nobias_d256_bwd", "kv_append", "kv_append_fp8", "rab_time", "rab_time_bwd", "rab_pos", "nmd_fwd", "nmd_bwd", "in_linear_silu", "in_linear_silu_bwd", "copy"],
                     help="'copy' runs a plain 256 MiB device copy: the known-size kernel the FETCH_SIZE/WRITE_SIZE counters are scaled by")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--timeline", action="store_true",
