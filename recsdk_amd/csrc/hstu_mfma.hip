@@ -1525,7 +1525,7 @@ bool mfma_self_scheduled(const KArgs& a) {
     return a.op == OP_JAGGED && (p.dtype == HSTU_BF16 || p.dtype == HSTU_F16) && p.dim_qk == p.dim_v &&
            (p.dim_qk == 32 || p.dim_qk == 64 || p.dim_qk == 128) &&
            p.batch >= 1 && p.batch <= 128 && p.seq_offset_q && p.seq_offset_q == p.seq_offset_k && !p.num_context &&
-           p.mask_type == HSTU_MASK_TRIL && (extra == 0 || (tables_too && extra >= 2 && extra <= 4)) &&
+           (p.mask_type == HSTU_MASK_TRIL || p.mask_type == HSTU_MASK_NONE) && (extra == 0 || (tables_too && extra >= 2 && extra <= 4)) &&
            p.max_seq_len_q == p.max_seq_len_k && p.max_seq_len_q <= 63 * BM &&
            !(p.flags & HSTU_FLAG_REUSE_WORKSPACE) && sched_dims(p).nsplit == 1;
 }

@@ -367,7 +367,7 @@ uint64_t mfma_fp8_workspace_bytes(const KArgs& a) { return work_list_shape(a.p).
 bool mfma_fp8_self_scheduled(const KArgs& a) {
     const hstu_fwd_params& p = a.p;
     return a.op == OP_JAGGED && p.batch >= 1 && p.batch <= 128 && p.seq_offset_q && p.seq_offset_q == p.seq_offset_k && !p.num_context &&
-           p.mask_type == HSTU_MASK_TRIL && p.max_seq_len_q == p.max_seq_len_k && p.max_seq_len_q <= 63 * FBM &&
+           (p.mask_type == HSTU_MASK_TRIL || p.mask_type == HSTU_MASK_NONE) && p.max_seq_len_q == p.max_seq_len_k && p.max_seq_len_q <= 63 * FBM &&
            !(p.flags & HSTU_FLAG_REUSE_WORKSPACE);
 }
 

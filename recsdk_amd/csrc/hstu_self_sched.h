@@ -24,10 +24,10 @@ __device__ __forceinline__ unsigned small_div(unsigned x, unsigned y) {
 
 // The record of workgroup blockIdx.x without a work list, computed by one wave on its own (the caller guarantees
 // batch <= 128, at most 63 Q tiles per sequence under the attribute, one set of offsets for q and k, no context rows, the
-// built-in causal mask; target rows are fine).  The order is the schedule kernel's with a coarser key: sequences by
+// built-in causal mask or no mask; target rows are fine).  The order is the schedule kernel's with a coarser key: sequences by
 // their number of Q tiles (longest first, then by batch index), (sequence, head) groups r = rank * heads + head dealt to
 // the XCDs in snake order (XCD x owns r = 16 u + x and 16 u + 15 - x), a group's tiles last tile first (the tiles of four
-// groups of one class in turn, see below), the first two tiles of a sequence of five or more tiles as one item.  Lane b first holds sequences b and b + 64, then lane k holds the
+// groups of one class in turn, see below), under the causal mask the first two tiles of a sequence of five or more tiles as one item.  Lane b first holds sequences b and b + 64, then lane k holds the
 // class of the sequences with cmax - k tiles (a histogram in `hist`, 64 words of LDS private to the wave): the sequences
 // and the list entries ahead of a class are two prefix sums over the lanes, so the cost does not grow with the number of
 // classes.  No list can exceed the grid: with entries per group falling along r, the lists differ by at most one group's
@@ -80,7 +80,9 @@ __device__ __forceinline__ void self_record(const KArgs& a, int ntiles_attr, int
     const unsigned x = blockIdx.x & 7u, pos = blockIdx.x >> 3;
     // r's of XCD x below m
     auto below = [&](unsigned m) -> unsigned { return 2u * (m >> 4) + ((m & 15u) > x ? 1u : 0u) + ((m & 15u) > 15u - x ? 1u : 0u); };
-    auto entries = [&](int cc) -> unsigned { return (unsigned)min(cc, ntiles_attr) - ((cc <= ntiles_attr && cc >= 5) ? 1u : 0u); };
+    // without a mask every tile of a sequence sees all of K: no pair of cheap first tiles to merge
+    const bool pairs = p.mask_type == HSTU_MASK_TRIL;
+    auto entries = [&](int cc) -> unsigned { return (unsigned)min(cc, ntiles_attr) - ((pairs && cc <= ntiles_attr && cc >= 5) ? 1u : 0u); };
     const unsigned seqs_incl = wave_inclusive_sum(n), seqs_before = seqs_incl - n;
     const unsigned g0 = below(seqs_before * (unsigned)H), g1 = below(seqs_incl * (unsigned)H);
     const unsigned span = n ? (g1 - g0) * entries(c) : 0u;
@@ -131,7 +133,7 @@ __device__ __forceinline__ void self_record(const KArgs& a, int ntiles_attr, int
     const unsigned lq = (unsigned)__builtin_amdgcn_readlane(second ? len[1] : len[0], fl);
     const unsigned tg = (unsigned)__builtin_amdgcn_readlane(second ? tgt[1] : tgt[0], fl);
     const unsigned fb = (unsigned)fl + (second ? 64u : 0u);
-    const bool sw = found_cls > ntiles_attr, pr = !sw && found_cls >= 5;
+    const bool sw = found_cls > ntiles_attr, pr = pairs && !sw && found_cls >= 5;
     const bool both = pr && found_i == found_e - 1;
     const unsigned tile = both ? 0u : (found_e - 1 - found_i) + (pr ? 1u : 0u), part = both ? 1u : 0u;
     rec[0] = fb | h << 12 | tile << 16 | ((found_i == 0 && sw) ? 1u << 24 : 0u) | part << 25 | 1u << 28;

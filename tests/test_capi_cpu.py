@@ -130,6 +130,7 @@ def test_describe_kernel_selection():
     lib = _capi.lib()
     for over, want in [(dict(), "mfma_bf16_d128_selfsched"), (dict(flags=_capi.FLAG_REUSE_WORKSPACE), "mfma_bf16_d128"), (dict(batch=128), "mfma_bf16_d128_selfsched"), (dict(batch=129), "mfma_bf16_d128"),
                        (dict(num_target=0x2000), "mfma_bf16_d128_selfsched"), (dict(num_context=0x2000), "mfma_bf16_d128"),
+                       (dict(mask_type=2), "mfma_bf16_d128_selfsched"),
                        (dict(dim_qk=64, dim_v=64, dtype=_capi.HSTU_F16), "mfma_f16_d64_selfsched"),
                        (dict(dtype=_capi.HSTU_F32), "generic_f32"), (dict(dim_v=64), "mfma_bf16_d128_padded"), (dict(dim_qk=64, dim_v=32), "mfma_bf16_d64_padded"),
                        (dict(dim_qk=72, dim_v=64), "generic_bf16"), (dict(dim_v=64, attn_bias=0x1000), "generic_bf16"),
@@ -167,7 +168,7 @@ def test_fp8_inputs_selection_and_rejections():
                        (dict(dim_qk=32, dim_v=32), "mfma_fp8_d64_padded"), (dict(dim_qk=96, dim_v=80), "mfma_fp8_d128_padded"),
                        (dict(dim_qk=72, dim_v=32), "generic_fp8"), (dict(dim_qk=96, dim_v=80, attn_bias=0x1000), "generic_fp8"),
                        (dict(attn_bias=0x1000), "generic_fp8"), (dict(mask_type=3, mask=0x1000), "generic_fp8"),
-                       (dict(mask_type=2), "mfma_fp8_d128"), (dict(k=0x1008), "generic_fp8"),
+                       (dict(mask_type=2), "mfma_fp8_d128_selfsched"), (dict(mask_type=2, num_context=0x2000), "mfma_fp8_d128"), (dict(k=0x1008), "generic_fp8"),
                        (dict(flags=_capi.FLAG_FORCE_GENERIC), "generic_fp8")]:
         p = _params(**fp8, **over)
         assert lib.hstu_hip_describe_kernel(C.byref(p), buf, 64) == 0, lib.hstu_hip_last_error()

@@ -221,7 +221,9 @@ def test_fp8_self_derived_launches_match_the_list_driven_launch_on_random_batche
         if rng.random() < 0.4:
             cfg["num_target"] = torch.tensor([min(l, int(t)) for l, t in zip(lens, rng.integers(0, 50, B))], dtype=idt)
             cfg["target_group_size"] = int(rng.integers(1, 4))
-        say("fp8_self_derived_random", it, B, H, d, kind, sum(lens), mx, cfg["max_seq_len"])
+        if rng.random() < 0.3:
+            cfg["mask_type"] = 2
+        say("fp8_self_derived_random", it, B, H, d, kind, sum(lens), mx, cfg["max_seq_len"], cfg["mask_type"])
         out, name = T.run_capi(cfg)
         if not name.endswith("_selfsched"):
             continue
