@@ -52,8 +52,8 @@ enum { HSTU_MASK_TRIL = 0, HSTU_MASK_TRIU = 1, HSTU_MASK_NONE = 2, HSTU_MASK_CUS
 /* The workspace still holds the work list an earlier call built for the same sequence offsets, num_context,
  * num_target, page offsets, shapes and attributes (e.g. the other layers of one model on one batch): do not
  * rebuild it.  Only q/k/v/out/bias/table contents may differ between such calls.  (Every call without the flag leaves
- * the list in the workspace, also the calls that need no schedule kernel of their own: causal self-attention on at most
- * 128 sequences at head dims 32, 64 and 128, whose workgroups derive their items from the offsets and write them down as
+ * the list in the workspace, also the calls that need no schedule kernel of their own: self-attention under the causal
+ * mask or none on at most 128 sequences at head dims 32, 64 and 128, whose workgroups derive their items from the offsets and write them down as
  * they go.) */
 #define HSTU_FLAG_REUSE_WORKSPACE 4u
 /* backward only: run all kernels of this call on `stream` itself (see hstu_hip_jagged_backward) */
