@@ -478,16 +478,16 @@ template <int D, int EXTRA, bool PAGED> struct Shape {
     static constexpr int MAXP = (PAGED && D == 128 && EXTRA != 8 && EXTRA != 9) ? MAXP_HALF : MAXP_ALL;
     static constexpr bool DMA = (!PAGED && D == 128 && !UNEVEN) || PDMA;
     // head dim 64, rows straight from k / v, no dense bias or custom mask: direct copies too, 8 rows per instruction
-    static constexpr bool DMA64 = !PAGED && D == 64 && (EXTRA == 0 || (EXTRA >= 2 && EXTRA <= 4));
+    static constexpr bool DMA64 = !PAGED && D == 64 && (EXTRA == 0 || (EXTRA >= 2 && EXTRA <= 7));
     // head dim 32, plain variant: 16 rows of 64 bytes per instruction
-    static constexpr bool DMA32 = !PAGED && D == 32 && EXTRA == 0;
+    static constexpr bool DMA32 = !PAGED && D == 32 && (EXTRA == 0 || (EXTRA >= 5 && EXTRA <= 7));
     static constexpr bool LEAN = DMA && (EXTRA == 0 || EXTRA == 8 || EXTRA == 9 || EXTRA == 10);
     // EXTRA 10: the plain variant on sequences whose rows are taken in reverse order (row i of q / k / v / out is row
     // L - 1 - i of its sequence in memory).  With K in the place of q, Q in the place of k and dO in the place of v the
     // causal forward then computes dV of the backward: dV[j] = sum over i >= j of P[i][j] dO[i].
     static constexpr bool REV = EXTRA == 10;
     // a dense bias (or, without one, a custom mask) next to direct K/V copies: its blocks are copied into LDS the same way, one tile ahead
-    static constexpr bool XDMA = DMA && EXTRA >= 5 && EXTRA <= 7;
+    static constexpr bool XDMA = (DMA || DMA64 || DMA32) && EXTRA >= 5 && EXTRA <= 7;
     static constexpr bool RDMA = DMA && REV;
     static constexpr int BNT = (LEAN || XDMA) ? 32 : 64;     // K columns per step
     // waves per SIMD; head dim 256 needs the registers of a whole SIMD lane for its 32 x 256 accumulator and Q fragments
@@ -830,10 +830,18 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
                 __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc((void*)(vview + tile_off), 0, (int)(view_bytes - tile_off), 0x00020000);
                 const int rho = lane >> 2;
                 const unsigned lo = (unsigned)rho * rowstride + ((((lane & 3) - (rho >> 2)) & 3) << 4);   // lane L fills slot L % 4 of row L / 4
-                static_assert(!DMA32 || NBLK16 == 4, "one block of K and one of V per wave");
-                const unsigned so = (unsigned)(16 * w) * rowstride;
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, LDS_PTR(void, dst + w * 1024), 16, lo + so, 0, 0, 0);
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, LDS_PTR(void, dst + (NBLK16 + w) * 1024), 16, lo + so, 0, 0, 0);
+                static_assert(!DMA32 || NBLK16 == 4 || NBLK16 == 2, "one block of K and one of V per wave, or one block per wave");
+                if constexpr (NBLK16 == 4) {
+                    const unsigned so = (unsigned)(16 * w) * rowstride;
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, LDS_PTR(void, dst + w * 1024), 16, lo + so, 0, 0, 0);
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, LDS_PTR(void, dst + (NBLK16 + w) * 1024), 16, lo + so, 0, 0, 0);
+                } else {
+                    // tiles of 32 keys: waves 0 and 1 copy the two blocks of K, waves 2 and 3 those of V
+                    const int b = w & 1;
+                    const unsigned so = (unsigned)(16 * b) * rowstride;
+                    if (w < 2) __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, LDS_PTR(void, dst + b * 1024), 16, lo + so, 0, 0, 0);
+                    else __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, LDS_PTR(void, dst + (NBLK16 + b) * 1024), 16, lo + so, 0, 0, 0);
+                }
             } else if (PAGED && p.page_size % BNT == 0 && k0 + BNT <= s.hist_k) {
                 // the whole tile lies in one page of the history (pages hold a multiple of the tile's columns and the
                 // history starts at column 0): one page lookup for the tile, rows at a fixed stride
@@ -1351,8 +1359,12 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
             // is free now (every wave is past the last barrier of the K loop), row stride 2*D + 8 bytes, and writes
             // it out 16 bytes per lane, 64 / (D / 8) rows per instruction.
             constexpr int ORS = 2 * D + 8;
-            static_assert(2 * 32 * ORS <= STAGE_BYTES, "two waves park their output tile in one stage");
-            char* park = ((w & 2) ? lds1 : lds0) + (w & 1) * (32 * ORS);
+            // (head dim 64 with the bias blocks copied: a stage of 32 keys holds one output tile, the other two waves use
+            // the stages of the bias blocks)
+            constexpr bool PARK_TWO = 2 * 32 * ORS <= STAGE_BYTES;
+            static_assert(PARK_TWO || (XDMA && 32 * ORS <= STAGE_BYTES && 32 * ORS <= XDS), "every wave parks its output tile in a stage that is free");
+            char* park = PARK_TWO ? ((w & 2) ? lds1 : lds0) + (w & 1) * (32 * ORS)
+                                  : ((w & 2) ? ((w & 1) ? lds_xd1 : lds_xd0) : ((w & 1) ? lds1 : lds0));
 #pragma unroll
             for (int db = 0; db < D / 32; db++) {
 #pragma unroll
