@@ -105,7 +105,7 @@ def build_workload(name, torch, W):
 
 def bench_kind(workload):
     """Which leg of this file measures a workload (the names of several legs end alike)."""
-    if workload in ("copy", "kv_append", "kv_append_fp8", "in_linear_silu", "in_linear_silu_bwd", "ref_grid"):
+    if workload in ("copy", "kv_append", "kv_append_fp8", "in_linear_silu", "in_linear_silu_bwd", "ref_grid", "ref_grid_bwd"):
         return workload
     if workload in ("rab_time", "rab_time_bwd", "rab_pos"):
         return "bias"
@@ -121,7 +121,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=1000)
-    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "config5_d32", "config5_d256", "ref_grid", "ref_bias", "ref_nobias", "ref_bias_unmasked", "ref_nobias_unmasked", "ref_nobias_d32", "ref_nobias_d64", "ref_nobias_d256", "ref_nobias_d64v32", "ref_nobias_d128v48", "config2_fp8", "ref_nobias_fp8", "config2_bwd", "ref_bias_bwd", "ref_nobias_bwd", "ref_nobias_d32_bwd", "ref_nobias_d64_bwd", "ref_nobias_d256_bwd", "kv_append", "kv_append_fp8", "rab_time", "rab_time_bwd", "rab_pos", "nmd_fwd", "nmd_bwd", "in_linear_silu", "in_linear_silu_bwd", "copy"],
+    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "config5_d32", "config5_d256", "ref_grid", "ref_grid_bwd", "ref_bias", "ref_nobias", "ref_bias_unmasked", "ref_nobias_unmasked", "ref_nobias_d32", "ref_nobias_d64", "ref_nobias_d256", "ref_nobias_d64v32", "ref_nobias_d128v48", "config2_fp8", "ref_nobias_fp8", "config2_bwd", "ref_bias_bwd", "ref_nobias_bwd", "ref_nobias_d32_bwd", "ref_nobias_d64_bwd", "ref_nobias_d256_bwd", "kv_append", "kv_append_fp8", "rab_time", "rab_time_bwd", "rab_pos", "nmd_fwd", "nmd_bwd", "in_linear_silu", "in_linear_silu_bwd", "copy"],
                     help="'copy' runs a plain 256 MiB device copy: the known-size kernel the FETCH_SIZE/WRITE_SIZE counters are scaled by")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--timeline", action="store_true",
@@ -143,8 +143,8 @@ def main():
     kind = bench_kind(args.workload)
     if kind == "copy":
         return copy_calibration(args, torch)
-    if kind == "ref_grid":
-        return reference_grid(args, torch, _capi)
+    if kind in ("ref_grid", "ref_grid_bwd"):
+        return reference_grid(args, torch, _capi, backward=kind == "ref_grid_bwd")
     if kind == "attention_backward":
         return backward_bench(args, torch, W, _capi)
     if kind == "kv_append":
@@ -790,8 +790,9 @@ def in_linear_silu_bwd_bench(args, torch):
     print(json.dumps(out), flush=True)
 
 
-def reference_grid(args, torch, _capi):
-    """The grid of the reference's own forward benchmark (cust_op/test/hstu_v2/test_forward_op_benchmark.py:246-259): B = 32,
+def reference_grid(args, torch, _capi, backward=False):
+    """The grid of the reference's own forward benchmark (cust_op/test/hstu_v2/test_forward_op_benchmark.py:246-259; with
+    `backward` that of test_backward_op_benchmark.py:246-259, the gradients dQ, dK, dV and, with a bias, dBias: 2.5 x the FLOPs): B = 32,
     h = 8, every sequence int(0.9 S) rows, S in {512, 1024, 2048, 4096} x head dim in {32, 64, 128, 256} x with / without a
     dense bias [B, h, S, S], no mask (its window_size (-1, -1)), alpha 0.5, silu_scale 1/1024, inputs uniform in (-1, 1) -- in
     bf16 (the reference also runs fp16).  One JSON line per point; --steps / --warmup apply to every point (capped at 50 / 20)."""
@@ -812,12 +813,22 @@ def reference_grid(args, torch, _capi):
                 p, keep = _capi.make_params(q, k, v, out, seq_offset_q=off, max_seq_len_q=S, mask_type=_capi.MASK_NONE, alpha=0.5,
                                             silu_scale=1.0 / 1024, attn_bias=bias)
                 n = C.c_uint64(0)
-                if L.hstu_hip_jagged_forward_get_workspace_size(C.byref(p), C.byref(n)) != 0:
+                if backward:
+                    if rab and S == 4096:
+                        continue          # bias and its gradient: 2 x 8.6 GB per point; left out
+                    grad, dq, dk, dv = uni(32 * l, 8, d), torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+                    dbias = torch.empty_like(bias) if rab else None
+                    p.out = None
+                    fwd, p = p, _capi.make_backward_params(p, grad, dq, dk, dv, dbias)
+                    size_fn, run_fn, name = L.hstu_hip_jagged_backward_get_workspace_size, L.hstu_hip_jagged_backward, _capi.describe_backward_kernel(p)
+                else:
+                    size_fn, run_fn, name = L.hstu_hip_jagged_forward_get_workspace_size, L.hstu_hip_jagged_forward, _capi.describe_kernel(p)
+                if size_fn(C.byref(p), C.byref(n)) != 0:
                     raise RuntimeError(L.hstu_hip_last_error().decode())
-                ws = torch.empty(max(int(n.value), 4), dtype=torch.uint8, device="cuda")
+                ws = torch.empty(max(int(n.value), 16), dtype=torch.uint8, device="cuda")
 
                 def step():
-                    if L.hstu_hip_jagged_forward(C.byref(p), C.c_void_p(ws.data_ptr()), n.value, stream) != 0:
+                    if run_fn(C.byref(p), C.c_void_p(ws.data_ptr()), n.value, stream) != 0:
                         raise RuntimeError(L.hstu_hip_last_error().decode())
                 settle_clocks(step, args.settle_ms, torch)
                 for _ in range(warm):
@@ -830,9 +841,9 @@ def reference_grid(args, torch, _capi):
                 e1.record()
                 torch.cuda.synchronize()
                 us = e0.elapsed_time(e1) / steps * 1e3
-                flops = 32 * 4.0 * l * l * 8 * d
-                print(json.dumps({"metric": "hstu_reference_benchmark_grid", "S": S, "head_dim": d, "dense_bias": rab, "mask": "none", "dtype": "bf16",
-                                  "batch": 32, "heads": 8, "rows_per_sequence": l, "kernel": _capi.describe_kernel(p), "us_per_call": round(us, 1),
+                flops = 32 * 4.0 * l * l * 8 * d * (2.5 if backward else 1.0)
+                print(json.dumps({"metric": "hstu_reference_benchmark_grid" + ("_backward" if backward else ""), "S": S, "head_dim": d, "dense_bias": rab, "mask": "none", "dtype": "bf16",
+                                  "batch": 32, "heads": 8, "rows_per_sequence": l, "kernel": name, "us_per_call": round(us, 1),
                                   "tflops": round(flops / us * 1e-6, 1), "pct_bf16_mfma_peak": round(flops / us * 1e-6 / PEAK_BF16_TFLOPS * 100, 1),
                                   "steps": steps, "warmup": warm, "n_gpus": 1}), flush=True)
                 del bias
