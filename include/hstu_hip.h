@@ -222,10 +222,12 @@ const char* hstu_hip_last_error(void);
 
 /* Name of the kernel variant the given arguments select ("mfma_bf16_d128", "generic_f32", ...);
  * written NUL-terminated into buf.  Diagnostic: lets a caller assert that the MFMA path is the one in use.  The
- * matrix-core kernels take bf16 / fp16 with dim_qk == dim_v in {32, 64, 128, 256} (paged: 64 or 128, and at most 320 pages
- * per user) and buffers on 16-byte boundaries, and FP8_E4M3 with dim_qk == dim_v in {64, 128, 256}, the built-in mask or
- * none and no bias ("mfma_fp8_d128"); everything else (fp32, other head dims, dim_qk != dim_v, fp8 bias or custom mask)
- * runs the plain fp32-FMA kernel, which is an order of magnitude slower. */
+ * matrix-core kernels take bf16 / fp16 with dim_qk == dim_v in {32, 64, 128, 256} (paged too, with at most 640 pages per
+ * user, 320 at head dim 128 when the page size is no multiple of 4) and buffers on 16-byte boundaries; other multiples of
+ * 16 up to 256 and dim_qk != dim_v under the built-in mask or none without a bias ("mfma_bf16_d128_padded"); FP8_E4M3
+ * with the built-in mask or none and no bias ("mfma_fp8_d128"); everything else (fp32, unaligned buffers, other head dims
+ * with a bias or pages, fp8 with a bias or a custom mask) runs the plain fp32-FMA kernel, which is an order of magnitude
+ * slower. */
 int hstu_hip_describe_kernel(const hstu_fwd_params* p, char* buf, size_t buf_bytes);
 
 /* The same for the backward: "mfma_bwd_bf16_d128", "mfma_bwd_f16_d64_bias", "generic_bwd_f32", ...  The matrix-core
