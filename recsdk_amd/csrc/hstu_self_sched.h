@@ -34,6 +34,7 @@ __device__ __forceinline__ unsigned small_div(unsigned x, unsigned y) {
 // entries.
 constexpr int SELF_TILE_ROWS = 128;
 
+template <bool FOUR_STREAMS = true>
 __device__ __forceinline__ void self_record(const KArgs& a, int ntiles_attr, int lane, unsigned* hist, unsigned (&rec)[WORK_RECORD_WORDS], int64_t& rows) {
     const hstu_fwd_params& p = a.p;
     const int B = p.batch, H = p.heads_q;
@@ -105,7 +106,8 @@ __device__ __forceinline__ void self_record(const KArgs& a, int ntiles_attr, int
     // is has no room: with four streams of equal cost the engines fill and drain together instead of holding each
     // other's free slots up.
     const unsigned g_first = (unsigned)__builtin_amdgcn_readlane((int)g0, fk), g_count = (unsigned)__builtin_amdgcn_readlane((int)g1, fk) - g_first;
-    const unsigned in_blocks = (g_count >> 2) * 4u * found_e;     // entries of the whole blocks
+    // (FOUR_STREAMS off: group by group, for the variants that lean on the L2 for the rows and bias planes a group shares)
+    const unsigned in_blocks = FOUR_STREAMS ? (g_count >> 2) * 4u * found_e : 0u;     // entries of the whole blocks
     unsigned found_g, found_i;
     if (d < in_blocks) {
         const unsigned blk = small_div(d, 4u * found_e), rem = d - blk * 4u * found_e;
@@ -114,7 +116,7 @@ __device__ __forceinline__ void self_record(const KArgs& a, int ntiles_attr, int
     } else {
         const unsigned td = d - in_blocks, gj = small_div(td, found_e);
         found_i = td - gj * found_e;
-        found_g = g_first + (g_count & ~3u) + gj;
+        found_g = g_first + (FOUR_STREAMS ? (g_count & ~3u) : 0u) + gj;
     }
     // group found_g of this XCD's list: r = 16 (g / 2) + (x or 15 - x); its sequence is the (rank - found_first)-th of its class
     const unsigned r = 16u * (found_g >> 1) + ((found_g & 1u) ? 15u - x : x);

@@ -135,7 +135,8 @@ def test_describe_kernel_selection():
                        (dict(dtype=_capi.HSTU_F32), "generic_f32"), (dict(dim_v=64), "mfma_bf16_d128_padded"), (dict(dim_qk=64, dim_v=32), "mfma_bf16_d64_padded"),
                        (dict(dim_qk=72, dim_v=64), "generic_bf16"), (dict(dim_v=64, attn_bias=0x1000), "generic_bf16"),
                        (dict(dim_qk=32, dim_v=32), "mfma_bf16_d32_selfsched"), (dict(dim_qk=256, dim_v=256, dtype=_capi.HSTU_F16), "mfma_f16_d256"),
-                       (dict(dim_qk=32, dim_v=32, attn_bias=0x1000), "mfma_bf16_d32"),
+                       (dict(dim_qk=32, dim_v=32, attn_bias=0x1000), "mfma_bf16_d32_selfsched"), (dict(dim_qk=32, dim_v=32, attn_bias=0x1002), "mfma_bf16_d32"),
+                       (dict(attn_bias=0x1000), "mfma_bf16_d128_selfsched"), (dict(attn_bias=0x1000, mask_type=3, mask=0x2000), "mfma_bf16_d128"),
                        (dict(dim_qk=96, dim_v=96), "mfma_bf16_d128_padded"),
                        (dict(q=0x1002), "generic_bf16"), (dict(out=0x1008), "generic_bf16"),   # not on a 16-byte boundary
                        (dict(flags=_capi.FLAG_FORCE_GENERIC), "generic_bf16")]:

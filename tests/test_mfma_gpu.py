@@ -39,7 +39,7 @@ def test_reference_benchmark_shape_unmasked_by_the_reference_criterion(has_rab):
     cfg = W.reference_benchmark_config(batch=8, has_rab=has_rab)
     cfg["mask_type"] = 2
     out, name = T.run_capi(cfg)
-    assert name == ("mfma_bf16_d128" if has_rab else "mfma_bf16_d128_selfsched"), name
+    assert name == "mfma_bf16_d128_selfsched", name
     T.assert_parity(out, T.oracle_jagged(cfg), dtype, what="unmasked reference shape vs oracle")
 
     def golden(dt):          # plain torch in one dtype throughout, like the reference's test backend
@@ -155,7 +155,7 @@ def test_reference_benchmark_shape_with_dense_bias():
     dtype = torch.bfloat16
     cfg = W.reference_benchmark_config()
     out, name = T.run_capi(cfg)
-    assert name == "mfma_bf16_d128", name
+    assert name == "mfma_bf16_d128_selfsched", name
     gen, _ = T.run_capi(cfg, flags=FORCE_GENERIC)
     T.assert_parity(out, gen.float(), dtype, what="reference benchmark shape vs generic kernel")
     l = cfg["lens"][0]
@@ -576,7 +576,7 @@ def _self_scheduled_wide(d, nseq, heads, tables, index_dtype):
 def test_self_scheduled_random_geometries_match_the_list_driven_launch(seed):
     """Random batches (1..128 sequences, 1..16 heads, head dims 32 / 64 / 128, uniform, heavy-tailed, half-empty, equal and
     tile-aligned lengths, attributes below / at / above the longest sequence, both offset dtypes, target rows, a position
-    table, no mask instead of the causal one): the launch that derives its items must produce the same bits as the same call made ineligible by a
+    table, no mask instead of the causal one, a dense bias): the launch that derives its items must produce the same bits as the same call made ineligible by a
     num_context of zeros (which runs over the schedule kernel's list), and as a second call over the list it left."""
     rng = np.random.default_rng(seed)
     taken = 0
@@ -604,6 +604,9 @@ def test_self_scheduled_random_geometries_match_the_list_driven_launch(seed):
             cfg["pos_table"] = torch.from_numpy(rng.normal(0, 0.5, 2 * cfg["max_seq_len"] - 1).astype(np.float32))
         if rng.random() < 0.3:
             cfg["mask_type"] = 2              # no mask: every tile of a sequence sees all of K, no merged first tiles
+        if "pos_table" not in cfg and rng.random() < 0.35 and B * H * cfg["max_seq_len"] ** 2 <= 48_000_000:
+            m = cfg["max_seq_len"] = (cfg["max_seq_len"] + 7) // 8 * 8        # rows of the bias on 16-byte boundaries: the variant for a dense bias alone
+            cfg["attn_bias"] = torch.from_numpy(rng.normal(0, 0.5, (B, H, m, m)).astype(np.float32)).to(cfg["q"].dtype)
         say("self_scheduled_random", seed, it, B, H, d, kind, sum(lens), mx, cfg["max_seq_len"], cfg["mask_type"])
         out, name = T.run_capi(cfg)
         if not name.endswith("_selfsched"):          # K ranges split: few tiles, long sequences
