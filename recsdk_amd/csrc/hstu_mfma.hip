@@ -590,7 +590,8 @@ void hstu_mfma_kernel(const KArgs a, const unsigned* __restrict__ ws, const floa
         // every wave derives the record by itself: no exchange through LDS, no barrier
         __shared__ unsigned lds_hist[4 * 64];
         unsigned rv[REC];
-        self_record<EXTRA != 5>(a, (p.max_seq_len_q + BM - 1) / BM, lane, lds_hist + 64 * w, rv, owned_rows);
+        if (p.seq_offset_k == p.seq_offset_q) self_record<EXTRA != 5, false>(a, (p.max_seq_len_q + BM - 1) / BM, lane, lds_hist + 64 * w, rv, owned_rows);
+        else self_record<EXTRA != 5, true>(a, (p.max_seq_len_q + BM - 1) / BM, lane, lds_hist + 64 * w, rv, owned_rows);
 #pragma unroll
         for (int i = 0; i < REC; i++) rw[i] = __builtin_amdgcn_readfirstlane(rv[i]);
         // the record also goes where the schedule kernel would have put it, so that the caller's workspace holds the list
@@ -1525,7 +1526,8 @@ static int forward_extra(const KArgs& a) {
 
 // Launches without a schedule kernel (see SELF): the variants with the built-in mask or none and at most the bias tables
 // or a dense bias alone at head dims 64 and 128 (the plain and the dense-bias variants also at 32), one or two sequences per lane, at most 64 tile-count classes (63 tile counts and the class of longer
-// sequences), and lists that cannot overflow (q and k share their offsets, so entries per group fall along the order).
+// sequences), and lists that cannot overflow (entries per group follow the Q tiles alone and fall along the order; K offsets in a
+// tensor of their own are fine when q and k have as many rows in total, the sign of plain self-attention).
 // A caller that already holds a list (HSTU_FLAG_REUSE_WORKSPACE) keeps using it.
 bool mfma_self_scheduled(const KArgs& a) {
     const hstu_fwd_params& p = a.p;
@@ -1536,7 +1538,7 @@ bool mfma_self_scheduled(const KArgs& a) {
     const bool tables_too = p.dim_qk == 128 || p.dim_qk == 64;
     return a.op == OP_JAGGED && (p.dtype == HSTU_BF16 || p.dtype == HSTU_F16) && p.dim_qk == p.dim_v &&
            (p.dim_qk == 32 || p.dim_qk == 64 || p.dim_qk == 128) &&
-           p.batch >= 1 && p.batch <= 128 && p.seq_offset_q && p.seq_offset_q == p.seq_offset_k && !p.num_context &&
+           p.batch >= 1 && p.batch <= 128 && p.seq_offset_q && p.seq_offset_k && p.total_q == p.total_k && !p.num_context &&
            (p.mask_type == HSTU_MASK_TRIL || p.mask_type == HSTU_MASK_NONE) && (extra == 0 || extra == 5 || (tables_too && extra >= 2 && extra <= 4)) &&
            p.max_seq_len_q == p.max_seq_len_k && p.max_seq_len_q <= 63 * BM &&
            !(p.flags & HSTU_FLAG_REUSE_WORKSPACE) && sched_dims(p).nsplit == 1;

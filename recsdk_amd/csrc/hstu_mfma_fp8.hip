@@ -77,7 +77,8 @@ void hstu_mfma_fp8_kernel(const KArgs a, const unsigned* __restrict__ ws) {
     if constexpr (SELF) {
         __shared__ unsigned lds_hist[4 * 64];
         unsigned rv[WORK_RECORD_WORDS];
-        self_record(a, (p.max_seq_len_q + FBM - 1) / FBM, lane, lds_hist + 64 * w, rv, owned_rows);
+        if (p.seq_offset_k == p.seq_offset_q) self_record<true, false>(a, (p.max_seq_len_q + FBM - 1) / FBM, lane, lds_hist + 64 * w, rv, owned_rows);
+        else self_record<true, true>(a, (p.max_seq_len_q + FBM - 1) / FBM, lane, lds_hist + 64 * w, rv, owned_rows);
 #pragma unroll
         for (int i = 0; i < WORK_RECORD_WORDS; i++) rw[i] = __builtin_amdgcn_readfirstlane(rv[i]);
         if (tid < WORK_RECORD_WORDS) {
@@ -366,7 +367,7 @@ uint64_t mfma_fp8_workspace_bytes(const KArgs& a) { return work_list_shape(a.p).
 // launches without the schedule kernel: the conditions of the 16-bit kernels (mfma_self_scheduled)
 bool mfma_fp8_self_scheduled(const KArgs& a) {
     const hstu_fwd_params& p = a.p;
-    return a.op == OP_JAGGED && p.batch >= 1 && p.batch <= 128 && p.seq_offset_q && p.seq_offset_q == p.seq_offset_k && !p.num_context &&
+    return a.op == OP_JAGGED && p.batch >= 1 && p.batch <= 128 && p.seq_offset_q && p.seq_offset_k && p.total_q == p.total_k && !p.num_context &&
            (p.mask_type == HSTU_MASK_TRIL || p.mask_type == HSTU_MASK_NONE) && p.max_seq_len_q == p.max_seq_len_k && p.max_seq_len_q <= 63 * FBM &&
            !(p.flags & HSTU_FLAG_REUSE_WORKSPACE);
 }

@@ -23,7 +23,7 @@ __device__ __forceinline__ unsigned small_div(unsigned x, unsigned y) {
 }
 
 // The record of workgroup blockIdx.x without a work list, computed by one wave on its own (the caller guarantees
-// batch <= 128, at most 63 Q tiles per sequence under the attribute, one set of offsets for q and k, no context rows, the
+// batch <= 128, at most 63 Q tiles per sequence under the attribute, the same attribute for q and k, no context rows, the
 // built-in causal mask or no mask; target rows are fine).  The order is the schedule kernel's with a coarser key: sequences by
 // their number of Q tiles (longest first, then by batch index), (sequence, head) groups r = rank * heads + head dealt to
 // the XCDs in snake order (XCD x owns r = 16 u + x and 16 u + 15 - x), a group's tiles last tile first (the tiles of four
@@ -34,7 +34,7 @@ __device__ __forceinline__ unsigned small_div(unsigned x, unsigned y) {
 // entries.
 constexpr int SELF_TILE_ROWS = 128;
 
-template <bool FOUR_STREAMS = true>
+template <bool FOUR_STREAMS = true, bool OWN_K = false>
 __device__ __forceinline__ void self_record(const KArgs& a, int ntiles_attr, int lane, unsigned* hist, unsigned (&rec)[WORK_RECORD_WORDS], int64_t& rows) {
     const hstu_fwd_params& p = a.p;
     const int B = p.batch, H = p.heads_q;
@@ -45,6 +45,10 @@ __device__ __forceinline__ void self_record(const KArgs& a, int ntiles_attr, int
     const int cmax = ntiles_attr + 1;
     int64_t o0[2], o1[2];
     int len[2], cls[2], tgt[2];
+    // OWN_K: the K offsets are a tensor of their own (the order follows the Q tiles either way; the record carries the K
+    // range).  A template argument, chosen by the caller ahead of everything: a test down here would split the loads below
+    // into two round trips, and loading them always costs the common case 0.4 us per call.
+    unsigned ks[OWN_K ? 2 : 1], kl[OWN_K ? 2 : 1];
 #pragma unroll
     for (int u = 0; u < 2; u++) {
         const bool mine = lane + 64 * u < B;
@@ -52,9 +56,17 @@ __device__ __forceinline__ void self_record(const KArgs& a, int ntiles_attr, int
         if (is64) {
             const I64x2 v = *reinterpret_cast<const I64x2*>(static_cast<const int64_t*>(p.seq_offset_q) + mb);
             o0[u] = v.lo; o1[u] = v.hi;
+            if constexpr (OWN_K) {
+                const I64x2 kv = *reinterpret_cast<const I64x2*>(static_cast<const int64_t*>(p.seq_offset_k) + mb);
+                ks[u] = (unsigned)kv.lo; kl[u] = (unsigned)(kv.hi - kv.lo);
+            }
         } else {
             const I32x2 v = *reinterpret_cast<const I32x2*>(static_cast<const int*>(p.seq_offset_q) + mb);
             o0[u] = v.lo; o1[u] = v.hi;
+            if constexpr (OWN_K) {
+                const I32x2 kv = *reinterpret_cast<const I32x2*>(static_cast<const int*>(p.seq_offset_k) + mb);
+                ks[u] = (unsigned)kv.lo; kl[u] = (unsigned)(kv.hi - kv.lo);
+            }
         }
         tgt[u] = p.num_target ? (int)ld_idx(p.num_target, mb, is64) : 0;
     }
@@ -134,12 +146,17 @@ __device__ __forceinline__ void self_record(const KArgs& a, int ntiles_attr, int
     const unsigned q0 = (unsigned)__builtin_amdgcn_readlane((int)(second ? o0[1] : o0[0]), fl);
     const unsigned lq = (unsigned)__builtin_amdgcn_readlane(second ? len[1] : len[0], fl);
     const unsigned tg = (unsigned)__builtin_amdgcn_readlane(second ? tgt[1] : tgt[0], fl);
+    unsigned k0 = q0, lk = lq;
+    if constexpr (OWN_K) {
+        k0 = (unsigned)__builtin_amdgcn_readlane((int)(second ? ks[1] : ks[0]), fl);
+        lk = (unsigned)__builtin_amdgcn_readlane((int)(second ? kl[1] : kl[0]), fl);
+    }
     const unsigned fb = (unsigned)fl + (second ? 64u : 0u);
     const bool sw = found_cls > ntiles_attr, pr = pairs && !sw && found_cls >= 5;
     const bool both = pr && found_i == found_e - 1;
     const unsigned tile = both ? 0u : (found_e - 1 - found_i) + (pr ? 1u : 0u), part = both ? 1u : 0u;
     rec[0] = fb | h << 12 | tile << 16 | ((found_i == 0 && sw) ? 1u << 24 : 0u) | part << 25 | 1u << 28;
-    rec[1] = q0; rec[2] = lq; rec[3] = q0; rec[4] = lq; rec[5] = 0u; rec[6] = tg; rec[7] = 0u;
+    rec[1] = q0; rec[2] = lq; rec[3] = k0; rec[4] = lk; rec[5] = 0u; rec[6] = tg; rec[7] = 0u;
 }
 
 }  // namespace hstu

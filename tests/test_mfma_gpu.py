@@ -621,6 +621,30 @@ def test_self_scheduled_random_geometries_match_the_list_driven_launch(seed):
     assert taken >= 40, taken
 
 
+def test_self_scheduled_with_k_offsets_in_a_tensor_of_their_own():
+    """Callers that pass seq_offset_k next to seq_offset_q (the reference's second-generation op always does) with as many
+    K rows as Q rows in total also run without the schedule kernel: same bits as with one tensor for both, and, when the
+    totals agree but the sequences differ, every row as the plain kernel computes it."""
+    say("self_scheduled_own_k_offsets")
+    dtype = torch.bfloat16
+    lens = [700, 0, 129, 513, 64, 300]
+    cfg, _ = _jag(88, lens, 4, 4, 128, 128, dtype)
+    out0, name0 = T.run_capi(cfg)
+    own = dict(cfg, seq_offset_k=cfg["seq_offset"].clone(), max_seq_len_k=cfg["max_seq_len"])
+    out1, name1 = T.run_capi(own)
+    assert name0.endswith("_selfsched") and name1.endswith("_selfsched"), (name0, name1)
+    assert torch.equal(out0, out1)
+    again, _ = T.run_capi(own, reuse_from=own)
+    assert torch.equal(out1, again)
+    cfg3, _ = _jag(89, [300, 100, 513, 8], 4, 4, 128, 128, dtype, lens_k=[100, 513, 300, 8])
+    out3, name3 = T.run_capi(cfg3)
+    assert name3.endswith("_selfsched"), name3
+    gen, _ = T.run_capi(cfg3, flags=FORCE_GENERIC)
+    assert torch.equal(torch.isnan(out3), torch.isnan(gen))
+    T.assert_parity(torch.nan_to_num(out3.float()).to(dtype), torch.nan_to_num(gen.float()), dtype, what="own K offsets, other lengths vs generic kernel")
+    T.assert_parity(torch.nan_to_num(out3.float()).to(dtype), torch.nan_to_num(T.oracle_jagged(cfg3).float()), dtype, what="own K offsets, other lengths vs oracle")
+
+
 def test_self_scheduling_is_left_to_the_work_list_where_it_does_not_apply():
     say("self_scheduled: not taken")
     dtype = torch.bfloat16
