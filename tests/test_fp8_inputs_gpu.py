@@ -235,3 +235,21 @@ def test_fp8_self_derived_launches_match_the_list_driven_launch_on_random_batche
         assert torch.equal(torch.isnan(out), torch.isnan(listed)), "other rows produced"
         assert torch.equal(torch.nan_to_num(out.float()), torch.nan_to_num(listed.float())), "other bits than over the schedule kernel's list"
     assert taken >= 40, taken
+
+
+@pytest.mark.parametrize("d", [64, 128, 256])
+def test_fp8_self_derived_launch_with_k_offsets_in_a_tensor_of_their_own(d):
+    """seq_offset_k given next to seq_offset_q with as many K rows in total: still no schedule kernel; same bits as with one
+    tensor for both, and with other lengths per sequence the plain kernel's rows."""
+    say("fp8_self_derived_own_k_offsets", d)
+    cfg, _ = _jag8(7, [700, 0, 129, 513, 64, 300], 4, 4, d, d, silu_scale=1.0 / 64)
+    out0, name0 = T.run_capi(cfg)
+    out1, name1 = T.run_capi(dict(cfg, seq_offset_k=cfg["seq_offset"].clone(), max_seq_len_k=cfg["max_seq_len"]))
+    assert name0.endswith("_selfsched") and name1.endswith("_selfsched"), (name0, name1)
+    assert torch.equal(out0, out1)
+    c3, _ = _jag8(8, [300, 100, 513, 8], 4, 4, d, d, lens_k=[100, 513, 300, 8], silu_scale=1.0 / 64)
+    out3, name3 = T.run_capi(c3)
+    assert name3.endswith("_selfsched"), name3
+    gen, gname = T.run_capi(c3, flags=FORCE_GENERIC)
+    assert gname == "generic_fp8"
+    _close(out3, gen, "fp8, own K offsets, other lengths: matrix-core vs plain kernel")
